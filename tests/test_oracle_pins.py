@@ -1,0 +1,432 @@
+"""Pins the CPU oracle (oracle/evo_oracle.c) without running the reference.
+
+The reference holds no golden vectors for this path (its tests are behavioural), so the
+oracle is anchored on: brute-force numpy re-derivations on small inputs (tests/brute.py),
+closed forms, the invariants the reference's own tests state (test/predict-leaf-idx.jl:25-49,
+test/metrics.jl:160-204, docs/src/overview.md tie rule) and hand-built edge cases chosen so
+that a dropped term, a wrong inequality or a transposed index fails.
+"""
+import numpy as np
+import pytest
+
+import brute
+from oracle import oracle as orc
+
+
+def make_data(seed, N, F, nbins, loss="mse", weights=False):
+    rng = np.random.default_rng(seed)
+    x_bin = rng.integers(1, nbins + 1, size=(F, N), dtype=np.uint8)
+    K = 2 if loss == "gaussian_mle" else 1
+    NK = 2 * K + 1
+    y = rng.random(N).astype(np.float32)
+    if loss == "logloss":
+        y = (y > 0.5).astype(np.float32)
+    pred = (rng.standard_normal((N, K)) * 0.3).astype(np.float32)
+    grad = np.zeros((N, NK), np.float32)
+    grad[:, NK - 1] = (rng.random(N).astype(np.float32) + 0.5) if weights else 1.0
+    return x_bin, y, pred, grad
+
+
+def trees_equal_struct(t, T):
+    return (np.array_equal(t.feat, T["feat"]) and np.array_equal(t.cond_bin, T["cond_bin"])
+            and np.array_equal(t.split, T["split"]))
+
+
+# ---------------------------------------------------------------- gradients
+def test_grads_mse_closed_form():
+    x_bin, y, pred, grad = make_data(1, 500, 3, 8, weights=True)
+    p = orc.make_params("mse")
+    w = grad[:, 2].copy()
+    orc.update_grads(p, pred, y, grad)
+    assert np.array_equal(grad[:, 0], (np.float32(2) * (pred[:, 0] - y)) * w)
+    assert np.array_equal(grad[:, 1], np.float32(2) * w)
+    assert np.array_equal(grad[:, 2], w)  # the weight row is only read
+
+
+def test_grads_logloss_vs_float64():
+    x_bin, y, pred, grad = make_data(2, 500, 3, 8, loss="logloss", weights=True)
+    p = orc.make_params("logloss")
+    w = grad[:, 2].astype(np.float64)
+    orc.update_grads(p, pred, y, grad)
+    s = 1.0 / (1.0 + np.exp(-pred[:, 0].astype(np.float64)))
+    np.testing.assert_allclose(grad[:, 0], (s - y) * w, rtol=0, atol=2e-7)
+    np.testing.assert_allclose(grad[:, 1], s * (1 - s) * w, rtol=2e-6)
+
+
+def test_grads_gaussian_fisher_and_finite_difference():
+    # test/metrics.jl:160-204: -d(logpdf)/d(loc) == g1, -d(logpdf)/d(raw) == g2, Fisher hessians
+    # 1/scale^2 and 2 (sigmoid(raw)/scale)^2 do not depend on the residual; link is softplus.
+    def lpdf(yv, loc, raw):
+        scale = np.log1p(np.exp(raw))
+        return -(np.log(scale) + (yv - loc) ** 2 / (2 * scale ** 2))
+
+    p = orc.make_params("gaussian_mle")
+    cases = [(0.5, 0.3, 1.5), (0.5, 0.3, 4.0), (-1.0, -0.7, -3.0), (0.0, 1.2, 0.0)]
+    N = len(cases)
+    pred = np.array([[c[0], c[1]] for c in cases], np.float32)
+    y = np.array([c[2] for c in cases], np.float32)
+    grad = np.zeros((N, 5), np.float32)
+    grad[:, 4] = 1.0
+    orc.update_grads(p, pred, y, grad)
+    h = 1e-6
+    for i, (loc, raw, yv) in enumerate(cases):
+        loc, raw, yv = float(np.float32(loc)), float(np.float32(raw)), float(np.float32(yv))
+        dloc = (lpdf(yv, loc + h, raw) - lpdf(yv, loc - h, raw)) / (2 * h)
+        draw = (lpdf(yv, loc, raw + h) - lpdf(yv, loc, raw - h)) / (2 * h)
+        assert abs(-dloc - grad[i, 0]) < 2e-5 * max(1, abs(dloc))
+        assert abs(-draw - grad[i, 1]) < 2e-5 * max(1, abs(draw))
+        scale = np.log1p(np.exp(raw))
+        ds = 1 / (1 + np.exp(-raw))
+        np.testing.assert_allclose(grad[i, 2], 1 / scale ** 2, rtol=1e-5)
+        np.testing.assert_allclose(grad[i, 3], 2 * (ds / scale) ** 2, rtol=1e-5)
+    # cases 0 and 1 share (loc, raw): hessians identical although residuals differ
+    assert grad[0, 2] == grad[1, 2] and grad[0, 3] == grad[1, 3]
+
+
+def test_grads_gaussian_weight_scales_all_rows():
+    p = orc.make_params("gaussian_mle")
+    pred = np.array([[0.2, -0.4]] * 2, np.float32)
+    y = np.array([1.0, 1.0], np.float32)
+    grad = np.zeros((2, 5), np.float32)
+    grad[:, 4] = [1.0, 3.0]
+    orc.update_grads(p, pred, y, grad)
+    np.testing.assert_allclose(grad[1, :4], 3 * grad[0, :4], rtol=1e-6)
+
+
+# ---------------------------------------------------------------- binarize / subsample
+def test_binarize_searchsortedfirst():
+    rng = np.random.default_rng(3)
+    edges = np.sort(rng.random(15))
+    x = np.concatenate([rng.random(200), edges, [-1.0, 2.0]])  # values equal to an edge go to that edge's bin
+    got = orc.binarize(x, edges)
+    want = np.searchsorted(edges, x, side="left") + 1
+    assert np.array_equal(got, want.astype(np.uint8))
+    assert got.min() >= 1 and got.max() <= 16
+
+
+def test_subsample_threshold_rule():
+    mask = np.arange(256, dtype=np.uint8)
+    # src/subsample.jl:9: cond = round(UInt8, 255*rowsample), half-to-even: 0.5 -> 128
+    cond = int(np.rint(255 * 0.5))
+    assert cond == 128
+    got = orc.subsample(mask, cond)
+    assert np.array_equal(got, np.arange(129, dtype=np.uint32))
+    assert orc.subsample(mask, 255).shape[0] == 256
+    assert orc.subsample(np.full(10, 7, np.uint8), 3).shape[0] == 0
+
+
+# ---------------------------------------------------------------- histogram
+@pytest.mark.parametrize("loss,weights", [("mse", False), ("mse", True), ("logloss", True), ("gaussian_mle", False)])
+def test_hist_against_dense_bruteforce_and_invariants(loss, weights):
+    N, F, B, D = 700, 5, 8, 4
+    x_bin, y, pred, grad = make_data(10, N, F, B, loss, weights)
+    p = orc.make_params(loss, nbins=B, max_depth=D, min_weight=1.0)
+    orc.update_grads(p, pred, y, grad)
+    rng = np.random.default_rng(11)
+    rows = np.sort(rng.choice(N, 500, replace=False)).astype(np.uint32)
+    js = np.array([1, 2, 4, 5], np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t, nidx = o.grow_tree(grad, rows, js, mode=0)
+    H = o.hist()
+    S = o.node_sums()
+    K, NK = p.K, 2 * p.K + 1
+    # walk the tree the oracle produced; every split node's histogram must equal the dense one of its rows
+    label = np.zeros(N, np.int64)
+    label[rows] = 1
+    checked = 0
+    for n in range(1, 2 ** (D - 1)):
+        if not t.split[n - 1]:
+            continue
+        r = np.flatnonzero(label == n)
+        dense = brute.dense_hist(x_bin, grad, r, B)
+        for j in js:
+            np.testing.assert_allclose(H[n - 1, j - 1], dense[j - 1], rtol=1e-12, atol=1e-12)
+            # sum over bins == node sums, for every sampled feature
+            np.testing.assert_allclose(H[n - 1, j - 1].sum(axis=0), S[n], rtol=1e-11, atol=1e-11)
+            if not weights:
+                cnt = np.bincount(x_bin[j - 1, r].astype(np.int64) - 1, minlength=B)
+                assert np.array_equal(H[n - 1, j - 1][:, NK - 1], cnt.astype(np.float64))
+        f, b = int(t.feat[n - 1]), int(t.cond_bin[n - 1])
+        go = x_bin[f - 1, r] <= b
+        label[r[go]] = 2 * n
+        label[r[~go]] = 2 * n + 1
+        checked += 1
+        # parent == left + right wherever both children were scanned
+        if 2 * n + 1 < 2 ** (D - 1) and (t.split[2 * n - 1] or t.split[2 * n]):
+            for j in js:
+                np.testing.assert_allclose(H[n - 1, j - 1], H[2 * n - 1, j - 1] + H[2 * n, j - 1], rtol=1e-11, atol=1e-11)
+    assert checked >= 3
+    o.close()
+
+
+# ---------------------------------------------------------------- split search / full tree vs brute force
+@pytest.mark.parametrize("loss,weights,lam,gamma,minw", [
+    ("mse", False, 0.0, 0.0, 1.0),
+    ("mse", True, 0.5, 0.1, 2.0),
+    ("logloss", False, 0.0, 0.0, 1.0),
+    ("logloss", True, 0.3, 0.0, 1.0),
+    ("gaussian_mle", False, 0.0, 0.0, 8.0),
+    ("gaussian_mle", True, 0.2, 0.05, 4.0),
+])
+def test_tree_against_bruteforce(loss, weights, lam, gamma, minw):
+    N, F, B, D = 900, 6, 16, 5
+    x_bin, y, pred, grad = make_data(20, N, F, B, loss, weights)
+    p = orc.make_params(loss, nbins=B, max_depth=D, lambda_=lam, gamma=gamma, min_weight=minw, eta=0.3)
+    orc.update_grads(p, pred, y, grad)
+    rng = np.random.default_rng(21)
+    rows = np.sort(rng.choice(N, 640, replace=False)).astype(np.uint32)
+    js = np.array([1, 3, 4, 6], np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t, nidx = o.grow_tree(grad, rows, js, mode=0)
+    T, label, hists, sums = brute.grow(x_bin, grad, rows, js, p.K, B, D, eta=0.3, lam=lam, L2=1.0, gamma=gamma, min_weight=minw)
+    assert trees_equal_struct(t, T)
+    assert t.split.sum() >= 3
+    np.testing.assert_allclose(t.gain, T["gain"], rtol=1e-5)
+    np.testing.assert_allclose(t.pred, T["pred"], rtol=1e-5, atol=1e-9)
+    np.testing.assert_allclose(t.w, T["w"], rtol=1e-6)
+    assert np.array_equal(nidx.astype(np.int64), label)  # node each sampled row ends in; 0 for unsampled rows
+    o.close()
+
+
+def test_root_gain_closed_form_unit_weights():
+    # w == 1, lambda == 0, mse => h = 2n: gain = GL^2/(2(2nL+L2)) + GR^2/(2(2nR+L2)) - G^2/(2(2n+L2))
+    N, F, B = 400, 3, 8
+    x_bin, y, pred, grad = make_data(30, N, F, B)
+    p = orc.make_params("mse", nbins=B, max_depth=2, L2=1.0)
+    orc.update_grads(p, pred, y, grad)
+    rows = np.arange(N, dtype=np.uint32)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t, _ = o.grow_tree(grad, rows, js)
+    g = grad[:, 0].astype(np.float64)
+    best = (-1.0, 0, 0)
+    for j in range(F):
+        for b in range(1, B):
+            L = x_bin[j] <= b
+            nL, nR = L.sum(), N - L.sum()
+            if not (nL > 1.0 and nR > 1.0):
+                continue
+            GL, GR, G = g[L].sum(), g[~L].sum(), g.sum()
+            gain = GL ** 2 / (2 * (2 * nL + 1)) + GR ** 2 / (2 * (2 * nR + 1)) - G ** 2 / (2 * (2 * N + 1))
+            if gain > best[0]:
+                best = (gain, j + 1, b)
+    assert (int(t.feat[0]), int(t.cond_bin[0])) == best[1:]
+    np.testing.assert_allclose(t.gain[0], best[0], rtol=1e-6)
+    # leaf value closed form and w == row count
+    for child in (2, 3):
+        sel = (x_bin[best[1] - 1] <= best[2]) if child == 2 else (x_bin[best[1] - 1] > best[2])
+        assert t.w[child - 1] == sel.sum()
+        np.testing.assert_allclose(t.pred[child - 1, 0], -0.1 * g[sel].sum() / (2 * sel.sum() + 1.0), rtol=1e-6)
+    o.close()
+
+
+def test_tie_rule_duplicate_columns_and_empty_bins():
+    # "the first one will be selected": duplicated columns give identical gains -> earliest feature in js;
+    # an empty bin repeats the previous cumulative sums -> identical gain -> lowest bin wins.
+    N, B = 300, 16
+    rng = np.random.default_rng(40)
+    col = rng.integers(1, B + 1, N).astype(np.uint8)
+    col[col == 7] = 8  # bin 7 empty: candidates at bin 6 and 7 have the same left set
+    noise = rng.integers(1, B + 1, N).astype(np.uint8)
+    x_bin = np.stack([noise, col, col.copy(), col.copy()])
+    y = (col > 6).astype(np.float32) + 0.01 * rng.random(N).astype(np.float32)
+    pred = np.zeros((N, 1), np.float32)
+    grad = np.zeros((N, 3), np.float32)
+    grad[:, 2] = 1
+    p = orc.make_params("mse", nbins=B, max_depth=2)
+    orc.update_grads(p, pred, y, grad)
+    rows = np.arange(N, dtype=np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t, _ = o.grow_tree(grad, rows, np.array([1, 2, 3, 4], np.uint32))
+    assert (int(t.feat[0]), int(t.cond_bin[0])) == (2, 6)
+    t, _ = o.grow_tree(grad, rows, np.array([1, 3, 4], np.uint32))
+    assert (int(t.feat[0]), int(t.cond_bin[0])) == (3, 6)
+    o.close()
+
+
+def test_min_weight_is_strict_and_gamma_is_strict():
+    # 4 rows, one feature: the only balanced split has w_l == w_r == 2.
+    x_bin = np.array([[1, 1, 2, 2]], np.uint8)
+    grad = np.array([[-1, 2, 1], [-1, 2, 1], [1, 2, 1], [1, 2, 1]], np.float32)
+    rows = np.arange(4, dtype=np.uint32)
+    js = np.array([1], np.uint32)
+    for minw, expect in [(1.999, 1), (2.0, 0), (2.5, 0)]:
+        p = orc.make_params("mse", nbins=4, max_depth=2, min_weight=minw)
+        o = orc.Oracle(p, x_bin)
+        t, _ = o.grow_tree(grad, rows, js)
+        assert int(t.split[0]) == expect, minw
+        o.close()
+    # gain of that split: 2 * (2^2 / (4+1) / 2) - 0 = 0.8 ; accepted only if gain > gamma
+    for gamma, expect in [(0.79, 1), (0.8, 0), (0.9, 0)]:
+        p = orc.make_params("mse", nbins=4, max_depth=2, min_weight=1.0, gamma=gamma)
+        o = orc.Oracle(p, x_bin)
+        t, _ = o.grow_tree(grad, rows, js)
+        assert int(t.split[0]) == expect, gamma
+        if expect:
+            np.testing.assert_allclose(t.gain[0], 0.8, rtol=1e-6)
+        o.close()
+
+
+def test_numeric_scan_excludes_last_bin_uses_nbins_param():
+    # all rows in bins {B-1, B}: the only separating split is at bin B-1 (allowed, <= B-1)
+    B = 8
+    x_bin = np.array([[B - 1] * 5 + [B] * 5], np.uint8)
+    grad = np.zeros((10, 3), np.float32)
+    grad[:, 2] = 1
+    grad[:, 1] = 2
+    grad[:5, 0] = -1
+    grad[5:, 0] = 1
+    p = orc.make_params("mse", nbins=B, max_depth=2)
+    o = orc.Oracle(p, x_bin)
+    t, _ = o.grow_tree(grad, np.arange(10, dtype=np.uint32), np.array([1], np.uint32))
+    assert int(t.cond_bin[0]) == B - 1 and t.split[0] == 1
+    o.close()
+
+
+def test_categorical_and_monotone_against_bruteforce():
+    N, F, B, D = 800, 4, 8, 4
+    x_bin, y, pred, grad = make_data(50, N, F, B, "mse", True)
+    y = (y + 0.3 * (x_bin[0] / B)).astype(np.float32)
+    feattypes = np.array([1, 0, 1, 0], np.uint8)
+    mono = np.array([1, 0, -1, 0], np.int32)
+    p = orc.make_params("mse", nbins=B, max_depth=D)
+    orc.update_grads(p, pred, y, grad)
+    rows = np.arange(N, dtype=np.uint32)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    o = orc.Oracle(p, x_bin, feattypes, mono)
+    t, nidx = o.grow_tree(grad, rows, js)
+    T, label, _, _ = brute.grow(x_bin, grad, rows, js, 1, B, D, feattypes=feattypes, mono=mono)
+    assert trees_equal_struct(t, T)
+    assert any(t.split[n] and feattypes[t.feat[n] - 1] == 0 for n in range(len(t.split)))
+    assert np.array_equal(nidx.astype(np.int64), label)
+    for i in (0, 6, 122, N - 1):
+        assert brute.walk(x_bin, feattypes, T, i) == nidx[i]
+    o.close()
+
+
+# ---------------------------------------------------------------- node index / traversal / predict
+def test_nidx_equals_independent_walk_and_leaves_are_not_split():
+    N, F, B, D = 1000, 5, 16, 5
+    x_bin, y, pred, grad = make_data(60, N, F, B)
+    p = orc.make_params("mse", nbins=B, max_depth=D, eta=0.2)
+    orc.update_grads(p, pred, y, grad)
+    rows = np.arange(N, dtype=np.uint32)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t, nidx = o.grow_tree(grad, rows, js)
+    ft = np.ones(F, np.uint8)
+    T = dict(feat=t.feat, cond_bin=t.cond_bin, split=t.split)
+    leaf = orc.predict_leaf_idx(x_bin, ft, t)
+    for i in range(N):
+        assert brute.walk(x_bin, ft, T, i) == leaf[i]
+    assert np.array_equal(leaf, nidx)
+    assert not t.split[leaf - 1].any()
+    # stable partition property: rows of each node, in the oracle's work buffer order, are ascending
+    before = pred.copy()
+    o.predict_tree(t, pred)
+    np.testing.assert_array_equal(pred[:, 0], before[:, 0] + t.pred[leaf - 1, 0])
+    o.close()
+
+
+def test_max_depth_one_is_a_single_leaf():
+    N, F, B = 200, 3, 8
+    x_bin, y, pred, grad = make_data(61, N, F, B)
+    p = orc.make_params("mse", nbins=B, max_depth=1)
+    orc.update_grads(p, pred, y, grad)
+    o = orc.Oracle(p, x_bin)
+    t, nidx = o.grow_tree(grad, np.arange(N, dtype=np.uint32), np.arange(1, F + 1, dtype=np.uint32))
+    assert t.split.shape == (1,) and t.split[0] == 0 and (nidx == 1).all()
+    g = grad[:, 0].astype(np.float64).sum()
+    np.testing.assert_allclose(t.pred[0, 0], -0.1 * g / (2 * N + 1.0), rtol=1e-6)
+    o.close()
+
+
+def test_predict_clamps():
+    x_bin = np.array([[1, 2, 2]], np.uint8)
+    ft = np.ones(1, np.uint8)
+    t = orc.Tree(1, 3)
+    t.feat[0], t.cond_bin[0], t.split[0] = 1, 1, 1
+    t.pred[1, 0], t.pred[2, 0] = 20.0, -20.0
+    pred = np.array([[1.0], [1.0], [-14.0]], np.float32)
+    orc.predict_tree(orc.LOSS_IDS["logloss"], 1, x_bin, ft, t, pred)
+    assert pred[:, 0].tolist() == [15.0, -15.0, -15.0]
+    pred = np.array([[1.0], [1.0], [-14.0]], np.float32)
+    orc.predict_tree(orc.LOSS_IDS["mse"], 1, x_bin, ft, t, pred)
+    assert pred[:, 0].tolist() == [21.0, -19.0, -34.0]
+    t2 = orc.Tree(2, 3)
+    t2.feat[0], t2.cond_bin[0], t2.split[0] = 1, 1, 1
+    t2.pred[1] = [100.0, 100.0]
+    t2.pred[2] = [-100.0, -100.0]
+    pred = np.zeros((3, 2), np.float32)
+    orc.predict_tree(orc.LOSS_IDS["gaussian_mle"], 2, x_bin, ft, t2, pred)
+    assert pred.tolist() == [[100.0, 100.0], [-100.0, -15.0], [-100.0, -15.0]]  # only the scale row has a floor
+    # link: sigmoid for logloss, softplus on the scale row only (test/metrics.jl:200-204)
+    pr = np.array([[0.0, -2.0], [1.0, 0.5]], np.float32)
+    orc.apply_link(orc.LOSS_IDS["gaussian_mle"], 2, pr)
+    assert pr[:, 0].tolist() == [0.0, 1.0]
+    np.testing.assert_allclose(pr[:, 1], np.log1p(np.exp(np.array([-2.0, 0.5]))), rtol=1e-6)
+
+
+# ---------------------------------------------------------------- oblivious
+@pytest.mark.parametrize("loss", ["mse", "gaussian_mle"])
+def test_oblivious_against_bruteforce(loss):
+    N, F, B, D = 1500, 5, 8, 4
+    x_bin, y, pred, grad = make_data(70, N, F, B, loss)
+    y = (y + 0.5 * (x_bin[1] > 4) + 0.3 * (x_bin[3] > 2)).astype(np.float32)
+    p = orc.make_params(loss, nbins=B, max_depth=D, tree_type="oblivious", min_weight=4.0)
+    orc.update_grads(p, pred, y, grad)
+    rows = np.arange(N, dtype=np.uint32)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t, nidx = o.grow_tree(grad, rows, js)
+    T, label, _, _ = brute.grow(x_bin, grad, rows, js, p.K, B, D, min_weight=4.0, oblivious=True)
+    assert trees_equal_struct(t, T)
+    assert t.split[:3].all()
+    for d in range(D - 1):  # every split node of a depth shares (feat, bin, gain)
+        lvl = slice(2 ** d - 1, 2 ** (d + 1) - 1)
+        s = t.split[lvl].astype(bool)
+        if s.any():
+            assert s.all()
+            assert len(set(t.feat[lvl])) == 1 and len(set(t.cond_bin[lvl])) == 1 and len(set(t.gain[lvl])) == 1
+    np.testing.assert_allclose(t.gain, T["gain"], rtol=1e-5)
+    np.testing.assert_allclose(t.pred, T["pred"], rtol=1e-5, atol=1e-9)
+    assert np.array_equal(nidx.astype(np.int64), label)
+    o.close()
+
+
+# ---------------------------------------------------------------- fixed-point mode vs reference arithmetic
+@pytest.mark.parametrize("loss,weights", [("mse", False), ("logloss", True), ("gaussian_mle", False)])
+def test_fixed_point_mode_matches_f64_mode(loss, weights):
+    N, F, B, D = 3000, 8, 32, 6
+    x_bin, y, pred, grad = make_data(80, N, F, B, loss, weights)
+    p = orc.make_params(loss, nbins=B, max_depth=D)
+    orc.update_grads(p, pred, y, grad)
+    rows = np.arange(N, dtype=np.uint32)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t0, n0 = o.grow_tree(grad, rows, js, mode=0)
+    H0 = o.hist().copy()
+    NK = 2 * p.K + 1
+    qbits = np.full(NK, 38, np.int32)
+    qbits[0] = 30
+    o.set_quant(grad, qbits)
+    qb, qe = o.get_quant()
+    for k in range(NK):
+        m = np.abs(grad[:, k]).max()
+        assert m < 2.0 ** qe[k] and (m == 0 or m >= 2.0 ** (qe[k] - 1))
+    t1, n1 = o.grow_tree(grad, rows, js, mode=1)
+    assert np.array_equal(t0.feat, t1.feat) and np.array_equal(t0.cond_bin, t1.cond_bin) and np.array_equal(t0.split, t1.split)
+    assert np.array_equal(n0, n1)
+    np.testing.assert_allclose(t1.gain, t0.gain, rtol=1e-5)
+    np.testing.assert_allclose(t1.pred, t0.pred, rtol=1e-5, atol=1e-9)
+    np.testing.assert_allclose(t1.w, t0.w, rtol=1e-6)
+    Hq = o.hist(fixed=True)
+    scale = np.ldexp(1.0, (qe - qb).astype(np.int64))
+    root = Hq[0].astype(np.float64) * scale
+    np.testing.assert_allclose(root, H0[0], rtol=0, atol=1e-5 * np.abs(grad).max())
+    # exact integer invariants of the fixed-point histogram
+    tot = Hq[0].sum(axis=1)
+    assert (tot == tot[0]).all()  # every feature's bins sum to the same node total, exactly
+    if t1.split[0]:
+        assert np.array_equal(Hq[0], Hq[1] + Hq[2])
+    o.close()
