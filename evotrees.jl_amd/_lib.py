@@ -1,0 +1,280 @@
+"""ctypes binding of libevotrees_hip.so (the C ABI declared in include/evotrees_hip.h).
+
+The library is mandatory: there is no CPU fallback.  Loading fails loudly when the shared
+object has not been built, and every compute entry point fails when no MI355X is visible.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libevotrees_hip.so")
+
+EVT_OK, EVT_ERR_ARG, EVT_ERR_HIP, EVT_ERR_STATE, EVT_ERR_EMPTY, EVT_ERR_NOMEM = 0, -1, -2, -3, -4, -5
+LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2}
+TREE_TYPES = {"binary": 0, "oblivious": 1}
+KERNEL_CLASSES = ["grad", "hist", "scan", "partition", "predict", "other"]
+
+# every symbol include/evotrees_hip.h declares
+EXPORTS = [
+    "evt_last_error", "evt_device_count", "evt_create", "evt_destroy", "evt_set_xbin", "evt_binarize_f64",
+    "evt_set_target", "evt_set_feature_meta", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
+    "evt_predict_tree", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
+    "evt_predict", "evt_predict_leaf_idx", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
+    "evt_set_option", "evt_synchronize", "evt_copy_bandwidth",
+]
+
+
+class EvtError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("libevotrees_hip error %d: %s" % (code, msg))
+        self.code = code
+
+
+class EvtParams(C.Structure):
+    _fields_ = [("eta", C.c_double), ("L2", C.c_double), ("lambda_", C.c_double), ("gamma", C.c_double),
+                ("min_weight", C.c_double), ("bagging_size", C.c_int32), ("update_pred", C.c_int32)]
+
+
+class EvtTreeOut(C.Structure):
+    _fields_ = [("feat", C.c_void_p), ("cond_bin", C.c_void_p), ("w", C.c_void_p), ("gain", C.c_void_p),
+                ("pred", C.c_void_p), ("split", C.c_void_p)]
+
+
+_lib = None
+
+
+def load():
+    """Loads the shared library (once).  Raises if it is missing: build it with
+    `python evotrees.jl_amd/build.py` (or `__graft_entry__.build()`)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("libevotrees_hip.so is not built (%s missing); run evotrees.jl_amd/build.py" % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    vp, i64, i32 = C.c_void_p, C.c_int64, C.c_int32
+    L.evt_last_error.restype = C.c_char_p
+    L.evt_last_error.argtypes = []
+    sigs = {
+        "evt_device_count": [vp],
+        "evt_create": [i64, i32, i32, i32, i32, i32, i32, vp],
+        "evt_destroy": [vp],
+        "evt_set_xbin": [vp, vp],
+        "evt_binarize_f64": [vp, vp, vp, vp],
+        "evt_set_target": [vp, vp, vp, vp, vp],
+        "evt_set_feature_meta": [vp, vp, vp],
+        "evt_update_grads": [vp],
+        "evt_set_grads": [vp, vp],
+        "evt_grow_tree": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams), C.POINTER(EvtTreeOut)],
+        "evt_predict_tree": [vp, i32, vp, vp, vp, vp],
+        "evt_get_pred": [vp, vp],
+        "evt_get_grads": [vp, vp],
+        "evt_get_nidx": [vp, vp],
+        "evt_get_hist": [vp, vp],
+        "evt_get_quant": [vp, vp, vp],
+        "evt_predict": [i64, i32, vp, vp, i32, i32, i32, vp, vp, vp, vp, vp, i32, vp],
+        "evt_predict_leaf_idx": [i64, i32, vp, vp, i32, vp, vp, vp, vp, vp],
+        "evt_set_profiling": [vp, i32],
+        "evt_get_profile": [vp, vp, vp, vp],
+        "evt_reset_profile": [vp],
+        "evt_set_option": [vp, C.c_char_p, i64],
+        "evt_synchronize": [vp],
+        "evt_copy_bandwidth": [i64, i32, vp],
+    }
+    for name, args in sigs.items():
+        f = getattr(L, name)
+        f.argtypes = args
+        f.restype = C.c_int
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != EVT_OK:
+        raise EvtError(rc, load().evt_last_error().decode("utf-8", "replace"))
+
+
+def ptr(a):
+    if a is None:
+        return None
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def device_count():
+    n = C.c_int32(0)
+    check(load().evt_device_count(C.byref(n)))
+    return n.value
+
+
+def copy_bandwidth(nbytes=1 << 30, iters=10):
+    out = C.c_double(0.0)
+    check(load().evt_copy_bandwidth(nbytes, iters, C.byref(out)))
+    return out.value
+
+
+class TreeArrays:
+    """Host arrays in the layout of Tree{L,K} (src/structs.jl:77-106)."""
+
+    def __init__(self, K, nnodes):
+        self.feat = np.zeros(nnodes, np.int64)
+        self.cond_bin = np.zeros(nnodes, np.uint8)
+        self.w = np.zeros(nnodes, np.float32)
+        self.gain = np.zeros(nnodes, np.float32)
+        self.pred = np.zeros((nnodes, K), np.float32)  # memory order of Julia's K x nnodes matrix
+        self.split = np.zeros(nnodes, np.uint8)
+
+    def as_out(self):
+        return EvtTreeOut(ptr(self.feat), ptr(self.cond_bin), ptr(self.w), ptr(self.gain), ptr(self.pred), ptr(self.split))
+
+
+class Handle:
+    """One training cache on the device (the reference's CacheGPU)."""
+
+    def __init__(self, nobs, nfeats, nbins, K, max_depth, loss, tree_type="binary"):
+        self._h = C.c_void_p(None)
+        self.N, self.F, self.B, self.K, self.D = int(nobs), int(nfeats), int(nbins), int(K), int(max_depth)
+        self.NK = 2 * self.K + 1
+        self.nnodes = (1 << self.D) - 1
+        self.loss = loss
+        check(load().evt_create(self.N, self.F, self.B, self.K, self.D, LOSS_IDS[loss], TREE_TYPES[tree_type], C.byref(self._h)))
+
+    def close(self):
+        if self._h:
+            load().evt_destroy(self._h)
+            self._h = C.c_void_p(None)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_xbin(self, x_bin_FN):
+        """x_bin_FN: (F, N) C-order uint8 == Julia's N x F column-major matrix."""
+        assert x_bin_FN.dtype == np.uint8 and x_bin_FN.flags.c_contiguous and x_bin_FN.shape == (self.F, self.N)
+        check(load().evt_set_xbin(self._h, ptr(x_bin_FN)))
+
+    def binarize(self, x_FN, edges):
+        """x_FN: (F, N) C-order float64; edges: list of F ascending float64 arrays."""
+        assert x_FN.dtype == np.float64 and x_FN.flags.c_contiguous and x_FN.shape == (self.F, self.N)
+        off = np.zeros(self.F + 1, np.int32)
+        off[1:] = np.cumsum([len(e) for e in edges])
+        flat = np.ascontiguousarray(np.concatenate([np.asarray(e, np.float64) for e in edges]))
+        check(load().evt_binarize_f64(self._h, ptr(x_FN), ptr(flat), ptr(off)))
+
+    def set_target(self, y, w, mu, offset=None):
+        y = np.ascontiguousarray(y, np.float32)
+        w = None if w is None else np.ascontiguousarray(w, np.float32)
+        mu = np.ascontiguousarray(mu, np.float32)
+        offset = None if offset is None else np.ascontiguousarray(offset, np.float32)
+        assert y.shape == (self.N,) and mu.shape == (self.K,)
+        check(load().evt_set_target(self._h, ptr(y), ptr(w), ptr(mu), ptr(offset)))
+
+    def set_feature_meta(self, feattypes=None, monotone=None):
+        ft = None if feattypes is None else np.ascontiguousarray(feattypes, np.uint8)
+        mo = None if monotone is None else np.ascontiguousarray(monotone, np.int32)
+        check(load().evt_set_feature_meta(self._h, ptr(ft), ptr(mo)))
+
+    def update_grads(self):
+        check(load().evt_update_grads(self._h))
+
+    def set_grads(self, grad):
+        grad = np.ascontiguousarray(grad, np.float32)
+        assert grad.shape == (self.N, self.NK)
+        check(load().evt_set_grads(self._h, ptr(grad)))
+
+    def grow_tree(self, js, params, mask=None, cond=255, want_tree=True):
+        js = np.ascontiguousarray(js, np.uint32)
+        if mask is not None:
+            mask = np.ascontiguousarray(mask, np.uint8)
+            assert mask.shape == (self.N,)
+        t = TreeArrays(self.K, self.nnodes) if want_tree else None
+        out = t.as_out() if want_tree else None
+        check(load().evt_grow_tree(self._h, ptr(mask), int(cond), ptr(js), js.shape[0], C.byref(params),
+                                   C.byref(out) if want_tree else None))
+        return t
+
+    def predict_tree(self, tree):
+        check(load().evt_predict_tree(self._h, tree.feat.shape[0], ptr(tree.feat), ptr(tree.cond_bin), ptr(tree.pred), ptr(tree.split)))
+
+    def get_pred(self):
+        out = np.empty((self.N, self.K), np.float32)
+        check(load().evt_get_pred(self._h, ptr(out)))
+        return out
+
+    def get_grads(self):
+        out = np.empty((self.N, self.NK), np.float32)
+        check(load().evt_get_grads(self._h, ptr(out)))
+        return out
+
+    def get_nidx(self):
+        out = np.empty(self.N, np.uint32)
+        check(load().evt_get_nidx(self._h, ptr(out)))
+        return out
+
+    def get_hist(self):
+        """[node, feature, bin, k] Float64 view of the reference's h∇[k, bin, feature, node]."""
+        out = np.empty((self.nnodes, self.F, self.B, self.NK), np.float64)
+        check(load().evt_get_hist(self._h, ptr(out)))
+        return out
+
+    def get_quant(self):
+        qb = np.zeros(self.NK, np.int32)
+        qe = np.zeros(self.NK, np.int32)
+        check(load().evt_get_quant(self._h, ptr(qb), ptr(qe)))
+        return qb, qe
+
+    def set_profiling(self, on):
+        check(load().evt_set_profiling(self._h, 1 if on else 0))
+
+    def reset_profile(self):
+        check(load().evt_reset_profile(self._h))
+
+    def get_profile(self):
+        n = len(KERNEL_CLASSES)
+        la = np.zeros(n, np.int64)
+        ms = np.zeros(n, np.float64)
+        un = np.zeros(n, np.int64)
+        check(load().evt_get_profile(self._h, ptr(la), ptr(ms), ptr(un)))
+        return {k: {"launches": int(la[i]), "ms": float(ms[i]), "units": int(un[i])} for i, k in enumerate(KERNEL_CLASSES)}
+
+    def set_option(self, name, value):
+        check(load().evt_set_option(self._h, name.encode(), int(value)))
+
+    def synchronize(self):
+        check(load().evt_synchronize(self._h))
+
+
+def make_params(eta=0.1, L2=1.0, lambda_=0.0, gamma=0.0, min_weight=1.0, bagging_size=1, update_pred=True):
+    return EvtParams(eta, L2, lambda_, gamma, min_weight, bagging_size, 1 if update_pred else 0)
+
+
+def predict_model(x_bin_FN, feattypes, loss, K, trees, apply_link=True):
+    """trees: list of objects with feat/cond_bin/pred/split arrays.  Returns (N, K) float32."""
+    F, N = x_bin_FN.shape
+    off = np.zeros(len(trees) + 1, np.int64)
+    off[1:] = np.cumsum([t.feat.shape[0] for t in trees])
+    feat = np.ascontiguousarray(np.concatenate([t.feat for t in trees]), np.int64)
+    cb = np.ascontiguousarray(np.concatenate([t.cond_bin for t in trees]), np.uint8)
+    sp = np.ascontiguousarray(np.concatenate([t.split for t in trees]), np.uint8)
+    pr = np.ascontiguousarray(np.concatenate([t.pred.reshape(-1, K) for t in trees]), np.float32)
+    ft = None if feattypes is None else np.ascontiguousarray(feattypes, np.uint8)
+    out = np.empty((N, K), np.float32)
+    check(load().evt_predict(N, F, ptr(x_bin_FN), ptr(ft), LOSS_IDS[loss], K, len(trees), ptr(off), ptr(feat), ptr(cb), ptr(pr),
+                             ptr(sp), 1 if apply_link else 0, ptr(out)))
+    return out
+
+
+def predict_leaf_idx(x_bin_FN, feattypes, trees):
+    F, N = x_bin_FN.shape
+    off = np.zeros(len(trees) + 1, np.int64)
+    off[1:] = np.cumsum([t.feat.shape[0] for t in trees])
+    feat = np.ascontiguousarray(np.concatenate([t.feat for t in trees]), np.int64)
+    cb = np.ascontiguousarray(np.concatenate([t.cond_bin for t in trees]), np.uint8)
+    sp = np.ascontiguousarray(np.concatenate([t.split for t in trees]), np.uint8)
+    ft = None if feattypes is None else np.ascontiguousarray(feattypes, np.uint8)
+    out = np.empty((len(trees), N), np.uint32)  # Julia: N x ntrees column-major
+    check(load().evt_predict_leaf_idx(N, F, ptr(x_bin_FN), ptr(ft), len(trees), ptr(off), ptr(feat), ptr(cb), ptr(sp), ptr(out)))
+    return out.T

@@ -1,0 +1,861 @@
+// C ABI of libevotrees_hip.so: handle lifecycle, uploads, the per-tree level loop, read-back.
+#include "evt_internal.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+#include <new>
+
+int launch_absmax_rows(evt_ctx *c, int k0, int k1);
+int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, const float *leaf_pred_dev);
+int launch_predict_model(hipStream_t s, const uint32_t *nodes, const float *leaf_pred, const int64_t *off, int ntrees, const uint8_t *xcm,
+                         const uint8_t *feattypes, int64_t N, int K, int loss, int apply_link, float *out);
+int launch_leaf_idx_model(hipStream_t s, const uint32_t *nodes, const int64_t *off, int ntrees, const uint8_t *xcm, const uint8_t *feattypes,
+                          int64_t N, uint32_t *out);
+
+static thread_local char g_err[512] = "";
+
+void evt_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char *evt_last_error(void) { return g_err; }
+
+extern "C" int evt_device_count(int32_t *count) {
+    ARGCHK(count, "count is NULL");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        *count = 0;
+        evt_set_error("no HIP device: %s", hipGetErrorString(e));
+        return EVT_ERR_HIP;
+    }
+    *count = n;
+    return EVT_OK;
+}
+
+// ---- profiling ------------------------------------------------------------------------------
+void prof_begin(evt_ctx *c, int cls, int level) {
+    if (!c->profiling) return;
+    ProfRec r;
+    r.cls = cls;
+    r.level = level;
+    auto get = [&]() {
+        hipEvent_t e;
+        if (!c->free_events.empty()) {
+            e = c->free_events.back();
+            c->free_events.pop_back();
+        } else {
+            (void)hipEventCreate(&e);
+        }
+        return e;
+    };
+    r.e0 = get();
+    r.e1 = get();
+    (void)hipEventRecord(r.e0, c->stream);
+    c->recs.push_back(r);
+}
+void prof_end(evt_ctx *c) {
+    if (!c->profiling || c->recs.empty()) return;
+    (void)hipEventRecord(c->recs.back().e1, c->stream);
+}
+// after a stream sync: fold finished event pairs into the per-class totals
+static void prof_collect(evt_ctx *c, const int64_t *stats_host) {
+    for (auto &r : c->recs) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, r.e0, r.e1) == hipSuccess) {
+            c->prof_launches[r.cls] += 1;
+            c->prof_ms[r.cls] += (double)ms;
+            if (r.cls == EVT_K_HIST && stats_host && r.level >= 1) c->prof_units[r.cls] += stats_host[r.level];
+        }
+        c->free_events.push_back(r.e0);
+        c->free_events.push_back(r.e1);
+    }
+    c->recs.clear();
+}
+
+template <typename T>
+static int dev_alloc(T **p, size_t n) {
+    *p = nullptr;
+    if (n == 0) n = 1;
+    hipError_t e = hipMalloc((void **)p, n * sizeof(T));
+    if (e != hipSuccess) {
+        evt_set_error("hipMalloc of %zu bytes failed: %s", n * sizeof(T), hipGetErrorString(e));
+        return EVT_ERR_NOMEM;
+    }
+    return EVT_OK;
+}
+#define ALLOC(ptr, n)                         \
+    do {                                      \
+        int _r = dev_alloc(&(ptr), (size_t)(n)); \
+        if (_r != EVT_OK) {                   \
+            evt_destroy(c);                   \
+            return _r;                        \
+        }                                     \
+    } while (0)
+
+static int record_stride(int F) {
+    if (F <= 16) return 16;
+    if (F <= 32) return 32;
+    if (F <= 64) return 64;
+    return ((F + 63) / 64) * 64;
+}
+
+static int ceil_log2_i64(int64_t v) {
+    int b = 0;
+    while (((int64_t)1 << b) < v) b++;
+    return b;
+}
+
+extern "C" int evt_destroy(evt_handle c) {
+    if (!c) return EVT_OK;
+    (void)hipSetDevice(c->device);
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
+                    c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree.feat, c->tree.cond_bin, c->tree.w, c->tree.gain,
+                    c->tree.pred, c->tree.split, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
+                    c->qscale, c->stats, c->errflag, c->ogains, c->obest};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    for (int l = 0; l < 2; l++) {
+        LevelTab &L = c->lvl[l];
+        void *lp[] = {L.hdr, L.act_node, L.cprefix, L.bnode, L.bstart, L.bprefix};
+        for (void *p : lp)
+            if (p) (void)hipFree(p);
+    }
+    if (c->h_stage) (void)hipHostFree(c->h_stage);
+    for (auto &r : c->recs) {
+        (void)hipEventDestroy(r.e0);
+        (void)hipEventDestroy(r.e1);
+    }
+    for (auto e : c->free_events) (void)hipEventDestroy(e);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    delete c;
+    return EVT_OK;
+}
+
+extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K, int32_t max_depth, int32_t loss, int32_t tree_type,
+                          evt_handle *out) {
+    ARGCHK(out, "out handle is NULL");
+    *out = nullptr;
+    ARGCHK(nobs >= 1 && nobs <= (int64_t)0xFFFFFFFFll, "nobs must be in [1, 2^32-1]");
+    ARGCHK(nfeats >= 1 && nfeats <= 1024, "nfeats must be in [1, 1024]");
+    ARGCHK(nbins >= 2 && nbins <= 255, "nbins must be in [2, 255]");
+    ARGCHK(max_depth >= 1 && max_depth <= EVT_MAX_DEPTH, "max_depth must be in [1, 16]");
+    ARGCHK(loss >= 0 && loss <= 2, "loss must be one of mse (0), logloss (1), gaussian_mle (2)");
+    ARGCHK(tree_type == EVT_TREE_BINARY || tree_type == EVT_TREE_OBLIVIOUS, "tree_type must be binary (0) or oblivious (1)");
+    ARGCHK(K == (loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1), "K must be 1 for mse/logloss and 2 for gaussian_mle");
+    int ndev = 0;
+    {
+        int r = evt_device_count(&ndev);
+        if (r != EVT_OK) return r;
+    }
+    evt_ctx *c = new (std::nothrow) evt_ctx();
+    if (!c) {
+        evt_set_error("out of host memory");
+        return EVT_ERR_NOMEM;
+    }
+    memset((void *)&c->device, 0, sizeof(int));
+    c->stream = nullptr;
+    c->N = nobs; c->F = nfeats; c->B = nbins; c->K = K; c->NK = 2 * K + 1; c->D = max_depth; c->loss = loss; c->tree_type = tree_type;
+    c->nnodes = (1 << max_depth) - 1;
+    c->maxlvl = 1 << (max_depth - 1);
+    c->RS = record_stride(nfeats);
+    c->LPR = c->RS / 16;
+    c->unit_w = true;
+    c->have_xbin = c->have_target = c->have_grads = false;
+    c->xcm = nullptr; c->xrm = nullptr; c->y = nullptr; c->pred = nullptr; c->grad = nullptr; c->gq = nullptr;
+    c->is_a = c->is_b = nullptr; c->nidx = nullptr; c->mask = nullptr; c->flagw = nullptr; c->chunk_nleft = nullptr; c->chunk_lpre = nullptr;
+    c->hist = nullptr; c->seg_start = c->seg_len = nullptr; c->status = nullptr; c->node_sum = nullptr;
+    memset(&c->tree, 0, sizeof(c->tree));
+    memset(c->lvl, 0, sizeof(c->lvl));
+    c->js = nullptr; c->jsmap = nullptr; c->feattypes = nullptr; c->mono = nullptr; c->absmax = nullptr; c->qexp = nullptr; c->qbits = nullptr;
+    c->qscale = nullptr; c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->obest = nullptr;
+    c->h_stage = nullptr; c->h_stage_bytes = 0;
+    c->n_js_last = 0;
+    c->last_all_rows = true;
+    c->hist_blocks = 512;
+    c->hist_threads = 1024;
+    c->profiling = false;
+    memset(c->prof_launches, 0, sizeof(c->prof_launches));
+    memset(c->prof_ms, 0, sizeof(c->prof_ms));
+    memset(c->prof_units, 0, sizeof(c->prof_units));
+    if (c->LPR > 64) {
+        delete c;
+        evt_set_error("nfeats too large for the record layout");
+        return EVT_ERR_ARG;
+    }
+    hipError_t e = hipGetDevice(&c->device);
+    if (e == hipSuccess) e = hipStreamCreate(&c->stream);
+    if (e != hipSuccess) {
+        evt_set_error("stream creation failed: %s", hipGetErrorString(e));
+        delete c;
+        return EVT_ERR_HIP;
+    }
+    const int64_t N = nobs;
+    const int NAgmax = c->NK; // upper bound over the weight modes
+    c->max_chunks = (N + EVT_CHUNK - 1) / EVT_CHUNK + c->maxlvl + 2;
+    ALLOC(c->xcm, (size_t)N * c->F);
+    ALLOC(c->xrm, (size_t)N * c->RS);
+    ALLOC(c->y, N);
+    ALLOC(c->pred, (size_t)N * K);
+    ALLOC(c->grad, (size_t)N * c->NK);
+    ALLOC(c->gq, (size_t)N * c->NK);
+    ALLOC(c->is_a, N);
+    ALLOC(c->is_b, N);
+    ALLOC(c->nidx, N);
+    ALLOC(c->mask, N);
+    ALLOC(c->flagw, (size_t)c->max_chunks * EVT_CHUNK_WORDS);
+    ALLOC(c->chunk_nleft, c->max_chunks + 1);
+    ALLOC(c->chunk_lpre, c->max_chunks + 1);
+    ALLOC(c->hist, (size_t)c->nnodes * c->F * NAgmax * c->B);
+    ALLOC(c->seg_start, c->nnodes + 2);
+    ALLOC(c->seg_len, c->nnodes + 2);
+    ALLOC(c->status, c->nnodes + 2);
+    ALLOC(c->node_sum, (size_t)(c->nnodes + 2) * NAgmax);
+    ALLOC(c->tree.feat, c->nnodes);
+    ALLOC(c->tree.cond_bin, c->nnodes);
+    ALLOC(c->tree.w, c->nnodes);
+    ALLOC(c->tree.gain, c->nnodes);
+    ALLOC(c->tree.pred, (size_t)c->nnodes * K);
+    ALLOC(c->tree.split, c->nnodes);
+    ALLOC(c->tree.packed, c->nnodes);
+    for (int l = 0; l < 2; l++) {
+        ALLOC(c->lvl[l].hdr, LH_SIZE);
+        ALLOC(c->lvl[l].act_node, c->maxlvl + 2);
+        ALLOC(c->lvl[l].cprefix, c->maxlvl + 2);
+        ALLOC(c->lvl[l].bnode, c->maxlvl + 2);
+        ALLOC(c->lvl[l].bstart, c->maxlvl + 2);
+        ALLOC(c->lvl[l].bprefix, c->maxlvl + 2);
+    }
+    ALLOC(c->js, c->F);
+    ALLOC(c->jsmap, c->RS);
+    ALLOC(c->feattypes, c->F);
+    ALLOC(c->mono, c->F);
+    ALLOC(c->absmax, 8);
+    ALLOC(c->qexp, 8);
+    ALLOC(c->qbits, 8);
+    ALLOC(c->qscale, 16);
+    ALLOC(c->stats, c->D + 2);
+    ALLOC(c->errflag, 1);
+    if (tree_type == EVT_TREE_OBLIVIOUS) ALLOC(c->ogains, (size_t)c->maxlvl * c->F * c->B);
+    // pinned staging: tree read-back + small per-tree uploads
+    c->h_stage_bytes = (size_t)c->nnodes * (4 + 1 + 4 + 4 + 4 * K + 1) + (size_t)(c->D + 2) * 8 + (size_t)c->F * 4 + (size_t)c->RS * 2 + 1024;
+    if (hipHostMalloc((void **)&c->h_stage, c->h_stage_bytes, hipHostMallocDefault) != hipSuccess) {
+        evt_set_error("hipHostMalloc failed");
+        evt_destroy(c);
+        return EVT_ERR_NOMEM;
+    }
+    // defaults: all numeric, no monotone constraint
+    {
+        std::vector<uint8_t> ft(c->F, 1);
+        hipError_t e2 = hipMemcpy(c->feattypes, ft.data(), c->F, hipMemcpyHostToDevice);
+        if (e2 == hipSuccess) e2 = hipMemset(c->mono, 0, sizeof(int32_t) * c->F);
+        if (e2 == hipSuccess) e2 = hipMemset(c->absmax, 0, sizeof(uint32_t) * 8);
+        if (e2 == hipSuccess) e2 = hipMemset(c->nidx, 0, sizeof(uint32_t) * N);
+        if (e2 == hipSuccess) e2 = hipMemset(c->errflag, 0, sizeof(int32_t));
+        if (e2 != hipSuccess) {
+            evt_set_error("initial fills failed: %s", hipGetErrorString(e2));
+            evt_destroy(c);
+            return EVT_ERR_HIP;
+        }
+    }
+    *out = c;
+    return EVT_OK;
+}
+
+#define CTXCHK(c)                             \
+    do {                                      \
+        ARGCHK((c) != nullptr, "handle is NULL"); \
+        HIPCHK(hipSetDevice((c)->device));    \
+    } while (0)
+
+static int check_errflag(evt_ctx *c, const char *what) {
+    int32_t f = 0;
+    HIPCHK(hipMemcpyAsync(&f, c->errflag, sizeof(int32_t), hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    if (f != 0) {
+        HIPCHK(hipMemsetAsync(c->errflag, 0, sizeof(int32_t), c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        evt_set_error("%s", what);
+        return EVT_ERR_ARG;
+    }
+    return EVT_OK;
+}
+
+extern "C" int evt_set_xbin(evt_handle c, const uint8_t *x_bin_colmajor) {
+    CTXCHK(c);
+    ARGCHK(x_bin_colmajor, "x_bin is NULL");
+    c->have_xbin = false;
+    HIPCHK(hipMemcpyAsync(c->xcm, x_bin_colmajor, (size_t)c->N * c->F, hipMemcpyDefault, c->stream));
+    int r = launch_transpose_validate(c);
+    if (r != EVT_OK) return r;
+    r = check_errflag(c, "x_bin holds values outside 1..nbins");
+    if (r != EVT_OK) return r;
+    c->have_xbin = true;
+    return EVT_OK;
+}
+
+extern "C" int evt_binarize_f64(evt_handle c, const double *x_colmajor, const double *edges, const int32_t *edge_off) {
+    CTXCHK(c);
+    ARGCHK(x_colmajor && edges && edge_off, "NULL argument");
+    c->have_xbin = false;
+    hipPointerAttribute_t attr;
+    bool on_dev = (hipPointerGetAttributes(&attr, x_colmajor) == hipSuccess) && attr.type == hipMemoryTypeDevice;
+    (void)hipGetLastError();
+    // edge_off is read on the host to size the edges upload (works for host pointers only)
+    std::vector<int32_t> off(c->F + 1);
+    HIPCHK(hipMemcpy(off.data(), edge_off, sizeof(int32_t) * (c->F + 1), hipMemcpyDefault));
+    for (int j = 0; j < c->F; j++) {
+        int ne = off[j + 1] - off[j];
+        ARGCHK(ne >= 1 && ne <= c->B - 1 && off[j] >= 0, "each feature needs 1..nbins-1 edges");
+    }
+    double *d_edges = nullptr;
+    int32_t *d_off = nullptr;
+    double *d_x = nullptr;
+    HIPCHK(hipMalloc((void **)&d_edges, sizeof(double) * std::max(1, off[c->F])));
+    hipError_t e = hipMalloc((void **)&d_off, sizeof(int32_t) * (c->F + 1));
+    if (e == hipSuccess) e = hipMemcpyAsync(d_edges, edges, sizeof(double) * off[c->F], hipMemcpyDefault, c->stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(d_off, off.data(), sizeof(int32_t) * (c->F + 1), hipMemcpyHostToDevice, c->stream);
+    const double *xsrc = x_colmajor;
+    if (e == hipSuccess && !on_dev) {
+        e = hipMalloc((void **)&d_x, sizeof(double) * (size_t)c->N * c->F);
+        if (e == hipSuccess) e = hipMemcpyAsync(d_x, x_colmajor, sizeof(double) * (size_t)c->N * c->F, hipMemcpyHostToDevice, c->stream);
+        xsrc = d_x;
+    }
+    int r = EVT_OK;
+    if (e == hipSuccess) {
+        r = launch_binarize(c, xsrc, d_edges, d_off);
+        if (r == EVT_OK) r = launch_transpose_validate(c);
+        e = hipStreamSynchronize(c->stream);
+    }
+    if (d_x) (void)hipFree(d_x);
+    if (d_off) (void)hipFree(d_off);
+    if (d_edges) (void)hipFree(d_edges);
+    if (e != hipSuccess) {
+        evt_set_error("binarize failed: %s", hipGetErrorString(e));
+        return EVT_ERR_HIP;
+    }
+    if (r != EVT_OK) return r;
+    r = check_errflag(c, "binarize produced values outside 1..nbins");
+    if (r != EVT_OK) return r;
+    c->have_xbin = true;
+    return EVT_OK;
+}
+
+static void set_channels(evt_ctx *c) {
+    // LDS channels (rows of the gradient matrix that need their own accumulator)
+    int na = 0;
+    if (c->loss == EVT_LOSS_MSE) {
+        c->chan_k[na++] = 0;                   // g ; h == 2w is derived
+        if (!c->unit_w) c->chan_k[na++] = 2;   // w
+    } else {
+        for (int k = 0; k < c->NK - 1; k++) c->chan_k[na++] = k;
+        if (!c->unit_w) c->chan_k[na++] = c->NK - 1;
+    }
+    c->NA = na;
+    for (int a = na; a < EVT_MAX_NA; a++) c->chan_k[a] = 0;
+    c->NAg = (c->loss == EVT_LOSS_MSE) ? 2 : c->NK;
+    int qbg = 62 - ceil_log2_i64(c->N);
+    if (qbg > 40) qbg = 40;
+    for (int k = 0; k < c->NK; k++) c->h_qbits[k] = qbg;
+    if (c->unit_w) c->h_qbits[0] = EVT_PACK_QBITS;
+    for (int k = c->NK; k < 8; k++) c->h_qbits[k] = 0;
+}
+
+extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, const float *mu, const float *offset) {
+    CTXCHK(c);
+    ARGCHK(y && mu, "y and mu must not be NULL");
+    c->have_target = false;
+    c->have_grads = false;
+    c->unit_w = (w == nullptr);
+    set_channels(c);
+    HIPCHK(hipMemcpyAsync(c->y, y, sizeof(float) * c->N, hipMemcpyDefault, c->stream));
+    HIPCHK(hipMemcpyAsync(c->qbits, c->h_qbits, sizeof(int32_t) * 8, hipMemcpyHostToDevice, c->stream));
+    // stage w / offset through the (not yet needed) fixed-point buffer
+    float *tmp = reinterpret_cast<float *>(c->gq);
+    if (w) {
+        HIPCHK(hipMemcpyAsync(tmp, w, sizeof(float) * c->N, hipMemcpyDefault, c->stream));
+        int r = launch_set_weight_row(c, tmp);
+        if (r != EVT_OK) return r;
+    } else {
+        int r = launch_set_weight_row(c, nullptr);
+        if (r != EVT_OK) return r;
+    }
+    {
+        int r = launch_absmax_rows(c, c->NK - 1, c->NK);
+        if (r != EVT_OK) return r;
+    }
+    float *mu_dev = reinterpret_cast<float *>(c->chunk_lpre); // small scratch
+    HIPCHK(hipMemcpyAsync(mu_dev, mu, sizeof(float) * c->K, hipMemcpyDefault, c->stream));
+    if (offset) {
+        HIPCHK(hipStreamSynchronize(c->stream));
+        HIPCHK(hipMemcpyAsync(tmp, offset, sizeof(float) * c->N * c->K, hipMemcpyDefault, c->stream));
+        int r = launch_init_pred(c, mu_dev, tmp);
+        if (r != EVT_OK) return r;
+    } else {
+        int r = launch_init_pred(c, mu_dev, nullptr);
+        if (r != EVT_OK) return r;
+    }
+    HIPCHK(hipStreamSynchronize(c->stream));
+    c->have_target = true;
+    return EVT_OK;
+}
+
+extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, const int32_t *monotone) {
+    CTXCHK(c);
+    std::vector<uint8_t> ft(c->F, 1);
+    std::vector<int32_t> mo(c->F, 0);
+    if (feattypes) HIPCHK(hipMemcpy(ft.data(), feattypes, c->F, hipMemcpyDefault));
+    if (monotone) HIPCHK(hipMemcpy(mo.data(), monotone, sizeof(int32_t) * c->F, hipMemcpyDefault));
+    for (int j = 0; j < c->F; j++) {
+        ft[j] = ft[j] ? 1 : 0;
+        ARGCHK(mo[j] >= -1 && mo[j] <= 1, "monotone constraints must be -1, 0 or 1");
+    }
+    HIPCHK(hipMemcpy(c->feattypes, ft.data(), c->F, hipMemcpyHostToDevice));
+    HIPCHK(hipMemcpy(c->mono, mo.data(), sizeof(int32_t) * c->F, hipMemcpyHostToDevice));
+    return EVT_OK;
+}
+
+extern "C" int evt_update_grads(evt_handle c) {
+    CTXCHK(c);
+    if (!c->have_target) {
+        evt_set_error("evt_set_target must be called before evt_update_grads");
+        return EVT_ERR_STATE;
+    }
+    prof_begin(c, EVT_K_GRAD, 0);
+    int r = launch_grads(c);
+    prof_end(c);
+    if (r != EVT_OK) return r;
+    if (c->profiling) c->prof_units[EVT_K_GRAD] += c->N;
+    prof_begin(c, EVT_K_OTHER, 0);
+    r = launch_quantize(c);
+    prof_end(c);
+    if (r != EVT_OK) return r;
+    c->have_grads = true;
+    return EVT_OK;
+}
+
+extern "C" int evt_set_grads(evt_handle c, const float *grad) {
+    CTXCHK(c);
+    ARGCHK(grad, "grad is NULL");
+    if (!c->have_target) {
+        evt_set_error("evt_set_target must be called before evt_set_grads");
+        return EVT_ERR_STATE;
+    }
+    HIPCHK(hipMemcpyAsync(c->grad, grad, sizeof(float) * (size_t)c->N * c->NK, hipMemcpyDefault, c->stream));
+    int r = launch_absmax_rows(c, 0, c->NK);
+    if (r != EVT_OK) return r;
+    r = launch_quantize(c);
+    if (r != EVT_OK) return r;
+    HIPCHK(hipStreamSynchronize(c->stream));
+    c->have_grads = true;
+    return EVT_OK;
+}
+
+extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p,
+                             evt_tree_out *tree) {
+    CTXCHK(c);
+    ARGCHK(js && p, "js and params must not be NULL");
+    ARGCHK(n_js >= 1 && n_js <= c->F, "n_js must be in [1, nfeats]");
+    ARGCHK(p->bagging_size >= 1, "bagging_size must be >= 1");
+    ARGCHK(p->lambda >= 0 && p->gamma >= 0 && p->min_weight >= 0 && p->eta >= 0, "lambda, gamma, min_weight, eta must be >= 0");
+    if (!c->have_xbin || !c->have_target || !c->have_grads) {
+        evt_set_error("x_bin, target and gradients must be set before evt_grow_tree");
+        return EVT_ERR_STATE;
+    }
+    // js: 1-based, strictly ascending
+    std::vector<uint32_t> jsv(n_js);
+    HIPCHK(hipMemcpy(jsv.data(), js, sizeof(uint32_t) * n_js, hipMemcpyDefault));
+    for (int i = 0; i < n_js; i++) {
+        ARGCHK(jsv[i] >= 1 && jsv[i] <= (uint32_t)c->F, "js entries must be in 1..nfeats");
+        ARGCHK(i == 0 || jsv[i] > jsv[i - 1], "js must be strictly ascending");
+    }
+    // LDS budget of one block: channels x bins of a single feature must fit
+    ARGCHK((size_t)c->NA * c->B * 8 <= 64 * 1024, "histogram of one feature exceeds the LDS budget");
+
+    // rows kept by the mask (the host owns the RNG; src/subsample.jl:7-9)
+    int64_t n_is = c->N;
+    std::vector<uint8_t> mask_host;
+    if (mask) {
+        hipPointerAttribute_t attr;
+        bool on_dev = (hipPointerGetAttributes(&attr, mask) == hipSuccess) && attr.type == hipMemoryTypeDevice;
+        (void)hipGetLastError();
+        const uint8_t *mh = mask;
+        if (on_dev) {
+            mask_host.resize(c->N);
+            HIPCHK(hipMemcpy(mask_host.data(), mask, c->N, hipMemcpyDeviceToHost));
+            mh = mask_host.data();
+        }
+        n_is = 0;
+        for (int64_t i = 0; i < c->N; i++) n_is += (mh[i] <= cond);
+        if (n_is == 0) {
+            evt_set_error("no subsample observation - choose larger rowsample");
+            return EVT_ERR_EMPTY;
+        }
+    }
+    const bool all_rows = (n_is == c->N);
+    c->last_all_rows = all_rows;
+
+    // per-tree small uploads through pinned memory
+    uint32_t *h_js = reinterpret_cast<uint32_t *>(c->h_stage);
+    uint16_t *h_map = reinterpret_cast<uint16_t *>(c->h_stage + (size_t)c->F * 4);
+    for (int f = 0; f < c->RS; f++) h_map[f] = 0xFFFF;
+    for (int i = 0; i < n_js; i++) {
+        h_js[i] = jsv[i];
+        h_map[jsv[i] - 1] = (uint16_t)i;
+    }
+    HIPCHK(hipMemcpyAsync(c->js, h_js, sizeof(uint32_t) * n_js, hipMemcpyHostToDevice, c->stream));
+    HIPCHK(hipMemcpyAsync(c->jsmap, h_map, sizeof(uint16_t) * c->RS, hipMemcpyHostToDevice, c->stream));
+    c->n_js_last = n_js;
+    c->js_last = jsv;
+
+    int r;
+    prof_begin(c, EVT_K_OTHER, 0);
+    if (all_rows) {
+        r = launch_iota(c, c->is_a, c->N);
+    } else {
+        HIPCHK(hipMemcpyAsync(c->mask, mask, c->N, hipMemcpyDefault, c->stream));
+        r = launch_compact_mask(c, cond, n_is);
+        if (r == EVT_OK) r = launch_fill_u32(c, c->nidx, 0u, c->N);
+    }
+    if (r == EVT_OK) r = launch_tree_begin(c, n_is);
+    prof_end(c);
+    if (r != EVT_OK) return r;
+
+    const bool fuse_pred = p->update_pred && all_rows;
+    const bool obliv = (c->tree_type == EVT_TREE_OBLIVIOUS);
+    uint32_t *is_cur = c->is_a, *is_next = c->is_b;
+    for (int level = 1; level <= c->D; level++) {
+        const bool leaf_level = (level == c->D);
+        if (!leaf_level || level == 1) {
+            prof_begin(c, EVT_K_HIST, level);
+            r = launch_hist_build(c, level, is_cur);
+            prof_end(c);
+            if (r != EVT_OK) return r;
+        }
+        prof_begin(c, EVT_K_SCAN, level);
+        r = launch_scan(c, level, p, leaf_level);
+        if (r == EVT_OK && obliv && !leaf_level) r = launch_obliv_select(c, level, p);
+        prof_end(c);
+        if (r != EVT_OK) return r;
+        prof_begin(c, EVT_K_PARTITION, level);
+        if (!leaf_level) {
+            r = launch_part_count(c, level, is_cur);
+            if (r == EVT_OK) r = launch_level_next(c, level);
+        }
+        if (r == EVT_OK) r = launch_part_scatter(c, level, is_cur, is_next, fuse_pred);
+        prof_end(c);
+        if (r != EVT_OK) return r;
+        std::swap(is_cur, is_next);
+    }
+    if (p->update_pred && !all_rows) {
+        // rows outside the sample are predicted too (src/fit.jl:37): walk the new tree for all rows
+        prof_begin(c, EVT_K_PREDICT, 0);
+        r = launch_predict_tree_cache(c);
+        prof_end(c);
+        if (r != EVT_OK) return r;
+        if (c->profiling) c->prof_units[EVT_K_PREDICT] += c->N;
+    }
+    if (c->profiling) {
+        c->prof_units[EVT_K_PARTITION] += n_is;
+    }
+
+    // read back the tree (and the per-level row counts) in one pinned transfer
+    const int nn = c->nnodes, K = c->K;
+    uint8_t *hs = c->h_stage;
+    size_t o_feat = 0, o_w = o_feat + (size_t)nn * 4, o_gain = o_w + (size_t)nn * 4, o_pred = o_gain + (size_t)nn * 4,
+           o_stats = ((o_pred + (size_t)nn * 4 * K + 7) / 8) * 8, o_bin = o_stats + (size_t)(c->D + 2) * 8, o_split = o_bin + nn;
+    HIPCHK(hipMemcpyAsync(hs + o_feat, c->tree.feat, (size_t)nn * 4, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipMemcpyAsync(hs + o_w, c->tree.w, (size_t)nn * 4, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipMemcpyAsync(hs + o_gain, c->tree.gain, (size_t)nn * 4, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipMemcpyAsync(hs + o_pred, c->tree.pred, (size_t)nn * 4 * K, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipMemcpyAsync(hs + o_stats, c->stats, (size_t)(c->D + 2) * 8, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipMemcpyAsync(hs + o_bin, c->tree.cond_bin, nn, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipMemcpyAsync(hs + o_split, c->tree.split, nn, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    if (c->profiling) {
+        prof_collect(c, reinterpret_cast<const int64_t *>(hs + o_stats));
+        c->prof_units[EVT_K_SCAN] += 0;
+    }
+    if (tree) {
+        ARGCHK(tree->feat && tree->cond_bin && tree->w && tree->gain && tree->pred && tree->split, "tree output arrays must not be NULL");
+        const int32_t *f32 = reinterpret_cast<const int32_t *>(hs + o_feat);
+        for (int n = 0; n < nn; n++) tree->feat[n] = (int64_t)f32[n];
+        memcpy(tree->w, hs + o_w, (size_t)nn * 4);
+        memcpy(tree->gain, hs + o_gain, (size_t)nn * 4);
+        memcpy(tree->pred, hs + o_pred, (size_t)nn * 4 * K);
+        memcpy(tree->cond_bin, hs + o_bin, nn);
+        memcpy(tree->split, hs + o_split, nn);
+    }
+    return EVT_OK;
+}
+
+// host tree -> packed device nodes; validates that every split node has both children in range
+static int pack_tree(int32_t nn, const int64_t *feat, const uint8_t *cond_bin, const uint8_t *split, int F, std::vector<uint32_t> &out) {
+    out.assign(nn, 0u);
+    for (int n = 1; n <= nn; n++) {
+        if (split[n - 1]) {
+            ARGCHK(2 * n + 1 <= nn, "split node without children inside the tree arrays");
+            ARGCHK(feat[n - 1] >= 1 && feat[n - 1] <= F, "tree feature id outside 1..nfeats");
+            out[n - 1] = (uint32_t)feat[n - 1] | ((uint32_t)cond_bin[n - 1] << 16) | (1u << 24);
+        }
+    }
+    return EVT_OK;
+}
+
+extern "C" int evt_predict_tree(evt_handle c, int32_t nnodes_tree, const int64_t *feat, const uint8_t *cond_bin, const float *pred,
+                                const uint8_t *split) {
+    CTXCHK(c);
+    ARGCHK(feat && cond_bin && pred && split && nnodes_tree >= 1, "NULL tree arrays");
+    if (!c->have_xbin || !c->have_target) {
+        evt_set_error("x_bin and target must be set before evt_predict_tree");
+        return EVT_ERR_STATE;
+    }
+    std::vector<uint32_t> nodes;
+    int r = pack_tree(nnodes_tree, feat, cond_bin, split, c->F, nodes);
+    if (r != EVT_OK) return r;
+    uint32_t *d_nodes = nullptr;
+    float *d_pred = nullptr;
+    HIPCHK(hipMalloc((void **)&d_nodes, sizeof(uint32_t) * nnodes_tree));
+    hipError_t e = hipMalloc((void **)&d_pred, sizeof(float) * (size_t)nnodes_tree * c->K);
+    if (e == hipSuccess) e = hipMemcpyAsync(d_nodes, nodes.data(), sizeof(uint32_t) * nnodes_tree, hipMemcpyHostToDevice, c->stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(d_pred, pred, sizeof(float) * (size_t)nnodes_tree * c->K, hipMemcpyHostToDevice, c->stream);
+    if (e == hipSuccess) {
+        prof_begin(c, EVT_K_PREDICT, 0);
+        r = launch_predict_tree_nodes(c, d_nodes, d_pred);
+        prof_end(c);
+        e = hipStreamSynchronize(c->stream);
+        if (c->profiling) {
+            c->prof_units[EVT_K_PREDICT] += c->N;
+            prof_collect(c, nullptr);
+        }
+    }
+    if (d_nodes) (void)hipFree(d_nodes);
+    if (d_pred) (void)hipFree(d_pred);
+    if (e != hipSuccess) {
+        evt_set_error("predict_tree failed: %s", hipGetErrorString(e));
+        return EVT_ERR_HIP;
+    }
+    return r;
+}
+
+extern "C" int evt_get_pred(evt_handle c, float *out) {
+    CTXCHK(c);
+    ARGCHK(out, "out is NULL");
+    HIPCHK(hipMemcpyAsync(out, c->pred, sizeof(float) * (size_t)c->N * c->K, hipMemcpyDefault, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return EVT_OK;
+}
+extern "C" int evt_get_grads(evt_handle c, float *out) {
+    CTXCHK(c);
+    ARGCHK(out, "out is NULL");
+    HIPCHK(hipMemcpyAsync(out, c->grad, sizeof(float) * (size_t)c->N * c->NK, hipMemcpyDefault, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return EVT_OK;
+}
+extern "C" int evt_get_nidx(evt_handle c, uint32_t *out) {
+    CTXCHK(c);
+    ARGCHK(out, "out is NULL");
+    HIPCHK(hipMemcpyAsync(out, c->nidx, sizeof(uint32_t) * (size_t)c->N, hipMemcpyDefault, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return EVT_OK;
+}
+extern "C" int evt_get_hist(evt_handle c, double *out) {
+    CTXCHK(c);
+    ARGCHK(out, "out is NULL");
+    if (c->n_js_last <= 0) {
+        evt_set_error("no tree has been grown yet");
+        return EVT_ERR_STATE;
+    }
+    const size_t n = (size_t)c->NK * c->B * c->F * c->nnodes;
+    double *d = nullptr;
+    HIPCHK(hipMalloc((void **)&d, sizeof(double) * n));
+    hipError_t e = hipMemsetAsync(d, 0, sizeof(double) * n, c->stream);
+    int r = EVT_OK;
+    if (e == hipSuccess) r = launch_hist_export(c, d);
+    if (e == hipSuccess) e = hipMemcpyAsync(out, d, sizeof(double) * n, hipMemcpyDefault, c->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    (void)hipFree(d);
+    if (e != hipSuccess) {
+        evt_set_error("hist export failed: %s", hipGetErrorString(e));
+        return EVT_ERR_HIP;
+    }
+    return r;
+}
+extern "C" int evt_get_quant(evt_handle c, int32_t *qbits, int32_t *qexp) {
+    CTXCHK(c);
+    ARGCHK(qbits && qexp, "NULL argument");
+    int32_t e[8];
+    HIPCHK(hipMemcpyAsync(e, c->qexp, sizeof(int32_t) * 8, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    for (int k = 0; k < c->NK; k++) {
+        qbits[k] = c->h_qbits[k];
+        qexp[k] = e[k];
+    }
+    return EVT_OK;
+}
+
+// ---- inference ------------------------------------------------------------------------------
+static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, const uint8_t *feattypes, int32_t loss, int32_t K, int32_t ntrees,
+                          const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const float *pred, const uint8_t *split,
+                          int32_t apply_link, float *out, uint32_t *leaf_out) {
+    ARGCHK(nobs >= 1 && nfeats >= 1 && ntrees >= 1, "nobs, nfeats, ntrees must be >= 1");
+    ARGCHK(x_bin && tree_off && feat && cond_bin && split, "NULL argument");
+    ARGCHK(leaf_out || (pred && out && K >= 1 && K <= 4 && loss >= 0 && loss <= 2), "invalid prediction arguments");
+    int ndev = 0;
+    int r = evt_device_count(&ndev);
+    if (r != EVT_OK) return r;
+    const int64_t total = tree_off[ntrees];
+    std::vector<uint32_t> nodes((size_t)total, 0u), one;
+    for (int t = 0; t < ntrees; t++) {
+        const int64_t o = tree_off[t];
+        const int64_t nn = tree_off[t + 1] - o;
+        ARGCHK(nn >= 1 && o >= 0, "tree_off must be ascending");
+        r = pack_tree((int32_t)nn, feat + o, cond_bin + o, split + o, nfeats, one);
+        if (r != EVT_OK) return r;
+        memcpy(nodes.data() + o, one.data(), sizeof(uint32_t) * nn);
+    }
+    std::vector<uint8_t> ft(nfeats, 1);
+    if (feattypes)
+        for (int j = 0; j < nfeats; j++) ft[j] = feattypes[j] ? 1 : 0;
+    hipStream_t s = nullptr;
+    uint8_t *d_x = nullptr, *d_ft = nullptr;
+    uint32_t *d_nodes = nullptr, *d_leaf = nullptr;
+    float *d_lp = nullptr, *d_out = nullptr;
+    int64_t *d_off = nullptr;
+    hipError_t e = hipMalloc((void **)&d_x, (size_t)nobs * nfeats);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_ft, nfeats);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_nodes, sizeof(uint32_t) * total);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_off, sizeof(int64_t) * (ntrees + 1));
+    if (e == hipSuccess && !leaf_out) e = hipMalloc((void **)&d_lp, sizeof(float) * (size_t)total * K);
+    if (e == hipSuccess && !leaf_out) e = hipMalloc((void **)&d_out, sizeof(float) * (size_t)nobs * K);
+    if (e == hipSuccess && leaf_out) e = hipMalloc((void **)&d_leaf, sizeof(uint32_t) * (size_t)nobs * ntrees);
+    if (e == hipSuccess) e = hipMemcpy(d_x, x_bin, (size_t)nobs * nfeats, hipMemcpyDefault);
+    if (e == hipSuccess) e = hipMemcpy(d_ft, ft.data(), nfeats, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(d_nodes, nodes.data(), sizeof(uint32_t) * total, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(d_off, tree_off, sizeof(int64_t) * (ntrees + 1), hipMemcpyDefault);
+    if (e == hipSuccess && !leaf_out) e = hipMemcpy(d_lp, pred, sizeof(float) * (size_t)total * K, hipMemcpyDefault);
+    if (e == hipSuccess) {
+        if (leaf_out) r = launch_leaf_idx_model(s, d_nodes, d_off, ntrees, d_x, d_ft, nobs, d_leaf);
+        else r = launch_predict_model(s, d_nodes, d_lp, d_off, ntrees, d_x, d_ft, nobs, K, loss, apply_link, d_out);
+        e = hipDeviceSynchronize();
+    }
+    if (e == hipSuccess && r == EVT_OK) {
+        if (leaf_out) e = hipMemcpy(leaf_out, d_leaf, sizeof(uint32_t) * (size_t)nobs * ntrees, hipMemcpyDefault);
+        else e = hipMemcpy(out, d_out, sizeof(float) * (size_t)nobs * K, hipMemcpyDefault);
+    }
+    void *ptrs[] = {d_x, d_ft, d_nodes, d_off, d_lp, d_out, d_leaf};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    if (e != hipSuccess) {
+        evt_set_error("predict failed: %s", hipGetErrorString(e));
+        return EVT_ERR_HIP;
+    }
+    return r;
+}
+
+extern "C" int evt_predict(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, const uint8_t *feattypes, int32_t loss, int32_t K, int32_t ntrees,
+                           const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const float *pred, const uint8_t *split,
+                           int32_t apply_link, float *out) {
+    return predict_common(nobs, nfeats, x_bin, feattypes, loss, K, ntrees, tree_off, feat, cond_bin, pred, split, apply_link, out, nullptr);
+}
+
+extern "C" int evt_predict_leaf_idx(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, const uint8_t *feattypes, int32_t ntrees,
+                                    const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const uint8_t *split, uint32_t *out) {
+    ARGCHK(out, "out is NULL");
+    return predict_common(nobs, nfeats, x_bin, feattypes, 0, 1, ntrees, tree_off, feat, cond_bin, nullptr, split, 0, nullptr, out);
+}
+
+// ---- measurement ----------------------------------------------------------------------------
+extern "C" int evt_set_profiling(evt_handle c, int32_t on) {
+    CTXCHK(c);
+    HIPCHK(hipStreamSynchronize(c->stream));
+    prof_collect(c, nullptr);
+    c->profiling = on != 0;
+    return EVT_OK;
+}
+extern "C" int evt_get_profile(evt_handle c, int64_t *launches, double *ms, int64_t *units) {
+    CTXCHK(c);
+    ARGCHK(launches && ms && units, "NULL argument");
+    HIPCHK(hipStreamSynchronize(c->stream));
+    prof_collect(c, nullptr);
+    for (int k = 0; k < EVT_K_COUNT; k++) {
+        launches[k] = c->prof_launches[k];
+        ms[k] = c->prof_ms[k];
+        units[k] = c->prof_units[k];
+    }
+    return EVT_OK;
+}
+extern "C" int evt_reset_profile(evt_handle c) {
+    CTXCHK(c);
+    HIPCHK(hipStreamSynchronize(c->stream));
+    prof_collect(c, nullptr);
+    memset(c->prof_launches, 0, sizeof(c->prof_launches));
+    memset(c->prof_ms, 0, sizeof(c->prof_ms));
+    memset(c->prof_units, 0, sizeof(c->prof_units));
+    return EVT_OK;
+}
+extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
+    CTXCHK(c);
+    ARGCHK(name, "name is NULL");
+    if (strcmp(name, "hist_blocks") == 0) {
+        ARGCHK(value >= 1 && value <= 65535, "hist_blocks must be in [1, 65535]");
+        c->hist_blocks = (int)value;
+    } else if (strcmp(name, "hist_threads") == 0) {
+        ARGCHK(value == 256 || value == 512 || value == 1024, "hist_threads must be 256, 512 or 1024");
+        c->hist_threads = (int)value;
+    } else {
+        evt_set_error("unknown option %s", name);
+        return EVT_ERR_ARG;
+    }
+    return EVT_OK;
+}
+extern "C" int evt_synchronize(evt_handle c) {
+    CTXCHK(c);
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return EVT_OK;
+}
+
+__global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = src[i];
+}
+
+extern "C" int evt_copy_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out) {
+    ARGCHK(gbps_out && nbytes >= 4096 && iters >= 1, "invalid arguments");
+    int ndev = 0;
+    int r = evt_device_count(&ndev);
+    if (r != EVT_OK) return r;
+    const int64_t n = nbytes / 16;
+    uint4 *a = nullptr, *b = nullptr;
+    HIPCHK(hipMalloc((void **)&a, n * 16));
+    hipError_t e = hipMalloc((void **)&b, n * 16);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipMemset(a, 1, n * 16);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(k_copy16, dim3(8192), dim3(256), 0, 0, a, b, n); // warm-up
+        e = hipEventRecord(e0, 0);
+        for (int i = 0; i < iters; i++) hipLaunchKernelGGL(k_copy16, dim3(8192), dim3(256), 0, 0, a, b, n);
+        if (e == hipSuccess) e = hipEventRecord(e1, 0);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (a) (void)hipFree(a);
+    if (b) (void)hipFree(b);
+    if (e != hipSuccess) {
+        evt_set_error("copy bandwidth probe failed: %s", hipGetErrorString(e));
+        return EVT_ERR_HIP;
+    }
+    *gbps_out = 2.0 * (double)(n * 16) * iters / ((double)ms * 1e-3) / 1e9;
+    return EVT_OK;
+}

@@ -1,0 +1,171 @@
+// Internal declarations shared by the HIP translation units of libevotrees_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string>
+#include <vector>
+
+#include "../../include/evotrees_hip.h"
+
+// ---- node status on device ------------------------------------------------------------
+#define ST_INACTIVE 0
+#define ST_BUILD 1    // active at its level, histogram built from rows
+#define ST_SUBTRACT 2 // active at its level, histogram = parent - sibling
+#define ST_SPLIT 3    // scanned, split found
+#define ST_LEAF 4     // scanned (or last level), leaf
+
+#define EVT_CHUNK 2048        // rows per partition chunk (8 per thread of a 256-thread block)
+#define EVT_CHUNK_WORDS 32    // 64-bit ballot words per chunk
+#define EVT_MAX_NK 5
+#define EVT_MAX_NA 5
+#define EVT_MAX_DEPTH 16
+#define EVT_PACK_QBITS 30     // fixed-point bits of the gradient channel that shares a word with the row count
+#define EVT_PACK_CNT_BITS 16
+#define EVT_HIST_MAX_ROWS_PER_BLOCK 32768
+
+// Level table header slots (int64 each)
+#define LH_N_ACT 0
+#define LH_N_CHUNKS 1
+#define LH_N_BUILD 2
+#define LH_TOTAL_BUILD 3
+#define LH_SIZE 8
+
+struct LevelTab {
+    int64_t *hdr;      // [LH_SIZE]
+    int32_t *act_node; // active nodes in node (= position) order
+    int64_t *cprefix;  // exclusive prefix of chunk counts over active nodes, n_act+1 entries
+    int32_t *bnode;    // build nodes
+    int64_t *bstart;   // their segment starts
+    int64_t *bprefix;  // exclusive prefix of their lengths, n_build+1 entries
+};
+
+struct TreeDev {
+    int32_t *feat;    // 1-based, 0 none
+    uint8_t *cond_bin;
+    float *w;
+    float *gain;
+    float *pred;      // K x nnodes
+    uint8_t *split;
+    uint32_t *packed; // feat | cond_bin << 16 | split << 24, for traversal
+};
+
+struct ProfRec {
+    int cls;
+    int level;
+    hipEvent_t e0, e1;
+};
+
+struct evt_ctx {
+    int device;
+    hipStream_t stream;
+    int64_t N;
+    int32_t F, B, K, NK, D, loss, tree_type;
+    int32_t nnodes;    // 2^D - 1
+    int32_t maxlvl;    // 2^(D-1)
+    int32_t RS;        // bytes per observation-major record
+    int32_t LPR;       // 16-byte lanes per record
+    bool unit_w;       // weights are all one (w == NULL at set_target)
+    int32_t NA;        // LDS accumulator channels per bin
+    int32_t NAg;       // global histogram channels per bin
+    int32_t chan_k[EVT_MAX_NA]; // gradient row of LDS channel a
+    bool have_xbin, have_target, have_grads;
+
+    // data
+    uint8_t *xcm;   // F x N bytes (column-major N x F)
+    uint8_t *xrm;   // N records of RS bytes
+    float *y;
+    float *pred;    // K x N
+    float *grad;    // NK x N
+    unsigned long long *gq; // NA planes of N packed fixed-point words
+    uint32_t *is_a, *is_b;
+    uint32_t *nidx;
+    uint8_t *mask;
+    unsigned long long *flagw;
+    int32_t *chunk_nleft;
+    int64_t *chunk_lpre;
+    int64_t max_chunks;
+    long long *hist; // [node][jp][ag][bin]
+    int64_t *seg_start, *seg_len;
+    int32_t *status;
+    long long *node_sum; // [node][NAg]
+    TreeDev tree;
+    LevelTab lvl[2];
+    uint32_t *js;      // [F]
+    uint16_t *jsmap;   // [RS] slot of feature f (0-based), 0xFFFF = not sampled / padding
+    uint8_t *feattypes;
+    int32_t *mono;
+    uint32_t *absmax;  // [8] float bits
+    int32_t *qexp;     // [8]
+    int32_t *qbits;    // [8]
+    double *qscale;    // [8] decode scale per global channel
+    int64_t *stats;    // [D+1] rows built per level
+    int32_t *errflag;  // device-side validation flag
+    double *ogains;    // oblivious: [maxlvl][F][B]
+    double *obest;     // oblivious: level decision {gain, jp, bin}
+
+    // host staging (pinned)
+    uint8_t *h_stage;
+    size_t h_stage_bytes;
+    int32_t h_qbits[8];
+    int32_t n_js_last;
+    std::vector<uint32_t> js_last;
+    bool last_all_rows;
+
+    // tunables
+    int hist_blocks, hist_threads;
+
+    // profiling
+    bool profiling;
+    std::vector<ProfRec> recs;
+    std::vector<hipEvent_t> free_events;
+    int64_t prof_launches[EVT_K_COUNT];
+    double prof_ms[EVT_K_COUNT];
+    int64_t prof_units[EVT_K_COUNT];
+};
+
+// ---- error plumbing ---------------------------------------------------------------------
+void evt_set_error(const char *fmt, ...);
+#define HIPCHK(call)                                                                       \
+    do {                                                                                   \
+        hipError_t _e = (call);                                                            \
+        if (_e != hipSuccess) {                                                            \
+            evt_set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(_e), __FILE__, __LINE__); \
+            return EVT_ERR_HIP;                                                            \
+        }                                                                                  \
+    } while (0)
+#define ARGCHK(cond, msg)                \
+    do {                                 \
+        if (!(cond)) {                   \
+            evt_set_error("%s", msg);    \
+            return EVT_ERR_ARG;          \
+        }                                \
+    } while (0)
+
+// ---- kernel launchers (each only enqueues on c->stream) -----------------------------------
+// grad
+int launch_grads(evt_ctx *c);
+int launch_quantize(evt_ctx *c);
+int launch_set_weight_row(evt_ctx *c, const float *w_dev);
+int launch_init_pred(evt_ctx *c, const float *mu_dev, const float *offset_dev);
+// data layout
+int launch_transpose_validate(evt_ctx *c);
+int launch_binarize(evt_ctx *c, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev);
+// tree
+int launch_tree_begin(evt_ctx *c, int64_t n_is);
+int launch_iota(evt_ctx *c, uint32_t *dst, int64_t n);
+int launch_compact_mask(evt_ctx *c, uint8_t cond, int64_t n_is);
+int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur);
+int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level);
+int launch_obliv_select(evt_ctx *c, int level, const evt_params *p);
+int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur);
+int launch_level_next(evt_ctx *c, int level);
+int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred);
+int launch_fill_u32(evt_ctx *c, uint32_t *dst, uint32_t v, int64_t n);
+int launch_fill_bytes(evt_ctx *c, void *dst, int64_t nbytes);
+// predict
+int launch_predict_tree_cache(evt_ctx *c);
+int launch_hist_export(evt_ctx *c, double *out_dev);
+
+// profiling helpers
+void prof_begin(evt_ctx *c, int cls, int level);
+void prof_end(evt_ctx *c);

@@ -1,0 +1,118 @@
+// Data-layout kernels: observation-major copy of x_bin, device binarize, small fills.
+#include "evt_internal.h"
+
+// One thread = one observation x one 16-feature group.  Reads are coalesced along rows of each
+// column; the 16 bytes are written as one 128-bit store into the observation-major record.
+// Bins outside 1..B raise the device error flag (the histogram kernels index LDS with them).
+__global__ __launch_bounds__(256) void k_transpose_validate(const uint8_t *__restrict__ xcm, uint8_t *__restrict__ xrm,
+                                                           int64_t N, int F, int B, int RS, int32_t *errflag) {
+    int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    int grp = blockIdx.y;
+    if (row >= N) return;
+    uint32_t w[4] = {0, 0, 0, 0};
+    bool bad = false;
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+        int f = grp * 16 + t;
+        uint32_t b = 0;
+        if (f < F) {
+            b = xcm[(size_t)f * N + row];
+            bad |= (b == 0 || b > (uint32_t)B);
+        }
+        w[t >> 2] |= b << (8 * (t & 3));
+    }
+    if (bad) atomicOr(errflag, 1);
+    uint4 v = make_uint4(w[0], w[1], w[2], w[3]);
+    *reinterpret_cast<uint4 *>(xrm + (size_t)row * RS + grp * 16) = v;
+}
+
+int launch_transpose_validate(evt_ctx *c) {
+    dim3 grid((unsigned)((c->N + 255) / 256), (unsigned)(c->RS / 16));
+    hipLaunchKernelGGL(k_transpose_validate, grid, dim3(256), 0, c->stream, c->xcm, c->xrm, c->N, c->F, c->B, c->RS, c->errflag);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+// searchsortedfirst(edges_j, x) = 1 + number of edges strictly below x.
+__global__ __launch_bounds__(256) void k_binarize(const double *__restrict__ x, const double *__restrict__ edges,
+                                                 const int32_t *__restrict__ edge_off, uint8_t *__restrict__ xcm, int64_t N) {
+    int j = blockIdx.y;
+    int e0 = edge_off[j], ne = edge_off[j + 1] - e0;
+    extern __shared__ double s_edges[];
+    for (int t = threadIdx.x; t < ne; t += 256) s_edges[t] = edges[e0 + t];
+    __syncthreads();
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
+        double v = x[(size_t)j * N + i];
+        int lo = 0, hi = ne;
+        while (lo < hi) {
+            int mid = (lo + hi) >> 1;
+            if (s_edges[mid] < v) lo = mid + 1; else hi = mid;
+        }
+        xcm[(size_t)j * N + i] = (uint8_t)(lo + 1);
+    }
+}
+
+int launch_binarize(evt_ctx *c, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev) {
+    int64_t nb = (c->N + 255) / 256;
+    if (nb > 4096) nb = 4096;
+    dim3 grid((unsigned)nb, (unsigned)c->F);
+    hipLaunchKernelGGL(k_binarize, grid, dim3(256), 256 * sizeof(double), c->stream, x_dev, edges_dev, edge_off_dev, c->xcm, c->N);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+__global__ __launch_bounds__(256) void k_iota(uint32_t *dst, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = (uint32_t)i;
+}
+int launch_iota(evt_ctx *c, uint32_t *dst, int64_t n) {
+    int64_t nb = (n + 255) / 256;
+    if (nb > 8192) nb = 8192;
+    if (nb < 1) nb = 1;
+    hipLaunchKernelGGL(k_iota, dim3((unsigned)nb), dim3(256), 0, c->stream, dst, n);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+__global__ __launch_bounds__(256) void k_fill_u32(uint32_t *dst, uint32_t v, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = v;
+}
+int launch_fill_u32(evt_ctx *c, uint32_t *dst, uint32_t v, int64_t n) {
+    if (n <= 0) return EVT_OK;
+    int64_t nb = (n + 255) / 256;
+    if (nb > 8192) nb = 8192;
+    hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)nb), dim3(256), 0, c->stream, dst, v, n);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+// zero-fill of a byte range whose size is a multiple of 4
+int launch_fill_bytes(evt_ctx *c, void *dst, int64_t nbytes) { return launch_fill_u32(c, (uint32_t *)dst, 0u, nbytes / 4); }
+
+// grad[NK-1, i] = w[i] (or 1): the weight row is written once (src/init.jl:173-174).
+__global__ __launch_bounds__(256) void k_set_weight_row(float *grad, const float *w, int64_t N, int NK) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N) return;
+    float *g = grad + (size_t)NK * i;
+    for (int k = 0; k < NK - 1; k++) g[k] = 0.0f;
+    g[NK - 1] = w ? w[i] : 1.0f;
+}
+int launch_set_weight_row(evt_ctx *c, const float *w_dev) {
+    hipLaunchKernelGGL(k_set_weight_row, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, w_dev, c->N, c->NK);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+// pred[:, i] = mu (+ offset[:, i])  (src/init.jl:168-170)
+__global__ __launch_bounds__(256) void k_init_pred(float *pred, const float *mu, const float *offset, int64_t N, int K) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N) return;
+    for (int k = 0; k < K; k++) {
+        float v = mu[k];
+        if (offset) v += offset[(size_t)K * i + k];
+        pred[(size_t)K * i + k] = v;
+    }
+}
+int launch_init_pred(evt_ctx *c, const float *mu_dev, const float *offset_dev) {
+    hipLaunchKernelGGL(k_init_pred, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->pred, mu_dev, offset_dev, c->N, c->K);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}

@@ -1,0 +1,158 @@
+// Gradient kernels: fused per-loss gradient + hessian rows, |max| reduction, fixed-point staging.
+//
+// Streaming work, HBM bound: per row the kernel reads pred (4K B), y (4 B) and the weight
+// (4 B, last row of the gradient matrix) and writes 8K B.
+#include "evt_internal.h"
+
+__device__ __forceinline__ float wave_max_f32(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+__device__ __forceinline__ float dev_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float dev_softplus(float x) { return fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x))); }
+
+// LOSS: 0 mse (src/loss.jl:52), 1 logloss (:54-57), 2 gaussian_mle (:194-203).
+// grad rows: [g_1..g_K, h_1..h_K, w]; every written value is multiplied by w (src/loss.jl:104-108, :223-233).
+template <int LOSS>
+__global__ __launch_bounds__(256) void k_grads(const float *__restrict__ pred, const float *__restrict__ y,
+                                              float *__restrict__ grad, int64_t N, uint32_t *absmax) {
+    constexpr int K = (LOSS == 2) ? 2 : 1;
+    constexpr int NK = 2 * K + 1;
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    float out[2 * K];
+#pragma unroll
+    for (int k = 0; k < 2 * K; k++) out[k] = 0.0f;
+    if (i < N) {
+        float *g = grad + (size_t)NK * i;
+        float w = g[NK - 1];
+        if (LOSS == 0) {
+            float gg = 2.0f * (pred[i] - y[i]);
+            out[0] = gg * w;
+            out[1] = 2.0f * w;
+        } else if (LOSS == 1) {
+            float s = dev_sigmoid(pred[i]);
+            out[0] = (s - y[i]) * w;
+            out[1] = (s * (1.0f - s)) * w;
+        } else {
+            float loc = pred[2 * i], raw = pred[2 * i + 1];
+            float scale = dev_softplus(raw);
+            float dscale = dev_sigmoid(raw);
+            float resid = loc - y[i];
+            float s2 = scale * scale;
+            float ds = dscale / scale;
+            out[0] = (resid / s2) * w;
+            out[1] = ((1.0f - (resid * resid) / s2) * dscale / scale) * w;
+            out[2] = (1.0f / s2) * w;
+            out[3] = (2.0f * (ds * ds)) * w;
+        }
+#pragma unroll
+        for (int k = 0; k < 2 * K; k++) g[k] = out[k];
+    }
+    // per gradient row max |v| -> exponent bound of the fixed-point histogram
+#pragma unroll
+    for (int k = 0; k < 2 * K; k++) {
+        float m = wave_max_f32(fabsf(out[k]));
+        if ((threadIdx.x & 63) == 0 && m > 0.0f) atomicMax(&absmax[k], __float_as_uint(m));
+    }
+}
+
+// max |v| of every gradient row of an existing gradient matrix (injected gradients, weight row)
+__global__ __launch_bounds__(256) void k_absmax(const float *__restrict__ grad, int64_t N, int NK, int k0, int k1, uint32_t *absmax) {
+    float m[EVT_MAX_NK];
+    for (int k = 0; k < EVT_MAX_NK; k++) m[k] = 0.0f;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256)
+        for (int k = k0; k < k1; k++) m[k] = fmaxf(m[k], fabsf(grad[(size_t)NK * i + k]));
+    for (int k = k0; k < k1; k++) {
+        float v = wave_max_f32(m[k]);
+        if ((threadIdx.x & 63) == 0 && v > 0.0f) atomicMax(&absmax[k], __float_as_uint(v));
+    }
+}
+
+// qexp[k] = ilogb(max) + 1 (0 for an all-zero row); qmul[k] = 2^(qbits-qexp) encodes, qscale decodes.
+__global__ void k_quant_setup(const uint32_t *absmax, const int32_t *qbits, int32_t *qexp, double *qmul, double *qscale_g,
+                              int NK, int NAg, int loss, int unit_w) {
+    int k = threadIdx.x;
+    if (k < NK) {
+        float m = __uint_as_float(absmax[k]);
+        int e = 0;
+        if (m > 0.0f) {
+            e = ilogbf(m) + 1;
+            if (e > 128) e = 128;
+            if (e < -140) e = -140;
+        }
+        qexp[k] = e;
+        qmul[k] = scalbn(1.0, qbits[k] - e);
+    }
+    __syncthreads();
+    if (k < NAg) {
+        // global channel ag -> gradient row: mse {g, w}; otherwise identity; last channel is w (or the row count)
+        int kk = (loss == 0) ? (k == 0 ? 0 : 2) : k;
+        if (k == NAg - 1 && unit_w) qscale_g[k] = 1.0;
+        else qscale_g[k] = scalbn(1.0, qexp[kk] - qbits[kk]);
+    }
+}
+
+// Stages the fixed-point words the histogram kernel adds: plane a of gq holds, per row,
+// q = rint(v * 2^(qbits-qexp)) of gradient row chan_k[a]; with unit weights plane 0 also carries
+// the row count in its low 16 bits ((q << 16) + 1) so that one 64-bit LDS add serves both.
+__global__ __launch_bounds__(256) void k_quantize(const float *__restrict__ grad, unsigned long long *__restrict__ gq, int64_t N,
+                                                 int NK, int NA, int4 chan03, int chan4, const double *__restrict__ qmul, int pack) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N) return;
+    const float *g = grad + (size_t)NK * i;
+    int chan[5] = {chan03.x, chan03.y, chan03.z, chan03.w, chan4};
+#pragma unroll
+    for (int a = 0; a < EVT_MAX_NA; a++) {
+        if (a < NA) {
+            int k = chan[a];
+            long long q = __double2ll_rn((double)g[k] * qmul[k]);
+            unsigned long long word = (unsigned long long)q;
+            if (a == 0 && pack) word = ((unsigned long long)q << EVT_PACK_CNT_BITS) + 1ull;
+            gq[(size_t)a * N + i] = word;
+        }
+    }
+}
+
+int launch_grads(evt_ctx *c) {
+    // absmax of the rows this kernel writes starts from zero; the weight row keeps its value
+    {
+        int r = launch_fill_u32(c, c->absmax, 0u, c->NK - 1);
+        if (r != EVT_OK) return r;
+    }
+    dim3 grid((unsigned)((c->N + 255) / 256));
+    if (c->loss == EVT_LOSS_MSE)
+        hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+    else if (c->loss == EVT_LOSS_LOGLOSS)
+        hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+    else
+        hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+// absmax over rows [k0, k1) of the current gradient matrix
+int launch_absmax_rows(evt_ctx *c, int k0, int k1) {
+    {
+        int r = launch_fill_u32(c, c->absmax + k0, 0u, k1 - k0);
+        if (r != EVT_OK) return r;
+    }
+    int64_t nb = (c->N + 255) / 256;
+    if (nb > 2048) nb = 2048;
+    hipLaunchKernelGGL(k_absmax, dim3((unsigned)nb), dim3(256), 0, c->stream, c->grad, c->N, c->NK, k0, k1, c->absmax);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+int launch_quantize(evt_ctx *c) {
+    double *qmul = c->qscale + 8; // qscale[0..7] decode scales per global channel, [8..15] encode multipliers per gradient row
+    hipLaunchKernelGGL(k_quant_setup, dim3(1), dim3(64), 0, c->stream, c->absmax, c->qbits, c->qexp, qmul, c->qscale, c->NK, c->NAg,
+                       c->loss, c->unit_w ? 1 : 0);
+    HIPCHK(hipGetLastError());
+    int4 c03 = make_int4(c->chan_k[0], c->chan_k[1], c->chan_k[2], c->chan_k[3]);
+    hipLaunchKernelGGL(k_quantize, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, c->gq, c->N, c->NK, c->NA, c03,
+                       c->chan_k[4], qmul, c->unit_w ? 1 : 0);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}

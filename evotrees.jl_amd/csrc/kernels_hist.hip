@@ -1,0 +1,236 @@
+// Histogram builder: the dominant kernel of tree growth (update_hist! / _hist!,
+// src/fit-utils.jl:345-394; device twin ext/EvoTreesKernelAbstractionsExt/fit-utils.jl:57-174).
+//
+// Layout and mapping (gfx950, wave64):
+//  * Rows are read from the observation-major copy of x_bin: one record of RS bytes per row,
+//    fetched as 128-bit loads, LPR = RS/16 lanes per record, 64/LPR rows per wave instruction.
+//    A node's rows are a contiguous, ascending segment of the row-id list, so consecutive lanes
+//    touch consecutive (root: adjacent) records.
+//  * Each lane owns 16 fixed features for the whole kernel; lanes of one record therefore add into
+//    different feature planes of the LDS histogram and same-address collisions inside a wave
+//    instruction can only come from the few rows that share the instruction.
+//  * Accumulators are 64-bit fixed-point integers in LDS (ds_add_u64), one word per
+//    (channel, sampled feature, bin).  Integer sums are exact and order independent, so the
+//    result is bit-identical from run to run and across launch shapes.  With unit weights the
+//    first gradient channel and the row count share one word (count in the low 16 bits), which
+//    makes mse with unit weights a single LDS atomic per (row, feature).
+//  * A block walks a contiguous span of the level's build rows (all build nodes concatenated)
+//    and flushes its LDS histogram to the node's global histogram with 64-bit atomics whenever
+//    the node changes, so the number of flushes is (#blocks + #build nodes) per level.
+//
+// Algorithmic HBM bytes per built row: RS-or-F bin bytes + 8*NA staged gradient bytes + 4 row-id bytes.
+#include "evt_internal.h"
+
+struct HistArgs {
+    const uint8_t *xrm;
+    const unsigned long long *gq;
+    const uint32_t *is;
+    const int64_t *hdr;
+    const int32_t *bnode;
+    const int64_t *bstart;
+    const int64_t *bprefix;
+    const uint16_t *jsmap;
+    long long *hist;
+    int64_t *stats;
+    int64_t N;
+    int64_t node_stride;
+    int RS, LPR, RPW, F, nfs, B, NAg, level;
+    int slots_per_tile;
+};
+
+template <int NA, bool PACK>
+__global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
+    extern __shared__ unsigned long long H[]; // [NA][tile slots][B]
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
+    const int n_build = (int)A.hdr[LH_N_BUILD];
+    const int64_t total = A.hdr[LH_TOTAL_BUILD];
+    if (n_build <= 0 || total <= 0) return;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) A.stats[A.level] = total;
+
+    const int step = nwaves * A.RPW; // rows per block iteration
+    int64_t T = (total + gridDim.x - 1) / gridDim.x;
+    T = ((T + step - 1) / step) * step;
+    int64_t start = (int64_t)blockIdx.x * T;
+    if (start >= total) return;
+    int64_t end = start + T < total ? start + T : total;
+
+    const int slot0 = blockIdx.y * A.slots_per_tile;
+    int nslots = A.nfs - slot0;
+    if (nslots > A.slots_per_tile) nslots = A.slots_per_tile;
+    const int plane = nslots * A.B;
+
+    for (int i = tid; i < NA * plane; i += nthr) H[i] = 0ull;
+
+    // the 16 features this lane owns -> LDS word offset of their first bin (-1: not in this tile)
+    const int sub = lane % A.LPR, rloc = lane / A.LPR;
+    int off[16];
+    bool any = false;
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+        int f = sub * 16 + t;
+        int s = (f < A.F) ? (int)A.jsmap[f] : 0xFFFF;
+        s = (s == 0xFFFF) ? -1 : s - slot0;
+        off[t] = (s >= 0 && s < nslots) ? s * A.B : -1;
+        any |= off[t] >= 0;
+    }
+    const bool lane_on = (rloc < A.RPW) && any;
+    __syncthreads();
+
+    // first node of this block's span: largest i with bprefix[i] <= start
+    int lo = 0, hi = n_build;
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (A.bprefix[mid] <= start) lo = mid; else hi = mid;
+    }
+    int i = lo;
+
+    while (start < end) {
+        const int64_t nxt = A.bprefix[i + 1];
+        const int64_t nend = end < nxt ? end : nxt;
+        const int64_t seg = A.bstart[i] - A.bprefix[i]; // position in the row list = seg + p
+        for (int64_t b0 = start + (int64_t)wave * A.RPW; b0 < nend; b0 += step) {
+            const int64_t p = b0 + rloc;
+            if (lane_on && p < nend) {
+                const uint32_t row = A.is[seg + p];
+                const uint4 v = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)row * A.RS + sub * 16);
+                unsigned long long g[NA];
+#pragma unroll
+                for (int a = 0; a < NA; a++) g[a] = A.gq[(size_t)a * A.N + row];
+                const uint32_t wds[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int t = 0; t < 16; t++) {
+                    const uint32_t bin = (wds[t >> 2] >> (8 * (t & 3))) & 0xFFu;
+                    if (off[t] >= 0 && bin != 0) {
+                        const int idx = off[t] + (int)bin - 1;
+#pragma unroll
+                        for (int a = 0; a < NA; a++) atomicAdd(&H[a * plane + idx], g[a]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        // flush this node's partial histogram: hist[node][slot][ag][bin]
+        long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
+        for (int idx = tid; idx < NA * plane; idx += nthr) {
+            const unsigned long long w = H[idx];
+            if (w != 0ull) {
+                H[idx] = 0ull;
+                const int a = idx / plane;
+                const int rem = idx - a * plane;
+                const int s = rem / A.B;
+                const int bin = rem - s * A.B;
+                unsigned long long *base = reinterpret_cast<unsigned long long *>(hn) + ((int64_t)(slot0 + s) * A.NAg) * A.B + bin;
+                if (PACK && a == 0) {
+                    const long long gsum = (long long)w >> EVT_PACK_CNT_BITS;
+                    const unsigned long long cnt = w & ((1ull << EVT_PACK_CNT_BITS) - 1ull);
+                    if (gsum != 0) atomicAdd(base, (unsigned long long)gsum);
+                    atomicAdd(base + (int64_t)(A.NAg - 1) * A.B, cnt);
+                } else {
+                    atomicAdd(base + (int64_t)a * A.B, w);
+                }
+            }
+        }
+        __syncthreads();
+        start = nend;
+        i++;
+    }
+}
+
+template <int NA, bool PACK>
+static int launch_hist_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
+    static bool attr_set = false;
+    if (!attr_set && lds > 64 * 1024) {
+        HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build<NA, PACK>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((k_hist_build<NA, PACK>), grid, dim3(threads), lds, c->stream, A);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
+    const LevelTab &L = c->lvl[level & 1];
+    const int nfs = c->n_js_last;
+    HistArgs A;
+    A.xrm = c->xrm;
+    A.gq = c->gq;
+    A.is = is_cur;
+    A.hdr = L.hdr;
+    A.bnode = L.bnode;
+    A.bstart = L.bstart;
+    A.bprefix = L.bprefix;
+    A.jsmap = c->jsmap;
+    A.hist = c->hist;
+    A.stats = c->stats;
+    A.N = c->N;
+    A.node_stride = (int64_t)c->F * c->NAg * c->B;
+    A.RS = c->RS;
+    A.LPR = c->LPR;
+    A.RPW = 64 / c->LPR;
+    A.F = c->F;
+    A.nfs = nfs;
+    A.B = c->B;
+    A.NAg = c->NAg;
+    A.level = level;
+    // feature tiling so that one block's LDS histogram stays within budget
+    const size_t budget = 64 * 1024;
+    size_t per_slot = (size_t)c->NA * c->B * 8;
+    int slots_per_tile = (int)(budget / per_slot);
+    if (slots_per_tile < 1) slots_per_tile = 1;
+    if (slots_per_tile > nfs) slots_per_tile = nfs;
+    int ntiles = (nfs + slots_per_tile - 1) / slots_per_tile;
+    slots_per_tile = (nfs + ntiles - 1) / ntiles;
+    A.slots_per_tile = slots_per_tile;
+    size_t lds = per_slot * slots_per_tile;
+    int threads = c->hist_threads;
+    int64_t blocks = c->hist_blocks;
+    int64_t need = (c->N + EVT_HIST_MAX_ROWS_PER_BLOCK - 1) / EVT_HIST_MAX_ROWS_PER_BLOCK;
+    if (blocks < need) blocks = need;
+    dim3 grid((unsigned)blocks, (unsigned)ntiles);
+    const bool pack = c->unit_w;
+#define HCASE(NA_) \
+    case NA_: return pack ? launch_hist_t<NA_, true>(c, A, grid, threads, lds) : launch_hist_t<NA_, false>(c, A, grid, threads, lds);
+    switch (c->NA) {
+        HCASE(1)
+        HCASE(2)
+        HCASE(3)
+        HCASE(4)
+        HCASE(5)
+    }
+#undef HCASE
+    evt_set_error("unsupported channel count %d", c->NA);
+    return EVT_ERR_ARG;
+}
+
+// Reference-layout export for parity checks: out[k, bin, feat, node] Float64 (src/init.jl:204).
+__global__ __launch_bounds__(256) void k_hist_export(const long long *__restrict__ hist, const uint32_t *__restrict__ js, int nfs, int F,
+                                                    int B, int NK, int NAg, int loss, const double *__restrict__ qscale,
+                                                    const int32_t *__restrict__ status, int nnodes, int last_level_first, double *out) {
+    int node = blockIdx.x; // 0-based
+    if (node + 1 >= last_level_first) return; // nodes of the last level never get a histogram
+    int st = status[node + 1];
+    if (st != ST_SPLIT && st != ST_LEAF) return;
+    const long long *hn = hist + (int64_t)node * F * NAg * B;
+    for (int idx = threadIdx.x; idx < nfs * B; idx += 256) {
+        int jp = idx / B, b = idx - jp * B;
+        int f = (int)js[jp] - 1;
+        double ch[EVT_MAX_NA];
+        for (int ag = 0; ag < NAg; ag++) ch[ag] = (double)hn[((int64_t)jp * NAg + ag) * B + b] * qscale[ag];
+        double *o = out + (((int64_t)node * F + f) * B + b) * NK;
+        if (loss == 0) {
+            o[0] = ch[0];
+            o[1] = 2.0 * ch[1];
+            o[2] = ch[1];
+        } else {
+            for (int k = 0; k < NK; k++) o[k] = ch[k];
+        }
+    }
+}
+
+int launch_hist_export(evt_ctx *c, double *out_dev) {
+    hipLaunchKernelGGL(k_hist_export, dim3((unsigned)c->nnodes), dim3(256), 0, c->stream, c->hist, c->js, c->n_js_last, c->F, c->B, c->NK,
+                       c->NAg, c->loss, c->qscale, c->status, c->nnodes, 1 << (c->D - 1), out_dev);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}

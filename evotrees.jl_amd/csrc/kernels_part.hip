@@ -1,0 +1,495 @@
+// Row partitioning and level bookkeeping, all device resident.
+//
+// split_set! (src/fit-utils.jl:93-312) is a stable partition of each split node's row-id segment;
+// update_nodes_idx_kernel! (ext/EvoTreesKernelAbstractionsExt/fit-utils.jl:9-31) is the same
+// decision written per row.  Here every node owns a contiguous segment [seg_start, seg_start+seg_len)
+// of the row-id list; a split rewrites the segment in place order (lefts first, both sides keeping
+// ascending row ids) into the other list buffer, so children are again contiguous segments.
+// Segments are cut into chunks of EVT_CHUNK rows that never cross a node boundary:
+//   count   : one block per chunk evaluates x_bin[row, feat] <= cond_bin, keeps the ballots,
+//             counts lefts;
+//   next    : one block scans the chunk counts, sets the children's segments, picks which child
+//             is built (fewer rows; tie -> left, src/fit.jl:123-129) and writes the next level's
+//             tables (active nodes, chunk prefix, build list);
+//   scatter : one block per chunk moves row ids to their stable destination; chunks of nodes that
+//             became leaves record the node id per row (and add the leaf value to the prediction).
+// No host round trip is needed between levels.
+#include "evt_internal.h"
+
+// largest i in [0, n) with pre[i] <= v   (pre ascending, pre[0] <= v)
+__device__ __forceinline__ int find_owner(const int64_t *pre, int n, int64_t v) {
+    int lo = 0, hi = n;
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (pre[mid] <= v) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+struct PartArgs {
+    const int64_t *hdr;
+    const int32_t *act_node;
+    const int64_t *cprefix;
+    const int32_t *status;
+    const int64_t *seg_start;
+    const int64_t *seg_len;
+    const int32_t *t_feat;
+    const uint8_t *t_bin;
+    const uint8_t *feattypes;
+    const uint8_t *xcm;
+    int64_t N;
+    const uint32_t *is_cur;
+    uint32_t *is_next;
+    unsigned long long *flagw;
+    int32_t *chunk_nleft;
+    const int64_t *chunk_lpre;
+    // leaf finalisation
+    uint32_t *nidx;
+    float *pred;
+    const float *t_pred;
+    int K, loss, fuse_pred;
+};
+
+__global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n_act = (int)A.hdr[LH_N_ACT];
+    const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
+    __shared__ int s_cnt[4];
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const int i = find_owner(A.cprefix, n_act, c);
+        const int n = A.act_node[i];
+        if (A.status[n] != ST_SPLIT) {
+            if (tid == 0) A.chunk_nleft[c] = 0;
+            continue;
+        }
+        const int64_t cl = c - A.cprefix[i];
+        const int64_t seg = A.seg_start[n], len = A.seg_len[n];
+        const int64_t p0 = seg + cl * EVT_CHUNK;
+        const int64_t pend = seg + len;
+        const int f = A.t_feat[n - 1] - 1;
+        const uint32_t cb = A.t_bin[n - 1];
+        const bool numeric = A.feattypes[f] != 0;
+        const uint8_t *col = A.xcm + (size_t)f * A.N;
+        int cnt = 0;
+#pragma unroll
+        for (int it = 0; it < EVT_CHUNK / 256; it++) {
+            const int64_t p = p0 + it * 256 + tid;
+            bool flag = false;
+            if (p < pend) {
+                const uint32_t xb = col[A.is_cur[p]];
+                flag = numeric ? (xb <= cb) : (xb == cb);
+            }
+            const unsigned long long bal = __ballot(flag);
+            if (lane == 0) A.flagw[c * EVT_CHUNK_WORDS + it * 4 + wave] = bal;
+            cnt += __popcll(bal);
+        }
+        if (lane == 0) s_cnt[wave] = cnt;
+        __syncthreads();
+        if (tid == 0) A.chunk_nleft[c] = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n_act = (int)A.hdr[LH_N_ACT];
+    const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
+    __shared__ unsigned long long s_w[EVT_CHUNK_WORDS];
+    __shared__ int s_pre[EVT_CHUNK_WORDS];
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const int i = find_owner(A.cprefix, n_act, c);
+        const int n = A.act_node[i];
+        const int st = A.status[n];
+        const int64_t cl = c - A.cprefix[i];
+        const int64_t seg = A.seg_start[n], len = A.seg_len[n];
+        const int64_t p0 = seg + cl * EVT_CHUNK;
+        const int64_t pend = seg + len;
+        if (st == ST_SPLIT) {
+            if (tid < EVT_CHUNK_WORDS) s_w[tid] = A.flagw[c * EVT_CHUNK_WORDS + tid];
+            __syncthreads();
+            if (tid == 0) {
+                int run = 0;
+                for (int t = 0; t < EVT_CHUNK_WORDS; t++) { s_pre[t] = run; run += __popcll(s_w[t]); }
+            }
+            __syncthreads();
+            const int64_t lbase = A.chunk_lpre[c] - A.chunk_lpre[A.cprefix[i]]; // lefts of this node before this chunk
+            const int64_t nl_node = A.seg_len[2 * n];
+            const int64_t dstL = seg + lbase;
+            const int64_t dstR = seg + nl_node + (cl * EVT_CHUNK - lbase);
+#pragma unroll
+            for (int it = 0; it < EVT_CHUNK / 256; it++) {
+                const int64_t p = p0 + it * 256 + tid;
+                if (p < pend) {
+                    const int wi = it * 4 + wave;
+                    const unsigned long long word = s_w[wi];
+                    const int lrank = s_pre[wi] + __popcll(word & ((1ull << lane) - 1ull));
+                    const bool flag = (word >> lane) & 1ull;
+                    const int within = it * 256 + tid;
+                    const uint32_t row = A.is_cur[p];
+                    const int64_t d = flag ? (dstL + lrank) : (dstR + (within - lrank));
+                    A.is_next[d] = row;
+                }
+            }
+            __syncthreads();
+        } else if (st == ST_LEAF) {
+            // rows of a node that stops here: record the node id; add the leaf value
+            // (predict!, src/predict.jl:1-46: plain add / clamp(-15,15) / floor -15 on scale rows)
+            const int K = A.K;
+#pragma unroll
+            for (int it = 0; it < EVT_CHUNK / 256; it++) {
+                const int64_t p = p0 + it * 256 + tid;
+                if (p < pend) {
+                    const uint32_t row = A.is_cur[p];
+                    A.nidx[row] = (uint32_t)n;
+                    if (A.fuse_pred) {
+                        float *pr = A.pred + (size_t)K * row;
+                        const float *lp = A.t_pred + (size_t)K * (n - 1);
+                        if (A.loss == EVT_LOSS_MSE) {
+                            for (int k = 0; k < K; k++) pr[k] += lp[k];
+                        } else if (A.loss == EVT_LOSS_LOGLOSS) {
+                            for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
+                        } else {
+                            for (int t = 0; t < K / 2; t++) {
+                                pr[2 * t] += lp[2 * t];
+                                pr[2 * t + 1] = fmaxf(-15.0f, pr[2 * t + 1] + lp[2 * t + 1]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- single-block scans -----------------------------------------------------------------------
+// Exclusive prefix over the 1024 threads of the block; returns the prefix, *total gets the sum.
+__device__ long long block_excl_scan(long long v, long long *total, long long *s_tmp /* [17] */) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    long long x = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        int lo = __shfl_up((int)(x & 0xffffffffll), o), hi = __shfl_up((int)(x >> 32), o);
+        long long y = ((long long)hi << 32) | (unsigned int)lo;
+        if (lane >= o) x += y;
+    }
+    __syncthreads(); // s_tmp may still be read from a previous call
+    if (lane == 63) s_tmp[wave] = x;
+    __syncthreads();
+    if (tid == 0) {
+        long long run = 0;
+        const int nw = blockDim.x >> 6;
+        for (int w = 0; w < nw; w++) { long long t = s_tmp[w]; s_tmp[w] = run; run += t; }
+        s_tmp[16] = run;
+    }
+    __syncthreads();
+    *total = s_tmp[16];
+    return s_tmp[wave] + x - v;
+}
+
+struct NextArgs {
+    const int64_t *hdr;
+    const int32_t *act_node;
+    const int64_t *cprefix;
+    int32_t *status;
+    int64_t *seg_start;
+    int64_t *seg_len;
+    const int32_t *chunk_nleft;
+    int64_t *chunk_lpre;
+    // next level
+    int64_t *n_hdr;
+    int32_t *n_act_node;
+    int64_t *n_cprefix;
+    int32_t *n_bnode;
+    int64_t *n_bstart;
+    int64_t *n_bprefix;
+};
+
+__global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
+    const int tid = threadIdx.x;
+    __shared__ long long s_tmp[17];
+    const int n_act = (int)A.hdr[LH_N_ACT];
+    const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
+    long long total;
+    // A: exclusive scan of the chunks' left counts
+    {
+        const int64_t span = (n_chunks + 1023) / 1024;
+        const int64_t c0 = (int64_t)tid * span, c1 = (c0 + span < n_chunks) ? c0 + span : n_chunks;
+        long long s = 0;
+        for (int64_t c = c0; c < c1; c++) s += A.chunk_nleft[c];
+        long long pre = block_excl_scan(s, &total, s_tmp);
+        for (int64_t c = c0; c < c1; c++) { A.chunk_lpre[c] = pre; pre += A.chunk_nleft[c]; }
+        if (tid == 0) A.chunk_lpre[n_chunks] = total;
+    }
+    __syncthreads();
+    // B: children segments + three scans over the active nodes (children count, chunks, build rows)
+    const int span = (n_act + 1023) / 1024;
+    const int i0 = tid * span, i1 = (i0 + span < n_act) ? i0 + span : n_act;
+    long long s_pos = 0, s_chunks = 0, s_brows = 0;
+    for (int i = i0; i < i1; i++) {
+        const int n = A.act_node[i];
+        if (A.status[n] != ST_SPLIT) continue;
+        const int64_t nl = A.chunk_lpre[A.cprefix[i + 1]] - A.chunk_lpre[A.cprefix[i]];
+        const int64_t len = A.seg_len[n], start = A.seg_start[n];
+        const int64_t nr = len - nl;
+        A.seg_start[2 * n] = start;
+        A.seg_len[2 * n] = nl;
+        A.seg_start[2 * n + 1] = start + nl;
+        A.seg_len[2 * n + 1] = nr;
+        const bool build_left = nr >= nl; // the smaller child is built, tie -> left (src/fit.jl:123-129)
+        A.status[2 * n] = build_left ? ST_BUILD : ST_SUBTRACT;
+        A.status[2 * n + 1] = build_left ? ST_SUBTRACT : ST_BUILD;
+        s_pos += 1;
+        s_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
+        s_brows += build_left ? nl : nr;
+    }
+    long long t_pos, t_chunks, t_brows;
+    long long p_pos = block_excl_scan(s_pos, &t_pos, s_tmp);
+    long long p_chunks = block_excl_scan(s_chunks, &t_chunks, s_tmp);
+    long long p_brows = block_excl_scan(s_brows, &t_brows, s_tmp);
+    for (int i = i0; i < i1; i++) {
+        const int n = A.act_node[i];
+        if (A.status[n] != ST_SPLIT) continue;
+        const int64_t nl = A.seg_len[2 * n], nr = A.seg_len[2 * n + 1];
+        const bool build_left = nr >= nl;
+        A.n_act_node[2 * p_pos] = 2 * n;
+        A.n_act_node[2 * p_pos + 1] = 2 * n + 1;
+        A.n_cprefix[2 * p_pos] = p_chunks;
+        A.n_cprefix[2 * p_pos + 1] = p_chunks + (nl + EVT_CHUNK - 1) / EVT_CHUNK;
+        A.n_bnode[p_pos] = build_left ? 2 * n : 2 * n + 1;
+        A.n_bstart[p_pos] = build_left ? A.seg_start[2 * n] : A.seg_start[2 * n + 1];
+        A.n_bprefix[p_pos] = p_brows;
+        p_pos += 1;
+        p_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
+        p_brows += build_left ? nl : nr;
+    }
+    if (tid == 0) {
+        A.n_cprefix[2 * t_pos] = t_chunks;
+        A.n_bprefix[t_pos] = t_brows;
+        A.n_hdr[LH_N_ACT] = 2 * t_pos;
+        A.n_hdr[LH_N_CHUNKS] = t_chunks;
+        A.n_hdr[LH_N_BUILD] = t_pos;
+        A.n_hdr[LH_TOTAL_BUILD] = t_brows;
+    }
+}
+
+// Start of a tree: zero the Tree arrays (Tree{L,K}(depth), src/structs.jl:97-106) and node states,
+// make the root the only active (build) node over rows [0, n_is), zero its histogram slice.
+struct BeginArgs {
+    TreeDev tree;
+    int32_t *status;
+    int64_t *seg_start;
+    int64_t *seg_len;
+    int64_t *hdr;
+    int32_t *act_node;
+    int64_t *cprefix;
+    int32_t *bnode;
+    int64_t *bstart;
+    int64_t *bprefix;
+    long long *hist;
+    int64_t *stats;
+    int64_t n_is;
+    int64_t root_words;
+    int nnodes, K, D;
+};
+
+__global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) {
+    const int tid = threadIdx.x;
+    for (int n = tid; n < A.nnodes; n += 1024) {
+        A.tree.feat[n] = 0;
+        A.tree.cond_bin[n] = 0;
+        A.tree.w[n] = 0.0f;
+        A.tree.gain[n] = 0.0f;
+        A.tree.split[n] = 0;
+        A.tree.packed[n] = 0u;
+        for (int k = 0; k < A.K; k++) A.tree.pred[(int64_t)A.K * n + k] = 0.0f;
+    }
+    for (int n = tid; n < A.nnodes + 2; n += 1024) A.status[n] = ST_INACTIVE;
+    for (int64_t i = tid; i < A.root_words; i += 1024) A.hist[i] = 0;
+    for (int d = tid; d <= A.D; d += 1024) A.stats[d] = 0;
+    __syncthreads();
+    if (tid == 0) {
+        A.status[1] = ST_BUILD;
+        A.seg_start[1] = 0;
+        A.seg_len[1] = A.n_is;
+        A.hdr[LH_N_ACT] = 1;
+        A.hdr[LH_N_CHUNKS] = (A.n_is + EVT_CHUNK - 1) / EVT_CHUNK;
+        A.hdr[LH_N_BUILD] = 1;
+        A.hdr[LH_TOTAL_BUILD] = A.n_is;
+        A.act_node[0] = 1;
+        A.cprefix[0] = 0;
+        A.cprefix[1] = (A.n_is + EVT_CHUNK - 1) / EVT_CHUNK;
+        A.bnode[0] = 1;
+        A.bstart[0] = 0;
+        A.bprefix[0] = 0;
+        A.bprefix[1] = A.n_is;
+    }
+}
+
+// ---- row subsampling: is = rows with mask <= cond, ascending (src/subsample.jl:6-38) -----------
+__global__ __launch_bounds__(256) void k_mask_count(const uint8_t *mask, uint8_t cond, int64_t N, int64_t n_chunks,
+                                                   unsigned long long *flagw, int32_t *chunk_nleft) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __shared__ int s_cnt[4];
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        int cnt = 0;
+#pragma unroll
+        for (int it = 0; it < EVT_CHUNK / 256; it++) {
+            const int64_t p = c * EVT_CHUNK + it * 256 + tid;
+            const bool flag = (p < N) && (mask[p] <= cond);
+            const unsigned long long bal = __ballot(flag);
+            if (lane == 0) flagw[c * EVT_CHUNK_WORDS + it * 4 + wave] = bal;
+            cnt += __popcll(bal);
+        }
+        if (lane == 0) s_cnt[wave] = cnt;
+        __syncthreads();
+        if (tid == 0) chunk_nleft[c] = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(1024) void k_mask_scan(const int32_t *chunk_nleft, int64_t *chunk_lpre, int64_t n_chunks) {
+    __shared__ long long s_tmp[17];
+    const int tid = threadIdx.x;
+    const int64_t span = (n_chunks + 1023) / 1024;
+    const int64_t c0 = (int64_t)tid * span, c1 = (c0 + span < n_chunks) ? c0 + span : n_chunks;
+    long long s = 0, total;
+    for (int64_t c = c0; c < c1; c++) s += chunk_nleft[c];
+    long long pre = block_excl_scan(s, &total, s_tmp);
+    for (int64_t c = c0; c < c1; c++) { chunk_lpre[c] = pre; pre += chunk_nleft[c]; }
+    if (tid == 0) chunk_lpre[n_chunks] = total;
+}
+
+__global__ __launch_bounds__(256) void k_mask_scatter(int64_t N, int64_t n_chunks, const unsigned long long *flagw,
+                                                     const int64_t *chunk_lpre, uint32_t *is_out) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __shared__ unsigned long long s_w[EVT_CHUNK_WORDS];
+    __shared__ int s_pre[EVT_CHUNK_WORDS];
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        if (tid < EVT_CHUNK_WORDS) s_w[tid] = flagw[c * EVT_CHUNK_WORDS + tid];
+        __syncthreads();
+        if (tid == 0) {
+            int run = 0;
+            for (int t = 0; t < EVT_CHUNK_WORDS; t++) { s_pre[t] = run; run += __popcll(s_w[t]); }
+        }
+        __syncthreads();
+        const int64_t base = chunk_lpre[c];
+#pragma unroll
+        for (int it = 0; it < EVT_CHUNK / 256; it++) {
+            const int64_t p = c * EVT_CHUNK + it * 256 + tid;
+            const int wi = it * 4 + wave;
+            const unsigned long long word = s_w[wi];
+            if ((word >> lane) & 1ull) is_out[base + s_pre[wi] + __popcll(word & ((1ull << lane) - 1ull))] = (uint32_t)p;
+        }
+        __syncthreads();
+    }
+}
+
+static unsigned grid_for_chunks(int64_t max_chunks) {
+    int64_t g = max_chunks;
+    if (g > 4096) g = 4096;
+    if (g < 1) g = 1;
+    return (unsigned)g;
+}
+
+int launch_compact_mask(evt_ctx *c, uint8_t cond, int64_t n_is) {
+    const int64_t n_chunks = (c->N + EVT_CHUNK - 1) / EVT_CHUNK;
+    unsigned g = grid_for_chunks(n_chunks);
+    hipLaunchKernelGGL(k_mask_count, dim3(g), dim3(256), 0, c->stream, c->mask, cond, c->N, n_chunks, c->flagw, c->chunk_nleft);
+    HIPCHK(hipGetLastError());
+    hipLaunchKernelGGL(k_mask_scan, dim3(1), dim3(1024), 0, c->stream, c->chunk_nleft, c->chunk_lpre, n_chunks);
+    HIPCHK(hipGetLastError());
+    hipLaunchKernelGGL(k_mask_scatter, dim3(g), dim3(256), 0, c->stream, c->N, n_chunks, c->flagw, c->chunk_lpre, c->is_a);
+    HIPCHK(hipGetLastError());
+    (void)n_is;
+    return EVT_OK;
+}
+
+int launch_tree_begin(evt_ctx *c, int64_t n_is) {
+    const LevelTab &L = c->lvl[1];
+    BeginArgs A;
+    A.tree = c->tree;
+    A.status = c->status;
+    A.seg_start = c->seg_start;
+    A.seg_len = c->seg_len;
+    A.hdr = L.hdr;
+    A.act_node = L.act_node;
+    A.cprefix = L.cprefix;
+    A.bnode = L.bnode;
+    A.bstart = L.bstart;
+    A.bprefix = L.bprefix;
+    A.hist = c->hist;
+    A.stats = c->stats;
+    A.n_is = n_is;
+    A.root_words = (int64_t)c->n_js_last * c->NAg * c->B;
+    A.nnodes = c->nnodes;
+    A.K = c->K;
+    A.D = c->D;
+    hipLaunchKernelGGL(k_tree_begin, dim3(1), dim3(1024), 0, c->stream, A);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred, PartArgs &A) {
+    const LevelTab &L = c->lvl[level & 1];
+    A.hdr = L.hdr;
+    A.act_node = L.act_node;
+    A.cprefix = L.cprefix;
+    A.status = c->status;
+    A.seg_start = c->seg_start;
+    A.seg_len = c->seg_len;
+    A.t_feat = c->tree.feat;
+    A.t_bin = c->tree.cond_bin;
+    A.feattypes = c->feattypes;
+    A.xcm = c->xcm;
+    A.N = c->N;
+    A.is_cur = is_cur;
+    A.is_next = is_next;
+    A.flagw = c->flagw;
+    A.chunk_nleft = c->chunk_nleft;
+    A.chunk_lpre = c->chunk_lpre;
+    A.nidx = c->nidx;
+    A.pred = c->pred;
+    A.t_pred = c->tree.pred;
+    A.K = c->K;
+    A.loss = c->loss;
+    A.fuse_pred = fuse_pred ? 1 : 0;
+}
+
+int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur) {
+    PartArgs A;
+    fill_part_args(c, level, is_cur, nullptr, false, A);
+    hipLaunchKernelGGL(k_part_count, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred) {
+    PartArgs A;
+    fill_part_args(c, level, is_cur, is_next, fuse_pred, A);
+    hipLaunchKernelGGL(k_part_scatter, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+int launch_level_next(evt_ctx *c, int level) {
+    const LevelTab &L = c->lvl[level & 1];
+    const LevelTab &Nx = c->lvl[(level + 1) & 1];
+    NextArgs A;
+    A.hdr = L.hdr;
+    A.act_node = L.act_node;
+    A.cprefix = L.cprefix;
+    A.status = c->status;
+    A.seg_start = c->seg_start;
+    A.seg_len = c->seg_len;
+    A.chunk_nleft = c->chunk_nleft;
+    A.chunk_lpre = c->chunk_lpre;
+    A.n_hdr = Nx.hdr;
+    A.n_act_node = Nx.act_node;
+    A.n_cprefix = Nx.cprefix;
+    A.n_bnode = Nx.bnode;
+    A.n_bstart = Nx.bstart;
+    A.n_bprefix = Nx.bprefix;
+    hipLaunchKernelGGL(k_level_next, dim3(1), dim3(1024), 0, c->stream, A);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}

@@ -1,0 +1,106 @@
+// Tree traversal: predict! (src/predict.jl:1-46), predict_leaf_idx! (:138-154), _predict (:118-136).
+//
+// A node is packed in one 32-bit word (feat | cond_bin << 16 | split << 24) so that each visited
+// node costs one cached 4-byte load.  Rows are independent; per row the walk reads one bin byte
+// per level from the column-major x_bin (neighbouring rows share 64-byte sectors of a column).
+#include "evt_internal.h"
+
+__device__ __forceinline__ int walk_packed(const uint32_t *__restrict__ nodes, const uint8_t *__restrict__ xcm, int64_t N, int64_t i,
+                                           const uint8_t *__restrict__ feattypes) {
+    int nid = 1;
+    uint32_t nd = nodes[0];
+    while (nd >> 24) {
+        const int feat = (int)(nd & 0xFFFFu);
+        const uint32_t cb = (nd >> 16) & 0xFFu;
+        const uint32_t xb = xcm[(size_t)(feat - 1) * N + i];
+        const bool cond = feattypes[feat - 1] ? (xb <= cb) : (xb == cb);
+        nid = (nid << 1) + (cond ? 0 : 1);
+        nd = nodes[nid - 1];
+    }
+    return nid;
+}
+
+__device__ __forceinline__ void add_leaf(float *pr, const float *lp, int K, int loss) {
+    if (loss == EVT_LOSS_MSE) {
+        for (int k = 0; k < K; k++) pr[k] += lp[k];
+    } else if (loss == EVT_LOSS_LOGLOSS) {
+        for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
+    } else {
+        for (int t = 0; t < K / 2; t++) {
+            pr[2 * t] += lp[2 * t];
+            pr[2 * t + 1] = fmaxf(-15.0f, pr[2 * t + 1] + lp[2 * t + 1]);
+        }
+    }
+}
+
+// one tree added to pred (K x N), all rows
+__global__ __launch_bounds__(256) void k_predict_tree(const uint32_t *__restrict__ nodes, const float *__restrict__ leaf_pred,
+                                                     const uint8_t *__restrict__ xcm, const uint8_t *__restrict__ feattypes, int64_t N,
+                                                     int K, int loss, float *pred) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N) return;
+    const int nid = walk_packed(nodes, xcm, N, i, feattypes);
+    add_leaf(pred + (size_t)K * i, leaf_pred + (size_t)K * (nid - 1), K, loss);
+}
+
+int launch_predict_tree_cache(evt_ctx *c) {
+    hipLaunchKernelGGL(k_predict_tree, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->tree.packed, c->tree.pred, c->xcm,
+                       c->feattypes, c->N, c->K, c->loss, c->pred);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, const float *leaf_pred_dev) {
+    hipLaunchKernelGGL(k_predict_tree, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, nodes_dev, leaf_pred_dev, c->xcm,
+                       c->feattypes, c->N, c->K, c->loss, c->pred);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+// whole model: trees concatenated, tree t owns nodes [off[t], off[t+1]); the running prediction
+// stays in registers and is written once.  The per-tree clamps are applied after every tree, as
+// predict! does.
+__global__ __launch_bounds__(256) void k_predict_model(const uint32_t *__restrict__ nodes, const float *__restrict__ leaf_pred,
+                                                      const int64_t *__restrict__ off, int ntrees, const uint8_t *__restrict__ xcm,
+                                                      const uint8_t *__restrict__ feattypes, int64_t N, int K, int loss, int apply_link,
+                                                      float *out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N) return;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int t = 0; t < ntrees; t++) {
+        const int64_t o = off[t];
+        const int nid = walk_packed(nodes + o, xcm, N, i, feattypes);
+        add_leaf(acc, leaf_pred + (size_t)K * (o + nid - 1), K, loss);
+    }
+    if (apply_link) { // apply_prediction_link!, src/predict.jl:105-116
+        if (loss == EVT_LOSS_LOGLOSS) {
+            for (int k = 0; k < K; k++) acc[k] = 1.0f / (1.0f + expf(-acc[k]));
+        } else if (loss == EVT_LOSS_GAUSSIAN_MLE) {
+            for (int k = 1; k < K; k += 2) acc[k] = fmaxf(acc[k], 0.0f) + log1pf(expf(-fabsf(acc[k])));
+        }
+    }
+    for (int k = 0; k < K; k++) out[(size_t)K * i + k] = acc[k];
+}
+
+__global__ __launch_bounds__(256) void k_leaf_idx_model(const uint32_t *__restrict__ nodes, const int64_t *__restrict__ off, int ntrees,
+                                                       const uint8_t *__restrict__ xcm, const uint8_t *__restrict__ feattypes, int64_t N,
+                                                       uint32_t *out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N) return;
+    for (int t = 0; t < ntrees; t++) out[(size_t)t * N + i] = (uint32_t)walk_packed(nodes + off[t], xcm, N, i, feattypes);
+}
+
+int launch_predict_model(hipStream_t s, const uint32_t *nodes, const float *leaf_pred, const int64_t *off, int ntrees, const uint8_t *xcm,
+                         const uint8_t *feattypes, int64_t N, int K, int loss, int apply_link, float *out) {
+    hipLaunchKernelGGL(k_predict_model, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, nodes, leaf_pred, off, ntrees, xcm, feattypes, N, K,
+                       loss, apply_link, out);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+int launch_leaf_idx_model(hipStream_t s, const uint32_t *nodes, const int64_t *off, int ntrees, const uint8_t *xcm, const uint8_t *feattypes,
+                          int64_t N, uint32_t *out) {
+    hipLaunchKernelGGL(k_leaf_idx_model, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, nodes, off, ntrees, xcm, feattypes, N, out);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}

@@ -1,0 +1,467 @@
+// Split search: subtract_hist! + _scan_node!/get_best_split + _child_sums! + leaf values
+// (src/fit-utils.jl:321-332, :403-486; src/split.jl:1, :58-66, :108-117; src/predict.jl:198-234).
+//
+// One block per node of the level; each wave takes sampled features round-robin; lanes are bins.
+// The left sums of all bins of one (node, feature) come from one wavefront inclusive prefix scan
+// of the int64 histogram (DPP row shifts + row broadcasts), the candidate gains are evaluated in
+// Float64 with the reference's expression order, and the best candidate is found with a
+// cross-lane arg-max whose ties go to the lowest bin, then the earliest feature of js — the
+// reference's "first maximum wins" (strict '>' at src/fit-utils.jl:447).
+#include "evt_internal.h"
+#include <float.h>
+
+#define NO_BIN 0x7fffffff
+
+struct ScanArgs {
+    long long *hist;
+    int64_t node_stride;
+    const uint32_t *js;
+    const uint8_t *feattypes;
+    const int32_t *mono;
+    int32_t *status;
+    long long *node_sum;
+    const double *qscale;
+    TreeDev tree;
+    double *ogains;
+    double eta, lambda, L2, gamma, min_weight;
+    int bagging;
+    int nfs, B, F, K, NK, NAg, loss, level, leaf_level, oblivious, zero_children;
+};
+
+// ---- wavefront primitives -----------------------------------------------------------------
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ long long dpp_move_i64(long long x) {
+    int lo = (int)(x & 0xffffffffll), hi = (int)(x >> 32);
+    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROW_MASK, 0xf, false);
+    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROW_MASK, 0xf, false);
+    return ((long long)hi << 32) | (unsigned int)lo;
+}
+
+// Inclusive prefix sum over the 64 lanes of a wavefront.
+// row_shr:1,2,4,8 scan each row of 16 lanes; row_bcast:15 then row_bcast:31 carry row totals forward.
+__device__ __forceinline__ long long wave_incl_scan_i64(long long x) {
+    x += dpp_move_i64<0x111, 0xf>(x); // row_shr:1
+    x += dpp_move_i64<0x112, 0xf>(x); // row_shr:2
+    x += dpp_move_i64<0x114, 0xf>(x); // row_shr:4
+    x += dpp_move_i64<0x118, 0xf>(x); // row_shr:8
+    x += dpp_move_i64<0x142, 0xa>(x); // row_bcast:15 into rows 1 and 3
+    x += dpp_move_i64<0x143, 0xc>(x); // row_bcast:31 into rows 2 and 3
+    return x;
+}
+
+__device__ __forceinline__ long long wave_sum_i64(long long x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        int lo = __shfl_xor((int)(x & 0xffffffffll), o), hi = __shfl_xor((int)(x >> 32), o);
+        x += ((long long)hi << 32) | (unsigned int)lo;
+    }
+    return x;
+}
+
+__device__ __forceinline__ double shfl_xor_f64(double v, int o) {
+    long long b = __double_as_longlong(v);
+    int lo = __shfl_xor((int)(b & 0xffffffffll), o), hi = __shfl_xor((int)(b >> 32), o);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
+// ---- Float64 gain algebra, expression order as in the reference ------------------------------
+__device__ __forceinline__ double term_gh(double g, double h, double w, double lambda, double L2) {
+    double d = h + lambda * w + L2;
+    if (!(d > DBL_EPSILON)) d = DBL_EPSILON;
+    return g * g / d / 2.0;
+}
+
+// fixed-point channel sums -> the 2K+1 Float64 statistics [g.., h.., w]
+__device__ __forceinline__ void decode_vals(const long long *q, const double *sc, int loss, int NK, double *out) {
+    if (loss == EVT_LOSS_MSE) {
+        double w = (double)q[1] * sc[1];
+        out[0] = (double)q[0] * sc[0];
+        out[1] = 2.0 * w;
+        out[2] = w;
+    } else {
+        for (int k = 0; k < NK; k++) out[k] = (double)q[k] * sc[k];
+    }
+}
+
+__device__ __forceinline__ double leaf_value(const double *S, int k, int K, double eta, int bagging, double lambda, double L2) {
+    double d = S[K + k] + lambda * S[2 * K] + L2;
+    if (!(d > DBL_EPSILON)) d = DBL_EPSILON;
+    return -eta / (double)bagging * S[k] / d;
+}
+
+template <int NAG>
+__global__ __launch_bounds__(1024) void k_scan(ScanArgs A) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int n = (1 << (A.level - 1)) + blockIdx.x; // 1-based node id
+    const int st = A.status[n];
+    if (st != ST_BUILD && st != ST_SUBTRACT) return;
+    const bool is_sub = (st == ST_SUBTRACT);
+    const int B = A.B, NK = A.NK, K = A.K;
+    const int BPL = (B + 63) >> 6; // bins per lane (<= 4)
+    long long *hn = A.hist + (int64_t)(n - 1) * A.node_stride;
+    const long long *hp = A.hist + (int64_t)((n >> 1) - 1) * A.node_stride;
+    const long long *hs = A.hist + (int64_t)((n ^ 1) - 1) * A.node_stride;
+
+    __shared__ long long s_Sq[EVT_MAX_NA];
+    __shared__ double s_S[EVT_MAX_NK];
+    __shared__ double s_sc[EVT_MAX_NA];
+    __shared__ double s_wg[16];
+    __shared__ int s_wjp[16], s_wbin[16];
+    __shared__ int s_dec[4]; // found, jp, bin
+    __shared__ double s_gain;
+
+    if (tid < NAG) s_sc[tid] = A.qscale[tid];
+    // node totals: carried from the parent's split, except the root whose totals are the bin sums
+    // of its first sampled feature (exact in integers, any feature gives the same total)
+    if (A.level == 1) {
+        if (wave == 0) {
+            for (int ag = 0; ag < NAG; ag++) {
+                long long s = 0;
+                for (int b = lane; b < B; b += 64) s += hn[(int64_t)ag * B + b];
+                s = wave_sum_i64(s);
+                if (lane == 0) { s_Sq[ag] = s; A.node_sum[(int64_t)n * NAG + ag] = s; }
+            }
+        }
+    } else if (tid < NAG) {
+        s_Sq[tid] = A.node_sum[(int64_t)n * NAG + tid];
+    }
+    __syncthreads();
+    if (tid == 0) {
+        double v[EVT_MAX_NK];
+        long long q[NAG];
+        for (int ag = 0; ag < NAG; ag++) q[ag] = s_Sq[ag];
+        decode_vals(q, s_sc, A.loss, NK, v);
+        for (int k = 0; k < NK; k++) s_S[k] = v[k];
+        A.tree.w[n - 1] = (float)v[NK - 1];
+    }
+    __syncthreads();
+    double S[EVT_MAX_NK];
+    for (int k = 0; k < NK; k++) S[k] = s_S[k];
+
+    if (A.leaf_level) {
+        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
+        if (tid == 0) A.status[n] = ST_LEAF;
+        return;
+    }
+
+    double gain_p = 0.0;
+    for (int k = 0; k < K; k++) gain_p += term_gh(S[k], S[K + k], S[2 * K], A.lambda, A.L2);
+    const double w_p = S[NK - 1];
+
+    double wbest = -INFINITY;
+    int wjp = NO_BIN, wbin = NO_BIN;
+    const int nodeidx = blockIdx.x;
+
+    for (int jp = wave; jp < A.nfs; jp += nwaves) {
+        const int f = (int)A.js[jp] - 1;
+        const bool numeric = A.feattypes[f] != 0;
+        const int constraint = A.mono[f];
+        const int bmax = numeric ? B - 1 : B;
+        long long pre[NAG][4];
+        long long excl[NAG];
+#pragma unroll
+        for (int ag = 0; ag < NAG; ag++) {
+            const int64_t o = ((int64_t)jp * NAG + ag) * B;
+            long long run = 0;
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const int b = lane * BPL + t;
+                long long v = 0;
+                if (t < BPL && b < B) {
+                    if (is_sub) {
+                        v = hp[o + b] - hs[o + b];
+                        hn[o + b] = v; // subtract_hist!: h[n] = h[parent] - h[sibling]
+                    } else {
+                        v = hn[o + b];
+                    }
+                }
+                run += v;
+                pre[ag][t] = run;
+            }
+            const long long incl = wave_incl_scan_i64(run);
+            excl[ag] = incl - run;
+#pragma unroll
+            for (int t = 0; t < 4; t++) pre[ag][t] += excl[ag];
+        }
+        double lg = -INFINITY;
+        int lb = NO_BIN;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int b = lane * BPL + t;
+            if (t < BPL && b < B) {
+                double gain = 0.0;
+                bool ok = false;
+                if (b + 1 <= bmax) {
+                    long long q[NAG];
+#pragma unroll
+                    for (int ag = 0; ag < NAG; ag++) {
+                        const long long prev = (t == 0) ? excl[ag] : pre[ag][t > 0 ? t - 1 : 0];
+                        q[ag] = numeric ? pre[ag][t] : (pre[ag][t] - prev); // _acc_left!: accumulate vs single bin
+                    }
+                    double SL[EVT_MAX_NK];
+                    decode_vals(q, s_sc, A.loss, NK, SL);
+                    const double w_l = SL[NK - 1];
+                    const double w_r = w_p - w_l;
+                    if (w_l > A.min_weight && w_r > A.min_weight) {
+                        ok = true;
+                        if (constraint != 0) {
+                            double SR[EVT_MAX_NK];
+                            for (int k = 0; k < NK; k++) SR[k] = S[k] - SL[k];
+                            const double predL = leaf_value(SL, 0, K, A.eta, A.bagging, A.lambda, A.L2);
+                            const double predR = leaf_value(SR, 0, K, A.eta, A.bagging, A.lambda, A.L2);
+                            ok = (constraint == -1 && predL > predR) || (constraint == 1 && predL < predR);
+                        }
+                        if (ok) {
+                            double sg = 0.0;
+                            for (int k = 0; k < K; k++) {
+                                const double g_l = SL[k], h_l = SL[K + k];
+                                sg += term_gh(g_l, h_l, w_l, A.lambda, A.L2) + term_gh(S[k] - g_l, S[K + k] - h_l, w_r, A.lambda, A.L2);
+                            }
+                            gain = sg - gain_p;
+                        }
+                    }
+                }
+                if (A.oblivious) {
+                    A.ogains[((int64_t)nodeidx * A.nfs + jp) * B + b] = ok ? gain : 0.0; // update_gains!
+                } else if (ok && gain > lg) {
+                    lg = gain;
+                    lb = b + 1;
+                }
+            }
+        }
+        if (!A.oblivious) {
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const double og = shfl_xor_f64(lg, o);
+                const int ob = __shfl_xor(lb, o);
+                if (og > lg || (og == lg && ob < lb)) { lg = og; lb = ob; }
+            }
+            if (lg > wbest) { wbest = lg; wjp = jp; wbin = lb; }
+        }
+    }
+    if (A.oblivious) return; // decision is taken for the whole level by k_obliv_select
+
+    if (lane == 0) { s_wg[wave] = wbest; s_wjp[wave] = wjp; s_wbin[wave] = wbin; }
+    __syncthreads();
+    if (tid == 0) {
+        double bg = -INFINITY;
+        int bj = NO_BIN, bb = NO_BIN;
+        for (int w = 0; w < nwaves; w++) {
+            if (s_wg[w] > bg || (s_wg[w] == bg && s_wjp[w] < bj)) { bg = s_wg[w]; bj = s_wjp[w]; bb = s_wbin[w]; }
+        }
+        const int found = (bb != NO_BIN && bg > A.gamma) ? 1 : 0;
+        s_dec[0] = found; s_dec[1] = bj; s_dec[2] = bb;
+        s_gain = bg;
+        if (found) {
+            const int feat = (int)A.js[bj];
+            A.tree.feat[n - 1] = feat;
+            A.tree.cond_bin[n - 1] = (uint8_t)bb;
+            A.tree.gain[n - 1] = (float)bg;
+            A.tree.split[n - 1] = 1;
+            A.tree.packed[n - 1] = (uint32_t)feat | ((uint32_t)bb << 16) | (1u << 24);
+            A.status[n] = ST_SPLIT;
+        } else {
+            for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (n - 1) + k] = (float)leaf_value(S, k, K, A.eta, A.bagging, A.lambda, A.L2);
+            A.status[n] = ST_LEAF;
+        }
+    }
+    __syncthreads();
+    if (!s_dec[0]) return;
+    const int bj = s_dec[1], bb = s_dec[2];
+    // _child_sums!: left = bins 1..bb of the parent histogram (numeric) or bin bb alone (categorical);
+    // right = parent - left.  Exact in integers.
+    if (wave == 0) {
+        const int f = (int)A.js[bj] - 1;
+        const bool numeric = A.feattypes[f] != 0;
+        for (int ag = 0; ag < NAG; ag++) {
+            const int64_t o = ((int64_t)bj * NAG + ag) * B;
+            long long s = 0;
+            for (int b = lane; b < B; b += 64) {
+                const bool in = numeric ? (b + 1 <= bb) : (b + 1 == bb);
+                if (in) s += is_sub ? (hp[o + b] - hs[o + b]) : hn[o + b];
+            }
+            s = wave_sum_i64(s);
+            if (lane == 0) {
+                A.node_sum[(int64_t)(2 * n) * NAG + ag] = s;
+                A.node_sum[(int64_t)(2 * n + 1) * NAG + ag] = s_Sq[ag] - s;
+            }
+        }
+    }
+    // the children's histogram slices start from zero (the build child is filled with atomics)
+    if (!A.zero_children) return;
+    long long *hc = A.hist + (int64_t)(2 * n - 1) * A.node_stride;
+    const int64_t used = (int64_t)A.nfs * NAG * B;
+    for (int64_t i = tid; i < used; i += blockDim.x) {
+        hc[i] = 0;
+        hc[A.node_stride + i] = 0;
+    }
+}
+
+// Oblivious trees (grow_otree!, src/fit.jl:190-257): per-level decision from the sum of the
+// nodes' gain matrices, masked where any node's gain is not positive; first maximum in
+// (feature position, bin) order; all nodes of the level split on it iff it exceeds gamma.
+struct OblivArgs {
+    long long *hist;
+    int64_t node_stride;
+    const uint32_t *js;
+    const uint8_t *feattypes;
+    int32_t *status;
+    long long *node_sum;
+    const double *qscale;
+    TreeDev tree;
+    const double *ogains;
+    const int64_t *hdr;
+    const int32_t *act_node;
+    double eta, lambda, L2, gamma;
+    int bagging, nfs, B, K, NK, NAg, loss, level, zero_children;
+};
+
+__global__ __launch_bounds__(1024) void k_obliv_select(OblivArgs A) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int n_act = (int)A.hdr[LH_N_ACT];
+    if (n_act <= 0) return;
+    const int B = A.B, K = A.K, NK = A.NK, NAG = A.NAg;
+    const int first = 1 << (A.level - 1);
+    __shared__ double s_g[1024];
+    __shared__ int s_i[1024];
+    __shared__ int s_dec[3];
+    __shared__ double s_gain;
+    __shared__ double s_sc[EVT_MAX_NA];
+    if (tid < NAG) s_sc[tid] = A.qscale[tid];
+    // level matrix and its first maximum
+    double bg = -INFINITY;
+    int bi = NO_BIN;
+    const int cells = A.nfs * B;
+    for (int c = tid; c < cells; c += blockDim.x) {
+        double acc = 0.0;
+        bool allpos = true;
+        for (int i = 0; i < n_act; i++) {
+            const int n = A.act_node[i];
+            const double g = A.ogains[(int64_t)(n - first) * cells + c];
+            acc += g;
+            if (n > 1) allpos = allpos && (g > 0.0);
+        }
+        const double v = allpos ? acc : 0.0;
+        if (v > bg) { bg = v; bi = c; } // c ascending per thread: first maximum kept
+    }
+    s_g[tid] = bg;
+    s_i[tid] = bi;
+    __syncthreads();
+    for (int o = blockDim.x >> 1; o > 0; o >>= 1) {
+        if (tid < o) {
+            if (s_g[tid + o] > s_g[tid] || (s_g[tid + o] == s_g[tid] && s_i[tid + o] < s_i[tid])) {
+                s_g[tid] = s_g[tid + o];
+                s_i[tid] = s_i[tid + o];
+            }
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        const int found = (s_i[0] != NO_BIN && s_g[0] > A.gamma) ? 1 : 0;
+        s_dec[0] = found;
+        s_dec[1] = found ? s_i[0] / B : 0;
+        s_dec[2] = found ? (s_i[0] % B) + 1 : 0;
+        s_gain = s_g[0];
+    }
+    __syncthreads();
+    const int found = s_dec[0], bj = s_dec[1], bb = s_dec[2];
+    const double bgain = s_gain;
+    for (int i = wave; i < n_act; i += nwaves) {
+        const int n = A.act_node[i];
+        long long Sq[EVT_MAX_NA];
+        double S[EVT_MAX_NK];
+        for (int ag = 0; ag < NAG; ag++) Sq[ag] = A.node_sum[(int64_t)n * NAG + ag];
+        decode_vals(Sq, s_sc, A.loss, NK, S);
+        if (!found) {
+            if (lane < K) A.tree.pred[(int64_t)K * (n - 1) + lane] = (float)leaf_value(S, lane, K, A.eta, A.bagging, A.lambda, A.L2);
+            if (lane == 0) A.status[n] = ST_LEAF;
+            continue;
+        }
+        const int feat = (int)A.js[bj];
+        const bool numeric = A.feattypes[feat - 1] != 0;
+        const long long *hn = A.hist + (int64_t)(n - 1) * A.node_stride;
+        for (int ag = 0; ag < NAG; ag++) {
+            const int64_t o = ((int64_t)bj * NAG + ag) * B;
+            long long s = 0;
+            for (int b = lane; b < B; b += 64) {
+                const bool in = numeric ? (b + 1 <= bb) : (b + 1 == bb);
+                if (in) s += hn[o + b];
+            }
+            s = wave_sum_i64(s);
+            if (lane == 0) {
+                A.node_sum[(int64_t)(2 * n) * NAG + ag] = s;
+                A.node_sum[(int64_t)(2 * n + 1) * NAG + ag] = Sq[ag] - s;
+            }
+        }
+        if (lane == 0) {
+            A.tree.feat[n - 1] = feat;
+            A.tree.cond_bin[n - 1] = (uint8_t)bb;
+            A.tree.gain[n - 1] = (float)bgain;
+            A.tree.split[n - 1] = 1;
+            A.tree.packed[n - 1] = (uint32_t)feat | ((uint32_t)bb << 16) | (1u << 24);
+            A.status[n] = ST_SPLIT;
+        }
+        if (!A.zero_children) continue;
+        long long *hc = A.hist + (int64_t)(2 * n - 1) * A.node_stride;
+        const int64_t used = (int64_t)A.nfs * NAG * B;
+        for (int64_t t = lane; t < used; t += 64) {
+            hc[t] = 0;
+            hc[A.node_stride + t] = 0;
+        }
+    }
+}
+
+int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
+    ScanArgs A;
+    A.hist = c->hist;
+    A.node_stride = (int64_t)c->F * c->NAg * c->B;
+    A.js = c->js;
+    A.feattypes = c->feattypes;
+    A.mono = c->mono;
+    A.status = c->status;
+    A.node_sum = c->node_sum;
+    A.qscale = c->qscale;
+    A.tree = c->tree;
+    A.ogains = c->ogains;
+    A.eta = p->eta; A.lambda = p->lambda; A.L2 = p->L2; A.gamma = p->gamma; A.min_weight = p->min_weight;
+    A.bagging = p->bagging_size;
+    A.nfs = c->n_js_last; A.B = c->B; A.F = c->F; A.K = c->K; A.NK = c->NK; A.NAg = c->NAg; A.loss = c->loss;
+    A.level = level;
+    A.leaf_level = leaf_level ? 1 : 0;
+    A.oblivious = (c->tree_type == EVT_TREE_OBLIVIOUS) ? 1 : 0;
+    A.zero_children = (level + 1 < c->D) ? 1 : 0; // children at the last level never get a histogram
+    dim3 grid(1u << (level - 1));
+    int threads = 1024;
+    if (level > 6) threads = 256; // many nodes per level: smaller blocks, same total parallelism
+    switch (c->NAg) {
+    case 2: hipLaunchKernelGGL(k_scan<2>, grid, dim3(threads), 0, c->stream, A); break;
+    case 3: hipLaunchKernelGGL(k_scan<3>, grid, dim3(threads), 0, c->stream, A); break;
+    case 5: hipLaunchKernelGGL(k_scan<5>, grid, dim3(threads), 0, c->stream, A); break;
+    default: evt_set_error("unsupported global channel count %d", c->NAg); return EVT_ERR_ARG;
+    }
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+int launch_obliv_select(evt_ctx *c, int level, const evt_params *p) {
+    const LevelTab &L = c->lvl[level & 1];
+    OblivArgs A;
+    A.hist = c->hist;
+    A.node_stride = (int64_t)c->F * c->NAg * c->B;
+    A.js = c->js;
+    A.feattypes = c->feattypes;
+    A.status = c->status;
+    A.node_sum = c->node_sum;
+    A.qscale = c->qscale;
+    A.tree = c->tree;
+    A.ogains = c->ogains;
+    A.hdr = L.hdr;
+    A.act_node = L.act_node;
+    A.eta = p->eta; A.lambda = p->lambda; A.L2 = p->L2; A.gamma = p->gamma;
+    A.bagging = p->bagging_size;
+    A.nfs = c->n_js_last; A.B = c->B; A.K = c->K; A.NK = c->NK; A.NAg = c->NAg; A.loss = c->loss; A.level = level;
+    A.zero_children = (level + 1 < c->D) ? 1 : 0;
+    hipLaunchKernelGGL(k_obliv_select, dim3(1), dim3(1024), 0, c->stream, A);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}

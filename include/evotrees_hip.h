@@ -1,0 +1,186 @@
+/*
+ * libevotrees_hip.so — C ABI of the MI355X (gfx950) tree-building backend.
+ *
+ * This is the drop-in boundary for the data-parallel hot path of EvoTrees.jl
+ * (gradients -> histogram -> split search -> row partition -> predict).  Host code in
+ * any language (Julia `ccall`, Python ctypes, C) owns the model (`EvoTree`, `Tree`) and the
+ * random streams; the library owns one opaque training cache per handle, which replaces the
+ * reference's device cache (ext/EvoTreesKernelAbstractionsExt/structs.jl:14-67).
+ *
+ * Conventions
+ *  - Every function returns 0 on success and a negative evt_status on failure; the message
+ *    is available from evt_last_error() (thread local).  No C++ exception crosses the ABI.
+ *  - Host arrays are owned by the caller; the library copies in/out before it returns and
+ *    never keeps a host pointer.  Input pointers may be host or device memory.
+ *  - Matrices use the reference's Julia memory order: x_bin is nobs x nfeats column-major
+ *    (x_bin[i + nobs*j]); pred is K x nobs and grad is (2K+1) x nobs with the first index
+ *    fastest.
+ *  - Feature ids and bins cross the boundary 1-based exactly as stored in Tree
+ *    (src/structs.jl:77-84): feat 0 / cond_bin 0 mean "no split".
+ *  - A handle is bound to the device that was current when it was created and to one HIP
+ *    stream.  Calls on one handle must not overlap; different handles may be used from
+ *    different threads.
+ */
+#ifndef EVOTREES_HIP_H
+#define EVOTREES_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct evt_ctx *evt_handle;
+
+typedef enum {
+    EVT_OK = 0,
+    EVT_ERR_ARG = -1,   /* invalid argument (null pointer, range, unsupported size)        */
+    EVT_ERR_HIP = -2,   /* a HIP runtime call or kernel launch failed                      */
+    EVT_ERR_STATE = -3, /* call order violated (e.g. grow before x_bin / target were set)  */
+    EVT_ERR_EMPTY = -4, /* "no subsample observation" (src/subsample.jl:36)                */
+    EVT_ERR_NOMEM = -5
+} evt_status;
+
+/* loss ids: the in-scope subset of src/loss.jl:20-34 */
+enum { EVT_LOSS_MSE = 0, EVT_LOSS_LOGLOSS = 1, EVT_LOSS_GAUSSIAN_MLE = 2 };
+/* params.tree_type, src/learners.jl:45 */
+enum { EVT_TREE_BINARY = 0, EVT_TREE_OBLIVIOUS = 1 };
+
+/* Per-tree hyper-parameters read by the kernels (fields of EvoTreeRegressor & co,
+ * src/learners.jl:1-23). */
+typedef struct {
+    double eta;
+    double L2;
+    double lambda;
+    double gamma;
+    double min_weight;
+    int32_t bagging_size;
+    int32_t update_pred; /* 1: also apply predict!(cache.pred, tree, ...) as grow_evotree! does
+                            (src/fit.jl:36-37); 0: only grow */
+} evt_params;
+
+/* Host arrays with the layout of Tree{L,K} (src/structs.jl:77-106), each of length
+ * 2^max_depth - 1 (pred: K * that).  Zero-filled by the library before it writes. */
+typedef struct {
+    int64_t *feat;     /* Vector{Int}: 1-based feature id, 0 = none                        */
+    uint8_t *cond_bin; /* Vector{UInt8}                                                    */
+    float *w;          /* Vector{Float32}: sum of weights reaching the node                */
+    float *gain;       /* Vector{Float32}                                                  */
+    float *pred;       /* Matrix{Float32} K x nnodes                                       */
+    uint8_t *split;    /* Vector{Bool}                                                     */
+} evt_tree_out;
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char *evt_last_error(void);
+
+/* Number of visible HIP devices; fails (EVT_ERR_HIP) when the runtime finds none. */
+int evt_device_count(int32_t *count);
+
+/* ---- training cache ------------------------------------------------------------------
+ * Replaces init_core(params, ::Type{<:GPU}, ...) device allocation
+ * (ext/EvoTreesKernelAbstractionsExt/init.jl:1-151): sizes every device buffer.
+ * nbins in [2,255] (src/learners.jl:527), K = 1 (mse, logloss) or 2 (gaussian_mle, one target). */
+int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K, int32_t max_depth, int32_t loss,
+               int32_t tree_type, evt_handle *out);
+/* Frees all device memory; the slot post_fit_gc has in the reference (src/fit.jl:340). */
+int evt_destroy(evt_handle h);
+
+/* Upload of the binned matrix: `_to_device(x_bin)` in ext/.../init.jl:4-6.  Values must be in
+ * 1..nbins (src/fit-utils.jl:66-72); anything else is rejected.  Also derives the
+ * observation-major copy the histogram kernel streams (the CPU path's x_bin_T, src/init.jl:155). */
+int evt_set_xbin(evt_handle h, const uint8_t *x_bin_colmajor);
+
+/* Device binarize: searchsortedfirst(edges[j], x[i,j]) for every cell (src/fit-utils.jl:66-72),
+ * written straight into the cache's x_bin.  x is nobs x nfeats column-major Float64; edges are
+ * concatenated per feature, edge_off has nfeats+1 entries. */
+int evt_binarize_f64(evt_handle h, const double *x_colmajor, const double *edges, const int32_t *edge_off);
+
+/* Target, weights and initial prediction: y Float32[nobs]; w Float32[nobs] or NULL for ones
+ * (device_ones, src/init.jl:300); pred[:, i] = mu (+ offset[:, i] if offset != NULL), offset is
+ * K x nobs (src/init.jl:168-174).  Writes the weight row of the gradient matrix. */
+int evt_set_target(evt_handle h, const float *y, const float *w, const float *mu, const float *offset);
+
+/* feattypes[j] != 0: numeric (<=), 0: categorical (==); monotone[j] in {-1,0,1}
+ * (cache.feattypes / cache.monotone_constraints, src/init.jl:183-187).  NULL = all numeric / none. */
+int evt_set_feature_meta(evt_handle h, const uint8_t *feattypes, const int32_t *monotone);
+
+/* update_grads!(cache.∇, cache.pred, cache.y, L, params): src/loss.jl:100-111, :219-236;
+ * device twin ext/.../loss.jl:183-191. */
+int evt_update_grads(evt_handle h);
+
+/* Overwrites the gradient matrix ((2K+1) x nobs Float32, weight row included) — used to feed
+ * identical gradients to the library and to a CPU run. */
+int evt_set_grads(evt_handle h, const float *grad);
+
+/*
+ * One tree: subsample (src/subsample.jl:6-38 / ext/.../subsample.jl:2-8) + grow_tree! or
+ * grow_otree! (src/fit.jl:45-263; device twin ext/.../fit.jl:132-342) + optionally predict!
+ * on the cache (src/fit.jl:37).
+ *  mask : UInt8[nobs] drawn by the host RNG, rows with mask[i] <= cond are kept; NULL keeps all.
+ *  js   : sampled feature ids, 1-based, ascending, n_js of them (src/fit.jl:16).
+ * Returns EVT_ERR_EMPTY when no row is kept.
+ */
+int evt_grow_tree(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js,
+                  const evt_params *params, evt_tree_out *tree);
+
+/* predict!(cache.pred, tree, cache.x_bin, feattypes): src/predict.jl:1-46; ext/.../predict.jl:60-75.
+ * Adds one host tree (arrays of length nnodes_tree) to the cache's prediction. */
+int evt_predict_tree(evt_handle h, int32_t nnodes_tree, const int64_t *feat, const uint8_t *cond_bin,
+                     const float *pred, const uint8_t *split);
+
+/* ---- read-back of cache state (parity tests, callbacks) ------------------------------ */
+int evt_get_pred(evt_handle h, float *pred_out /* K x nobs */);
+int evt_get_grads(evt_handle h, float *grad_out /* (2K+1) x nobs */);
+/* Node each sampled row ended in for the last tree (update_nodes_idx!, ext/.../fit-utils.jl:9-31),
+ * 1-based node id; 0 for rows outside the sample. */
+int evt_get_nidx(evt_handle h, uint32_t *nidx_out /* nobs */);
+/* Histogram of the last tree in the reference layout h∇[k, bin, feat, node] Float64
+ * ((2K+1) x nbins x nfeats x (2^max_depth-1), src/init.jl:204); only slices of nodes that were
+ * scanned and features in js are defined, the rest is zero. */
+int evt_get_hist(evt_handle h, double *hist_out);
+/* Fixed-point parameters of the last update: gradient row k is accumulated as
+ * rint(v * 2^(qbits[k]-qexp[k])) in int64. */
+int evt_get_quant(evt_handle h, int32_t *qbits /* 2K+1 */, int32_t *qexp /* 2K+1 */);
+
+/* ---- inference: _predict(m, data, ::Type{<:GPU}) (ext/.../predict.jl:115-135) ----------
+ * x_bin: nobs x nfeats column-major; trees concatenated: tree t owns entries
+ * [tree_off[t], tree_off[t+1]) of feat / cond_bin / split and K times that of pred.
+ * out: K x nobs raw sums, link applied when apply_link != 0 (src/predict.jl:105-116).
+ * The transposition to nobs x K (src/predict.jl:134) is left to the host. */
+int evt_predict(int64_t nobs, int32_t nfeats, const uint8_t *x_bin_colmajor, const uint8_t *feattypes,
+                int32_t loss, int32_t K, int32_t ntrees, const int64_t *tree_off, const int64_t *feat,
+                const uint8_t *cond_bin, const float *pred, const uint8_t *split, int32_t apply_link,
+                float *out);
+/* predict_leaf_idx (src/predict.jl:138-185): out is nobs x ntrees column-major UInt32. */
+int evt_predict_leaf_idx(int64_t nobs, int32_t nfeats, const uint8_t *x_bin_colmajor, const uint8_t *feattypes,
+                         int32_t ntrees, const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin,
+                         const uint8_t *split, uint32_t *out);
+
+/* ---- measurement ---------------------------------------------------------------------
+ * Kernel classes timed with HIP events on the handle's stream when profiling is on. */
+enum {
+    EVT_K_GRAD = 0,
+    EVT_K_HIST = 1,
+    EVT_K_SCAN = 2,
+    EVT_K_PARTITION = 3,
+    EVT_K_PREDICT = 4,
+    EVT_K_OTHER = 5,
+    EVT_K_COUNT = 6
+};
+int evt_set_profiling(evt_handle h, int32_t on);
+/* Accumulated since the last reset: per class number of launches, milliseconds, and units
+ * (GRAD/PREDICT: rows; HIST: rows built; SCAN: nodes scanned; PARTITION: rows moved). */
+int evt_get_profile(evt_handle h, int64_t *launches, double *ms, int64_t *units);
+int evt_reset_profile(evt_handle h);
+/* Tunables for sweeps: "hist_blocks", "hist_threads". */
+int evt_set_option(evt_handle h, const char *name, int64_t value);
+/* Blocks until all work queued on the handle's stream is done. */
+int evt_synchronize(evt_handle h);
+/* Plain device copy of nbytes (read + write) timed with HIP events: the box's streaming
+ * ceiling that roofline figures are quoted beside. */
+int evt_copy_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EVOTREES_HIP_H */
