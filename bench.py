@@ -1,0 +1,236 @@
+"""Benchmark of the tree-building hot path on one MI355X.
+
+A step is one boosting round (gradients -> one tree: histograms, split search, row partition ->
+prediction update) over a synthetic matrix that is already binned and resident in HBM when the
+timed region starts.  Default workload: BASELINE.json configs[2], the configuration the metric is
+quoted on (mse, 10M x 100 Float64 iid U(0,1), y ~ U(0,1), nbins 64, max_depth 11, eta 0.1, full
+row and column sampling, 200 rounds).
+
+Prints one JSON line.  `value` = seconds per 200 rounds (lower is better), scaled from the K timed
+rounds.  `roofline` = histogram kernel: algorithmic bytes rows_built*(Fs + 4*(2K+1) + 4) over the
+HIP-event time of its launches inside the timed region, against 8 TB/s.  `cpu_baseline` = the CPU
+oracle (a restatement of the reference's CPU algorithm, OpenMP over node x feature tiles) timed
+on this box's host cores on a few rounds of the same workload.
+"""
+import argparse
+import importlib.util
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: loss, N, F, nbins, depth, eta, rowsample, colsample, tree_type, min_weight
+    "cfg1": dict(loss="mse", N=100_000, F=10, nbins=64, depth=6, eta=0.1, rowsample=1.0, colsample=1.0, tree_type="binary", min_weight=1.0),
+    "cfg2": dict(loss="mse", N=1_000_000, F=100, nbins=64, depth=6, eta=0.1, rowsample=0.5, colsample=0.5, tree_type="binary", min_weight=1.0),
+    "cfg3": dict(loss="mse", N=10_000_000, F=100, nbins=64, depth=11, eta=0.1, rowsample=1.0, colsample=1.0, tree_type="binary", min_weight=1.0),
+    "cfg4": dict(loss="logloss", N=1_000_000, F=28, nbins=128, depth=8, eta=0.05, rowsample=0.8, colsample=1.0, tree_type="binary", min_weight=1.0),
+    "cfg5": dict(loss="gaussian_mle", N=2_000_000, F=50, nbins=64, depth=7, eta=0.1, rowsample=1.0, colsample=1.0, tree_type="binary", min_weight=8.0),
+    "cfg5o": dict(loss="gaussian_mle", N=2_000_000, F=50, nbins=64, depth=7, eta=0.1, rowsample=1.0, colsample=1.0, tree_type="oblivious", min_weight=8.0),
+}
+
+
+def load_package():
+    name = "evotrees_jl_amd"
+    if name in sys.modules:
+        return sys.modules[name]
+    pkg_dir = os.path.join(ROOT, "evotrees.jl_amd")
+    spec = importlib.util.spec_from_file_location(name, os.path.join(pkg_dir, "__init__.py"), submodule_search_locations=[pkg_dir])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def synth(cfg, seed=123):
+    """Float64 features in (F, N) order and the Float32 target of the named configuration."""
+    rng = np.random.default_rng(seed)
+    N, F = cfg["N"], cfg["F"]
+    loss = cfg["loss"]
+    if loss == "mse" and cfg["colsample"] < 1.0:  # cfg2: linear signal on 10 random columns
+        x = rng.random((F, N))
+        cols = rng.choice(F, 10, replace=False)
+        coef = rng.standard_normal(10)
+        y = (coef[:, None] * x[cols]).sum(axis=0) + 0.1 * rng.standard_normal(N)
+    elif loss == "mse":
+        x = rng.random((F, N))
+        y = rng.random(N)
+    elif loss == "logloss":
+        x = rng.standard_normal((F, N))
+        wv = 0.5 * rng.standard_normal(F)
+        z = (wv[:, None] * x).sum(axis=0) + 0.5 * x[0] * x[1]
+        y = (rng.random(N) < 1 / (1 + np.exp(-z))).astype(np.float64)
+    else:
+        x = rng.uniform(-1, 1, (F, N))
+        y = np.sin(3 * x[0]) + x[1] + np.exp(0.5 * x[2]) * rng.standard_normal(N)
+    return x, y.astype(np.float32), rng
+
+
+def edges_from_sample(x_FN, nbins, rng):
+    """Quantile edges on <= 1000*nbins sampled rows (src/fit-utils.jl:9-16)."""
+    F, N = x_FN.shape
+    nobs = min(N, 1000 * nbins)
+    idx = np.sort(rng.choice(N, nobs, replace=False)) if nobs < N else np.arange(N)
+    q = np.arange(1, nbins) / nbins
+    return [np.ascontiguousarray(np.quantile(x_FN[j, idx], q)) for j in range(F)]
+
+
+def bias(loss, y):
+    if loss == "logloss":
+        m = float(y.mean())
+        return np.array([np.log(m / (1 - m))], np.float32)
+    if loss == "gaussian_mle":
+        s = float(y.std(ddof=1))
+        return np.array([y.mean(), s + np.log(-np.expm1(-s))], np.float32)
+    return np.array([y.mean()], np.float32)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--rows", type=int, default=0, help="override the number of rows (smoke runs)")
+    ap.add_argument("--cpu-rounds", type=int, default=3, help="rounds of the CPU oracle to time (0: skip)")
+    ap.add_argument("--no-profile", action="store_true", help="do not record HIP events around kernels")
+    ap.add_argument("--hist-blocks", type=int, default=0)
+    ap.add_argument("--hist-threads", type=int, default=0)
+    ap.add_argument("--predict", action="store_true", help="also time model inference on the training rows")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no multi-GPU path is built)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    evt = load_package()
+    evt._lib.load()
+    cfg = dict(WORKLOADS[args.workload])
+    if args.rows:
+        cfg["N"] = args.rows
+    N, F, B, D, loss = cfg["N"], cfg["F"], cfg["nbins"], cfg["depth"], cfg["loss"]
+    K = 2 if loss == "gaussian_mle" else 1
+    NK = 2 * K + 1
+
+    t0 = time.time()
+    x, y, rng = synth(cfg)
+    edges = edges_from_sample(x, B, rng)
+    h = evt.Handle(N, F, B, K, D, loss, cfg["tree_type"])
+    h.binarize(x, edges)
+    del x
+    mu = bias(loss, y)
+    h.set_target(y, None, mu)
+    if args.hist_blocks:
+        h.set_option("hist_blocks", args.hist_blocks)
+    if args.hist_threads:
+        h.set_option("hist_threads", args.hist_threads)
+    t_setup = time.time() - t0
+
+    params = evt.make_params(eta=cfg["eta"], min_weight=cfg["min_weight"], update_pred=True)
+    cond = int(np.rint(255 * cfg["rowsample"]))
+    nfs = int(np.ceil(cfg["colsample"] * F))
+    L = evt._lib.load()
+    tree = evt.Tree(K, h.nnodes)
+    tree_out = tree.as_out()
+
+    def one_round():
+        h.update_grads()
+        mask = None if cond >= 255 else rng.integers(0, 256, N, dtype=np.uint8)
+        js = np.arange(1, F + 1, dtype=np.uint32) if nfs >= F else (np.sort(rng.choice(F, nfs, replace=False)) + 1).astype(np.uint32)
+        evt._lib.check(L.evt_grow_tree(h._h, evt._lib.ptr(mask), cond, evt._lib.ptr(js), js.shape[0], params, tree_out))
+
+    for _ in range(args.warmup):
+        one_round()
+    h.synchronize()
+    h.set_profiling(not args.no_profile)
+    h.reset_profile()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        one_round()
+    h.synchronize()
+    t2 = time.perf_counter()
+    prof = h.get_profile()
+    h.set_profiling(False)
+    elapsed = t2 - t1
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = ms_per_step * 200 / 1e3
+
+    # roofline of the dominant kernel (histogram build)
+    rows_built = prof["hist"]["units"]
+    hist_ms = prof["hist"]["ms"]
+    bytes_per_row = nfs + 4 * NK + 4
+    roofline = None
+    if hist_ms > 0:
+        achieved = rows_built * bytes_per_row / (hist_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": "k_hist_build", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "launches": prof["hist"]["launches"], "avg_launch_ms": round(hist_ms / max(1, prof["hist"]["launches"]), 4),
+                    "rows_built_per_round": rows_built // max(1, args.steps), "bytes_per_row": bytes_per_row,
+                    "rows_features_per_s": round(rows_built * nfs / (hist_ms * 1e-3), 1)}
+    kernels = {k: {"ms_per_round": round(v["ms"] / args.steps, 4), "launches_per_round": v["launches"] / args.steps} for k, v in prof.items()}
+    if prof["grad"]["ms"] > 0:
+        gb = N * (4 * K + 4 + 4 + 8 * K)
+        kernels["grad"]["GBps"] = round(gb * args.steps / (prof["grad"]["ms"] * 1e-3) / 1e9, 1)
+
+    out = {
+        "metric": "train s/200 rounds @10Mx100 depth 11 (1 GPU)" if args.workload == "cfg3" and not args.rows
+        else "train s/200 rounds (%s)" % args.workload,
+        "value": round(value, 4), "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int64 fixed-point histograms, f64 gains, f32 gradients/predictions", "data": "synthetic",
+        "config": {"workload": "%s: %s %dx%d nbins=%d max_depth=%d eta=%g rowsample=%g colsample=%g tree_type=%s" % (
+            args.workload, loss, N, F, B, D, cfg["eta"], cfg["rowsample"], cfg["colsample"], cfg["tree_type"])},
+        "roofline": roofline, "kernels": kernels, "setup_s": round(t_setup, 2),
+    }
+    try:
+        out["copy_kernel_GBps"] = round(evt._lib.copy_bandwidth(1 << 30, 10), 1)
+    except Exception as e:  # measurement aid only
+        out["copy_kernel_GBps"] = None
+
+    if args.predict:
+        m_trees = []
+        # a model of `steps` copies of the last tree has the same traversal cost as a trained one of that size
+        b = evt.Tree.bias(mu)
+        m_trees = [b] + [tree] * min(args.steps, 200)
+        xb = h.get_xbin()
+        tp = time.perf_counter()
+        evt._lib.predict_model(xb, None, loss, K, m_trees, apply_link=True)
+        out["predict"] = {"rows_per_s_incl_transfers": round(N / (time.perf_counter() - tp), 1), "trees": len(m_trees)}
+
+    if args.cpu_rounds > 0:
+        from oracle import oracle as orc
+        xb = h.get_xbin()
+        op = orc.make_params(loss, nbins=B, max_depth=D, tree_type=cfg["tree_type"], eta=cfg["eta"], min_weight=cfg["min_weight"])
+        o = orc.Oracle(op, xb, with_fixed=False)
+        pred = np.tile(mu, (N, 1)).astype(np.float32)
+        grad = np.zeros((N, NK), np.float32)
+        grad[:, NK - 1] = 1.0
+        rows = np.arange(N, dtype=np.uint32)
+        tc = time.perf_counter()
+        for _ in range(args.cpu_rounds):
+            orc.update_grads(op, pred, y, grad)
+            if cond < 255:
+                rows = orc.subsample(rng.integers(0, 256, N, dtype=np.uint8), cond)
+            js = np.arange(1, F + 1, dtype=np.uint32) if nfs >= F else (np.sort(rng.choice(F, nfs, replace=False)) + 1).astype(np.uint32)
+            t_cpu, _ = o.grow_tree(grad, rows, js, mode=0, want_nidx=False)
+            o.predict_tree(t_cpu, pred)
+        cpu_s = (time.perf_counter() - tc) / args.cpu_rounds
+        out["cpu_baseline"] = {"value": round(cpu_s * 200, 2), "unit": "s", "cores": o.nthreads, "kind": "port",
+                               "sample": "%d rounds of the same workload (first rounds of boosting), scaled to 200 rounds; "
+                                         "restated CPU path (OpenMP, %d threads), not EvoTrees.jl" % (args.cpu_rounds, o.nthreads)}
+        out["speedup_vs_cpu_baseline"] = round(cpu_s * 200 / value, 1)
+        o.close()
+    h.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

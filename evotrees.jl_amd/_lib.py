@@ -20,7 +20,7 @@ KERNEL_CLASSES = ["grad", "hist", "scan", "partition", "predict", "other"]
 EXPORTS = [
     "evt_last_error", "evt_device_count", "evt_create", "evt_destroy", "evt_set_xbin", "evt_binarize_f64",
     "evt_set_target", "evt_set_feature_meta", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
-    "evt_predict_tree", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
+    "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
     "evt_predict", "evt_predict_leaf_idx", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
     "evt_set_option", "evt_synchronize", "evt_copy_bandwidth",
 ]
@@ -69,6 +69,7 @@ def load():
         "evt_set_grads": [vp, vp],
         "evt_grow_tree": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams), C.POINTER(EvtTreeOut)],
         "evt_predict_tree": [vp, i32, vp, vp, vp, vp],
+        "evt_get_xbin": [vp, vp],
         "evt_get_pred": [vp, vp],
         "evt_get_grads": [vp, vp],
         "evt_get_nidx": [vp, vp],
@@ -198,6 +199,11 @@ class Handle:
 
     def predict_tree(self, tree):
         check(load().evt_predict_tree(self._h, tree.feat.shape[0], ptr(tree.feat), ptr(tree.cond_bin), ptr(tree.pred), ptr(tree.split)))
+
+    def get_xbin(self):
+        out = np.empty((self.F, self.N), np.uint8)
+        check(load().evt_get_xbin(self._h, ptr(out)))
+        return out
 
     def get_pred(self):
         out = np.empty((self.N, self.K), np.float32)

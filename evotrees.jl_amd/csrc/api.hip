@@ -645,6 +645,17 @@ extern "C" int evt_predict_tree(evt_handle c, int32_t nnodes_tree, const int64_t
     return r;
 }
 
+extern "C" int evt_get_xbin(evt_handle c, uint8_t *out) {
+    CTXCHK(c);
+    ARGCHK(out, "out is NULL");
+    if (!c->have_xbin) {
+        evt_set_error("x_bin has not been set");
+        return EVT_ERR_STATE;
+    }
+    HIPCHK(hipMemcpyAsync(out, c->xcm, (size_t)c->N * c->F, hipMemcpyDefault, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return EVT_OK;
+}
 extern "C" int evt_get_pred(evt_handle c, float *out) {
     CTXCHK(c);
     ARGCHK(out, "out is NULL");

@@ -20,41 +20,52 @@ __global__ __launch_bounds__(256) void k_grads(const float *__restrict__ pred, c
                                               float *__restrict__ grad, int64_t N, uint32_t *absmax) {
     constexpr int K = (LOSS == 2) ? 2 : 1;
     constexpr int NK = 2 * K + 1;
-    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    float out[2 * K];
+    float mx[2 * K];
 #pragma unroll
-    for (int k = 0; k < 2 * K; k++) out[k] = 0.0f;
-    if (i < N) {
+    for (int k = 0; k < 2 * K; k++) mx[k] = 0.0f;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
+        float out[2 * K];
         float *g = grad + (size_t)NK * i;
-        float w = g[NK - 1];
+        const float w = g[NK - 1];
         if (LOSS == 0) {
-            float gg = 2.0f * (pred[i] - y[i]);
+            const float gg = 2.0f * (pred[i] - y[i]);
             out[0] = gg * w;
             out[1] = 2.0f * w;
         } else if (LOSS == 1) {
-            float s = dev_sigmoid(pred[i]);
+            const float s = dev_sigmoid(pred[i]);
             out[0] = (s - y[i]) * w;
             out[1] = (s * (1.0f - s)) * w;
         } else {
-            float loc = pred[2 * i], raw = pred[2 * i + 1];
-            float scale = dev_softplus(raw);
-            float dscale = dev_sigmoid(raw);
-            float resid = loc - y[i];
-            float s2 = scale * scale;
-            float ds = dscale / scale;
+            const float loc = pred[2 * i], raw = pred[2 * i + 1];
+            const float scale = dev_softplus(raw);
+            const float dscale = dev_sigmoid(raw);
+            const float resid = loc - y[i];
+            const float s2 = scale * scale;
+            const float ds = dscale / scale;
             out[0] = (resid / s2) * w;
             out[1] = ((1.0f - (resid * resid) / s2) * dscale / scale) * w;
             out[2] = (1.0f / s2) * w;
             out[3] = (2.0f * (ds * ds)) * w;
         }
 #pragma unroll
-        for (int k = 0; k < 2 * K; k++) g[k] = out[k];
+        for (int k = 0; k < 2 * K; k++) {
+            g[k] = out[k];
+            mx[k] = fmaxf(mx[k], fabsf(out[k]));
+        }
     }
-    // per gradient row max |v| -> exponent bound of the fixed-point histogram
+    // per gradient row max |v| -> exponent bound of the fixed-point histogram.
+    // One atomic per block and row: contended same-address atomics serialise in L2.
+    __shared__ float s_m[4][2 * K];
 #pragma unroll
     for (int k = 0; k < 2 * K; k++) {
-        float m = wave_max_f32(fabsf(out[k]));
-        if ((threadIdx.x & 63) == 0 && m > 0.0f) atomicMax(&absmax[k], __float_as_uint(m));
+        const float m = wave_max_f32(mx[k]);
+        if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6][k] = m;
+    }
+    __syncthreads();
+    if (threadIdx.x < 2 * K) {
+        const int k = threadIdx.x;
+        const float m = fmaxf(fmaxf(s_m[0][k], s_m[1][k]), fmaxf(s_m[2][k], s_m[3][k]));
+        if (m > 0.0f) atomicMax(&absmax[k], __float_as_uint(m));
     }
 }
 
@@ -121,7 +132,9 @@ int launch_grads(evt_ctx *c) {
         int r = launch_fill_u32(c, c->absmax, 0u, c->NK - 1);
         if (r != EVT_OK) return r;
     }
-    dim3 grid((unsigned)((c->N + 255) / 256));
+    int64_t nb = (c->N + 255) / 256;
+    if (nb > 2048) nb = 2048;
+    dim3 grid((unsigned)nb);
     if (c->loss == EVT_LOSS_MSE)
         hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
     else if (c->loss == EVT_LOSS_LOGLOSS)

@@ -129,6 +129,8 @@ int evt_predict_tree(evt_handle h, int32_t nnodes_tree, const int64_t *feat, con
                      const float *pred, const uint8_t *split);
 
 /* ---- read-back of cache state (parity tests, callbacks) ------------------------------ */
+/* The cache's binned matrix (nobs x nfeats column-major), e.g. after evt_binarize_f64. */
+int evt_get_xbin(evt_handle h, uint8_t *x_bin_out);
 int evt_get_pred(evt_handle h, float *pred_out /* K x nobs */);
 int evt_get_grads(evt_handle h, float *grad_out /* (2K+1) x nobs */);
 /* Node each sampled row ended in for the last tree (update_nodes_idx!, ext/.../fit-utils.jl:9-31),
