@@ -104,6 +104,7 @@ def main():
     ap.add_argument("--no-profile", action="store_true", help="do not record HIP events around kernels")
     ap.add_argument("--hist-blocks", type=int, default=0)
     ap.add_argument("--hist-threads", type=int, default=0)
+    ap.add_argument("--hist-min-rows", type=int, default=0)
     ap.add_argument("--predict", action="store_true", help="also time model inference on the training rows")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -132,6 +133,8 @@ def main():
         h.set_option("hist_blocks", args.hist_blocks)
     if args.hist_threads:
         h.set_option("hist_threads", args.hist_threads)
+    if args.hist_min_rows:
+        h.set_option("hist_min_rows", args.hist_min_rows)
     t_setup = time.time() - t0
 
     params = evt.make_params(eta=cfg["eta"], min_weight=cfg["min_weight"], update_pred=True)
@@ -190,6 +193,15 @@ def main():
             args.workload, loss, N, F, B, D, cfg["eta"], cfg["rowsample"], cfg["colsample"], cfg["tree_type"])},
         "roofline": roofline, "kernels": kernels, "setup_s": round(t_setup, 2),
     }
+    # rows built per level of the last tree (unit weights: Tree.w holds row counts): the smaller child of every split
+    per_level = [int(N if cond >= 255 else tree.w[0])]
+    for d in range(1, D - 1):
+        tot = 0
+        for n in range(1 << (d - 1), 1 << d):
+            if tree.split[n - 1]:
+                tot += int(min(tree.w[2 * n - 1], tree.w[2 * n]))
+        per_level.append(tot)
+    out["last_tree_rows_built_per_level"] = per_level
     try:
         out["copy_kernel_GBps"] = round(evt._lib.copy_bandwidth(1 << 30, 10), 1)
     except Exception as e:  # measurement aid only

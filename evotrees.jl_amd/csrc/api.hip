@@ -119,7 +119,7 @@ extern "C" int evt_destroy(evt_handle c) {
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree.feat, c->tree.cond_bin, c->tree.w, c->tree.gain,
                     c->tree.pred, c->tree.split, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->stats, c->errflag, c->ogains, c->obest};
+                    c->qscale, c->stats, c->errflag, c->ogains, c->obest, c->sbest};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -175,12 +175,16 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     memset(&c->tree, 0, sizeof(c->tree));
     memset(c->lvl, 0, sizeof(c->lvl));
     c->js = nullptr; c->jsmap = nullptr; c->feattypes = nullptr; c->mono = nullptr; c->absmax = nullptr; c->qexp = nullptr; c->qbits = nullptr;
-    c->qscale = nullptr; c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->obest = nullptr;
+    c->qscale = nullptr; c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->obest = nullptr; c->sbest = nullptr;
     c->h_stage = nullptr; c->h_stage_bytes = 0;
     c->n_js_last = 0;
     c->last_all_rows = true;
     c->hist_blocks = 512;
     c->hist_threads = 1024;
+    c->hist_min_rows = 2048;
+    c->record_nidx = false;
+    c->nidx_valid = false;
+    c->last_cond = 255;
     c->profiling = false;
     memset(c->prof_launches, 0, sizeof(c->prof_launches));
     memset(c->prof_ms, 0, sizeof(c->prof_ms));
@@ -244,6 +248,11 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->stats, c->D + 2);
     ALLOC(c->errflag, 1);
     if (tree_type == EVT_TREE_OBLIVIOUS) ALLOC(c->ogains, (size_t)c->maxlvl * c->F * c->B);
+    {
+        uint8_t *sb = nullptr;
+        ALLOC(sb, (size_t)c->maxlvl * ((c->F + 3) / 4) * 16);
+        c->sbest = sb;
+    }
     // pinned staging: tree read-back + small per-tree uploads
     c->h_stage_bytes = (size_t)c->nnodes * (4 + 1 + 4 + 4 + 4 * K + 1) + (size_t)(c->D + 2) * 8 + (size_t)c->F * 4 + (size_t)c->RS * 2 + 1024;
     if (hipHostMalloc((void **)&c->h_stage, c->h_stage_bytes, hipHostMallocDefault) != hipSuccess) {
@@ -501,6 +510,8 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     }
     const bool all_rows = (n_is == c->N);
     c->last_all_rows = all_rows;
+    c->last_cond = cond;
+    c->nidx_valid = c->record_nidx;
 
     // per-tree small uploads through pinned memory
     uint32_t *h_js = reinterpret_cast<uint32_t *>(c->h_stage);
@@ -522,7 +533,7 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     } else {
         HIPCHK(hipMemcpyAsync(c->mask, mask, c->N, hipMemcpyDefault, c->stream));
         r = launch_compact_mask(c, cond, n_is);
-        if (r == EVT_OK) r = launch_fill_u32(c, c->nidx, 0u, c->N);
+        if (r == EVT_OK && c->record_nidx) r = launch_fill_u32(c, c->nidx, 0u, c->N);
     }
     if (r == EVT_OK) r = launch_tree_begin(c, n_is);
     prof_end(c);
@@ -673,6 +684,15 @@ extern "C" int evt_get_grads(evt_handle c, float *out) {
 extern "C" int evt_get_nidx(evt_handle c, uint32_t *out) {
     CTXCHK(c);
     ARGCHK(out, "out is NULL");
+    if (c->n_js_last <= 0) {
+        evt_set_error("no tree has been grown yet");
+        return EVT_ERR_STATE;
+    }
+    if (!c->nidx_valid) { // not recorded while growing: walk the last tree (same decisions, row by row)
+        int r = launch_nidx_from_tree(c, !c->last_all_rows, c->last_cond);
+        if (r != EVT_OK) return r;
+        c->nidx_valid = true;
+    }
     HIPCHK(hipMemcpyAsync(out, c->nidx, sizeof(uint32_t) * (size_t)c->N, hipMemcpyDefault, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     return EVT_OK;
@@ -818,6 +838,11 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
     if (strcmp(name, "hist_blocks") == 0) {
         ARGCHK(value >= 1 && value <= 65535, "hist_blocks must be in [1, 65535]");
         c->hist_blocks = (int)value;
+    } else if (strcmp(name, "hist_min_rows") == 0) {
+        ARGCHK(value >= 1 && value <= EVT_HIST_MAX_ROWS_PER_BLOCK, "hist_min_rows must be in [1, 32768]");
+        c->hist_min_rows = (int)value;
+    } else if (strcmp(name, "record_nidx") == 0) {
+        c->record_nidx = value != 0;
     } else if (strcmp(name, "hist_threads") == 0) {
         ARGCHK(value == 256 || value == 512 || value == 1024, "hist_threads must be 256, 512 or 1024");
         c->hist_threads = (int)value;

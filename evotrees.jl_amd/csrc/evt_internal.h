@@ -101,7 +101,8 @@ struct evt_ctx {
     int64_t *stats;    // [D+1] rows built per level
     int32_t *errflag;  // device-side validation flag
     double *ogains;    // oblivious: [maxlvl][F][B]
-    double *obest;     // oblivious: level decision {gain, jp, bin}
+    double *obest;     // unused
+    void *sbest;       // split search: best candidate per (node of the level, feature group), 16 B each
 
     // host staging (pinned)
     uint8_t *h_stage;
@@ -112,7 +113,10 @@ struct evt_ctx {
     bool last_all_rows;
 
     // tunables
-    int hist_blocks, hist_threads;
+    int hist_blocks, hist_threads, hist_min_rows;
+    bool record_nidx;  // leaf finalisation also writes the node id of every sampled row
+    bool nidx_valid;   // nidx holds the last tree's node ids
+    uint8_t last_cond;
 
     // profiling
     bool profiling;
@@ -165,6 +169,7 @@ int launch_fill_bytes(evt_ctx *c, void *dst, int64_t nbytes);
 // predict
 int launch_predict_tree_cache(evt_ctx *c);
 int launch_hist_export(evt_ctx *c, double *out_dev);
+int launch_nidx_from_tree(evt_ctx *c, bool use_mask, uint8_t cond);
 
 // profiling helpers
 void prof_begin(evt_ctx *c, int cls, int level);

@@ -36,6 +36,7 @@ struct HistArgs {
     int64_t node_stride;
     int RS, LPR, RPW, F, nfs, B, NAg, level;
     int slots_per_tile;
+    int min_rows;
 };
 
 template <int NA, bool PACK>
@@ -49,8 +50,11 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) A.stats[A.level] = total;
 
     const int step = nwaves * A.RPW; // rows per block iteration
+    // rows per block: an even share, but never so few that the flush of a whole LDS histogram
+    // (and the chain of same-address global atomics it joins) outweighs the rows it covers
     int64_t T = (total + gridDim.x - 1) / gridDim.x;
-    T = ((T + step - 1) / step) * step;
+    if (T < A.min_rows) T = A.min_rows;
+    T = ((T + 2 * step - 1) / (2 * step)) * (2 * step);
     int64_t start = (int64_t)blockIdx.x * T;
     if (start >= total) return;
     int64_t end = start + T < total ? start + T : total;
@@ -62,19 +66,20 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
 
     for (int i = tid; i < NA * plane; i += nthr) H[i] = 0ull;
 
-    // the 16 features this lane owns -> LDS word offset of their first bin (-1: not in this tile)
+    // the 16 features this lane owns -> LDS word offset of their first bin (vmask bit t: in this tile)
     const int sub = lane % A.LPR, rloc = lane / A.LPR;
     int off[16];
-    bool any = false;
+    unsigned vmask = 0;
 #pragma unroll
     for (int t = 0; t < 16; t++) {
         int f = sub * 16 + t;
         int s = (f < A.F) ? (int)A.jsmap[f] : 0xFFFF;
         s = (s == 0xFFFF) ? -1 : s - slot0;
-        off[t] = (s >= 0 && s < nslots) ? s * A.B : -1;
-        any |= off[t] >= 0;
+        const bool ok = (s >= 0 && s < nslots);
+        off[t] = ok ? s * A.B - 1 : 0; // bins are 1-based
+        vmask |= ok ? (1u << t) : 0u;
     }
-    const bool lane_on = (rloc < A.RPW) && any;
+    const bool lane_on = (rloc < A.RPW) && vmask != 0;
     __syncthreads();
 
     // first node of this block's span: largest i with bprefix[i] <= start
@@ -84,35 +89,68 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
         if (A.bprefix[mid] <= start) lo = mid; else hi = mid;
     }
     int i = lo;
+    const int64_t blk_start = start, blk_end = end;
 
     while (start < end) {
+        const int64_t nbeg = A.bprefix[i];
         const int64_t nxt = A.bprefix[i + 1];
         const int64_t nend = end < nxt ? end : nxt;
-        const int64_t seg = A.bstart[i] - A.bprefix[i]; // position in the row list = seg + p
-        for (int64_t b0 = start + (int64_t)wave * A.RPW; b0 < nend; b0 += step) {
-            const int64_t p = b0 + rloc;
-            if (lane_on && p < nend) {
-                const uint32_t row = A.is[seg + p];
-                const uint4 v = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)row * A.RS + sub * 16);
-                unsigned long long g[NA];
+        const int64_t seg = A.bstart[i] - nbeg; // position in the row list = seg + p
+        // two row groups per iteration: all loads are issued before the first LDS atomic
+        for (int64_t b0 = start + (int64_t)wave * A.RPW; b0 < nend; b0 += 2 * step) {
+            const int64_t p0 = b0 + rloc, p1 = p0 + step;
+            const bool a0 = lane_on && p0 < nend, a1 = lane_on && p1 < nend;
+            uint32_t r0 = 0, r1 = 0;
+            if (a0) r0 = A.is[seg + p0];
+            if (a1) r1 = A.is[seg + p1];
+            uint4 v0 = make_uint4(0, 0, 0, 0), v1 = make_uint4(0, 0, 0, 0);
+            unsigned long long g0[NA], g1[NA];
+            if (a0) {
+                v0 = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)r0 * A.RS + sub * 16);
 #pragma unroll
-                for (int a = 0; a < NA; a++) g[a] = A.gq[(size_t)a * A.N + row];
-                const uint32_t wds[4] = {v.x, v.y, v.z, v.w};
+                for (int a = 0; a < NA; a++) g0[a] = A.gq[(size_t)a * A.N + r0];
+            }
+            if (a1) {
+                v1 = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)r1 * A.RS + sub * 16);
+#pragma unroll
+                for (int a = 0; a < NA; a++) g1[a] = A.gq[(size_t)a * A.N + r1];
+            }
+            if (a0) {
+                const uint32_t wds[4] = {v0.x, v0.y, v0.z, v0.w};
 #pragma unroll
                 for (int t = 0; t < 16; t++) {
-                    const uint32_t bin = (wds[t >> 2] >> (8 * (t & 3))) & 0xFFu;
-                    if (off[t] >= 0 && bin != 0) {
-                        const int idx = off[t] + (int)bin - 1;
+                    if (vmask & (1u << t)) {
+                        const int idx = off[t] + (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu);
 #pragma unroll
-                        for (int a = 0; a < NA; a++) atomicAdd(&H[a * plane + idx], g[a]);
+                        for (int a = 0; a < NA; a++) atomicAdd(&H[a * plane + idx], g0[a]);
+                    }
+                }
+            }
+            if (a1) {
+                const uint32_t wds[4] = {v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+                for (int t = 0; t < 16; t++) {
+                    if (vmask & (1u << t)) {
+                        const int idx = off[t] + (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu);
+#pragma unroll
+                        for (int a = 0; a < NA; a++) atomicAdd(&H[a * plane + idx], g1[a]);
                     }
                 }
             }
         }
         __syncthreads();
-        // flush this node's partial histogram: hist[node][slot][ag][bin]
+        // flush this node's partial histogram: hist[node][slot][ag][bin].  A node whose rows all lie in
+        // this block's span has a single writer: plain stores into its zero-initialised slice; a node
+        // shared with other blocks is accumulated with 64-bit global atomics.
+        const bool sole = (nbeg >= blk_start) && (nxt <= blk_end);
         long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
-        for (int idx = tid; idx < NA * plane; idx += nthr) {
+        // blocks start at different words so that concurrent flushes of one node do not queue on the
+        // same addresses
+        const int nwords = NA * plane;
+        const int rot = (int)(((int64_t)blockIdx.x * 1021) % nwords);
+        for (int k = tid; k < nwords; k += nthr) {
+            int idx = k + rot;
+            if (idx >= nwords) idx -= nwords;
             const unsigned long long w = H[idx];
             if (w != 0ull) {
                 H[idx] = 0ull;
@@ -124,8 +162,15 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
                 if (PACK && a == 0) {
                     const long long gsum = (long long)w >> EVT_PACK_CNT_BITS;
                     const unsigned long long cnt = w & ((1ull << EVT_PACK_CNT_BITS) - 1ull);
-                    if (gsum != 0) atomicAdd(base, (unsigned long long)gsum);
-                    atomicAdd(base + (int64_t)(A.NAg - 1) * A.B, cnt);
+                    if (sole) {
+                        base[0] = (unsigned long long)gsum;
+                        base[(int64_t)(A.NAg - 1) * A.B] = cnt;
+                    } else {
+                        if (gsum != 0) atomicAdd(base, (unsigned long long)gsum);
+                        atomicAdd(base + (int64_t)(A.NAg - 1) * A.B, cnt);
+                    }
+                } else if (sole) {
+                    base[(int64_t)a * A.B] = w;
                 } else {
                     atomicAdd(base + (int64_t)a * A.B, w);
                 }
@@ -182,6 +227,7 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
     int ntiles = (nfs + slots_per_tile - 1) / slots_per_tile;
     slots_per_tile = (nfs + ntiles - 1) / ntiles;
     A.slots_per_tile = slots_per_tile;
+    A.min_rows = c->hist_min_rows;
     size_t lds = per_slot * slots_per_tile;
     int threads = c->hist_threads;
     int64_t blocks = c->hist_blocks;

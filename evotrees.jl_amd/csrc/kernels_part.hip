@@ -47,7 +47,7 @@ struct PartArgs {
     uint32_t *nidx;
     float *pred;
     const float *t_pred;
-    int K, loss, fuse_pred;
+    int K, loss, fuse_pred, write_nidx;
 };
 
 __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
                 }
             }
             __syncthreads();
-        } else if (st == ST_LEAF) {
+        } else if (st == ST_LEAF && (A.write_nidx || A.fuse_pred)) {
             // rows of a node that stops here: record the node id; add the leaf value
             // (predict!, src/predict.jl:1-46: plain add / clamp(-15,15) / floor -15 on scale rows)
             const int K = A.K;
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
                 const int64_t p = p0 + it * 256 + tid;
                 if (p < pend) {
                     const uint32_t row = A.is_cur[p];
-                    A.nidx[row] = (uint32_t)n;
+                    if (A.write_nidx) A.nidx[row] = (uint32_t)n;
                     if (A.fuse_pred) {
                         float *pr = A.pred + (size_t)K * row;
                         const float *lp = A.t_pred + (size_t)K * (n - 1);
@@ -453,6 +453,7 @@ static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32
     A.K = c->K;
     A.loss = c->loss;
     A.fuse_pred = fuse_pred ? 1 : 0;
+    A.write_nidx = c->record_nidx ? 1 : 0;
 }
 
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur) {

@@ -43,6 +43,25 @@ __global__ __launch_bounds__(256) void k_predict_tree(const uint32_t *__restrict
     add_leaf(pred + (size_t)K * i, leaf_pred + (size_t)K * (nid - 1), K, loss);
 }
 
+// node each sampled row of the last tree ended in (0 outside the sample): the walk reproduces the
+// partition's decisions row by row (update_nodes_idx!, ext/EvoTreesKernelAbstractionsExt/fit-utils.jl:9-31)
+__global__ __launch_bounds__(256) void k_nidx_from_tree(const uint32_t *__restrict__ nodes, const uint8_t *__restrict__ xcm,
+                                                       const uint8_t *__restrict__ feattypes, int64_t N, const uint8_t *__restrict__ mask,
+                                                       uint32_t cond, uint32_t *out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N) return;
+    uint32_t r = 0;
+    if (!mask || mask[i] <= cond) r = (uint32_t)walk_packed(nodes, xcm, N, i, feattypes);
+    out[i] = r;
+}
+
+int launch_nidx_from_tree(evt_ctx *c, bool use_mask, uint8_t cond) {
+    hipLaunchKernelGGL(k_nidx_from_tree, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->tree.packed, c->xcm, c->feattypes,
+                       c->N, use_mask ? c->mask : nullptr, (uint32_t)cond, c->nidx);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
 int launch_predict_tree_cache(evt_ctx *c) {
     hipLaunchKernelGGL(k_predict_tree, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->tree.packed, c->tree.pred, c->xcm,
                        c->feattypes, c->N, c->K, c->loss, c->pred);

@@ -12,7 +12,13 @@
 
 #define NO_BIN 0x7fffffff
 
+struct ScanBest {
+    double gain;
+    int jp, bin;
+};
+
 struct ScanArgs {
+    ScanBest *sbest;
     long long *hist;
     int64_t node_stride;
     const uint32_t *js;
@@ -89,8 +95,45 @@ __device__ __forceinline__ double leaf_value(const double *S, int k, int K, doub
     return -eta / (double)bagging * S[k] / d;
 }
 
+// shared prologue: node totals -> Float64 statistics.  Root totals are the bin sums of its first
+// sampled feature (exact in integers: every feature's bins sum to the same total); other nodes carry
+// the totals their parent's split gave them.
 template <int NAG>
-__global__ __launch_bounds__(1024) void k_scan(ScanArgs A) {
+__device__ __forceinline__ void node_totals(const ScanArgs &A, int n, const long long *hn, bool writer, long long *s_Sq, double *s_S,
+                                            double *s_sc) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid < NAG) s_sc[tid] = A.qscale[tid];
+    if (A.level == 1) {
+        if (wave == 0) {
+            for (int ag = 0; ag < NAG; ag++) {
+                long long s = 0;
+                for (int b = lane; b < A.B; b += 64) s += hn[(int64_t)ag * A.B + b];
+                s = wave_sum_i64(s);
+                if (lane == 0) {
+                    s_Sq[ag] = s;
+                    if (writer) A.node_sum[(int64_t)n * NAG + ag] = s;
+                }
+            }
+        }
+    } else if (tid < NAG) {
+        s_Sq[tid] = A.node_sum[(int64_t)n * NAG + tid];
+    }
+    __syncthreads();
+    if (tid == 0) {
+        double v[EVT_MAX_NK];
+        long long q[NAG];
+        for (int ag = 0; ag < NAG; ag++) q[ag] = s_Sq[ag];
+        decode_vals(q, s_sc, A.loss, A.NK, v);
+        for (int k = 0; k < A.NK; k++) s_S[k] = v[k];
+    }
+    __syncthreads();
+}
+
+// Pass 1: grid (nodes of the level, feature groups); one wave per (node, sampled feature).
+// Writes the group's best candidate to sbest[node][group] (or the gain matrix for oblivious trees)
+// and, for subtract nodes, materialises h[n] = h[parent] - h[sibling].
+template <int NAG>
+__global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const int n = (1 << (A.level - 1)) + blockIdx.x; // 1-based node id
     const int st = A.status[n];
@@ -105,44 +148,12 @@ __global__ __launch_bounds__(1024) void k_scan(ScanArgs A) {
     __shared__ long long s_Sq[EVT_MAX_NA];
     __shared__ double s_S[EVT_MAX_NK];
     __shared__ double s_sc[EVT_MAX_NA];
-    __shared__ double s_wg[16];
-    __shared__ int s_wjp[16], s_wbin[16];
-    __shared__ int s_dec[4]; // found, jp, bin
-    __shared__ double s_gain;
+    __shared__ double s_wg[4];
+    __shared__ int s_wjp[4], s_wbin[4];
 
-    if (tid < NAG) s_sc[tid] = A.qscale[tid];
-    // node totals: carried from the parent's split, except the root whose totals are the bin sums
-    // of its first sampled feature (exact in integers, any feature gives the same total)
-    if (A.level == 1) {
-        if (wave == 0) {
-            for (int ag = 0; ag < NAG; ag++) {
-                long long s = 0;
-                for (int b = lane; b < B; b += 64) s += hn[(int64_t)ag * B + b];
-                s = wave_sum_i64(s);
-                if (lane == 0) { s_Sq[ag] = s; A.node_sum[(int64_t)n * NAG + ag] = s; }
-            }
-        }
-    } else if (tid < NAG) {
-        s_Sq[tid] = A.node_sum[(int64_t)n * NAG + tid];
-    }
-    __syncthreads();
-    if (tid == 0) {
-        double v[EVT_MAX_NK];
-        long long q[NAG];
-        for (int ag = 0; ag < NAG; ag++) q[ag] = s_Sq[ag];
-        decode_vals(q, s_sc, A.loss, NK, v);
-        for (int k = 0; k < NK; k++) s_S[k] = v[k];
-        A.tree.w[n - 1] = (float)v[NK - 1];
-    }
-    __syncthreads();
+    node_totals<NAG>(A, n, hn, blockIdx.y == 0, s_Sq, s_S, s_sc);
     double S[EVT_MAX_NK];
     for (int k = 0; k < NK; k++) S[k] = s_S[k];
-
-    if (A.leaf_level) {
-        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
-        if (tid == 0) A.status[n] = ST_LEAF;
-        return;
-    }
 
     double gain_p = 0.0;
     for (int k = 0; k < K; k++) gain_p += term_gh(S[k], S[K + k], S[2 * K], A.lambda, A.L2);
@@ -152,7 +163,8 @@ __global__ __launch_bounds__(1024) void k_scan(ScanArgs A) {
     int wjp = NO_BIN, wbin = NO_BIN;
     const int nodeidx = blockIdx.x;
 
-    for (int jp = wave; jp < A.nfs; jp += nwaves) {
+    const int jp = blockIdx.y * nwaves + wave;
+    if (jp < A.nfs) {
         const int f = (int)A.js[jp] - 1;
         const bool numeric = A.feattypes[f] != 0;
         const int constraint = A.mono[f];
@@ -249,9 +261,63 @@ __global__ __launch_bounds__(1024) void k_scan(ScanArgs A) {
         for (int w = 0; w < nwaves; w++) {
             if (s_wg[w] > bg || (s_wg[w] == bg && s_wjp[w] < bj)) { bg = s_wg[w]; bj = s_wjp[w]; bb = s_wbin[w]; }
         }
+        ScanBest r;
+        r.gain = bg; r.jp = bj; r.bin = bb;
+        A.sbest[(int64_t)nodeidx * gridDim.y + blockIdx.y] = r;
+    }
+}
+
+// Pass 2: one block per node.  Leaf level: leaf value only.  Otherwise: arg-max over the feature
+// groups (first maximum: highest gain, then earliest feature, whose bin is already the lowest),
+// split iff gain > gamma; writes the Tree arrays, the children's totals (_child_sums!: left = bins
+// 1..bin of the parent histogram, or that bin alone for categorical features; right = parent - left,
+// exact in integers) and zeroes the children's histogram slices.
+template <int NAG>
+__global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = (1 << (A.level - 1)) + blockIdx.x;
+    const int st = A.status[n];
+    if (st != ST_BUILD && st != ST_SUBTRACT) return;
+    const int B = A.B, NK = A.NK, K = A.K;
+    long long *hn = A.hist + (int64_t)(n - 1) * A.node_stride;
+
+    __shared__ long long s_Sq[EVT_MAX_NA];
+    __shared__ double s_S[EVT_MAX_NK];
+    __shared__ double s_sc[EVT_MAX_NA];
+    __shared__ double s_g[256];
+    __shared__ int s_j[256], s_b[256];
+    __shared__ int s_dec[3];
+
+    node_totals<NAG>(A, n, hn, true, s_Sq, s_S, s_sc);
+    double S[EVT_MAX_NK];
+    for (int k = 0; k < NK; k++) S[k] = s_S[k];
+    if (tid == 0) A.tree.w[n - 1] = (float)S[NK - 1];
+
+    if (A.leaf_level) {
+        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
+        if (tid == 0) A.status[n] = ST_LEAF;
+        return;
+    }
+    double bg = -INFINITY;
+    int bj = NO_BIN, bb = NO_BIN;
+    if (tid < ngroups) {
+        const ScanBest r = A.sbest[(int64_t)blockIdx.x * ngroups + tid];
+        bg = r.gain; bj = r.jp; bb = r.bin;
+    }
+    s_g[tid] = bg; s_j[tid] = bj; s_b[tid] = bb;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (tid < o) {
+            if (s_g[tid + o] > s_g[tid] || (s_g[tid + o] == s_g[tid] && s_j[tid + o] < s_j[tid])) {
+                s_g[tid] = s_g[tid + o]; s_j[tid] = s_j[tid + o]; s_b[tid] = s_b[tid + o];
+            }
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        bg = s_g[0]; bj = s_j[0]; bb = s_b[0];
         const int found = (bb != NO_BIN && bg > A.gamma) ? 1 : 0;
         s_dec[0] = found; s_dec[1] = bj; s_dec[2] = bb;
-        s_gain = bg;
         if (found) {
             const int feat = (int)A.js[bj];
             A.tree.feat[n - 1] = feat;
@@ -267,10 +333,8 @@ __global__ __launch_bounds__(1024) void k_scan(ScanArgs A) {
     }
     __syncthreads();
     if (!s_dec[0]) return;
-    const int bj = s_dec[1], bb = s_dec[2];
-    // _child_sums!: left = bins 1..bb of the parent histogram (numeric) or bin bb alone (categorical);
-    // right = parent - left.  Exact in integers.
-    if (wave == 0) {
+    bj = s_dec[1]; bb = s_dec[2];
+    if (wave == 0) { // pass 1 already materialised h[n] for subtract nodes
         const int f = (int)A.js[bj] - 1;
         const bool numeric = A.feattypes[f] != 0;
         for (int ag = 0; ag < NAG; ag++) {
@@ -278,7 +342,7 @@ __global__ __launch_bounds__(1024) void k_scan(ScanArgs A) {
             long long s = 0;
             for (int b = lane; b < B; b += 64) {
                 const bool in = numeric ? (b + 1 <= bb) : (b + 1 == bb);
-                if (in) s += is_sub ? (hp[o + b] - hs[o + b]) : hn[o + b];
+                if (in) s += hn[o + b];
             }
             s = wave_sum_i64(s);
             if (lane == 0) {
@@ -287,7 +351,7 @@ __global__ __launch_bounds__(1024) void k_scan(ScanArgs A) {
             }
         }
     }
-    // the children's histogram slices start from zero (the build child is filled with atomics)
+    // the children's histogram slices start from zero (the build child accumulates into it)
     if (!A.zero_children) return;
     long long *hc = A.hist + (int64_t)(2 * n - 1) * A.node_stride;
     const int64_t used = (int64_t)A.nfs * NAG * B;
@@ -372,6 +436,7 @@ __global__ __launch_bounds__(1024) void k_obliv_select(OblivArgs A) {
         double S[EVT_MAX_NK];
         for (int ag = 0; ag < NAG; ag++) Sq[ag] = A.node_sum[(int64_t)n * NAG + ag];
         decode_vals(Sq, s_sc, A.loss, NK, S);
+        if (lane == 0) A.tree.w[n - 1] = (float)S[NK - 1];
         if (!found) {
             if (lane < K) A.tree.pred[(int64_t)K * (n - 1) + lane] = (float)leaf_value(S, lane, K, A.eta, A.bagging, A.lambda, A.L2);
             if (lane == 0) A.status[n] = ST_LEAF;
@@ -413,6 +478,7 @@ __global__ __launch_bounds__(1024) void k_obliv_select(OblivArgs A) {
 
 int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     ScanArgs A;
+    A.sbest = reinterpret_cast<ScanBest *>(c->sbest);
     A.hist = c->hist;
     A.node_stride = (int64_t)c->F * c->NAg * c->B;
     A.js = c->js;
@@ -430,15 +496,21 @@ int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     A.leaf_level = leaf_level ? 1 : 0;
     A.oblivious = (c->tree_type == EVT_TREE_OBLIVIOUS) ? 1 : 0;
     A.zero_children = (level + 1 < c->D) ? 1 : 0; // children at the last level never get a histogram
-    dim3 grid(1u << (level - 1));
-    int threads = 1024;
-    if (level > 6) threads = 256; // many nodes per level: smaller blocks, same total parallelism
+    const unsigned nodes = 1u << (level - 1);
+    const int ngroups = (A.nfs + 3) / 4; // 4 waves per block, one sampled feature each
+    dim3 grid(nodes, (unsigned)ngroups);
+#define SCASE(NAG_)                                                                                     \
+    case NAG_:                                                                                          \
+        if (!leaf_level) hipLaunchKernelGGL(k_scan<NAG_>, grid, dim3(256), 0, c->stream, A);            \
+        if (!A.oblivious || leaf_level) hipLaunchKernelGGL(k_scan_fin<NAG_>, dim3(nodes), dim3(256), 0, c->stream, A, ngroups); \
+        break;
     switch (c->NAg) {
-    case 2: hipLaunchKernelGGL(k_scan<2>, grid, dim3(threads), 0, c->stream, A); break;
-    case 3: hipLaunchKernelGGL(k_scan<3>, grid, dim3(threads), 0, c->stream, A); break;
-    case 5: hipLaunchKernelGGL(k_scan<5>, grid, dim3(threads), 0, c->stream, A); break;
+        SCASE(2)
+        SCASE(3)
+        SCASE(5)
     default: evt_set_error("unsupported global channel count %d", c->NAg); return EVT_ERR_ARG;
     }
+#undef SCASE
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

@@ -125,6 +125,7 @@ def test_grow_tree_matches_oracle(evt, loss, weights, N, F, B, D, tt, n_js, rows
         rows = orc.subsample(mask, cond)
     else:
         mask, cond, rows = None, 255, np.arange(N, dtype=np.uint32)
+    h.set_option("record_nidx", 1)  # node ids written by the partition itself while the tree grows
     t_gpu = h.grow_tree(js, gp, mask=mask, cond=cond)
     nidx_gpu = h.get_nidx()
     # fixed-point oracle: bit exact
@@ -157,6 +158,15 @@ def test_grow_tree_matches_oracle(evt, loss, weights, N, F, B, D, tt, n_js, rows
     p_orc = pred0.copy()
     o.predict_tree(t_fx, p_orc)
     assert np.array_equal(p_gpu.view(np.uint32), p_orc.view(np.uint32))
+    # without recording, the node ids are derived by walking the finished tree: same answer
+    h.set_option("record_nidx", 0)
+    t_again = h.grow_tree(js, gp, mask=mask, cond=cond)
+    assert_tree_bits(t_again, t_fx)
+    assert np.array_equal(h.get_nidx(), nidx_fx)
+    # launch shape must not change a bit of the result (integer accumulation is order independent)
+    h.set_option("hist_blocks", 37)
+    h.set_option("hist_threads", 256)
+    assert_tree_bits(h.grow_tree(js, gp, mask=mask, cond=cond), t_fx)
     h.close()
     o.close()
 
@@ -177,7 +187,7 @@ def test_categorical_and_monotone(evt):
     o.set_quant(grad, qb)
     t_fx, nidx_fx = o.grow_tree(grad, rows, js, mode=1)
     assert_tree_bits(t_gpu, t_fx)
-    assert np.array_equal(h.get_nidx(), nidx_fx)
+    assert np.array_equal(h.get_nidx(), nidx_fx)  # derived by walking the finished tree
     t_ref, _ = o.grow_tree(grad, rows, js, mode=0)
     assert_tree_close(t_gpu, t_ref)
     assert any(t_gpu.split[n] and feattypes[t_gpu.feat[n] - 1] == 0 for n in range(len(t_gpu.split)))
