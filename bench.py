@@ -105,6 +105,8 @@ def main():
     ap.add_argument("--hist-blocks", type=int, default=0)
     ap.add_argument("--hist-threads", type=int, default=0)
     ap.add_argument("--hist-min-rows", type=int, default=0)
+    ap.add_argument("--hist-variant", type=int, default=0)
+    ap.add_argument("--hist-small-rows", type=int, default=-1)
     ap.add_argument("--predict", action="store_true", help="also time model inference on the training rows")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -135,6 +137,10 @@ def main():
         h.set_option("hist_threads", args.hist_threads)
     if args.hist_min_rows:
         h.set_option("hist_min_rows", args.hist_min_rows)
+    if args.hist_variant:
+        h.set_option("hist_variant", args.hist_variant)
+    if args.hist_small_rows >= 0:
+        h.set_option("hist_small_rows", args.hist_small_rows)
     t_setup = time.time() - t0
 
     params = evt.make_params(eta=cfg["eta"], min_weight=cfg["min_weight"], update_pred=True)
@@ -203,8 +209,9 @@ def main():
         per_level.append(tot)
     out["last_tree_rows_built_per_level"] = per_level
     try:
-        out["copy_kernel_GBps"] = round(evt._lib.copy_bandwidth(1 << 30, 10), 1)
-    except Exception as e:  # measurement aid only
+        out["copy_kernel_GBps"] = round(evt._lib.copy_bandwidth(1 << 30, 10), 1)  # read + write bytes of a plain copy
+        out["read_kernel_GBps"] = round(evt._lib.read_bandwidth(1 << 30, 10), 1)  # read-only stream
+    except Exception:  # measurement aid only
         out["copy_kernel_GBps"] = None
 
     if args.predict:

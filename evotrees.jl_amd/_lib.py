@@ -22,7 +22,7 @@ EXPORTS = [
     "evt_set_target", "evt_set_feature_meta", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
     "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
     "evt_predict", "evt_predict_leaf_idx", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
-    "evt_set_option", "evt_synchronize", "evt_copy_bandwidth",
+    "evt_set_option", "evt_synchronize", "evt_copy_bandwidth", "evt_read_bandwidth",
 ]
 
 
@@ -83,6 +83,7 @@ def load():
         "evt_set_option": [vp, C.c_char_p, i64],
         "evt_synchronize": [vp],
         "evt_copy_bandwidth": [i64, i32, vp],
+        "evt_read_bandwidth": [i64, i32, vp],
     }
     for name, args in sigs.items():
         f = getattr(L, name)
@@ -112,6 +113,12 @@ def device_count():
 def copy_bandwidth(nbytes=1 << 30, iters=10):
     out = C.c_double(0.0)
     check(load().evt_copy_bandwidth(nbytes, iters, C.byref(out)))
+    return out.value
+
+
+def read_bandwidth(nbytes=1 << 30, iters=10):
+    out = C.c_double(0.0)
+    check(load().evt_read_bandwidth(nbytes, iters, C.byref(out)))
     return out.value
 
 

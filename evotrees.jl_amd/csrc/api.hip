@@ -180,8 +180,10 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->n_js_last = 0;
     c->last_all_rows = true;
     c->hist_blocks = 512;
-    c->hist_threads = 1024;
+    c->hist_threads = 512;
     c->hist_min_rows = 2048;
+    c->hist_variant = 1;
+    c->hist_small_rows = 0;
     c->record_nidx = false;
     c->nidx_valid = false;
     c->last_cond = 255;
@@ -841,6 +843,12 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
     } else if (strcmp(name, "hist_min_rows") == 0) {
         ARGCHK(value >= 1 && value <= EVT_HIST_MAX_ROWS_PER_BLOCK, "hist_min_rows must be in [1, 32768]");
         c->hist_min_rows = (int)value;
+    } else if (strcmp(name, "hist_small_rows") == 0) {
+        ARGCHK(value >= 0 && value <= 65536, "hist_small_rows must be in [0, 65536]");
+        c->hist_small_rows = (int)value;
+    } else if (strcmp(name, "hist_variant") == 0) {
+        ARGCHK(value >= 0 && value <= 2, "hist_variant must be 0 (auto), 1 (generic) or 2 (conflict-free)");
+        c->hist_variant = (int)value;
     } else if (strcmp(name, "record_nidx") == 0) {
         c->record_nidx = value != 0;
     } else if (strcmp(name, "hist_threads") == 0) {
@@ -860,6 +868,50 @@ extern "C" int evt_synchronize(evt_handle c) {
 
 __global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = src[i];
+}
+
+__global__ __launch_bounds__(256) void k_read16(const uint4 *__restrict__ src, int64_t n, unsigned int *sink) {
+    unsigned int acc = 0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const uint4 v = src[i];
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x12345678u) sink[0] = acc; // keeps the loads alive without a write stream
+}
+
+extern "C" int evt_read_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out) {
+    ARGCHK(gbps_out && nbytes >= 4096 && iters >= 1, "invalid arguments");
+    int ndev = 0;
+    int r = evt_device_count(&ndev);
+    if (r != EVT_OK) return r;
+    const int64_t n = nbytes / 16;
+    uint4 *a = nullptr;
+    unsigned int *sink = nullptr;
+    HIPCHK(hipMalloc((void **)&a, n * 16));
+    hipError_t e = hipMalloc((void **)&sink, 64);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipMemset(a, 1, n * 16);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(k_read16, dim3(8192), dim3(256), 0, 0, a, n, sink);
+        e = hipEventRecord(e0, 0);
+        for (int i = 0; i < iters; i++) hipLaunchKernelGGL(k_read16, dim3(8192), dim3(256), 0, 0, a, n, sink);
+        if (e == hipSuccess) e = hipEventRecord(e1, 0);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (a) (void)hipFree(a);
+    if (sink) (void)hipFree(sink);
+    if (e != hipSuccess) {
+        evt_set_error("read bandwidth probe failed: %s", hipGetErrorString(e));
+        return EVT_ERR_HIP;
+    }
+    *gbps_out = (double)(n * 16) * iters / ((double)ms * 1e-3) / 1e9;
+    return EVT_OK;
 }
 
 extern "C" int evt_copy_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out) {

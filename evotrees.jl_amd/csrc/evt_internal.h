@@ -113,7 +113,8 @@ struct evt_ctx {
     bool last_all_rows;
 
     // tunables
-    int hist_blocks, hist_threads, hist_min_rows;
+    int hist_blocks, hist_threads, hist_min_rows, hist_small_rows;
+    int hist_variant;  // 0 auto, 1 generic 16-byte-piece kernel, 2 conflict-free 8-byte-piece kernel where it applies
     bool record_nidx;  // leaf finalisation also writes the node id of every sampled row
     bool nidx_valid;   // nidx holds the last tree's node ids
     uint8_t last_cond;

@@ -37,6 +37,7 @@ struct HistArgs {
     int RS, LPR, RPW, F, nfs, B, NAg, level;
     int slots_per_tile;
     int min_rows;
+    int small_rows;
 };
 
 template <int NA, bool PACK>
@@ -96,45 +97,109 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
         const int64_t nxt = A.bprefix[i + 1];
         const int64_t nend = end < nxt ? end : nxt;
         const int64_t seg = A.bstart[i] - nbeg; // position in the row list = seg + p
-        // two row groups per iteration: all loads are issued before the first LDS atomic
-        for (int64_t b0 = start + (int64_t)wave * A.RPW; b0 < nend; b0 += 2 * step) {
-            const int64_t p0 = b0 + rloc, p1 = p0 + step;
-            const bool a0 = lane_on && p0 < nend, a1 = lane_on && p1 < nend;
-            uint32_t r0 = 0, r1 = 0;
-            if (a0) r0 = A.is[seg + p0];
-            if (a1) r1 = A.is[seg + p1];
-            uint4 v0 = make_uint4(0, 0, 0, 0), v1 = make_uint4(0, 0, 0, 0);
-            unsigned long long g0[NA], g1[NA];
-            if (a0) {
-                v0 = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)r0 * A.RS + sub * 16);
+        if (nend - start <= A.small_rows) {
+            // a short run of this node's rows: cheaper to add straight into the global histogram than
+            // to scan and flush a whole LDS histogram for it
+            unsigned long long *hg = reinterpret_cast<unsigned long long *>(A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride);
+            for (int64_t b0 = start + (int64_t)wave * A.RPW; b0 < nend; b0 += step) {
+                const int64_t p = b0 + rloc;
+                if (lane_on && p < nend) {
+                    const uint32_t row = A.is[seg + p];
+                    const uint4 v = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)row * A.RS + sub * 16);
+                    unsigned long long g[NA];
 #pragma unroll
-                for (int a = 0; a < NA; a++) g0[a] = A.gq[(size_t)a * A.N + r0];
-            }
-            if (a1) {
-                v1 = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)r1 * A.RS + sub * 16);
+                    for (int a = 0; a < NA; a++) g[a] = A.gq[(size_t)a * A.N + row];
+                    const uint32_t wds[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                for (int a = 0; a < NA; a++) g1[a] = A.gq[(size_t)a * A.N + r1];
-            }
-            if (a0) {
-                const uint32_t wds[4] = {v0.x, v0.y, v0.z, v0.w};
+                    for (int t = 0; t < 16; t++) {
+                        if (vmask & (1u << t)) {
+                            const int slot = A.jsmap[sub * 16 + t];
+                            const int bin = (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu) - 1;
+                            unsigned long long *base = hg + ((int64_t)slot * A.NAg) * A.B + bin;
 #pragma unroll
-                for (int t = 0; t < 16; t++) {
-                    if (vmask & (1u << t)) {
-                        const int idx = off[t] + (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu);
-#pragma unroll
-                        for (int a = 0; a < NA; a++) atomicAdd(&H[a * plane + idx], g0[a]);
+                            for (int a = 0; a < NA; a++) {
+                                if (PACK && a == 0) {
+                                    const long long gs = (long long)g[0] >> EVT_PACK_CNT_BITS;
+                                    if (gs != 0) atomicAdd(base, (unsigned long long)gs);
+                                    atomicAdd(base + (int64_t)(A.NAg - 1) * A.B, 1ull);
+                                } else {
+                                    atomicAdd(base + (int64_t)a * A.B, g[a]);
+                                }
+                            }
+                        }
                     }
                 }
             }
-            if (a1) {
-                const uint32_t wds[4] = {v1.x, v1.y, v1.z, v1.w};
+            start = nend;
+            i++;
+            continue;
+        }
+        // software pipeline over U row groups per wave: the row ids of iteration k+2 and the records of
+        // iteration k+1 are in flight while the LDS atomics of iteration k are issued
+        {
+            constexpr int U = 2;
+            constexpr uint32_t INV = 0xFFFFFFFFu;
+            const int64_t itstride = (int64_t)U * step;
+            uint32_t rc[U], rn[U];
+            uint4 vc[U], vn[U];
+            unsigned long long gc[U][NA], gn[U][NA];
+            int64_t b0 = start + (int64_t)wave * A.RPW;
 #pragma unroll
-                for (int t = 0; t < 16; t++) {
-                    if (vmask & (1u << t)) {
-                        const int idx = off[t] + (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu);
+            for (int u = 0; u < U; u++) {
+                const int64_t p = b0 + (int64_t)u * step + rloc;
+                rc[u] = (lane_on && p < nend) ? A.is[seg + p] : INV;
+            }
 #pragma unroll
-                        for (int a = 0; a < NA; a++) atomicAdd(&H[a * plane + idx], g1[a]);
+            for (int u = 0; u < U; u++) {
+                vc[u] = make_uint4(0, 0, 0, 0);
+                if (rc[u] != INV) {
+                    vc[u] = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)rc[u] * A.RS + sub * 16);
+#pragma unroll
+                    for (int a = 0; a < NA; a++) gc[u][a] = A.gq[(size_t)a * A.N + rc[u]];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int64_t p = b0 + itstride + (int64_t)u * step + rloc;
+                rn[u] = (lane_on && p < nend) ? A.is[seg + p] : INV;
+            }
+            for (; b0 < nend; b0 += itstride) {
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    vn[u] = make_uint4(0, 0, 0, 0);
+                    if (rn[u] != INV) {
+                        vn[u] = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)rn[u] * A.RS + sub * 16);
+#pragma unroll
+                        for (int a = 0; a < NA; a++) gn[u][a] = A.gq[(size_t)a * A.N + rn[u]];
                     }
+                }
+                uint32_t rnn[U];
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const int64_t p = b0 + 2 * itstride + (int64_t)u * step + rloc;
+                    rnn[u] = (lane_on && p < nend) ? A.is[seg + p] : INV;
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    if (rc[u] != INV) {
+                        const uint32_t wds[4] = {vc[u].x, vc[u].y, vc[u].z, vc[u].w};
+#pragma unroll
+                        for (int t = 0; t < 16; t++) {
+                            if (vmask & (1u << t)) {
+                                const int idx = off[t] + (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu);
+#pragma unroll
+                                for (int a = 0; a < NA; a++) atomicAdd(&H[a * plane + idx], gc[u][a]);
+                            }
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    rc[u] = rn[u];
+                    vc[u] = vn[u];
+#pragma unroll
+                    for (int a = 0; a < NA; a++) gc[u][a] = gn[u][a];
+                    rn[u] = rnn[u];
                 }
             }
         }
@@ -180,6 +245,233 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
         start = nend;
         i++;
     }
+}
+
+// Bank-conflict-free variant for records of 128 / 256 / 512 bytes.
+//
+// A record is read as 8-byte pieces, NS = RS/8 lanes per row (a multiple of 16), so every group of
+// 16 consecutive lanes — the unit the LDS serves per cycle for 64-bit operations — holds 16 different
+// pieces `sub` of ONE row.  The LDS histogram is laid out as word(a, t, bin, sub) =
+// ((a*8 + t)*B + bin)*NS + sub for feature f = 8*sub + t, i.e. `sub` selects the bank pair, so the 16
+// lanes of a group always fall on 16 different bank pairs whatever their bins are.  Rows that share a
+// wave instruction sit in different groups and cannot collide inside one LDS pass either.
+template <int NA, bool PACK>
+__global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
+    extern __shared__ unsigned long long H[]; // [NA][8][B][NS]
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
+    const int n_build = (int)A.hdr[LH_N_BUILD];
+    const int64_t total = A.hdr[LH_TOTAL_BUILD];
+    if (n_build <= 0 || total <= 0) return;
+    if (blockIdx.x == 0 && tid == 0) A.stats[A.level] = total;
+
+    const int NS = A.RS >> 3;     // 8-byte pieces per record
+    const int RPW = 64 / NS;      // rows per wave instruction
+    const int step = nwaves * RPW;
+    int64_t T = (total + gridDim.x - 1) / gridDim.x;
+    if (T < A.min_rows) T = A.min_rows;
+    T = ((T + 4 * step - 1) / (4 * step)) * (4 * step);
+    int64_t start = (int64_t)blockIdx.x * T;
+    if (start >= total) return;
+    int64_t end = start + T < total ? start + T : total;
+
+    const int B = A.B;
+    const int plane = 8 * B * NS; // words per channel
+    for (int i = tid; i < NA * plane; i += nthr) H[i] = 0ull;
+
+    const int sub = lane % NS, rloc = lane / NS;
+    // byte offset of (t, bin 0) for this lane; bins are 1-based so bin*NS*8 is added on top
+    int coff[8];
+    unsigned vmask = 0;
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        const int f = sub * 8 + t;
+        const bool ok = (f < A.F) && (A.jsmap[f] != 0xFFFF);
+        coff[t] = ((t * B - 1) * NS + sub) * 8;
+        vmask |= ok ? (1u << t) : 0u;
+    }
+    const int binmul = NS * 8;
+    const bool lane_on = vmask != 0;
+    __syncthreads();
+
+    int lo = 0, hi = n_build;
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (A.bprefix[mid] <= start) lo = mid; else hi = mid;
+    }
+    int i = lo;
+    const int64_t blk_start = start, blk_end = end;
+    char *Hb = reinterpret_cast<char *>(H);
+
+    while (start < end) {
+        const int64_t nbeg = A.bprefix[i];
+        const int64_t nxt = A.bprefix[i + 1];
+        const int64_t nend = end < nxt ? end : nxt;
+        const int64_t seg = A.bstart[i] - nbeg;
+        if (nend - start <= A.small_rows) {
+            // a short run of this node's rows: cheaper to add straight into the global histogram than
+            // to scan and flush a whole LDS histogram for it
+            unsigned long long *hg = reinterpret_cast<unsigned long long *>(A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride);
+            for (int64_t b0 = start + (int64_t)wave * RPW; b0 < nend; b0 += step) {
+                const int64_t p = b0 + rloc;
+                if (lane_on && p < nend) {
+                    const uint32_t row = A.is[seg + p];
+                    const uint2 v = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)row * A.RS + sub * 8);
+                    unsigned long long g[NA];
+#pragma unroll
+                    for (int a = 0; a < NA; a++) g[a] = A.gq[(size_t)a * A.N + row];
+                    const uint32_t wds[2] = {v.x, v.y};
+#pragma unroll
+                    for (int t = 0; t < 8; t++) {
+                        if (vmask & (1u << t)) {
+                            const int slot = A.jsmap[sub * 8 + t];
+                            const int bin = (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu) - 1;
+                            unsigned long long *base = hg + ((int64_t)slot * A.NAg) * B + bin;
+#pragma unroll
+                            for (int a = 0; a < NA; a++) {
+                                if (PACK && a == 0) {
+                                    const long long gs = (long long)g[0] >> EVT_PACK_CNT_BITS;
+                                    if (gs != 0) atomicAdd(base, (unsigned long long)gs);
+                                    atomicAdd(base + (int64_t)(A.NAg - 1) * B, 1ull);
+                                } else {
+                                    atomicAdd(base + (int64_t)a * B, g[a]);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+            start = nend;
+            i++;
+            continue;
+        }
+        // software pipeline over U row groups per wave: the row ids of iteration k+2 and the records of
+        // iteration k+1 are in flight while the LDS atomics of iteration k are issued
+        {
+            constexpr int U = 4;
+            constexpr uint32_t INV = 0xFFFFFFFFu;
+            const int64_t itstride = (int64_t)U * step;
+            uint32_t rc[U], rn[U];
+            uint2 vc[U], vn[U];
+            unsigned long long gc[U][NA], gn[U][NA];
+            int64_t b0 = start + (int64_t)wave * RPW;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int64_t p = b0 + (int64_t)u * step + rloc;
+                rc[u] = (lane_on && p < nend) ? A.is[seg + p] : INV;
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                vc[u] = make_uint2(0, 0);
+                if (rc[u] != INV) {
+                    vc[u] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)rc[u] * A.RS + sub * 8);
+#pragma unroll
+                    for (int a = 0; a < NA; a++) gc[u][a] = A.gq[(size_t)a * A.N + rc[u]];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int64_t p = b0 + itstride + (int64_t)u * step + rloc;
+                rn[u] = (lane_on && p < nend) ? A.is[seg + p] : INV;
+            }
+            for (; b0 < nend; b0 += itstride) {
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    vn[u] = make_uint2(0, 0);
+                    if (rn[u] != INV) {
+                        vn[u] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)rn[u] * A.RS + sub * 8);
+#pragma unroll
+                        for (int a = 0; a < NA; a++) gn[u][a] = A.gq[(size_t)a * A.N + rn[u]];
+                    }
+                }
+                uint32_t rnn[U];
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const int64_t p = b0 + 2 * itstride + (int64_t)u * step + rloc;
+                    rnn[u] = (lane_on && p < nend) ? A.is[seg + p] : INV;
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    if (rc[u] != INV) {
+                        const uint32_t wds[2] = {vc[u].x, vc[u].y};
+#pragma unroll
+                        for (int t = 0; t < 8; t++) {
+                            if (vmask & (1u << t)) {
+                                const int bo = coff[t] + (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu) * binmul;
+#pragma unroll
+                                for (int a = 0; a < NA; a++)
+                                    atomicAdd(reinterpret_cast<unsigned long long *>(Hb + bo + a * plane * 8), gc[u][a]);
+                            }
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    rc[u] = rn[u];
+                    vc[u] = vn[u];
+#pragma unroll
+                    for (int a = 0; a < NA; a++) gc[u][a] = gn[u][a];
+                    rn[u] = rnn[u];
+                }
+            }
+        }
+        __syncthreads();
+        // flush: a wave covers 8 consecutive bins x 8 consecutive pieces `sub` of one (channel, t): global
+        // accesses are whole 64-byte runs of one feature's bins, LDS reads spread over 8 bank pairs.  Blocks
+        // start at different items so that concurrent flushes of one node do not queue on the same addresses.
+        const bool sole = (nbeg >= blk_start) && (nxt <= blk_end);
+        long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
+        const int nchunks = (B + 7) >> 3;
+        const int nsg = NS >> 3;
+        const int nitems = NA * 8 * nchunks * nsg * 64;
+        const int rot = (int)(((int64_t)blockIdx.x * 1031) % (nitems >> 6)) << 6;
+        for (int k0 = tid; k0 < nitems; k0 += nthr) {
+            int k = k0 + rot;
+            if (k >= nitems) k -= nitems;
+            const int bl = k & 7, sl = (k >> 3) & 7;
+            int rest = k >> 6;
+            const int chunk = rest % nchunks; rest /= nchunks;
+            const int sg = rest % nsg; rest /= nsg;
+            const int t = rest & 7;
+            const int a = rest >> 3;
+            const int b = chunk * 8 + bl;
+            const int sidx = sg * 8 + sl;
+            const int f = sidx * 8 + t;
+            if (b >= B || f >= A.F) continue;
+            unsigned long long *hw = &H[(size_t)a * plane + ((size_t)t * B + b) * NS + sidx];
+            const unsigned long long w = *hw;
+            if (w == 0ull) continue;
+            *hw = 0ull;
+            const int slot = A.jsmap[f];
+            if (slot == 0xFFFF) continue;
+            unsigned long long *base = reinterpret_cast<unsigned long long *>(hn) + ((int64_t)slot * A.NAg) * B + b;
+            if (PACK && a == 0) {
+                const long long gsum = (long long)w >> EVT_PACK_CNT_BITS;
+                const unsigned long long cnt = w & ((1ull << EVT_PACK_CNT_BITS) - 1ull);
+                if (sole) {
+                    base[0] = (unsigned long long)gsum;
+                    base[(int64_t)(A.NAg - 1) * B] = cnt;
+                } else {
+                    if (gsum != 0) atomicAdd(base, (unsigned long long)gsum);
+                    atomicAdd(base + (int64_t)(A.NAg - 1) * B, cnt);
+                }
+            } else if (sole) {
+                base[(int64_t)a * B] = w;
+            } else {
+                atomicAdd(base + (int64_t)a * B, w);
+            }
+        }
+        __syncthreads();
+        start = nend;
+        i++;
+    }
+}
+
+template <int NA, bool PACK>
+static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
+    hipLaunchKernelGGL((k_hist_build16<NA, PACK>), grid, dim3(threads), lds, c->stream, A);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
 }
 
 template <int NA, bool PACK>
@@ -228,6 +520,7 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
     slots_per_tile = (nfs + ntiles - 1) / ntiles;
     A.slots_per_tile = slots_per_tile;
     A.min_rows = c->hist_min_rows;
+    A.small_rows = c->hist_small_rows;
     size_t lds = per_slot * slots_per_tile;
     int threads = c->hist_threads;
     int64_t blocks = c->hist_blocks;
@@ -235,6 +528,23 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
     if (blocks < need) blocks = need;
     dim3 grid((unsigned)blocks, (unsigned)ntiles);
     const bool pack = c->unit_w;
+    // conflict-free variant: records of 128/256/512 bytes whose whole LDS histogram fits 64 KB
+    const size_t lds16 = (size_t)c->NA * 8 * c->B * (c->RS / 8) * 8;
+    const bool can16 = (c->RS % 128 == 0) && c->RS <= 512 && lds16 <= 64 * 1024;
+    const bool use16 = (c->hist_variant == 2) ? can16 : (c->hist_variant == 1 ? false : can16);
+    if (use16) {
+        dim3 grid16((unsigned)blocks, 1u);
+#define H16CASE(NA_) \
+    case NA_: return pack ? launch_hist16_t<NA_, true>(c, A, grid16, threads, lds16) : launch_hist16_t<NA_, false>(c, A, grid16, threads, lds16);
+        switch (c->NA) {
+            H16CASE(1)
+            H16CASE(2)
+            H16CASE(3)
+            H16CASE(4)
+            H16CASE(5)
+        }
+#undef H16CASE
+    }
 #define HCASE(NA_) \
     case NA_: return pack ? launch_hist_t<NA_, true>(c, A, grid, threads, lds) : launch_hist_t<NA_, false>(c, A, grid, threads, lds);
     switch (c->NA) {

@@ -183,6 +183,8 @@ int evt_synchronize(evt_handle h);
 /* Plain device copy of nbytes (read + write) timed with HIP events: the box's streaming
  * ceiling that roofline figures are quoted beside. */
 int evt_copy_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out);
+/* Same for a read-only stream of nbytes (no write traffic). */
+int evt_read_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out);
 
 #ifdef __cplusplus
 }

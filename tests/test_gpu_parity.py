@@ -104,6 +104,10 @@ CASES = [
     ("mse", False, 30000, 12, 32, 6, "oblivious", 12, 1.0, {}),
     ("logloss", True, 30000, 12, 32, 5, "oblivious", 8, 0.6, {}),
     ("mse", False, 5000, 200, 8, 4, "binary", 200, 1.0, {}),
+    ("mse", True, 40000, 120, 32, 6, "binary", 120, 1.0, {}),
+    ("logloss", False, 40000, 100, 32, 6, "binary", 70, 0.7, {}),
+    ("gaussian_mle", False, 30000, 128, 8, 5, "binary", 128, 1.0, dict(min_weight=8.0)),
+    ("mse", False, 20000, 300, 16, 5, "binary", 300, 1.0, {}),
     ("mse", False, 1000, 3, 4, 1, "binary", 3, 1.0, {}),
     ("mse", False, 300, 1, 2, 3, "binary", 1, 1.0, dict(min_weight=0.0)),
 ]
@@ -167,6 +171,14 @@ def test_grow_tree_matches_oracle(evt, loss, weights, N, F, B, D, tt, n_js, rows
     h.set_option("hist_blocks", 37)
     h.set_option("hist_threads", 256)
     assert_tree_bits(h.grow_tree(js, gp, mask=mask, cond=cond), t_fx)
+    # both histogram kernels (generic 16-byte pieces / conflict-free 8-byte pieces) give the same bits
+    h.set_option("hist_variant", 1)
+    assert_tree_bits(h.grow_tree(js, gp, mask=mask, cond=cond), t_fx)
+    # short runs of rows go straight to the global histogram: every row that way / none that way
+    for variant, small in ((1, 65536), (0, 65536), (0, 0)):
+        h.set_option("hist_variant", variant)
+        h.set_option("hist_small_rows", small)
+        assert_tree_bits(h.grow_tree(js, gp, mask=mask, cond=cond), t_fx)
     h.close()
     o.close()
 
