@@ -1,0 +1,74 @@
+"""Size-independent properties at the benchmark's full size (10M x 100, nbins 64, max_depth 11),
+where the CPU oracle would take too long to be the checker."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_full_size_invariants(evt):
+    N, F, B, D = 10_000_000, 100, 64, 11
+    rng = np.random.default_rng(2024)
+    print("generating", N, "x", F, flush=True)
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    y = rng.random(N, dtype=np.float32)
+    mu = np.array([y.mean()], np.float32)
+    h = evt.Handle(N, F, B, 1, D, "mse")
+    h.set_xbin(x_bin)
+    h.set_target(y, None, mu)
+    gp = evt.make_params(eta=0.1)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    h.update_grads()
+    grad = h.get_grads()
+    assert np.array_equal(grad[:, 0], np.float32(2) * (mu[0] - y)) and (grad[:, 1] == 2).all() and (grad[:, 2] == 1).all()
+    print("growing tree 1 (node ids recorded by the partition)", flush=True)
+    h.set_option("record_nidx", 1)
+    t1 = h.grow_tree(js, gp)
+    nidx_rec = h.get_nidx()
+    pred1 = h.get_pred()[:, 0]
+    nn = (1 << D) - 1
+    split = t1.split.astype(bool)
+    # structure: children of split nodes exist, weights are row counts and add up
+    assert split[0] and split.sum() > 500
+    for n in np.flatnonzero(split) + 1:
+        assert t1.w[n - 1] == t1.w[2 * n - 1] + t1.w[2 * n]
+        assert 1 <= t1.feat[n - 1] <= F and 1 <= t1.cond_bin[n - 1] <= B - 1 and t1.gain[n - 1] > 0
+    assert t1.w[0] == N
+    leaves = np.array([n for n in range(1, nn + 1) if t1.w[n - 1] > 0 and not split[n - 1]])
+    assert t1.w[leaves - 1].sum() == N
+    # every row sits in a leaf, and the partition's node ids equal an independent walk of the finished tree
+    assert not split[nidx_rec - 1].any()
+    counts = np.bincount(nidx_rec, minlength=nn + 1)
+    assert np.array_equal(counts[1:].astype(np.float32)[leaves - 1], t1.w[leaves - 1])
+    leaf_walk = evt._lib.predict_leaf_idx(x_bin, None, [t1])[:, 0]
+    assert np.array_equal(leaf_walk, nidx_rec)
+    # the prediction update applied by the partition equals mu + leaf value of the walked leaf, bit for bit
+    assert np.array_equal(pred1, mu[0] + t1.pred[leaf_walk - 1, 0])
+    # histogram invariants (exact integer accumulation): for the root, every feature's bins sum to the
+    # node totals; count channel equals the bin populations of x_bin
+    H = h.get_hist()
+    root = H[0]
+    tot = root.sum(axis=1)
+    assert (tot == tot[0]).all()
+    assert tot[0, 2] == N and tot[0, 1] == 2 * N
+    for j in (0, 37, 99):
+        assert np.array_equal(root[j, :, 2], np.bincount(x_bin[j], minlength=B + 1)[1:].astype(np.float64))
+    for n in (1, 2, 3):
+        if split[n - 1] and split[2 * n - 1] and split[2 * n]:
+            assert np.array_equal(H[n - 1], H[2 * n - 1] + H[2 * n])  # parent == left + right, exactly
+    del H
+    # determinism across launch shapes and kernels: the same gradients give the same tree, bit for bit
+    print("re-growing with other launch shapes", flush=True)
+    h.set_option("record_nidx", 0)
+    for blocks, threads, variant in ((333, 256, 1), (1024, 1024, 2)):
+        h.set_option("hist_blocks", blocks)
+        h.set_option("hist_threads", threads)
+        h.set_option("hist_variant", variant)
+        h.set_grads(grad)
+        t2 = h.grow_tree(js, gp)
+        for a in ("feat", "cond_bin", "split"):
+            assert np.array_equal(getattr(t1, a), getattr(t2, a))
+        for a in ("gain", "pred", "w"):
+            assert np.array_equal(getattr(t1, a).view(np.uint32), getattr(t2, a).view(np.uint32))
+        assert np.array_equal(h.get_nidx(), nidx_rec)  # derived by walking the tree this time
+    h.close()
