@@ -93,6 +93,21 @@ def bias(loss, y):
     return np.array([y.mean()], np.float32)
 
 
+def measured_traffic_per_launch(path):
+    """Average HBM bytes per k_hist_build launch (scaled FETCH_SIZE + WRITE_SIZE) from the committed
+    rocprofv3 --pmc summary of the same workload; None if the summary is absent."""
+    try:
+        tot, n = 0.0, 0
+        for line in open(path):
+            p = line.split()
+            if len(p) == 11 and p[0].isdigit():
+                tot += (float(p[7]) + float(p[9])) * 1e6
+                n += 1
+        return tot / n if n else None
+    except OSError:
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -179,8 +194,12 @@ def main():
     roofline = None
     if hist_ms > 0:
         achieved = rows_built * bytes_per_row / (hist_ms * 1e-3) / 1e9
+        traffic = None
+        if args.workload == "cfg3" and not args.rows:
+            traffic = measured_traffic_per_launch(os.path.join(ROOT, "profiles", "cfg3_k_hist_build_pmc.txt"))
         roofline = {"bound": "hbm", "kernel": "k_hist_build", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None if traffic is None else round(traffic),
+                    "algorithmic_bytes_per_launch": round(rows_built * bytes_per_row / max(1, prof["hist"]["launches"])),
                     "launches": prof["hist"]["launches"], "avg_launch_ms": round(hist_ms / max(1, prof["hist"]["launches"]), 4),
                     "rows_built_per_round": rows_built // max(1, args.steps), "bytes_per_row": bytes_per_row,
                     "rows_features_per_s": round(rows_built * nfs / (hist_ms * 1e-3), 1)}
