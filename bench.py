@@ -121,7 +121,7 @@ def main():
     ap.add_argument("--hist-threads", type=int, default=0)
     ap.add_argument("--hist-min-rows", type=int, default=0)
     ap.add_argument("--hist-variant", type=int, default=0)
-    ap.add_argument("--hist-small-rows", type=int, default=-1)
+    ap.add_argument("--hist-seg-cost", type=int, default=-1)
     ap.add_argument("--predict", action="store_true", help="also time model inference on the training rows")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -154,8 +154,8 @@ def main():
         h.set_option("hist_min_rows", args.hist_min_rows)
     if args.hist_variant:
         h.set_option("hist_variant", args.hist_variant)
-    if args.hist_small_rows >= 0:
-        h.set_option("hist_small_rows", args.hist_small_rows)
+    if args.hist_seg_cost >= 0:
+        h.set_option("hist_seg_cost", args.hist_seg_cost)
     t_setup = time.time() - t0
 
     params = evt.make_params(eta=cfg["eta"], min_weight=cfg["min_weight"], update_pred=True)

@@ -183,7 +183,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->hist_threads = 512;
     c->hist_min_rows = 2048;
     c->hist_variant = 1;
-    c->hist_small_rows = 0;
+    c->hist_seg_cost = 1024;
     c->record_nidx = false;
     c->nidx_valid = false;
     c->last_cond = 255;
@@ -843,9 +843,9 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
     } else if (strcmp(name, "hist_min_rows") == 0) {
         ARGCHK(value >= 1 && value <= EVT_HIST_MAX_ROWS_PER_BLOCK, "hist_min_rows must be in [1, 32768]");
         c->hist_min_rows = (int)value;
-    } else if (strcmp(name, "hist_small_rows") == 0) {
-        ARGCHK(value >= 0 && value <= 65536, "hist_small_rows must be in [0, 65536]");
-        c->hist_small_rows = (int)value;
+    } else if (strcmp(name, "hist_seg_cost") == 0) {
+        ARGCHK(value >= 0 && value <= 65536, "hist_seg_cost must be in [0, 65536]");
+        c->hist_seg_cost = (int)value;
     } else if (strcmp(name, "hist_variant") == 0) {
         ARGCHK(value >= 0 && value <= 2, "hist_variant must be 0 (auto), 1 (generic) or 2 (conflict-free)");
         c->hist_variant = (int)value;

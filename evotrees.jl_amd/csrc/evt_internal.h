@@ -27,7 +27,7 @@
 #define LH_N_ACT 0
 #define LH_N_CHUNKS 1
 #define LH_N_BUILD 2
-#define LH_TOTAL_BUILD 3
+#define LH_TOTAL_BUILD 3 // build rows of the level + hist_seg_cost per build node
 #define LH_SIZE 8
 
 struct LevelTab {
@@ -113,7 +113,7 @@ struct evt_ctx {
     bool last_all_rows;
 
     // tunables
-    int hist_blocks, hist_threads, hist_min_rows, hist_small_rows;
+    int hist_blocks, hist_threads, hist_min_rows, hist_seg_cost;
     int hist_variant;  // 0 auto, 1 generic 16-byte-piece kernel, 2 conflict-free 8-byte-piece kernel where it applies
     bool record_nidx;  // leaf finalisation also writes the node id of every sampled row
     bool nidx_valid;   // nidx holds the last tree's node ids

@@ -37,7 +37,7 @@ struct HistArgs {
     int RS, LPR, RPW, F, nfs, B, NAg, level;
     int slots_per_tile;
     int min_rows;
-    int small_rows;
+    int seg_cost;
 };
 
 template <int NA, bool PACK>
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     const int n_build = (int)A.hdr[LH_N_BUILD];
     const int64_t total = A.hdr[LH_TOTAL_BUILD];
     if (n_build <= 0 || total <= 0) return;
-    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) A.stats[A.level] = total;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
 
     const int step = nwaves * A.RPW; // rows per block iteration
     // rows per block: an even share, but never so few that the flush of a whole LDS histogram
@@ -93,47 +93,20 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     const int64_t blk_start = start, blk_end = end;
 
     while (start < end) {
+        // spans are cut in a cost space where node i occupies [bprefix[i], bprefix[i+1]): its rows first,
+        // then seg_cost units standing for the fixed cost of one flush, so that a span holding many tiny
+        // nodes carries proportionally fewer rows
         const int64_t nbeg = A.bprefix[i];
         const int64_t nxt = A.bprefix[i + 1];
-        const int64_t nend = end < nxt ? end : nxt;
-        const int64_t seg = A.bstart[i] - nbeg; // position in the row list = seg + p
-        if (nend - start <= A.small_rows) {
-            // a short run of this node's rows: cheaper to add straight into the global histogram than
-            // to scan and flush a whole LDS histogram for it
-            unsigned long long *hg = reinterpret_cast<unsigned long long *>(A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride);
-            for (int64_t b0 = start + (int64_t)wave * A.RPW; b0 < nend; b0 += step) {
-                const int64_t p = b0 + rloc;
-                if (lane_on && p < nend) {
-                    const uint32_t row = A.is[seg + p];
-                    const uint4 v = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)row * A.RS + sub * 16);
-                    unsigned long long g[NA];
-#pragma unroll
-                    for (int a = 0; a < NA; a++) g[a] = A.gq[(size_t)a * A.N + row];
-                    const uint32_t wds[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                    for (int t = 0; t < 16; t++) {
-                        if (vmask & (1u << t)) {
-                            const int slot = A.jsmap[sub * 16 + t];
-                            const int bin = (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu) - 1;
-                            unsigned long long *base = hg + ((int64_t)slot * A.NAg) * A.B + bin;
-#pragma unroll
-                            for (int a = 0; a < NA; a++) {
-                                if (PACK && a == 0) {
-                                    const long long gs = (long long)g[0] >> EVT_PACK_CNT_BITS;
-                                    if (gs != 0) atomicAdd(base, (unsigned long long)gs);
-                                    atomicAdd(base + (int64_t)(A.NAg - 1) * A.B, 1ull);
-                                } else {
-                                    atomicAdd(base + (int64_t)a * A.B, g[a]);
-                                }
-                            }
-                        }
-                    }
-                }
-            }
-            start = nend;
+        const int64_t nrows_end = nxt - A.seg_cost;
+        const int64_t cend = end < nxt ? end : nxt;
+        const int64_t nend = cend < nrows_end ? cend : nrows_end;
+        if (start >= nend) { // only this node's padding lies in the span
+            start = cend;
             i++;
             continue;
         }
+        const int64_t seg = A.bstart[i] - nbeg; // position in the row list = seg + p
         // software pipeline over U row groups per wave: the row ids of iteration k+2 and the records of
         // iteration k+1 are in flight while the LDS atomics of iteration k are issued
         {
@@ -207,7 +180,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
         // flush this node's partial histogram: hist[node][slot][ag][bin].  A node whose rows all lie in
         // this block's span has a single writer: plain stores into its zero-initialised slice; a node
         // shared with other blocks is accumulated with 64-bit global atomics.
-        const bool sole = (nbeg >= blk_start) && (nxt <= blk_end);
+        const bool sole = (nbeg >= blk_start) && (nrows_end <= blk_end);
         long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
         // blocks start at different words so that concurrent flushes of one node do not queue on the
         // same addresses
@@ -242,7 +215,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
             }
         }
         __syncthreads();
-        start = nend;
+        start = cend;
         i++;
     }
 }
@@ -263,7 +236,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     const int n_build = (int)A.hdr[LH_N_BUILD];
     const int64_t total = A.hdr[LH_TOTAL_BUILD];
     if (n_build <= 0 || total <= 0) return;
-    if (blockIdx.x == 0 && tid == 0) A.stats[A.level] = total;
+    if (blockIdx.x == 0 && tid == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
 
     const int NS = A.RS >> 3;     // 8-byte pieces per record
     const int RPW = 64 / NS;      // rows per wave instruction
@@ -304,47 +277,20 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     char *Hb = reinterpret_cast<char *>(H);
 
     while (start < end) {
+        // spans are cut in a cost space where node i occupies [bprefix[i], bprefix[i+1]): its rows first,
+        // then seg_cost units standing for the fixed cost of one flush, so that a span holding many tiny
+        // nodes carries proportionally fewer rows
         const int64_t nbeg = A.bprefix[i];
         const int64_t nxt = A.bprefix[i + 1];
-        const int64_t nend = end < nxt ? end : nxt;
-        const int64_t seg = A.bstart[i] - nbeg;
-        if (nend - start <= A.small_rows) {
-            // a short run of this node's rows: cheaper to add straight into the global histogram than
-            // to scan and flush a whole LDS histogram for it
-            unsigned long long *hg = reinterpret_cast<unsigned long long *>(A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride);
-            for (int64_t b0 = start + (int64_t)wave * RPW; b0 < nend; b0 += step) {
-                const int64_t p = b0 + rloc;
-                if (lane_on && p < nend) {
-                    const uint32_t row = A.is[seg + p];
-                    const uint2 v = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)row * A.RS + sub * 8);
-                    unsigned long long g[NA];
-#pragma unroll
-                    for (int a = 0; a < NA; a++) g[a] = A.gq[(size_t)a * A.N + row];
-                    const uint32_t wds[2] = {v.x, v.y};
-#pragma unroll
-                    for (int t = 0; t < 8; t++) {
-                        if (vmask & (1u << t)) {
-                            const int slot = A.jsmap[sub * 8 + t];
-                            const int bin = (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu) - 1;
-                            unsigned long long *base = hg + ((int64_t)slot * A.NAg) * B + bin;
-#pragma unroll
-                            for (int a = 0; a < NA; a++) {
-                                if (PACK && a == 0) {
-                                    const long long gs = (long long)g[0] >> EVT_PACK_CNT_BITS;
-                                    if (gs != 0) atomicAdd(base, (unsigned long long)gs);
-                                    atomicAdd(base + (int64_t)(A.NAg - 1) * B, 1ull);
-                                } else {
-                                    atomicAdd(base + (int64_t)a * B, g[a]);
-                                }
-                            }
-                        }
-                    }
-                }
-            }
-            start = nend;
+        const int64_t nrows_end = nxt - A.seg_cost;
+        const int64_t cend = end < nxt ? end : nxt;
+        const int64_t nend = cend < nrows_end ? cend : nrows_end;
+        if (start >= nend) { // only this node's padding lies in the span
+            start = cend;
             i++;
             continue;
         }
+        const int64_t seg = A.bstart[i] - nbeg;
         // software pipeline over U row groups per wave: the row ids of iteration k+2 and the records of
         // iteration k+1 are in flight while the LDS atomics of iteration k are issued
         {
@@ -419,7 +365,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         // flush: a wave covers 8 consecutive bins x 8 consecutive pieces `sub` of one (channel, t): global
         // accesses are whole 64-byte runs of one feature's bins, LDS reads spread over 8 bank pairs.  Blocks
         // start at different items so that concurrent flushes of one node do not queue on the same addresses.
-        const bool sole = (nbeg >= blk_start) && (nxt <= blk_end);
+        const bool sole = (nbeg >= blk_start) && (nrows_end <= blk_end);
         long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
         const int nchunks = (B + 7) >> 3;
         const int nsg = NS >> 3;
@@ -462,7 +408,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             }
         }
         __syncthreads();
-        start = nend;
+        start = cend;
         i++;
     }
 }
@@ -520,11 +466,12 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
     slots_per_tile = (nfs + ntiles - 1) / ntiles;
     A.slots_per_tile = slots_per_tile;
     A.min_rows = c->hist_min_rows;
-    A.small_rows = c->hist_small_rows;
+    A.seg_cost = c->hist_seg_cost;
     size_t lds = per_slot * slots_per_tile;
     int threads = c->hist_threads;
     int64_t blocks = c->hist_blocks;
-    int64_t need = (c->N + EVT_HIST_MAX_ROWS_PER_BLOCK - 1) / EVT_HIST_MAX_ROWS_PER_BLOCK;
+    // a block's span must stay below the row count the packed 16-bit counter can hold
+    int64_t need = (c->N + (int64_t)c->maxlvl * c->hist_seg_cost + EVT_HIST_MAX_ROWS_PER_BLOCK - 1) / EVT_HIST_MAX_ROWS_PER_BLOCK;
     if (blocks < need) blocks = need;
     dim3 grid((unsigned)blocks, (unsigned)ntiles);
     const bool pack = c->unit_w;

@@ -202,6 +202,7 @@ struct NextArgs {
     int32_t *n_bnode;
     int64_t *n_bstart;
     int64_t *n_bprefix;
+    int64_t seg_cost; // cost units added per build node in the histogram kernel's span space
 };
 
 __global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
         A.status[2 * n + 1] = build_left ? ST_SUBTRACT : ST_BUILD;
         s_pos += 1;
         s_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
-        s_brows += build_left ? nl : nr;
+        s_brows += (build_left ? nl : nr) + A.seg_cost;
     }
     long long t_pos, t_chunks, t_brows;
     long long p_pos = block_excl_scan(s_pos, &t_pos, s_tmp);
@@ -260,7 +261,7 @@ __global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
         A.n_bprefix[p_pos] = p_brows;
         p_pos += 1;
         p_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
-        p_brows += build_left ? nl : nr;
+        p_brows += (build_left ? nl : nr) + A.seg_cost;
     }
     if (tid == 0) {
         A.n_cprefix[2 * t_pos] = t_chunks;
@@ -288,6 +289,7 @@ struct BeginArgs {
     long long *hist;
     int64_t *stats;
     int64_t n_is;
+    int64_t seg_cost;
     int64_t root_words;
     int nnodes, K, D;
 };
@@ -314,14 +316,14 @@ __global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) {
         A.hdr[LH_N_ACT] = 1;
         A.hdr[LH_N_CHUNKS] = (A.n_is + EVT_CHUNK - 1) / EVT_CHUNK;
         A.hdr[LH_N_BUILD] = 1;
-        A.hdr[LH_TOTAL_BUILD] = A.n_is;
+        A.hdr[LH_TOTAL_BUILD] = A.n_is + A.seg_cost;
         A.act_node[0] = 1;
         A.cprefix[0] = 0;
         A.cprefix[1] = (A.n_is + EVT_CHUNK - 1) / EVT_CHUNK;
         A.bnode[0] = 1;
         A.bstart[0] = 0;
         A.bprefix[0] = 0;
-        A.bprefix[1] = A.n_is;
+        A.bprefix[1] = A.n_is + A.seg_cost;
     }
 }
 
@@ -420,6 +422,7 @@ int launch_tree_begin(evt_ctx *c, int64_t n_is) {
     A.hist = c->hist;
     A.stats = c->stats;
     A.n_is = n_is;
+    A.seg_cost = c->hist_seg_cost;
     A.root_words = (int64_t)c->n_js_last * c->NAg * c->B;
     A.nnodes = c->nnodes;
     A.K = c->K;
@@ -490,6 +493,7 @@ int launch_level_next(evt_ctx *c, int level) {
     A.n_bnode = Nx.bnode;
     A.n_bstart = Nx.bstart;
     A.n_bprefix = Nx.bprefix;
+    A.seg_cost = c->hist_seg_cost;
     hipLaunchKernelGGL(k_level_next, dim3(1), dim3(1024), 0, c->stream, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;

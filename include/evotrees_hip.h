@@ -174,7 +174,8 @@ int evt_set_profiling(evt_handle h, int32_t on);
  * (GRAD/PREDICT: rows; HIST: rows built; SCAN: nodes scanned; PARTITION: rows moved). */
 int evt_get_profile(evt_handle h, int64_t *launches, double *ms, int64_t *units);
 int evt_reset_profile(evt_handle h);
-/* Options: "hist_blocks", "hist_threads" (launch shape of the histogram kernel, for sweeps);
+/* Options: "hist_blocks", "hist_threads", "hist_min_rows", "hist_seg_cost", "hist_variant" (launch shape,
+ * work split and kernel variant of the histogram builder, for sweeps; results do not depend on them);
  * "record_nidx" (1: the partition also records every sampled row's final node while the tree grows;
  * 0, default: evt_get_nidx derives it afterwards by walking the finished tree). */
 int evt_set_option(evt_handle h, const char *name, int64_t value);

@@ -174,10 +174,10 @@ def test_grow_tree_matches_oracle(evt, loss, weights, N, F, B, D, tt, n_js, rows
     # both histogram kernels (generic 16-byte pieces / conflict-free 8-byte pieces) give the same bits
     h.set_option("hist_variant", 1)
     assert_tree_bits(h.grow_tree(js, gp, mask=mask, cond=cond), t_fx)
-    # short runs of rows go straight to the global histogram: every row that way / none that way
-    for variant, small in ((1, 65536), (0, 65536), (0, 0)):
+    # the per-node padding of the span space only moves work between blocks
+    for variant, cost in ((1, 0), (2, 7), (1, 5000)):
         h.set_option("hist_variant", variant)
-        h.set_option("hist_small_rows", small)
+        h.set_option("hist_seg_cost", cost)
         assert_tree_bits(h.grow_tree(js, gp, mask=mask, cond=cond), t_fx)
     h.close()
     o.close()
