@@ -182,7 +182,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->hist_blocks = 512;
     c->hist_threads = 512;
     c->hist_min_rows = 2048;
-    c->hist_variant = 1;
+    c->hist_variant = 0;
     c->hist_seg_cost = 1024;
     c->record_nidx = false;
     c->nidx_valid = false;

@@ -228,8 +228,8 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
 // ((a*8 + t)*B + bin)*NS + sub for feature f = 8*sub + t, i.e. `sub` selects the bank pair, so the 16
 // lanes of a group always fall on 16 different bank pairs whatever their bins are.  Rows that share a
 // wave instruction sit in different groups and cannot collide inside one LDS pass either.
-template <int NA, bool PACK>
-__global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
+template <int NA, bool PACK, int U, int MAXT>
+__global__ __launch_bounds__(MAXT) void k_hist_build16(HistArgs A) {
     extern __shared__ unsigned long long H[]; // [NA][8][B][NS]
     const int tid = threadIdx.x, nthr = blockDim.x;
     const int lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     const int step = nwaves * RPW;
     int64_t T = (total + gridDim.x - 1) / gridDim.x;
     if (T < A.min_rows) T = A.min_rows;
-    T = ((T + 4 * step - 1) / (4 * step)) * (4 * step);
+    T = ((T + U * step - 1) / (U * step)) * (U * step);
     int64_t start = (int64_t)blockIdx.x * T;
     if (start >= total) return;
     int64_t end = start + T < total ? start + T : total;
@@ -294,7 +294,6 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         // software pipeline over U row groups per wave: the row ids of iteration k+2 and the records of
         // iteration k+1 are in flight while the LDS atomics of iteration k are issued
         {
-            constexpr int U = 4;
             constexpr uint32_t INV = 0xFFFFFFFFu;
             const int64_t itstride = (int64_t)U * step;
             uint32_t rc[U], rn[U];
@@ -415,7 +414,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
 
 template <int NA, bool PACK>
 static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
-    hipLaunchKernelGGL((k_hist_build16<NA, PACK>), grid, dim3(threads), lds, c->stream, A);
+    hipLaunchKernelGGL((k_hist_build16<NA, PACK, 4, 1024>), grid, dim3(threads), lds, c->stream, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
