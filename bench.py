@@ -174,7 +174,8 @@ def main():
     for _ in range(args.warmup):
         one_round()
     h.synchronize()
-    h.set_profiling(not args.no_profile)
+    # timed region: HIP events only around the histogram launches (the kernel the roofline is quoted on)
+    h.set_profiling(False if args.no_profile else ["hist"])
     h.reset_profile()
     t1 = time.perf_counter()
     for _ in range(args.steps):
@@ -183,6 +184,18 @@ def main():
     t2 = time.perf_counter()
     prof = h.get_profile()
     h.set_profiling(False)
+    # per-class breakdown from a few extra rounds with events around every kernel (outside the timed region)
+    extra = 0 if args.no_profile else min(10, args.steps)
+    if extra:
+        h.set_profiling(True)
+        h.reset_profile()
+        for _ in range(extra):
+            one_round()
+        h.synchronize()
+        prof_all = h.get_profile()
+        h.set_profiling(False)
+    else:
+        prof_all = prof
     elapsed = t2 - t1
     ms_per_step = elapsed * 1e3 / args.steps
     value = ms_per_step * 200 / 1e3
@@ -203,10 +216,11 @@ def main():
                     "launches": prof["hist"]["launches"], "avg_launch_ms": round(hist_ms / max(1, prof["hist"]["launches"]), 4),
                     "rows_built_per_round": rows_built // max(1, args.steps), "bytes_per_row": bytes_per_row,
                     "rows_features_per_s": round(rows_built * nfs / (hist_ms * 1e-3), 1)}
-    kernels = {k: {"ms_per_round": round(v["ms"] / args.steps, 4), "launches_per_round": v["launches"] / args.steps} for k, v in prof.items()}
-    if prof["grad"]["ms"] > 0:
+    nb = max(1, extra)
+    kernels = {k: {"ms_per_round": round(v["ms"] / nb, 4), "launches_per_round": v["launches"] / nb} for k, v in prof_all.items()}
+    if prof_all["grad"]["ms"] > 0:
         gb = N * (4 * K + 4 + 4 + 8 * K)
-        kernels["grad"]["GBps"] = round(gb * args.steps / (prof["grad"]["ms"] * 1e-3) / 1e9, 1)
+        kernels["grad"]["GBps"] = round(gb * nb / (prof_all["grad"]["ms"] * 1e-3) / 1e9, 1)
 
     out = {
         "metric": "train s/200 rounds @10Mx100 depth 11 (1 GPU)" if args.workload == "cfg3" and not args.rows
@@ -216,7 +230,7 @@ def main():
         "dtype": "int64 fixed-point histograms, f64 gains, f32 gradients/predictions", "data": "synthetic",
         "config": {"workload": "%s: %s %dx%d nbins=%d max_depth=%d eta=%g rowsample=%g colsample=%g tree_type=%s" % (
             args.workload, loss, N, F, B, D, cfg["eta"], cfg["rowsample"], cfg["colsample"], cfg["tree_type"])},
-        "roofline": roofline, "kernels": kernels, "setup_s": round(t_setup, 2),
+        "roofline": roofline, "kernels_breakdown_%d_extra_rounds" % extra: kernels, "setup_s": round(t_setup, 2),
     }
     # rows built per level of the last tree (unit weights: Tree.w holds row counts): the smaller child of every split
     per_level = [int(N if cond >= 255 else tree.w[0])]

@@ -240,7 +240,16 @@ class Handle:
         return qb, qe
 
     def set_profiling(self, on):
-        check(load().evt_set_profiling(self._h, 1 if on else 0))
+        """on: False/True, or a list of kernel class names to time (e.g. ["hist"])."""
+        if isinstance(on, (list, tuple)):
+            mask = 0
+            for name in on:
+                mask |= 1 << KERNEL_CLASSES.index(name)
+            if mask == 1:
+                mask |= 1 << 30  # keep the value distinct from the "every class" code 1
+            check(load().evt_set_profiling(self._h, mask))
+        else:
+            check(load().evt_set_profiling(self._h, 1 if on else 0))
 
     def reset_profile(self):
         check(load().evt_reset_profile(self._h))

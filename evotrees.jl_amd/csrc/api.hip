@@ -41,7 +41,9 @@ extern "C" int evt_device_count(int32_t *count) {
 
 // ---- profiling ------------------------------------------------------------------------------
 void prof_begin(evt_ctx *c, int cls, int level) {
-    if (!c->profiling) return;
+    c->prof_open = false;
+    if (!((c->profiling >> cls) & 1)) return;
+    c->prof_open = true;
     ProfRec r;
     r.cls = cls;
     r.level = level;
@@ -61,7 +63,8 @@ void prof_begin(evt_ctx *c, int cls, int level) {
     c->recs.push_back(r);
 }
 void prof_end(evt_ctx *c) {
-    if (!c->profiling || c->recs.empty()) return;
+    if (!c->prof_open || c->recs.empty()) return;
+    c->prof_open = false;
     (void)hipEventRecord(c->recs.back().e1, c->stream);
 }
 // after a stream sync: fold finished event pairs into the per-class totals
@@ -117,9 +120,8 @@ extern "C" int evt_destroy(evt_handle c) {
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
-                    c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree.feat, c->tree.cond_bin, c->tree.w, c->tree.gain,
-                    c->tree.pred, c->tree.split, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->stats, c->errflag, c->ogains, c->obest, c->sbest};
+                    c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
+                    c->qscale, c->errflag, c->ogains, c->obest, c->sbest};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -173,6 +175,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->is_a = c->is_b = nullptr; c->nidx = nullptr; c->mask = nullptr; c->flagw = nullptr; c->chunk_nleft = nullptr; c->chunk_lpre = nullptr;
     c->hist = nullptr; c->seg_start = c->seg_len = nullptr; c->status = nullptr; c->node_sum = nullptr;
     memset(&c->tree, 0, sizeof(c->tree));
+    c->tree_blob = nullptr;
     memset(c->lvl, 0, sizeof(c->lvl));
     c->js = nullptr; c->jsmap = nullptr; c->feattypes = nullptr; c->mono = nullptr; c->absmax = nullptr; c->qexp = nullptr; c->qbits = nullptr;
     c->qscale = nullptr; c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->obest = nullptr; c->sbest = nullptr;
@@ -187,7 +190,8 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->record_nidx = false;
     c->nidx_valid = false;
     c->last_cond = 255;
-    c->profiling = false;
+    c->profiling = 0;
+    c->prof_open = false;
     memset(c->prof_launches, 0, sizeof(c->prof_launches));
     memset(c->prof_ms, 0, sizeof(c->prof_ms));
     memset(c->prof_units, 0, sizeof(c->prof_units));
@@ -224,12 +228,27 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->seg_len, c->nnodes + 2);
     ALLOC(c->status, c->nnodes + 2);
     ALLOC(c->node_sum, (size_t)(c->nnodes + 2) * NAgmax);
-    ALLOC(c->tree.feat, c->nnodes);
-    ALLOC(c->tree.cond_bin, c->nnodes);
-    ALLOC(c->tree.w, c->nnodes);
-    ALLOC(c->tree.gain, c->nnodes);
-    ALLOC(c->tree.pred, (size_t)c->nnodes * K);
-    ALLOC(c->tree.split, c->nnodes);
+    {
+        // the Tree arrays and the per-level row counts live in one allocation so that a finished tree is
+        // read back with a single copy
+        const size_t nn = (size_t)c->nnodes;
+        c->blob_feat = 0;
+        c->blob_w = c->blob_feat + nn * 4;
+        c->blob_gain = c->blob_w + nn * 4;
+        c->blob_pred = c->blob_gain + nn * 4;
+        c->blob_stats = ((c->blob_pred + nn * 4 * K + 7) / 8) * 8;
+        c->blob_bin = c->blob_stats + (size_t)(c->D + 2) * 8;
+        c->blob_split = c->blob_bin + nn;
+        c->blob_bytes = ((c->blob_split + nn + 15) / 16) * 16;
+        ALLOC(c->tree_blob, c->blob_bytes);
+        c->tree.feat = reinterpret_cast<int32_t *>(c->tree_blob + c->blob_feat);
+        c->tree.w = reinterpret_cast<float *>(c->tree_blob + c->blob_w);
+        c->tree.gain = reinterpret_cast<float *>(c->tree_blob + c->blob_gain);
+        c->tree.pred = reinterpret_cast<float *>(c->tree_blob + c->blob_pred);
+        c->stats = reinterpret_cast<int64_t *>(c->tree_blob + c->blob_stats);
+        c->tree.cond_bin = c->tree_blob + c->blob_bin;
+        c->tree.split = c->tree_blob + c->blob_split;
+    }
     ALLOC(c->tree.packed, c->nnodes);
     for (int l = 0; l < 2; l++) {
         ALLOC(c->lvl[l].hdr, LH_SIZE);
@@ -247,7 +266,6 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->qexp, 8);
     ALLOC(c->qbits, 8);
     ALLOC(c->qscale, 16);
-    ALLOC(c->stats, c->D + 2);
     ALLOC(c->errflag, 1);
     if (tree_type == EVT_TREE_OBLIVIOUS) ALLOC(c->ogains, (size_t)c->maxlvl * c->F * c->B);
     {
@@ -256,7 +274,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
         c->sbest = sb;
     }
     // pinned staging: tree read-back + small per-tree uploads
-    c->h_stage_bytes = (size_t)c->nnodes * (4 + 1 + 4 + 4 + 4 * K + 1) + (size_t)(c->D + 2) * 8 + (size_t)c->F * 4 + (size_t)c->RS * 2 + 1024;
+    c->h_stage_bytes = c->blob_bytes + (size_t)c->F * 4 + (size_t)c->RS * 2 + 1024;
     if (hipHostMalloc((void **)&c->h_stage, c->h_stage_bytes, hipHostMallocDefault) != hipSuccess) {
         evt_set_error("hipHostMalloc failed");
         evt_destroy(c);
@@ -482,7 +500,13 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     }
     // js: 1-based, strictly ascending
     std::vector<uint32_t> jsv(n_js);
-    HIPCHK(hipMemcpy(jsv.data(), js, sizeof(uint32_t) * n_js, hipMemcpyDefault));
+    {
+        hipPointerAttribute_t attr;
+        const bool on_dev = (hipPointerGetAttributes(&attr, js) == hipSuccess) && attr.type == hipMemoryTypeDevice;
+        (void)hipGetLastError();
+        if (on_dev) HIPCHK(hipMemcpy(jsv.data(), js, sizeof(uint32_t) * n_js, hipMemcpyDeviceToHost));
+        else memcpy(jsv.data(), js, sizeof(uint32_t) * n_js);
+    }
     for (int i = 0; i < n_js; i++) {
         ARGCHK(jsv[i] >= 1 && jsv[i] <= (uint32_t)c->F, "js entries must be in 1..nfeats");
         ARGCHK(i == 0 || jsv[i] > jsv[i - 1], "js must be strictly ascending");
@@ -516,17 +540,19 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     c->nidx_valid = c->record_nidx;
 
     // per-tree small uploads through pinned memory
-    uint32_t *h_js = reinterpret_cast<uint32_t *>(c->h_stage);
-    uint16_t *h_map = reinterpret_cast<uint16_t *>(c->h_stage + (size_t)c->F * 4);
-    for (int f = 0; f < c->RS; f++) h_map[f] = 0xFFFF;
-    for (int i = 0; i < n_js; i++) {
-        h_js[i] = jsv[i];
-        h_map[jsv[i] - 1] = (uint16_t)i;
+    if (c->n_js_last != n_js || c->js_last != jsv) { // the column sample changed: refresh the device copies
+        uint32_t *h_js = reinterpret_cast<uint32_t *>(c->h_stage + c->blob_bytes);
+        uint16_t *h_map = reinterpret_cast<uint16_t *>(c->h_stage + c->blob_bytes + (size_t)c->F * 4);
+        for (int f = 0; f < c->RS; f++) h_map[f] = 0xFFFF;
+        for (int i = 0; i < n_js; i++) {
+            h_js[i] = jsv[i];
+            h_map[jsv[i] - 1] = (uint16_t)i;
+        }
+        HIPCHK(hipMemcpyAsync(c->js, h_js, sizeof(uint32_t) * n_js, hipMemcpyHostToDevice, c->stream));
+        HIPCHK(hipMemcpyAsync(c->jsmap, h_map, sizeof(uint16_t) * c->RS, hipMemcpyHostToDevice, c->stream));
+        c->n_js_last = n_js;
+        c->js_last = jsv;
     }
-    HIPCHK(hipMemcpyAsync(c->js, h_js, sizeof(uint32_t) * n_js, hipMemcpyHostToDevice, c->stream));
-    HIPCHK(hipMemcpyAsync(c->jsmap, h_map, sizeof(uint16_t) * c->RS, hipMemcpyHostToDevice, c->stream));
-    c->n_js_last = n_js;
-    c->js_last = jsv;
 
     int r;
     prof_begin(c, EVT_K_OTHER, 0);
@@ -544,25 +570,31 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     const bool fuse_pred = p->update_pred && all_rows;
     const bool obliv = (c->tree_type == EVT_TREE_OBLIVIOUS);
     uint32_t *is_cur = c->is_a, *is_next = c->is_b;
-    for (int level = 1; level <= c->D; level++) {
-        const bool leaf_level = (level == c->D);
-        if (!leaf_level || level == 1) {
-            prof_begin(c, EVT_K_HIST, level);
-            r = launch_hist_build(c, level, is_cur);
-            prof_end(c);
-            if (r != EVT_OK) return r;
-        }
+    // levels 1 .. D-1 split; the last of them sends its rows straight to the leaves of level D
+    const int last_split = (c->D > 1) ? c->D - 1 : 1;
+    for (int level = 1; level <= last_split; level++) {
+        prof_begin(c, EVT_K_HIST, level);
+        r = launch_hist_build(c, level, is_cur);
+        prof_end(c);
+        if (r != EVT_OK) return r;
         prof_begin(c, EVT_K_SCAN, level);
-        r = launch_scan(c, level, p, leaf_level);
-        if (r == EVT_OK && obliv && !leaf_level) r = launch_obliv_select(c, level, p);
+        if (c->D == 1) {
+            r = launch_scan(c, 1, p, true); // a stump: the root is the only leaf
+        } else {
+            r = launch_scan(c, level, p, false);
+            if (r == EVT_OK && obliv) r = launch_obliv_select(c, level, p);
+            if (r == EVT_OK && level == last_split) r = launch_scan(c, c->D, p, true); // leaf values of level D
+        }
         prof_end(c);
         if (r != EVT_OK) return r;
         prof_begin(c, EVT_K_PARTITION, level);
-        if (!leaf_level) {
+        if (level < last_split) {
             r = launch_part_count(c, level, is_cur);
             if (r == EVT_OK) r = launch_level_next(c, level);
+            if (r == EVT_OK) r = launch_part_scatter(c, level, is_cur, is_next, fuse_pred);
+        } else {
+            r = launch_final_fused(c, level, is_cur, fuse_pred);
         }
-        if (r == EVT_OK) r = launch_part_scatter(c, level, is_cur, is_next, fuse_pred);
         prof_end(c);
         if (r != EVT_OK) return r;
         std::swap(is_cur, is_next);
@@ -582,15 +614,9 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     // read back the tree (and the per-level row counts) in one pinned transfer
     const int nn = c->nnodes, K = c->K;
     uint8_t *hs = c->h_stage;
-    size_t o_feat = 0, o_w = o_feat + (size_t)nn * 4, o_gain = o_w + (size_t)nn * 4, o_pred = o_gain + (size_t)nn * 4,
-           o_stats = ((o_pred + (size_t)nn * 4 * K + 7) / 8) * 8, o_bin = o_stats + (size_t)(c->D + 2) * 8, o_split = o_bin + nn;
-    HIPCHK(hipMemcpyAsync(hs + o_feat, c->tree.feat, (size_t)nn * 4, hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipMemcpyAsync(hs + o_w, c->tree.w, (size_t)nn * 4, hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipMemcpyAsync(hs + o_gain, c->tree.gain, (size_t)nn * 4, hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipMemcpyAsync(hs + o_pred, c->tree.pred, (size_t)nn * 4 * K, hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipMemcpyAsync(hs + o_stats, c->stats, (size_t)(c->D + 2) * 8, hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipMemcpyAsync(hs + o_bin, c->tree.cond_bin, nn, hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipMemcpyAsync(hs + o_split, c->tree.split, nn, hipMemcpyDeviceToHost, c->stream));
+    const size_t o_feat = c->blob_feat, o_w = c->blob_w, o_gain = c->blob_gain, o_pred = c->blob_pred, o_stats = c->blob_stats,
+                 o_bin = c->blob_bin, o_split = c->blob_split;
+    HIPCHK(hipMemcpyAsync(hs, c->tree_blob, c->blob_bytes, hipMemcpyDeviceToHost, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     if (c->profiling) {
         prof_collect(c, reinterpret_cast<const int64_t *>(hs + o_stats));
@@ -810,7 +836,7 @@ extern "C" int evt_set_profiling(evt_handle c, int32_t on) {
     CTXCHK(c);
     HIPCHK(hipStreamSynchronize(c->stream));
     prof_collect(c, nullptr);
-    c->profiling = on != 0;
+    c->profiling = (on == 1) ? 0x7fffffff : on; // 1: every class; otherwise a bit mask of EVT_K_* classes
     return EVT_OK;
 }
 extern "C" int evt_get_profile(evt_handle c, int64_t *launches, double *ms, int64_t *units) {

@@ -89,6 +89,8 @@ struct evt_ctx {
     int32_t *status;
     long long *node_sum; // [node][NAg]
     TreeDev tree;
+    uint8_t *tree_blob; // one allocation behind tree.{feat,w,gain,pred,cond_bin,split} and stats
+    size_t blob_feat, blob_w, blob_gain, blob_pred, blob_stats, blob_bin, blob_split, blob_bytes;
     LevelTab lvl[2];
     uint32_t *js;      // [F]
     uint16_t *jsmap;   // [RS] slot of feature f (0-based), 0xFFFF = not sampled / padding
@@ -120,7 +122,8 @@ struct evt_ctx {
     uint8_t last_cond;
 
     // profiling
-    bool profiling;
+    int profiling;     // bit mask of kernel classes timed with events
+    bool prof_open;
     std::vector<ProfRec> recs;
     std::vector<hipEvent_t> free_events;
     int64_t prof_launches[EVT_K_COUNT];
@@ -165,6 +168,7 @@ int launch_obliv_select(evt_ctx *c, int level, const evt_params *p);
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_level_next(evt_ctx *c, int level);
 int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred);
+int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred);
 int launch_fill_u32(evt_ctx *c, uint32_t *dst, uint32_t v, int64_t n);
 int launch_fill_bytes(evt_ctx *c, void *dst, int64_t nbytes);
 // predict

@@ -161,6 +161,66 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
     }
 }
 
+// Last pass of a tree: rows of the deepest split level go straight to their leaf.  For a node that split,
+// the child is decided from x_bin[row, feat] exactly as the partition would (left iff <= cond_bin, or ==
+// for a categorical feature) but the row list is not rewritten: nothing reads it afterwards.  Each row
+// gets its leaf's value added to the prediction (predict!, src/predict.jl:1-46) and, on request, its
+// node id recorded.
+__global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
+    const int tid = threadIdx.x;
+    const int n_act = (int)A.hdr[LH_N_ACT];
+    const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
+    const int K = A.K;
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const int i = find_owner(A.cprefix, n_act, c);
+        const int n = A.act_node[i];
+        const int st = A.status[n];
+        if (st != ST_SPLIT && st != ST_LEAF) continue;
+        const int64_t cl = c - A.cprefix[i];
+        const int64_t seg = A.seg_start[n], len = A.seg_len[n];
+        const int64_t p0 = seg + cl * EVT_CHUNK;
+        const int64_t pend = seg + len;
+        const bool is_split = (st == ST_SPLIT);
+        int f = 0;
+        uint32_t cb = 0;
+        bool numeric = true;
+        if (is_split) {
+            f = A.t_feat[n - 1] - 1;
+            cb = A.t_bin[n - 1];
+            numeric = A.feattypes[f] != 0;
+        }
+        const uint8_t *col = A.xcm + (size_t)f * A.N;
+#pragma unroll
+        for (int it = 0; it < EVT_CHUNK / 256; it++) {
+            const int64_t p = p0 + it * 256 + tid;
+            if (p < pend) {
+                const uint32_t row = A.is_cur[p];
+                int leaf = n;
+                if (is_split) {
+                    const uint32_t xb = col[row];
+                    const bool left = numeric ? (xb <= cb) : (xb == cb);
+                    leaf = 2 * n + (left ? 0 : 1);
+                }
+                if (A.write_nidx) A.nidx[row] = (uint32_t)leaf;
+                if (A.fuse_pred) {
+                    float *pr = A.pred + (size_t)K * row;
+                    const float *lp = A.t_pred + (size_t)K * (leaf - 1);
+                    if (A.loss == EVT_LOSS_MSE) {
+                        for (int k = 0; k < K; k++) pr[k] += lp[k];
+                    } else if (A.loss == EVT_LOSS_LOGLOSS) {
+                        for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
+                    } else {
+                        for (int t = 0; t < K / 2; t++) {
+                            pr[2 * t] += lp[2 * t];
+                            pr[2 * t + 1] = fmaxf(-15.0f, pr[2 * t + 1] + lp[2 * t + 1]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
 // ---- single-block scans -----------------------------------------------------------------------
 // Exclusive prefix over the 1024 threads of the block; returns the prefix, *total gets the sum.
 __device__ long long block_excl_scan(long long v, long long *total, long long *s_tmp /* [17] */) {
@@ -471,6 +531,15 @@ int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t 
     PartArgs A;
     fill_part_args(c, level, is_cur, is_next, fuse_pred, A);
     hipLaunchKernelGGL(k_part_scatter, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred) {
+    if (!fuse_pred && !c->record_nidx) return EVT_OK;
+    PartArgs A;
+    fill_part_args(c, level, is_cur, nullptr, fuse_pred, A);
+    hipLaunchKernelGGL(k_final_fused, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

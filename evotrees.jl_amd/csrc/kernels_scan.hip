@@ -276,8 +276,13 @@ template <int NAG>
 __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = (1 << (A.level - 1)) + blockIdx.x;
-    const int st = A.status[n];
-    if (st != ST_BUILD && st != ST_SUBTRACT) return;
+    if (A.leaf_level) {
+        // nodes of the last level are the children of the split nodes above them (the root when max_depth == 1)
+        if (n > 1 && A.status[n >> 1] != ST_SPLIT) return;
+    } else {
+        const int st = A.status[n];
+        if (st != ST_BUILD && st != ST_SUBTRACT) return;
+    }
     const int B = A.B, NK = A.NK, K = A.K;
     long long *hn = A.hist + (int64_t)(n - 1) * A.node_stride;
 

@@ -169,6 +169,7 @@ enum {
     EVT_K_OTHER = 5,
     EVT_K_COUNT = 6
 };
+/* on = 0: off; 1: every class; any other value: bit mask (1 << EVT_K_*) of the classes to time. */
 int evt_set_profiling(evt_handle h, int32_t on);
 /* Accumulated since the last reset: per class number of launches, milliseconds, and units
  * (GRAD/PREDICT: rows; HIST: rows built; SCAN: nodes scanned; PARTITION: rows moved). */
