@@ -514,27 +514,9 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     // LDS budget of one block: channels x bins of a single feature must fit
     ARGCHK((size_t)c->NA * c->B * 8 <= 64 * 1024, "histogram of one feature exceeds the LDS budget");
 
-    // rows kept by the mask (the host owns the RNG; src/subsample.jl:7-9)
-    int64_t n_is = c->N;
-    std::vector<uint8_t> mask_host;
-    if (mask) {
-        hipPointerAttribute_t attr;
-        bool on_dev = (hipPointerGetAttributes(&attr, mask) == hipSuccess) && attr.type == hipMemoryTypeDevice;
-        (void)hipGetLastError();
-        const uint8_t *mh = mask;
-        if (on_dev) {
-            mask_host.resize(c->N);
-            HIPCHK(hipMemcpy(mask_host.data(), mask, c->N, hipMemcpyDeviceToHost));
-            mh = mask_host.data();
-        }
-        n_is = 0;
-        for (int64_t i = 0; i < c->N; i++) n_is += (mh[i] <= cond);
-        if (n_is == 0) {
-            evt_set_error("no subsample observation - choose larger rowsample");
-            return EVT_ERR_EMPTY;
-        }
-    }
-    const bool all_rows = (n_is == c->N);
+    // rows kept by the mask (the host owns the RNG; src/subsample.jl:7-9).  The threshold, the count and the
+    // compaction run on the device; the count comes back with the finished tree.
+    const bool all_rows = (mask == nullptr) || (cond == 255);
     c->last_all_rows = all_rows;
     c->last_cond = cond;
     c->nidx_valid = c->record_nidx;
@@ -560,10 +542,10 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
         r = launch_iota(c, c->is_a, c->N);
     } else {
         HIPCHK(hipMemcpyAsync(c->mask, mask, c->N, hipMemcpyDefault, c->stream));
-        r = launch_compact_mask(c, cond, n_is);
+        r = launch_compact_mask(c, cond);
         if (r == EVT_OK && c->record_nidx) r = launch_fill_u32(c, c->nidx, 0u, c->N);
     }
-    if (r == EVT_OK) r = launch_tree_begin(c, n_is);
+    if (r == EVT_OK) r = launch_tree_begin(c, all_rows);
     prof_end(c);
     if (r != EVT_OK) return r;
 
@@ -608,7 +590,6 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
         if (c->profiling) c->prof_units[EVT_K_PREDICT] += c->N;
     }
     if (c->profiling) {
-        c->prof_units[EVT_K_PARTITION] += n_is;
     }
 
     // read back the tree (and the per-level row counts) in one pinned transfer
@@ -618,9 +599,15 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
                  o_bin = c->blob_bin, o_split = c->blob_split;
     HIPCHK(hipMemcpyAsync(hs, c->tree_blob, c->blob_bytes, hipMemcpyDeviceToHost, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
+    const int64_t n_is = reinterpret_cast<const int64_t *>(hs + o_stats)[0];
     if (c->profiling) {
+        c->prof_units[EVT_K_PARTITION] += n_is;
         prof_collect(c, reinterpret_cast<const int64_t *>(hs + o_stats));
         c->prof_units[EVT_K_SCAN] += 0;
+    }
+    if (n_is == 0) { // the tree grown on no rows is a single zero leaf; report it as the reference does
+        evt_set_error("no subsample observation - choose larger rowsample");
+        return EVT_ERR_EMPTY;
     }
     if (tree) {
         ARGCHK(tree->feat && tree->cond_bin && tree->w && tree->gain && tree->pred && tree->split, "tree output arrays must not be NULL");

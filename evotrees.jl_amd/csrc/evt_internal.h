@@ -159,9 +159,9 @@ int launch_init_pred(evt_ctx *c, const float *mu_dev, const float *offset_dev);
 int launch_transpose_validate(evt_ctx *c);
 int launch_binarize(evt_ctx *c, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev);
 // tree
-int launch_tree_begin(evt_ctx *c, int64_t n_is);
+int launch_tree_begin(evt_ctx *c, bool all_rows);
 int launch_iota(evt_ctx *c, uint32_t *dst, int64_t n);
-int launch_compact_mask(evt_ctx *c, uint8_t cond, int64_t n_is);
+int launch_compact_mask(evt_ctx *c, uint8_t cond);
 int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level);
 int launch_obliv_select(evt_ctx *c, int level, const evt_params *p);

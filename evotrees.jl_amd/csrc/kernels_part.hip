@@ -349,6 +349,7 @@ struct BeginArgs {
     long long *hist;
     int64_t *stats;
     int64_t n_is;
+    const int64_t *n_is_dev; // non-null: the number of sampled rows is the total the mask compaction left on the device
     int64_t seg_cost;
     int64_t root_words;
     int nnodes, K, D;
@@ -370,6 +371,8 @@ __global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) {
     for (int d = tid; d <= A.D; d += 1024) A.stats[d] = 0;
     __syncthreads();
     if (tid == 0) {
+        if (A.n_is_dev) A.n_is = *A.n_is_dev;
+        A.stats[0] = A.n_is; // read back with the tree: the host learns how many rows the mask kept
         A.status[1] = ST_BUILD;
         A.seg_start[1] = 0;
         A.seg_len[1] = A.n_is;
@@ -453,7 +456,7 @@ static unsigned grid_for_chunks(int64_t max_chunks) {
     return (unsigned)g;
 }
 
-int launch_compact_mask(evt_ctx *c, uint8_t cond, int64_t n_is) {
+int launch_compact_mask(evt_ctx *c, uint8_t cond) {
     const int64_t n_chunks = (c->N + EVT_CHUNK - 1) / EVT_CHUNK;
     unsigned g = grid_for_chunks(n_chunks);
     hipLaunchKernelGGL(k_mask_count, dim3(g), dim3(256), 0, c->stream, c->mask, cond, c->N, n_chunks, c->flagw, c->chunk_nleft);
@@ -462,11 +465,10 @@ int launch_compact_mask(evt_ctx *c, uint8_t cond, int64_t n_is) {
     HIPCHK(hipGetLastError());
     hipLaunchKernelGGL(k_mask_scatter, dim3(g), dim3(256), 0, c->stream, c->N, n_chunks, c->flagw, c->chunk_lpre, c->is_a);
     HIPCHK(hipGetLastError());
-    (void)n_is;
     return EVT_OK;
 }
 
-int launch_tree_begin(evt_ctx *c, int64_t n_is) {
+int launch_tree_begin(evt_ctx *c, bool all_rows) {
     const LevelTab &L = c->lvl[1];
     BeginArgs A;
     A.tree = c->tree;
@@ -481,7 +483,8 @@ int launch_tree_begin(evt_ctx *c, int64_t n_is) {
     A.bprefix = L.bprefix;
     A.hist = c->hist;
     A.stats = c->stats;
-    A.n_is = n_is;
+    A.n_is = c->N;
+    A.n_is_dev = all_rows ? nullptr : c->chunk_lpre + (c->N + EVT_CHUNK - 1) / EVT_CHUNK;
     A.seg_cost = c->hist_seg_cost;
     A.root_words = (int64_t)c->n_js_last * c->NAg * c->B;
     A.nnodes = c->nnodes;

@@ -132,7 +132,7 @@ __device__ __forceinline__ void node_totals(const ScanArgs &A, int n, const long
 // Pass 1: grid (nodes of the level, feature groups); one wave per (node, sampled feature).
 // Writes the group's best candidate to sbest[node][group] (or the gain matrix for oblivious trees)
 // and, for subtract nodes, materialises h[n] = h[parent] - h[sibling].
-template <int NAG>
+template <int NAG, int BPL>
 __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const int n = (1 << (A.level - 1)) + blockIdx.x; // 1-based node id
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     if (st != ST_BUILD && st != ST_SUBTRACT) return;
     const bool is_sub = (st == ST_SUBTRACT);
     const int B = A.B, NK = A.NK, K = A.K;
-    const int BPL = (B + 63) >> 6; // bins per lane (<= 4)
+    // BPL = bins per lane = ceil(nbins / 64), a template parameter so that nbins <= 64 keeps one bin per lane in registers
     long long *hn = A.hist + (int64_t)(n - 1) * A.node_stride;
     const long long *hp = A.hist + (int64_t)((n >> 1) - 1) * A.node_stride;
     const long long *hs = A.hist + (int64_t)((n ^ 1) - 1) * A.node_stride;
@@ -169,17 +169,17 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
         const bool numeric = A.feattypes[f] != 0;
         const int constraint = A.mono[f];
         const int bmax = numeric ? B - 1 : B;
-        long long pre[NAG][4];
+        long long pre[NAG][BPL];
         long long excl[NAG];
 #pragma unroll
         for (int ag = 0; ag < NAG; ag++) {
             const int64_t o = ((int64_t)jp * NAG + ag) * B;
             long long run = 0;
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
+            for (int t = 0; t < BPL; t++) {
                 const int b = lane * BPL + t;
                 long long v = 0;
-                if (t < BPL && b < B) {
+                if (b < B) {
                     if (is_sub) {
                         v = hp[o + b] - hs[o + b];
                         hn[o + b] = v; // subtract_hist!: h[n] = h[parent] - h[sibling]
@@ -193,14 +193,14 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
             const long long incl = wave_incl_scan_i64(run);
             excl[ag] = incl - run;
 #pragma unroll
-            for (int t = 0; t < 4; t++) pre[ag][t] += excl[ag];
+            for (int t = 0; t < BPL; t++) pre[ag][t] += excl[ag];
         }
         double lg = -INFINITY;
         int lb = NO_BIN;
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
+        for (int t = 0; t < BPL; t++) {
             const int b = lane * BPL + t;
-            if (t < BPL && b < B) {
+            if (b < B) {
                 double gain = 0.0;
                 bool ok = false;
                 if (b + 1 <= bmax) {
@@ -504,9 +504,14 @@ int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     const unsigned nodes = 1u << (level - 1);
     const int ngroups = (A.nfs + 3) / 4; // 4 waves per block, one sampled feature each
     dim3 grid(nodes, (unsigned)ngroups);
+    const int bpl = (c->B + 63) / 64;
 #define SCASE(NAG_)                                                                                     \
     case NAG_:                                                                                          \
-        if (!leaf_level) hipLaunchKernelGGL(k_scan<NAG_>, grid, dim3(256), 0, c->stream, A);            \
+        if (!leaf_level) {                                                                              \
+            if (bpl == 1) hipLaunchKernelGGL((k_scan<NAG_, 1>), grid, dim3(256), 0, c->stream, A);      \
+            else if (bpl == 2) hipLaunchKernelGGL((k_scan<NAG_, 2>), grid, dim3(256), 0, c->stream, A); \
+            else hipLaunchKernelGGL((k_scan<NAG_, 4>), grid, dim3(256), 0, c->stream, A);               \
+        }                                                                                               \
         if (!A.oblivious || leaf_level) hipLaunchKernelGGL(k_scan_fin<NAG_>, dim3(nodes), dim3(256), 0, c->stream, A, ngroups); \
         break;
     switch (c->NAg) {
