@@ -17,11 +17,15 @@ import numpy as np
 from . import _lib
 from ._lib import EvtError, Handle, TreeArrays, make_params  # noqa: F401
 
-__all__ = ["EvoTreeRegressor", "EvoTreeMLE", "EvoTree", "Tree", "fit", "predict", "predict_leaf_idx", "init", "grow_evotree",
-           "get_edges", "check_args", "EvtError"]
+__all__ = ["EvoTreeRegressor", "EvoTreeCount", "EvoTreeMLE", "EvoTree", "Tree", "fit", "predict", "predict_leaf_idx", "init",
+           "grow_evotree", "get_edges", "check_args", "CallBack", "init_logger", "update_logger", "EvtError"]
 
 _GPU_DEVICES = ("gpu", "rocm", "amd", "hip")
-_LOSS_K = {"mse": 1, "logloss": 1, "gaussian_mle": 2}
+_LOSS_K = {"mse": 1, "logloss": 1, "gaussian_mle": 2, "poisson": 1, "gamma": 1, "tweedie": 1}
+_EXP_LINK = ("poisson", "gamma", "tweedie")
+# is_maximise, src/metrics.jl:195-207
+_MAXIMISE = {"mse": False, "rmse": False, "mae": False, "logloss": False, "poisson": False, "gamma": False, "tweedie": False,
+             "gaussian_mle": True}
 
 
 def _device_check(device):
@@ -51,11 +55,14 @@ def check_args(args):
         raise ValueError("Invalid input for `tree_type` parameter: `%s`. Must be of one of `binary` or `oblivious`" % args["tree_type"])
     if args["bagging_size"] < 1:
         raise ValueError("bagging_size must be >= 1")
+    rng("early_stopping_rounds", 1, float("inf"))
+    rng("early_stopping_tolerance", 0.0, float("inf"))
 
 
 class _Learner:
     _losses = ()
-    _defaults = dict(loss="mse", nrounds=100, bagging_size=1, L2=1.0, lambda_=0.0, gamma=0.0, eta=0.1, max_depth=6, min_weight=1.0,
+    _metrics = ()
+    _defaults = dict(loss="mse", metric=None, early_stopping_rounds=2 ** 62, early_stopping_tolerance=0.0, nrounds=100, bagging_size=1, L2=1.0, lambda_=0.0, gamma=0.0, eta=0.1, max_depth=6, min_weight=1.0,
                      rowsample=1.0, colsample=1.0, nbins=64, monotone_constraints=None, tree_type="binary", seed=123, device="gpu")
 
     def __init__(self, **kwargs):
@@ -70,19 +77,31 @@ class _Learner:
         args["tree_type"] = str(args["tree_type"]).lstrip(":")
         if args["loss"] not in self._losses:
             raise ValueError("Invalid loss. Must be one of: %s" % (list(self._losses),))
+        args["metric"] = args["loss"] if args["metric"] is None else str(args["metric"]).lstrip(":")
+        if args["metric"] not in self._metrics:
+            raise ValueError("Invalid metric. Must be one of: %s" % (list(self._metrics),))
         args["monotone_constraints"] = dict(args["monotone_constraints"] or {})
         check_args(args)
         self.__dict__.update(args)
 
 
 class EvoTreeRegressor(_Learner):
-    """EvoTreeRegressor (src/learners.jl:1-119), losses mse and logloss."""
-    _losses = ("mse", "logloss")
+    """EvoTreeRegressor (src/learners.jl:1-119); losses mse, logloss, poisson, gamma, tweedie."""
+    _losses = ("mse", "logloss", "poisson", "gamma", "tweedie")
+    _metrics = ("mse", "rmse", "mae", "logloss", "poisson", "gamma", "tweedie")
+
+
+class EvoTreeCount(_Learner):
+    """EvoTreeCount (src/learners.jl:121-205): poisson loss and metric."""
+    _losses = ("poisson",)
+    _metrics = ("poisson",)
+    _defaults = dict(_Learner._defaults, loss="poisson")
 
 
 class EvoTreeMLE(_Learner):
     """EvoTreeMLE (src/learners.jl:300-400), loss gaussian_mle; min_weight defaults to 8."""
     _losses = ("gaussian_mle",)
+    _metrics = ("gaussian_mle",)
     _defaults = dict(_Learner._defaults, loss="gaussian_mle", min_weight=8.0)
 
 
@@ -146,9 +165,23 @@ def _init_target(loss, y):
         m = np.float32(y32.mean(dtype=np.float32))
         s = np.float32(y32.std(ddof=1, dtype=np.float32))
         mu = np.array([m, _invsoftplus(s)], np.float32)
+    elif loss in _EXP_LINK:
+        mu = np.array([np.log(np.float32(y32.mean(dtype=np.float32)))], np.float32)
     else:
         mu = np.array([y32.mean(dtype=np.float32)], np.float32)
     return _LOSS_K[loss], y32, mu.astype(np.float32)
+
+
+def _link_offset(loss, offset, N, K):
+    """Offsets are given on the response scale and moved to the linear one (src/init.jl:30, :43, :69; src/callback.jl:76-80)."""
+    offset = np.array(offset, np.float32).reshape(N, K)
+    if loss == "logloss":
+        offset = _logit(offset)
+    elif loss in _EXP_LINK:
+        offset = np.log(offset)
+    elif loss == "gaussian_mle":
+        offset[:, 1] = _invsoftplus(offset[:, 1])
+    return offset.astype(np.float32)
 
 
 class Cache:
@@ -180,11 +213,7 @@ def init(config, x_train, y_train, w_train=None, offset_train=None, feature_name
             raise AssertionError("weights must be positive and match the number of rows")
     offset = None
     if offset_train is not None:
-        offset = np.array(offset_train, np.float32).reshape(N, K)
-        if config.loss == "logloss":
-            offset = _logit(offset)
-        elif config.loss == "gaussian_mle":
-            offset[:, 1] = _invsoftplus(offset[:, 1])
+        offset = _link_offset(config.loss, offset_train, N, K)
         mu = np.zeros_like(mu)  # neutral bias when an offset is given (src/init.jl:164)
     h = Handle(N, F, config.nbins, K, config.max_depth, config.loss, config.tree_type)
     x_FN = np.ascontiguousarray(x.T, np.float64)
@@ -226,19 +255,94 @@ def grow_evotree(m, cache, config):
     m.info["nrounds"] += 1
 
 
-def fit(config, x_train=None, y_train=None, w_train=None, offset_train=None, feature_names=None, device=None, verbosity=1,
-        return_cache=False):
-    """fit(params; x_train, y_train, ...), src/fit.jl:388-437 (no eval set: the callback is outside this backend)."""
+class CallBack:
+    """CallBack (src/callback.jl:21-135) on the device: a second handle holds the binned eval rows, their
+    running prediction, target and weights; each call adds one tree and evaluates the metric there."""
+
+    def __init__(self, config, m, x_eval, y_eval, w_eval=None, offset_eval=None):
+        x = np.asarray(x_eval)
+        N, F = x.shape
+        self.metric = config.metric
+        self.maximise = _MAXIMISE[config.metric]
+        y32 = np.asarray(y_eval).astype(np.float32)
+        if y32.shape != (N,):
+            raise AssertionError("y_eval length must equal the number of eval rows")
+        w = None if w_eval is None else np.asarray(w_eval, np.float32)
+        offset = None if offset_eval is None else _link_offset(m.loss_type, offset_eval, N, m.K)
+        h = Handle(N, F, config.nbins, m.K, 1, m.loss_type, "binary")
+        try:
+            h.binarize(np.ascontiguousarray(x.T, np.float64), m.info["edges"])
+            h.set_feature_meta(m.info["feattypes"], None)
+            h.set_target(y32, w, np.zeros(m.K, np.float32), offset)  # p = zeros (+ offset'), src/callback.jl:104, :82
+        except Exception:
+            h.close()
+            raise
+        self.handle = h
+
+    def __call__(self, logger, it, tree):
+        self.handle.predict_tree(tree)
+        update_logger(logger, it, self.handle.eval_metric(self.metric))
+
+    def close(self):
+        self.handle.close()
+
+
+def init_logger(metric, maximise, early_stopping_rounds, early_stopping_tolerance=0.0):
+    """init_logger, src/callback.jl:137-151."""
+    return dict(name=str(metric), maximise=maximise, early_stopping_rounds=early_stopping_rounds,
+                early_stopping_tolerance=early_stopping_tolerance, nrounds=0, iter=[], metrics=[], iter_since_best=0, best_iter=0,
+                best_metric=0.0)
+
+
+def update_logger(logger, it, metric):
+    """update_logger!, src/callback.jl:153-171."""
+    logger["nrounds"] = it
+    logger["iter"].append(it)
+    logger["metrics"].append(metric)
+    if it == 0:
+        logger["best_metric"] = metric
+        return
+    tol = logger["early_stopping_tolerance"]
+    improved = metric > logger["best_metric"] + tol if logger["maximise"] else metric < logger["best_metric"] - tol
+    if improved:
+        logger["best_metric"] = metric
+        logger["best_iter"] = it
+        logger["iter_since_best"] = 0
+    else:
+        logger["iter_since_best"] += logger["iter"][-1] - logger["iter"][-2]
+
+
+def fit(config, x_train=None, y_train=None, w_train=None, offset_train=None, x_eval=None, y_eval=None, w_eval=None, offset_eval=None,
+        feature_names=None, print_every_n=9999, device=None, verbosity=1, return_cache=False):
+    """fit(params; x_train, y_train, ..., x_eval, y_eval, ...), src/fit.jl:388-437."""
     if x_train is None or y_train is None:
         raise TypeError("x_train and y_train are required")
     m, cache = init(config, x_train, y_train, w_train=w_train, offset_train=offset_train, feature_names=feature_names, device=device)
+    logger, cb = None, None
     try:
-        for _ in range(config.nrounds):
+        if x_eval is not None and y_eval is not None:
+            cb = CallBack(config, m, x_eval, y_eval, w_eval=w_eval, offset_eval=offset_eval)
+            logger = init_logger(config.metric, cb.maximise, config.early_stopping_rounds, config.early_stopping_tolerance)
+            cb(logger, 0, m.trees[-1])
+            if verbosity > 0:
+                print("initialization: %s = %.6g" % (config.metric, logger["metrics"][-1]))
+        elif x_eval is not None or y_eval is not None:
+            import warnings
+            warnings.warn("To track eval metric in logger, both `x_eval` and `y_eval` must be provided.")
+        for i in range(1, config.nrounds + 1):
             grow_evotree(m, cache, config)
+            if logger is not None:
+                cb(logger, i, m.trees[-1])  # as the reference: only the round's last tree reaches the eval prediction
+                if i % print_every_n == 0 and verbosity > 0:
+                    print("iter %d: %s = %.6g" % (i, config.metric, logger["metrics"][-1]))
+                if logger["iter_since_best"] >= logger["early_stopping_rounds"]:
+                    break
     finally:
+        if cb is not None:
+            cb.close()
         if not return_cache:
             cache.handle.close()  # post_fit_gc slot, src/fit.jl:340
-    m.info["logger"] = None
+    m.info["logger"] = logger
     return (m, cache) if return_cache else m
 
 
@@ -259,8 +363,8 @@ def predict(m, data, ntree_limit=None, device="gpu"):
     ntree_limit = ntrees if ntree_limit is None else ntree_limit
     if ntree_limit > ntrees:
         raise RuntimeError("ntree_limit is larger than number of trees %d." % ntrees)
-    x_bin = binarize(data, m.info["edges"])
-    p = _lib.predict_model(x_bin, m.info["feattypes"], m.loss_type, m.K, m.trees[:ntree_limit], apply_link=True)
+    x_FN = np.ascontiguousarray(np.asarray(data).T, np.float64)
+    p = _lib.predict_model_f64(x_FN, m.info["edges"], m.info["feattypes"], m.loss_type, m.K, m.trees[:ntree_limit], apply_link=True)
     return p[:, 0].copy() if m.K == 1 else p
 
 

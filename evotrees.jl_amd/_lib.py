@@ -12,7 +12,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libevotrees_hip.so")
 
 EVT_OK, EVT_ERR_ARG, EVT_ERR_HIP, EVT_ERR_STATE, EVT_ERR_EMPTY, EVT_ERR_NOMEM = 0, -1, -2, -3, -4, -5
-LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2}
+LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5}
+METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7}
 TREE_TYPES = {"binary": 0, "oblivious": 1}
 KERNEL_CLASSES = ["grad", "hist", "scan", "partition", "predict", "other"]
 
@@ -21,7 +22,7 @@ EXPORTS = [
     "evt_last_error", "evt_device_count", "evt_create", "evt_destroy", "evt_set_xbin", "evt_binarize_f64",
     "evt_set_target", "evt_set_feature_meta", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
     "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
-    "evt_predict", "evt_predict_leaf_idx", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
+    "evt_predict", "evt_predict_f64", "evt_predict_leaf_idx", "evt_eval_metric", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
     "evt_set_option", "evt_synchronize", "evt_copy_bandwidth", "evt_read_bandwidth",
 ]
 
@@ -77,6 +78,8 @@ def load():
         "evt_get_quant": [vp, vp, vp],
         "evt_predict": [i64, i32, vp, vp, i32, i32, i32, vp, vp, vp, vp, vp, i32, vp],
         "evt_predict_leaf_idx": [i64, i32, vp, vp, i32, vp, vp, vp, vp, vp],
+        "evt_predict_f64": [i64, i32, vp, vp, vp, vp, i32, i32, i32, vp, vp, vp, vp, vp, i32, vp],
+        "evt_eval_metric": [vp, i32, vp],
         "evt_set_profiling": [vp, i32],
         "evt_get_profile": [vp, vp, vp, vp],
         "evt_reset_profile": [vp],
@@ -207,6 +210,12 @@ class Handle:
     def predict_tree(self, tree):
         check(load().evt_predict_tree(self._h, tree.feat.shape[0], ptr(tree.feat), ptr(tree.cond_bin), ptr(tree.pred), ptr(tree.split)))
 
+    def eval_metric(self, metric):
+        """Metric of the handle's prediction against its target and weights (the eval CallBack's feval)."""
+        v = C.c_double(0.0)
+        check(load().evt_eval_metric(self._h, METRIC_IDS[metric], C.byref(v)))
+        return v.value
+
     def get_xbin(self):
         out = np.empty((self.F, self.N), np.uint8)
         check(load().evt_get_xbin(self._h, ptr(out)))
@@ -286,6 +295,26 @@ def predict_model(x_bin_FN, feattypes, loss, K, trees, apply_link=True):
     out = np.empty((N, K), np.float32)
     check(load().evt_predict(N, F, ptr(x_bin_FN), ptr(ft), LOSS_IDS[loss], K, len(trees), ptr(off), ptr(feat), ptr(cb), ptr(pr),
                              ptr(sp), 1 if apply_link else 0, ptr(out)))
+    return out
+
+
+def predict_model_f64(x_FN, edges, feattypes, loss, K, trees, apply_link=True):
+    """As predict_model, from raw features: x_FN (F, N) C-order float64, edges a list of F ascending arrays."""
+    assert x_FN.dtype == np.float64 and x_FN.flags.c_contiguous
+    F, N = x_FN.shape
+    eoff = np.zeros(F + 1, np.int32)
+    eoff[1:] = np.cumsum([len(e) for e in edges])
+    eflat = np.ascontiguousarray(np.concatenate([np.asarray(e, np.float64) for e in edges]))
+    off = np.zeros(len(trees) + 1, np.int64)
+    off[1:] = np.cumsum([t.feat.shape[0] for t in trees])
+    feat = np.ascontiguousarray(np.concatenate([t.feat for t in trees]), np.int64)
+    cb = np.ascontiguousarray(np.concatenate([t.cond_bin for t in trees]), np.uint8)
+    sp = np.ascontiguousarray(np.concatenate([t.split for t in trees]), np.uint8)
+    pr = np.ascontiguousarray(np.concatenate([t.pred.reshape(-1, K) for t in trees]), np.float32)
+    ft = None if feattypes is None else np.ascontiguousarray(feattypes, np.uint8)
+    out = np.empty((N, K), np.float32)
+    check(load().evt_predict_f64(N, F, ptr(x_FN), ptr(eflat), ptr(eoff), ptr(ft), LOSS_IDS[loss], K, len(trees), ptr(off), ptr(feat),
+                                 ptr(cb), ptr(pr), ptr(sp), 1 if apply_link else 0, ptr(out)))
     return out
 
 

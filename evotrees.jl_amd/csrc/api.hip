@@ -121,7 +121,7 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->errflag, c->ogains, c->obest, c->sbest};
+                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->obest, c->sbest};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -149,9 +149,9 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ARGCHK(nfeats >= 1 && nfeats <= 1024, "nfeats must be in [1, 1024]");
     ARGCHK(nbins >= 2 && nbins <= 255, "nbins must be in [2, 255]");
     ARGCHK(max_depth >= 1 && max_depth <= EVT_MAX_DEPTH, "max_depth must be in [1, 16]");
-    ARGCHK(loss >= 0 && loss <= 2, "loss must be one of mse (0), logloss (1), gaussian_mle (2)");
+    ARGCHK(loss >= 0 && loss <= EVT_LOSS_TWEEDIE, "loss must be one of mse (0), logloss (1), gaussian_mle (2), poisson (3), gamma (4), tweedie (5)");
     ARGCHK(tree_type == EVT_TREE_BINARY || tree_type == EVT_TREE_OBLIVIOUS, "tree_type must be binary (0) or oblivious (1)");
-    ARGCHK(K == (loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1), "K must be 1 for mse/logloss and 2 for gaussian_mle");
+    ARGCHK(K == (loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1), "K must be 2 for gaussian_mle and 1 for the other losses");
     int ndev = 0;
     {
         int r = evt_device_count(&ndev);
@@ -266,6 +266,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->qexp, 8);
     ALLOC(c->qbits, 8);
     ALLOC(c->qscale, 16);
+    ALLOC(c->metric_partial, 2 * EVT_METRIC_BLOCKS + 1);
     ALLOC(c->errflag, 1);
     if (tree_type == EVT_TREE_OBLIVIOUS) ALLOC(c->ogains, (size_t)c->maxlvl * c->F * c->B);
     {
@@ -747,13 +748,45 @@ extern "C" int evt_get_quant(evt_handle c, int32_t *qbits, int32_t *qexp) {
     return EVT_OK;
 }
 
+// ---- evaluation metric ------------------------------------------------------------------------
+extern "C" int evt_eval_metric(evt_handle c, int32_t metric, double *value_out) {
+    CTXCHK(c);
+    ARGCHK(value_out, "value_out is NULL");
+    ARGCHK(metric >= 0 && metric <= EVT_METRIC_TWEEDIE, "unknown metric");
+    ARGCHK((metric == EVT_METRIC_GAUSSIAN_MLE) == (c->loss == EVT_LOSS_GAUSSIAN_MLE),
+           "gaussian_mle is the metric of the gaussian_mle loss and of no other");
+    if (!c->have_target) {
+        evt_set_error("evt_eval_metric: set the target first");
+        return EVT_ERR_STATE;
+    }
+    prof_begin(c, EVT_K_OTHER, 0);
+    int r = launch_eval_metric(c, metric, c->metric_partial);
+    prof_end(c);
+    if (r != EVT_OK) return r;
+    HIPCHK(hipMemcpyAsync(c->h_stage, c->metric_partial + 2 * EVT_METRIC_BLOCKS, sizeof(double), hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    memcpy(value_out, c->h_stage, sizeof(double));
+    return EVT_OK;
+}
+
 // ---- inference ------------------------------------------------------------------------------
+// Rows binned per pass of evt_predict_f64: bounds the Float64 staging buffer to chunk * nfeats * 8 bytes.
+static const int64_t PREDICT_F64_CHUNK = 1 << 20;
+
 static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, const uint8_t *feattypes, int32_t loss, int32_t K, int32_t ntrees,
                           const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const float *pred, const uint8_t *split,
-                          int32_t apply_link, float *out, uint32_t *leaf_out) {
+                          int32_t apply_link, float *out, uint32_t *leaf_out, const double *x_f64 = nullptr, const double *edges = nullptr,
+                          const int32_t *edge_off = nullptr) {
     ARGCHK(nobs >= 1 && nfeats >= 1 && ntrees >= 1, "nobs, nfeats, ntrees must be >= 1");
-    ARGCHK(x_bin && tree_off && feat && cond_bin && split, "NULL argument");
-    ARGCHK(leaf_out || (pred && out && K >= 1 && K <= 4 && loss >= 0 && loss <= 2), "invalid prediction arguments");
+    ARGCHK((x_bin || x_f64) && tree_off && feat && cond_bin && split, "NULL argument");
+    ARGCHK(leaf_out || (pred && out && K >= 1 && K <= 4 && loss >= 0 && loss <= EVT_LOSS_TWEEDIE), "invalid prediction arguments");
+    std::vector<int32_t> eoff;
+    if (x_f64) {
+        ARGCHK(edges && edge_off, "NULL argument");
+        eoff.assign(edge_off, edge_off + nfeats + 1);
+        for (int j = 0; j < nfeats; j++)
+            ARGCHK(eoff[j] >= 0 && eoff[j + 1] - eoff[j] >= 1 && eoff[j + 1] - eoff[j] <= 254, "each feature needs 1..254 edges");
+    }
     int ndev = 0;
     int r = evt_device_count(&ndev);
     if (r != EVT_OK) return r;
@@ -782,12 +815,33 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
     if (e == hipSuccess && !leaf_out) e = hipMalloc((void **)&d_lp, sizeof(float) * (size_t)total * K);
     if (e == hipSuccess && !leaf_out) e = hipMalloc((void **)&d_out, sizeof(float) * (size_t)nobs * K);
     if (e == hipSuccess && leaf_out) e = hipMalloc((void **)&d_leaf, sizeof(uint32_t) * (size_t)nobs * ntrees);
-    if (e == hipSuccess) e = hipMemcpy(d_x, x_bin, (size_t)nobs * nfeats, hipMemcpyDefault);
+    if (e == hipSuccess && !x_f64) e = hipMemcpy(d_x, x_bin, (size_t)nobs * nfeats, hipMemcpyDefault);
+    if (e == hipSuccess && x_f64) {
+        // binarize on the device, PREDICT_F64_CHUNK rows at a time: each pass copies the rows' slice of every
+        // column (a strided 2-D copy) and bins it into place
+        const int64_t chunk = std::min(nobs, PREDICT_F64_CHUNK);
+        double *d_xf = nullptr, *d_edges = nullptr;
+        int32_t *d_eoff = nullptr;
+        e = hipMalloc((void **)&d_xf, sizeof(double) * (size_t)chunk * nfeats);
+        if (e == hipSuccess) e = hipMalloc((void **)&d_edges, sizeof(double) * eoff[nfeats]);
+        if (e == hipSuccess) e = hipMalloc((void **)&d_eoff, sizeof(int32_t) * (nfeats + 1));
+        if (e == hipSuccess) e = hipMemcpy(d_edges, edges, sizeof(double) * eoff[nfeats], hipMemcpyDefault);
+        if (e == hipSuccess) e = hipMemcpy(d_eoff, eoff.data(), sizeof(int32_t) * (nfeats + 1), hipMemcpyHostToDevice);
+        for (int64_t r0 = 0; r0 < nobs && e == hipSuccess && r == EVT_OK; r0 += chunk) {
+            const int64_t n = std::min(chunk, nobs - r0);
+            e = hipMemcpy2D(d_xf, sizeof(double) * chunk, x_f64 + r0, sizeof(double) * nobs, sizeof(double) * n, nfeats, hipMemcpyDefault);
+            if (e == hipSuccess) r = launch_binarize_cols(s, d_xf, d_edges, d_eoff, d_x + r0, n, nfeats, chunk, nobs);
+            if (e == hipSuccess) e = hipStreamSynchronize(s);
+        }
+        void *tmp[] = {d_xf, d_edges, d_eoff};
+        for (void *p : tmp)
+            if (p) (void)hipFree(p);
+    }
     if (e == hipSuccess) e = hipMemcpy(d_ft, ft.data(), nfeats, hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemcpy(d_nodes, nodes.data(), sizeof(uint32_t) * total, hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemcpy(d_off, tree_off, sizeof(int64_t) * (ntrees + 1), hipMemcpyDefault);
     if (e == hipSuccess && !leaf_out) e = hipMemcpy(d_lp, pred, sizeof(float) * (size_t)total * K, hipMemcpyDefault);
-    if (e == hipSuccess) {
+    if (e == hipSuccess && r == EVT_OK) {
         if (leaf_out) r = launch_leaf_idx_model(s, d_nodes, d_off, ntrees, d_x, d_ft, nobs, d_leaf);
         else r = launch_predict_model(s, d_nodes, d_lp, d_off, ntrees, d_x, d_ft, nobs, K, loss, apply_link, d_out);
         e = hipDeviceSynchronize();
@@ -810,6 +864,14 @@ extern "C" int evt_predict(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, c
                            const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const float *pred, const uint8_t *split,
                            int32_t apply_link, float *out) {
     return predict_common(nobs, nfeats, x_bin, feattypes, loss, K, ntrees, tree_off, feat, cond_bin, pred, split, apply_link, out, nullptr);
+}
+
+extern "C" int evt_predict_f64(int64_t nobs, int32_t nfeats, const double *x_colmajor, const double *edges, const int32_t *edge_off,
+                               const uint8_t *feattypes, int32_t loss, int32_t K, int32_t ntrees, const int64_t *tree_off, const int64_t *feat,
+                               const uint8_t *cond_bin, const float *pred, const uint8_t *split, int32_t apply_link, float *out) {
+    ARGCHK(x_colmajor, "x is NULL");
+    return predict_common(nobs, nfeats, nullptr, feattypes, loss, K, ntrees, tree_off, feat, cond_bin, pred, split, apply_link, out, nullptr,
+                          x_colmajor, edges, edge_off);
 }
 
 extern "C" int evt_predict_leaf_idx(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, const uint8_t *feattypes, int32_t ntrees,

@@ -18,6 +18,7 @@
 #define EVT_CHUNK_WORDS 32    // 64-bit ballot words per chunk
 #define EVT_MAX_NK 5
 #define EVT_MAX_NA 5
+#define EVT_METRIC_BLOCKS 1024 // partial sums of the evaluation metric
 #define EVT_MAX_DEPTH 16
 #define EVT_PACK_QBITS 30     // fixed-point bits of the gradient channel that shares a word with the row count
 #define EVT_PACK_CNT_BITS 16
@@ -100,6 +101,7 @@ struct evt_ctx {
     int32_t *qexp;     // [8]
     int32_t *qbits;    // [8]
     double *qscale;    // [8] decode scale per global channel
+    double *metric_partial; // [2 * EVT_METRIC_BLOCKS + 1] evaluation-metric partial sums, result last
     int64_t *stats;    // [D+1] rows built per level
     int32_t *errflag;  // device-side validation flag
     double *ogains;    // oblivious: [maxlvl][F][B]
@@ -158,6 +160,9 @@ int launch_init_pred(evt_ctx *c, const float *mu_dev, const float *offset_dev);
 // data layout
 int launch_transpose_validate(evt_ctx *c);
 int launch_binarize(evt_ctx *c, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev);
+int launch_binarize_cols(hipStream_t s, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev, uint8_t *xcm, int64_t n,
+                         int F, int64_t ldx, int64_t ldo);
+int launch_eval_metric(evt_ctx *c, int metric, double *partial);
 // tree
 int launch_tree_begin(evt_ctx *c, bool all_rows);
 int launch_iota(evt_ctx *c, uint32_t *dst, int64_t n);

@@ -35,30 +35,36 @@ int launch_transpose_validate(evt_ctx *c) {
 
 // searchsortedfirst(edges_j, x) = 1 + number of edges strictly below x.
 __global__ __launch_bounds__(256) void k_binarize(const double *__restrict__ x, const double *__restrict__ edges,
-                                                 const int32_t *__restrict__ edge_off, uint8_t *__restrict__ xcm, int64_t N) {
+                                                 const int32_t *__restrict__ edge_off, uint8_t *__restrict__ xcm, int64_t N,
+                                                 int64_t ldx, int64_t ldo) {
     int j = blockIdx.y;
     int e0 = edge_off[j], ne = edge_off[j + 1] - e0;
     extern __shared__ double s_edges[];
     for (int t = threadIdx.x; t < ne; t += 256) s_edges[t] = edges[e0 + t];
     __syncthreads();
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
-        double v = x[(size_t)j * N + i];
+        double v = x[(size_t)j * ldx + i];
         int lo = 0, hi = ne;
         while (lo < hi) {
             int mid = (lo + hi) >> 1;
             if (s_edges[mid] < v) lo = mid + 1; else hi = mid;
         }
-        xcm[(size_t)j * N + i] = (uint8_t)(lo + 1);
+        xcm[(size_t)j * ldo + i] = (uint8_t)(lo + 1);
     }
 }
 
-int launch_binarize(evt_ctx *c, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev) {
-    int64_t nb = (c->N + 255) / 256;
+// n rows of F columns: column j is read at x_dev + j * ldx and written at xcm + j * ldo
+int launch_binarize_cols(hipStream_t s, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev, uint8_t *xcm, int64_t n,
+                         int F, int64_t ldx, int64_t ldo) {
+    int64_t nb = (n + 255) / 256;
     if (nb > 4096) nb = 4096;
-    dim3 grid((unsigned)nb, (unsigned)c->F);
-    hipLaunchKernelGGL(k_binarize, grid, dim3(256), 256 * sizeof(double), c->stream, x_dev, edges_dev, edge_off_dev, c->xcm, c->N);
+    dim3 grid((unsigned)nb, (unsigned)F);
+    hipLaunchKernelGGL(k_binarize, grid, dim3(256), 256 * sizeof(double), s, x_dev, edges_dev, edge_off_dev, xcm, n, ldx, ldo);
     HIPCHK(hipGetLastError());
     return EVT_OK;
+}
+int launch_binarize(evt_ctx *c, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev) {
+    return launch_binarize_cols(c->stream, x_dev, edges_dev, edge_off_dev, c->xcm, c->N, c->F, c->N, c->N);
 }
 
 __global__ __launch_bounds__(256) void k_iota(uint32_t *dst, int64_t n) {

@@ -13,7 +13,8 @@ __device__ __forceinline__ float wave_max_f32(float v) {
 __device__ __forceinline__ float dev_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float dev_softplus(float x) { return fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x))); }
 
-// LOSS: 0 mse (src/loss.jl:52), 1 logloss (:54-57), 2 gaussian_mle (:194-203).
+// LOSS: 0 mse (src/loss.jl:52), 1 logloss (:54-57), 2 gaussian_mle (:194-203), 3 poisson (:59-62),
+// 4 gamma (:64-67), 5 tweedie with rho = 1.5 (:69-76).
 // grad rows: [g_1..g_K, h_1..h_K, w]; every written value is multiplied by w (src/loss.jl:104-108, :223-233).
 template <int LOSS>
 __global__ __launch_bounds__(256) void k_grads(const float *__restrict__ pred, const float *__restrict__ y,
@@ -35,6 +36,19 @@ __global__ __launch_bounds__(256) void k_grads(const float *__restrict__ pred, c
             const float s = dev_sigmoid(pred[i]);
             out[0] = (s - y[i]) * w;
             out[1] = (s * (1.0f - s)) * w;
+        } else if (LOSS == 3) {
+            const float e = expf(pred[i]);
+            out[0] = (e - y[i]) * w;
+            out[1] = e * w;
+        } else if (LOSS == 4) {
+            const float e = expf(pred[i]);
+            out[0] = (2.0f * (1.0f - y[i] / e)) * w;
+            out[1] = (2.0f * y[i] / e) * w;
+        } else if (LOSS == 5) {
+            const float e = expf(pred[i]);
+            const float a = powf(e, 0.5f), b = powf(e, -0.5f);
+            out[0] = (2.0f * (a - y[i] * b)) * w;
+            out[1] = (2.0f * (0.5f * a - (-0.5f) * y[i] * b)) * w;
         } else {
             const float loc = pred[2 * i], raw = pred[2 * i + 1];
             const float scale = dev_softplus(raw);
@@ -139,8 +153,14 @@ int launch_grads(evt_ctx *c) {
         hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
     else if (c->loss == EVT_LOSS_LOGLOSS)
         hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
-    else
+    else if (c->loss == EVT_LOSS_GAUSSIAN_MLE)
         hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+    else if (c->loss == EVT_LOSS_POISSON)
+        hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+    else if (c->loss == EVT_LOSS_GAMMA)
+        hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+    else
+        hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -166,6 +186,96 @@ int launch_quantize(evt_ctx *c) {
     int4 c03 = make_int4(c->chan_k[0], c->chan_k[1], c->chan_k[2], c->chan_k[3]);
     hipLaunchKernelGGL(k_quantize, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, c->gq, c->N, c->NK, c->NA, c03,
                        c->chan_k[4], qmul, c->unit_w ? 1 : 0);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+// ---- evaluation metric ------------------------------------------------------------------------
+// Per row value of src/metrics.jl:1-28 (:88-91 for gaussian_mle) in Float32, weighted as eval[i] = w * v / K
+// (:43, :111), accumulated in Float64.  Two stages with a fixed shape (EVT_METRIC_BLOCKS partial sums, then one
+// block) keep the summation order, hence the result, independent of scheduling.
+__device__ __forceinline__ float metric_value(int metric, const float *__restrict__ pred, const float *__restrict__ y, int64_t i) {
+    if (metric == EVT_METRIC_GAUSSIAN_MLE) {
+        const float loc = pred[2 * i], scale = dev_softplus(pred[2 * i + 1]);
+        const float d = y[i] - loc;
+        return -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+    }
+    const float pk = pred[i], yk = y[i];
+    switch (metric) {
+    case EVT_METRIC_MSE:
+    case EVT_METRIC_RMSE: return (pk - yk) * (pk - yk);
+    case EVT_METRIC_MAE: return fabsf(pk - yk);
+    case EVT_METRIC_LOGLOSS: {
+        const float s = dev_sigmoid(pk);
+        return -yk * logf(s) + (yk - 1.0f) * logf(1.0f - s);
+    }
+    case EVT_METRIC_POISSON: {
+        const float e = expf(pk);
+        return 2.0f * (yk * logf(yk / e + 7.105427357601002e-15f) + e - yk); // eps(Float32(1e-7)) = 2^-47
+    }
+    case EVT_METRIC_GAMMA: {
+        const float e = expf(pk);
+        return 2.0f * (logf(e / yk) + yk / e - 1.0f);
+    }
+    default: {
+        const float e = expf(pk);
+        return 2.0f * (powf(yk, 0.5f) / (-0.5f) / 0.5f - yk * powf(e, -0.5f) / (-0.5f) + powf(e, 0.5f) / 0.5f);
+    }
+    }
+}
+
+__device__ __forceinline__ double block_sum_f64(double v, double *s_red) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+}
+
+__global__ __launch_bounds__(256) void k_metric_partial(const float *__restrict__ pred, const float *__restrict__ y,
+                                                       const float *__restrict__ grad, int64_t N, int NK, int metric, float kdiv,
+                                                       double *__restrict__ partial) {
+    __shared__ double s_red[4];
+    double num = 0.0, den = 0.0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
+        const float w = grad[(size_t)NK * i + NK - 1];
+        const float ev = w * metric_value(metric, pred, y, i) / kdiv;
+        num += (double)ev;
+        den += (double)w;
+    }
+    num = block_sum_f64(num, s_red);
+    den = block_sum_f64(den, s_red);
+    if (threadIdx.x == 0) {
+        partial[2 * blockIdx.x] = num;
+        partial[2 * blockIdx.x + 1] = den;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_metric_final(const double *__restrict__ partial, int nblocks, int metric, double *out) {
+    __shared__ double s_red[4];
+    double num = 0.0, den = 0.0;
+    for (int b = threadIdx.x; b < nblocks; b += 256) {
+        num += partial[2 * b];
+        den += partial[2 * b + 1];
+    }
+    num = block_sum_f64(num, s_red);
+    den = block_sum_f64(den, s_red);
+    if (threadIdx.x == 0) {
+        const double r = num / den;
+        out[0] = (metric == EVT_METRIC_RMSE) ? sqrt(r) : r;
+    }
+}
+
+// partial: 2 * EVT_METRIC_BLOCKS + 1 doubles; the metric lands in the last one
+int launch_eval_metric(evt_ctx *c, int metric, double *partial) {
+    int64_t nb = (c->N + 255) / 256;
+    if (nb > EVT_METRIC_BLOCKS) nb = EVT_METRIC_BLOCKS;
+    const float kdiv = (float)(metric == EVT_METRIC_GAUSSIAN_MLE ? c->K / 2 : c->K);
+    hipLaunchKernelGGL(k_metric_partial, dim3((unsigned)nb), dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->NK, metric, kdiv,
+                       partial);
+    HIPCHK(hipGetLastError());
+    hipLaunchKernelGGL(k_metric_final, dim3(1), dim3(256), 0, c->stream, partial, (int)nb, metric, partial + 2 * EVT_METRIC_BLOCKS);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

@@ -517,7 +517,7 @@ static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32
     A.pred = c->pred;
     A.t_pred = c->tree.pred;
     A.K = c->K;
-    A.loss = c->loss;
+    A.loss = (c->loss >= EVT_LOSS_POISSON) ? EVT_LOSS_MSE : c->loss; // only selects the leaf-add rule: plain sum like mse
     A.fuse_pred = fuse_pred ? 1 : 0;
     A.write_nidx = c->record_nidx ? 1 : 0;
 }

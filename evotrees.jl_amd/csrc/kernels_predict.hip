@@ -21,7 +21,7 @@ __device__ __forceinline__ int walk_packed(const uint32_t *__restrict__ nodes, c
 }
 
 __device__ __forceinline__ void add_leaf(float *pr, const float *lp, int K, int loss) {
-    if (loss == EVT_LOSS_MSE) {
+    if (loss == EVT_LOSS_MSE || loss >= EVT_LOSS_POISSON) { // every GradientRegression loss but logloss: plain sum
         for (int k = 0; k < K; k++) pr[k] += lp[k];
     } else if (loss == EVT_LOSS_LOGLOSS) {
         for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
@@ -96,6 +96,8 @@ __global__ __launch_bounds__(256) void k_predict_model(const uint32_t *__restric
             for (int k = 0; k < K; k++) acc[k] = 1.0f / (1.0f + expf(-acc[k]));
         } else if (loss == EVT_LOSS_GAUSSIAN_MLE) {
             for (int k = 1; k < K; k += 2) acc[k] = fmaxf(acc[k], 0.0f) + log1pf(expf(-fabsf(acc[k])));
+        } else if (loss >= EVT_LOSS_POISSON) {
+            for (int k = 0; k < K; k++) acc[k] = expf(acc[k]);
         }
     }
     for (int k = 0; k < K; k++) out[(size_t)K * i + k] = acc[k];

@@ -42,7 +42,25 @@ typedef enum {
 } evt_status;
 
 /* loss ids: the in-scope subset of src/loss.jl:20-34 */
-enum { EVT_LOSS_MSE = 0, EVT_LOSS_LOGLOSS = 1, EVT_LOSS_GAUSSIAN_MLE = 2 };
+enum {
+    EVT_LOSS_MSE = 0,
+    EVT_LOSS_LOGLOSS = 1,
+    EVT_LOSS_GAUSSIAN_MLE = 2,
+    EVT_LOSS_POISSON = 3,
+    EVT_LOSS_GAMMA = 4,
+    EVT_LOSS_TWEEDIE = 5
+};
+/* evaluation metrics, metric_dict of src/metrics.jl:209-224 (in-scope subset) */
+enum {
+    EVT_METRIC_MSE = 0,
+    EVT_METRIC_RMSE = 1,
+    EVT_METRIC_MAE = 2,
+    EVT_METRIC_LOGLOSS = 3,
+    EVT_METRIC_GAUSSIAN_MLE = 4,
+    EVT_METRIC_POISSON = 5,
+    EVT_METRIC_GAMMA = 6,
+    EVT_METRIC_TWEEDIE = 7
+};
 /* params.tree_type, src/learners.jl:45 */
 enum { EVT_TREE_BINARY = 0, EVT_TREE_OBLIVIOUS = 1 };
 
@@ -79,7 +97,7 @@ int evt_device_count(int32_t *count);
 /* ---- training cache ------------------------------------------------------------------
  * Replaces init_core(params, ::Type{<:GPU}, ...) device allocation
  * (ext/EvoTreesKernelAbstractionsExt/init.jl:1-151): sizes every device buffer.
- * nbins in [2,255] (src/learners.jl:527), K = 1 (mse, logloss) or 2 (gaussian_mle, one target). */
+ * nbins in [2,255] (src/learners.jl:527), K = 2 for gaussian_mle (one target), 1 for every other loss. */
 int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K, int32_t max_depth, int32_t loss,
                int32_t tree_type, evt_handle *out);
 /* Frees all device memory; the slot post_fit_gc has in the reference (src/fit.jl:340). */
@@ -128,6 +146,14 @@ int evt_grow_tree(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_
 int evt_predict_tree(evt_handle h, int32_t nnodes_tree, const int64_t *feat, const uint8_t *cond_bin,
                      const float *pred, const uint8_t *split);
 
+/* The eval CallBack's metric (src/callback.jl:130-135 -> src/metrics.jl:30-48, :100-116) on the
+ * handle's own state: sum_i(Float32(w[i] * value(pred[:, i], y[i]) / K)) / sum_i(w[i]), both sums in
+ * Float64; rmse = sqrt(mse).  A handle created on the eval rows (evt_create + evt_set_xbin /
+ * evt_binarize_f64 + evt_set_target with the eval y, w, offset and mu = 0) plays the CallBack: each
+ * new tree is added with evt_predict_tree, then this call returns the metric.  The sum order is
+ * fixed, so the result is bit-reproducible. */
+int evt_eval_metric(evt_handle h, int32_t metric, double *value_out);
+
 /* ---- read-back of cache state (parity tests, callbacks) ------------------------------ */
 /* The cache's binned matrix (nobs x nfeats column-major), e.g. after evt_binarize_f64. */
 int evt_get_xbin(evt_handle h, uint8_t *x_bin_out);
@@ -153,6 +179,14 @@ int evt_predict(int64_t nobs, int32_t nfeats, const uint8_t *x_bin_colmajor, con
                 int32_t loss, int32_t K, int32_t ntrees, const int64_t *tree_off, const int64_t *feat,
                 const uint8_t *cond_bin, const float *pred, const uint8_t *split, int32_t apply_link,
                 float *out);
+/* The same from raw features: binarize(data; edges) (src/fit-utils.jl:66-72, searchsortedfirst per
+ * column) on the device, in row chunks, followed by the traversal above — the whole of
+ * _predict(m, data, ::Type{<:GPU}).  x is nobs x nfeats column-major Float64; edges / edge_off as in
+ * evt_binarize_f64 (at most 254 edges per feature). */
+int evt_predict_f64(int64_t nobs, int32_t nfeats, const double *x_colmajor, const double *edges,
+                    const int32_t *edge_off, const uint8_t *feattypes, int32_t loss, int32_t K, int32_t ntrees,
+                    const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const float *pred,
+                    const uint8_t *split, int32_t apply_link, float *out);
 /* predict_leaf_idx (src/predict.jl:138-185): out is nobs x ntrees column-major UInt32. */
 int evt_predict_leaf_idx(int64_t nobs, int32_t nfeats, const uint8_t *x_bin_colmajor, const uint8_t *feattypes,
                          int32_t ntrees, const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin,

@@ -42,6 +42,9 @@
 #define ORC_MSE 0
 #define ORC_LOGLOSS 1
 #define ORC_GAUSSIAN_MLE 2
+#define ORC_POISSON 3
+#define ORC_GAMMA 4
+#define ORC_TWEEDIE 5
 
 typedef struct {
     int32_t loss;         /* ORC_MSE / ORC_LOGLOSS / ORC_GAUSSIAN_MLE                      */
@@ -105,6 +108,19 @@ void orc_update_grads(const orc_params *p, int64_t N, const float *pred, const f
             float gg = s - y[i], hh = s * (1.0f - s);
             g[0] = gg * w;
             g[1] = hh * w;
+        } else if (p->loss == ORC_POISSON) { /* src/loss.jl:59-62 */
+            float e = expf(pred[i]);
+            g[0] = (e - y[i]) * w;
+            g[1] = e * w;
+        } else if (p->loss == ORC_GAMMA) { /* src/loss.jl:64-67 */
+            float e = expf(pred[i]);
+            g[0] = (2.0f * (1.0f - y[i] / e)) * w;
+            g[1] = (2.0f * y[i] / e) * w;
+        } else if (p->loss == ORC_TWEEDIE) { /* src/loss.jl:69-76, rho = 1.5 */
+            float e = expf(pred[i]);
+            float a = powf(e, 0.5f), b = powf(e, -0.5f);
+            g[0] = (2.0f * (a - y[i] * b)) * w;
+            g[1] = (2.0f * (0.5f * a - (-0.5f) * y[i] * b)) * w;
         } else { /* gaussian_mle, one target: rows [g_loc, g_scale, h_loc, h_scale, w] */
             float loc = pred[2 * i], raw = pred[2 * i + 1];
             float scale = orc_softplusf(raw);
@@ -652,7 +668,7 @@ void orc_predict_tree(int32_t loss, int32_t K, int64_t N, const uint8_t *x_bin, 
         int nid = walk(x_bin, N, i, feattypes, t_feat, t_cond_bin, t_split);
         const float *lp = t_pred + (size_t)K * (nid - 1);
         float *pr = pred + (size_t)K * i;
-        if (loss == ORC_MSE) {
+        if (loss == ORC_MSE || loss >= ORC_POISSON) {
             for (int k = 0; k < K; k++) pr[k] += lp[k];
         } else if (loss == ORC_LOGLOSS) {
             for (int k = 0; k < K; k++) {
@@ -684,6 +700,40 @@ void orc_apply_link(int32_t loss, int32_t K, int64_t N, float *pred) {
             for (int k = 0; k < K; k++) pred[(size_t)K * i + k] = orc_sigmoidf(pred[(size_t)K * i + k]);
         } else if (loss == ORC_GAUSSIAN_MLE) {
             for (int k = 1; k < K; k += 2) pred[(size_t)K * i + k] = orc_softplusf(pred[(size_t)K * i + k]);
+        } else if (loss >= ORC_POISSON) {
+            for (int k = 0; k < K; k++) pred[(size_t)K * i + k] = expf(pred[(size_t)K * i + k]);
         }
     }
+}
+
+/*
+ * Evaluation metrics — src/metrics.jl:1-48 (_eval_metric: eval[i] = w[i] * value / K in Float32, result
+ * sum(Float64, eval) / sum(Float64, w)) and :88-112 (gaussian_mle: mean log-likelihood).
+ * metric: 0 mse, 1 rmse, 2 mae, 3 logloss, 4 gaussian_mle, 5 poisson, 6 gamma, 7 tweedie.
+ */
+double orc_eval_metric(int32_t metric, int32_t K, int64_t N, const float *pred, const float *y, const float *w) {
+    double num = 0.0, den = 0.0;
+    for (int64_t i = 0; i < N; i++) {
+        float wi = w ? w[i] : 1.0f;
+        float v;
+        if (metric == 4) {
+            float loc = pred[2 * i], scale = orc_softplusf(pred[2 * i + 1]);
+            float d = y[i] - loc;
+            v = -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+        } else {
+            float pk = pred[i], yk = y[i];
+            if (metric == 0 || metric == 1) v = (pk - yk) * (pk - yk);
+            else if (metric == 2) v = fabsf(pk - yk);
+            else if (metric == 3) { float s = orc_sigmoidf(pk); v = -yk * logf(s) + (yk - 1.0f) * logf(1.0f - s); }
+            else if (metric == 5) { float e = expf(pk); const float eps = 7.105427357601002e-15f; /* eps(Float32(1e-7)) = 2^-47 */
+                                    v = 2.0f * (yk * logf(yk / e + eps) + e - yk); }
+            else if (metric == 6) { float e = expf(pk); v = 2.0f * (logf(e / yk) + yk / e - 1.0f); }
+            else { float e = expf(pk); v = 2.0f * (powf(yk, 0.5f) / (-0.5f) / 0.5f - yk * powf(e, -0.5f) / (-0.5f) + powf(e, 0.5f) / 0.5f); }
+        }
+        float ev = wi * v / (float)((metric == 4) ? K / 2 : K);
+        num += (double)ev;
+        den += (double)wi;
+    }
+    double r = num / den;
+    return metric == 1 ? sqrt(r) : r;
 }

@@ -12,7 +12,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libevo_oracle.so")
 
-LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2}
+LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5}
+METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7}
 TREE_TYPES = {"binary": 0, "oblivious": 1}
 
 
@@ -80,6 +81,8 @@ def lib():
         L.orc_predict_leaf_idx.restype = None
         L.orc_apply_link.argtypes = [i32, i32, i64, vp]
         L.orc_apply_link.restype = None
+        L.orc_eval_metric.argtypes = [i32, i32, i64, vp, vp, vp]
+        L.orc_eval_metric.restype = C.c_double
         _lib = L
     return _lib
 
@@ -216,3 +219,9 @@ def predict_leaf_idx(x_bin_FN, feattypes, tree):
 
 def apply_link(loss_id, K, pred):
     lib().orc_apply_link(loss_id, K, pred.shape[0], _p(pred))
+
+
+def eval_metric(metric, K, pred, y, w=None):
+    """pred (N, K) f32 raw (link not applied), y (N,) f32, w (N,) f32 or None."""
+    w = None if w is None else np.ascontiguousarray(w, np.float32)
+    return lib().orc_eval_metric(METRIC_IDS[metric], K, pred.shape[0], _p(pred), _p(y), _p(w))

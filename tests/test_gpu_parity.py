@@ -28,6 +28,10 @@ def make_data(seed, N, F, nbins, loss="mse", weights=False, signal=True):
         y = (y + 0.5 * (x_bin[0] / nbins) + 0.25 * (x_bin[F // 2] > nbins // 3)).astype(np.float32)
     if loss == "logloss":
         y = (y > np.median(y)).astype(np.float32)
+    elif loss == "poisson":
+        y = np.floor(y * 3).astype(np.float32)  # counts, zeros included
+    elif loss in ("gamma", "tweedie"):
+        y = (y + 0.1).astype(np.float32)  # strictly positive
     w = (rng.random(N).astype(np.float32) + 0.5) if weights else None
     mu = (rng.standard_normal(K) * 0.1).astype(np.float32)
     return x_bin, y, w, mu
@@ -59,18 +63,18 @@ def assert_tree_bits(t_gpu, t_orc):
     assert np.array_equal(t_gpu.w.view(np.uint32), t_orc.w.view(np.uint32))
 
 
-def assert_tree_close(t_gpu, t_ref):
+def assert_tree_close(t_gpu, t_ref, pred_atol=1e-9):
     assert np.array_equal(t_gpu.feat, t_ref.feat)
     assert np.array_equal(t_gpu.cond_bin, t_ref.cond_bin)
     assert np.array_equal(t_gpu.split, t_ref.split)
     np.testing.assert_allclose(t_gpu.gain, t_ref.gain, rtol=RTOL, atol=1e-7)
-    np.testing.assert_allclose(t_gpu.pred, t_ref.pred, rtol=RTOL, atol=1e-9)
+    np.testing.assert_allclose(t_gpu.pred, t_ref.pred, rtol=RTOL, atol=pred_atol)
     np.testing.assert_allclose(t_gpu.w, t_ref.w, rtol=RTOL)
 
 
 # --------------------------------------------------------------------------- gradients
 @pytest.mark.parametrize("loss,weights", [("mse", False), ("mse", True), ("logloss", True), ("gaussian_mle", False),
-                                          ("gaussian_mle", True)])
+                                          ("gaussian_mle", True), ("poisson", True), ("gamma", False), ("tweedie", True)])
 def test_gradient_kernel(evt, loss, weights):
     N, F, B = 70001, 5, 16
     x_bin, y, w, mu = make_data(1, N, F, B, loss, weights)
@@ -110,6 +114,9 @@ CASES = [
     ("mse", False, 20000, 300, 16, 5, "binary", 300, 1.0, {}),
     ("mse", False, 1000, 3, 4, 1, "binary", 3, 1.0, {}),
     ("mse", False, 300, 1, 2, 3, "binary", 1, 1.0, dict(min_weight=0.0)),
+    ("poisson", True, 30000, 12, 32, 6, "binary", 9, 0.8, {}),
+    ("gamma", False, 30000, 20, 64, 6, "binary", 20, 1.0, dict(lambda_=0.2)),
+    ("tweedie", False, 30000, 12, 32, 5, "oblivious", 12, 1.0, {}),
 ]
 
 
@@ -279,7 +286,7 @@ def test_free_running_rounds_bit_exact_mse(evt, loss, tt, rowsample, colsample):
     o.close()
 
 
-@pytest.mark.parametrize("loss", ["logloss", "gaussian_mle"])
+@pytest.mark.parametrize("loss", ["logloss", "gaussian_mle", "poisson", "gamma", "tweedie"])
 def test_free_running_rounds_tolerance(evt, loss):
     # device exp/log1p differ from the host's by an ulp: structure must still agree with the
     # reference arithmetic and predictions stay within 1e-5 over several rounds.
@@ -296,7 +303,9 @@ def test_free_running_rounds_tolerance(evt, loss):
         orc.update_grads(op, p_orc, y, grad)
         t_gpu = h.grow_tree(js, gp)
         t_ref, _ = o.grow_tree(grad, rows, js, mode=0)
-        assert_tree_close(t_gpu, t_ref)
+        # here the two sides' gradients already differ by an ulp (device vs host exp), and a leaf whose gradient sum
+        # nearly cancels amplifies that: leaf values of ~1e-2 typical size get an absolute floor of 1e-5 of that size
+        assert_tree_close(t_gpu, t_ref, pred_atol=1e-7)
         o.predict_tree(t_ref, p_orc)
     np.testing.assert_allclose(h.get_pred(), p_orc, rtol=RTOL, atol=1e-6)
     h.close()
@@ -306,7 +315,7 @@ def test_free_running_rounds_tolerance(evt, loss):
 # --------------------------------------------------------------------------- inference
 def test_model_predict_and_leaf_idx(evt):
     N, F, B, D, R = 20000, 8, 32, 5, 6
-    for loss in ("mse", "logloss", "gaussian_mle"):
+    for loss in ("mse", "logloss", "gaussian_mle", "poisson"):
         x_bin, y, w, mu = make_data(31, N, F, B, loss, False)
         pk = dict(min_weight=8.0) if loss == "gaussian_mle" else {}
         h, o, op, gp, pred0, grad0 = setup_pair(evt, loss, x_bin, y, w, mu, B, D, **pk)

@@ -430,3 +430,99 @@ def test_fixed_point_mode_matches_f64_mode(loss, weights):
     if t1.split[0]:
         assert np.array_equal(Hq[0], Hq[1] + Hq[2])
     o.close()
+
+
+# ---------------------------------------------------------------- exp-link losses and metrics
+def _deviance64(name, p, y):
+    """Unit deviances in float64 from the textbook forms (McCullagh & Nelder), mu = exp(p)."""
+    mu = np.exp(p)
+    if name == "poisson":
+        return 2 * (y * np.log(y / mu) + mu - y)
+    if name == "gamma":
+        return 2 * (np.log(mu / y) + y / mu - 1)
+    rho = 1.5
+    return 2 * (y ** (2 - rho) / ((1 - rho) * (2 - rho)) - y * mu ** (1 - rho) / (1 - rho) + mu ** (2 - rho) / (2 - rho))
+
+
+@pytest.mark.parametrize("loss", ["poisson", "gamma", "tweedie"])
+def test_exp_link_grads_are_derivatives_of_the_deviance(loss):
+    # gamma and tweedie use (D', D''); poisson uses half of them (src/loss.jl:59-76).  Central differences of the
+    # float64 textbook deviance pin sign, terms and the role of y in both rows; the weight multiplies both.
+    rng = np.random.default_rng(11)
+    N = 400
+    y = (rng.random(N) * 3 + 0.2).astype(np.float32)
+    pred = (rng.standard_normal((N, 1)) * 0.5).astype(np.float32)
+    grad = np.zeros((N, 3), np.float32)
+    grad[:, 2] = rng.random(N).astype(np.float32) + 0.5
+    w = grad[:, 2].astype(np.float64)
+    orc.update_grads(orc.make_params(loss), pred, y, grad)
+    p64, y64, e = pred[:, 0].astype(np.float64), y.astype(np.float64), 1e-4
+    d1 = (_deviance64(loss, p64 + e, y64) - _deviance64(loss, p64 - e, y64)) / (2 * e)
+    d2 = (_deviance64(loss, p64 + e, y64) - 2 * _deviance64(loss, p64, y64) + _deviance64(loss, p64 - e, y64)) / e ** 2
+    scale = 0.5 if loss == "poisson" else 1.0
+    np.testing.assert_allclose(grad[:, 0], scale * d1 * w, rtol=2e-5, atol=2e-6)
+    np.testing.assert_allclose(grad[:, 1], scale * d2 * w, rtol=2e-4, atol=1e-5)
+    assert np.all(grad[:, 1] > 0)
+
+
+@pytest.mark.parametrize("metric", ["poisson", "gamma", "tweedie"])
+def test_deviance_metrics_vs_float64_and_zero_at_perfect_fit(metric):
+    rng = np.random.default_rng(12)
+    N = 1000
+    y = (rng.random(N) * 3 + 0.2).astype(np.float32)
+    pred = (rng.standard_normal((N, 1)) * 0.5).astype(np.float32)
+    w = (rng.random(N) + 0.5).astype(np.float32)
+    ref = np.sum(w.astype(np.float64) * _deviance64(metric, pred[:, 0].astype(np.float64), y.astype(np.float64))) / np.sum(w, dtype=np.float64)
+    np.testing.assert_allclose(orc.eval_metric(metric, 1, pred, y, w), ref, rtol=3e-6)
+    perfect = np.log(y).reshape(N, 1).astype(np.float32)
+    assert abs(orc.eval_metric(metric, 1, perfect, y, w)) < 2e-6
+    # y = 0 is a legal count: the poisson value is finite thanks to the epsilon inside the log
+    if metric == "poisson":
+        v = orc.eval_metric("poisson", 1, np.zeros((4, 1), np.float32), np.zeros(4, np.float32), None)
+        np.testing.assert_allclose(v, 2.0, rtol=1e-6)
+
+
+def test_mse_rmse_mae_logloss_metrics_vs_library_forms():
+    from sklearn.metrics import log_loss, mean_absolute_error, mean_squared_error
+    rng = np.random.default_rng(13)
+    N = 2000
+    y = rng.random(N).astype(np.float32)
+    pred = rng.standard_normal((N, 1)).astype(np.float32)
+    w = (rng.random(N) + 0.5).astype(np.float32)
+    mse = mean_squared_error(y, pred[:, 0], sample_weight=w)
+    np.testing.assert_allclose(orc.eval_metric("mse", 1, pred, y, w), mse, rtol=2e-6)
+    np.testing.assert_allclose(orc.eval_metric("rmse", 1, pred, y, w), np.sqrt(mse), rtol=2e-6)
+    np.testing.assert_allclose(orc.eval_metric("mae", 1, pred, y, w), mean_absolute_error(y, pred[:, 0], sample_weight=w), rtol=2e-6)
+    np.testing.assert_allclose(orc.eval_metric("mse", 1, pred, y, None), mean_squared_error(y, pred[:, 0]), rtol=2e-6)
+    yb = (y > 0.5).astype(np.float32)
+    prob = 1 / (1 + np.exp(-pred[:, 0].astype(np.float64)))
+    np.testing.assert_allclose(orc.eval_metric("logloss", 1, pred, yb, w), log_loss(yb, prob, sample_weight=w), rtol=1e-5)
+
+
+def test_gaussian_mle_metric_is_mean_logpdf_up_to_the_constant():
+    from scipy.stats import norm
+    rng = np.random.default_rng(14)
+    N = 2000
+    y = rng.standard_normal(N).astype(np.float32)
+    pred = np.stack([rng.standard_normal(N) * 0.3, rng.standard_normal(N)], axis=1).astype(np.float32)
+    w = (rng.random(N) + 0.5).astype(np.float32)
+    scale = np.log1p(np.exp(pred[:, 1].astype(np.float64)))
+    lp = norm.logpdf(y.astype(np.float64), pred[:, 0].astype(np.float64), scale) + 0.5 * np.log(2 * np.pi)
+    ref = np.sum(w * lp) / np.sum(w, dtype=np.float64)
+    np.testing.assert_allclose(orc.eval_metric("gaussian_mle", 2, pred, y, w), ref, rtol=1e-5, atol=1e-6)
+
+
+def test_exp_link_predict_and_apply_link():
+    # predict! adds leaf values without clamping for every GradientRegression loss but logloss (src/predict.jl:1-14);
+    # the response is exp of the sum (src/predict.jl:108-109)
+    x_bin = np.array([[1, 2, 3, 4]], np.uint8)
+    t = orc.Tree(1, 3)
+    t.feat[0], t.cond_bin[0], t.split[0] = 1, 2, 1
+    t.pred[1, 0], t.pred[2, 0] = 40.0, -40.0
+    pred = np.zeros((4, 1), np.float32)
+    orc.predict_tree(orc.LOSS_IDS["poisson"], 1, x_bin, np.ones(1, np.uint8), t, pred)
+    assert np.array_equal(pred[:, 0], np.float32([40, 40, -40, -40]))
+    small = np.float32([[0.5], [-1.25]])
+    out = small.copy()
+    orc.apply_link(orc.LOSS_IDS["gamma"], 1, out)
+    np.testing.assert_allclose(out, np.exp(small.astype(np.float64)), rtol=2e-7)
