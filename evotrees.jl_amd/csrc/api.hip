@@ -182,11 +182,13 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->h_stage = nullptr; c->h_stage_bytes = 0;
     c->n_js_last = 0;
     c->last_all_rows = true;
-    c->hist_blocks = 512;
-    c->hist_threads = 512;
+    // one block of 16 waves per CU: as many waves as two blocks of 8 (the LDS histogram caps a CU at 128 KB), half
+    // the flushes per node
+    c->hist_blocks = 256;
+    c->hist_threads = 1024;
     c->hist_min_rows = 2048;
     c->hist_variant = 0;
-    c->hist_seg_cost = 1024;
+    c->hist_seg_cost = 2048;
     c->record_nidx = false;
     c->nidx_valid = false;
     c->last_cond = 255;
@@ -916,7 +918,7 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
         ARGCHK(value >= 1 && value <= 65535, "hist_blocks must be in [1, 65535]");
         c->hist_blocks = (int)value;
     } else if (strcmp(name, "hist_min_rows") == 0) {
-        ARGCHK(value >= 1 && value <= EVT_HIST_MAX_ROWS_PER_BLOCK, "hist_min_rows must be in [1, 32768]");
+        ARGCHK(value >= 1 && value <= EVT_HIST_MAX_ROWS_PER_BLOCK, "hist_min_rows must be in [1, 65535]");
         c->hist_min_rows = (int)value;
     } else if (strcmp(name, "hist_seg_cost") == 0) {
         ARGCHK(value >= 0 && value <= 65536, "hist_seg_cost must be in [0, 65536]");

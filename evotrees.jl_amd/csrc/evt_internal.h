@@ -22,7 +22,9 @@
 #define EVT_MAX_DEPTH 16
 #define EVT_PACK_QBITS 30     // fixed-point bits of the gradient channel that shares a word with the row count
 #define EVT_PACK_CNT_BITS 16
-#define EVT_HIST_MAX_ROWS_PER_BLOCK 32768
+// rows one LDS histogram may take between two flushes: the packed row counter has EVT_PACK_CNT_BITS bits, and
+// 65535 * 2^EVT_PACK_QBITS < 2^46 leaves the gradient sum inside its 48 signed bits
+#define EVT_HIST_MAX_ROWS_PER_BLOCK 65535
 
 // Level table header slots (int64 each)
 #define LH_N_ACT 0

@@ -4,6 +4,7 @@
 // One thread = one observation x one 16-feature group.  Reads are coalesced along rows of each
 // column; the 16 bytes are written as one 128-bit store into the observation-major record.
 // Bins outside 1..B raise the device error flag (the histogram kernels index LDS with them).
+// Padding bytes of a record are set to 1, so that a kernel may index with them unchecked.
 __global__ __launch_bounds__(256) void k_transpose_validate(const uint8_t *__restrict__ xcm, uint8_t *__restrict__ xrm,
                                                            int64_t N, int F, int B, int RS, int32_t *errflag) {
     int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -14,7 +15,7 @@ __global__ __launch_bounds__(256) void k_transpose_validate(const uint8_t *__res
 #pragma unroll
     for (int t = 0; t < 16; t++) {
         int f = grp * 16 + t;
-        uint32_t b = 0;
+        uint32_t b = 1; // padding behind the last feature reads as bin 1: always a valid histogram index
         if (f < F) {
             b = xcm[(size_t)f * N + row];
             bad |= (b == 0 || b > (uint32_t)B);

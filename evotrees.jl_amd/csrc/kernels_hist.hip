@@ -100,12 +100,14 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
         const int64_t nxt = A.bprefix[i + 1];
         const int64_t nrows_end = nxt - A.seg_cost;
         const int64_t cend = end < nxt ? end : nxt;
-        const int64_t nend = cend < nrows_end ? cend : nrows_end;
-        if (start >= nend) { // only this node's padding lies in the span
+        const int64_t nend_all = cend < nrows_end ? cend : nrows_end;
+        if (start >= nend_all) { // only this node's padding lies in the span
             start = cend;
             i++;
             continue;
         }
+        // the packed row counter holds 16 bits: a longer run of one node is flushed in several parts
+        const int64_t nend = (PACK && nend_all - start > EVT_HIST_MAX_ROWS_PER_BLOCK) ? start + EVT_HIST_MAX_ROWS_PER_BLOCK : nend_all;
         const int64_t seg = A.bstart[i] - nbeg; // position in the row list = seg + p
         // software pipeline over U row groups per wave: the row ids of iteration k+2 and the records of
         // iteration k+1 are in flight while the LDS atomics of iteration k are issued
@@ -180,7 +182,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
         // flush this node's partial histogram: hist[node][slot][ag][bin].  A node whose rows all lie in
         // this block's span has a single writer: plain stores into its zero-initialised slice; a node
         // shared with other blocks is accumulated with 64-bit global atomics.
-        const bool sole = (nbeg >= blk_start) && (nrows_end <= blk_end);
+        const bool sole = (nbeg >= blk_start) && (nrows_end <= blk_end) && !(PACK && nrows_end - nbeg > EVT_HIST_MAX_ROWS_PER_BLOCK);
         long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
         // blocks start at different words so that concurrent flushes of one node do not queue on the
         // same addresses
@@ -215,8 +217,12 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
             }
         }
         __syncthreads();
-        start = cend;
-        i++;
+        if (nend < nend_all) {
+            start = nend; // same node again
+        } else {
+            start = cend;
+            i++;
+        }
     }
 }
 
@@ -228,8 +234,8 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
 // ((a*8 + t)*B + bin)*NS + sub for feature f = 8*sub + t, i.e. `sub` selects the bank pair, so the 16
 // lanes of a group always fall on 16 different bank pairs whatever their bins are.  Rows that share a
 // wave instruction sit in different groups and cannot collide inside one LDS pass either.
-template <int NA, bool PACK, int U, int MAXT>
-__global__ __launch_bounds__(MAXT) void k_hist_build16(HistArgs A) {
+template <int NA, bool PACK, int U, bool FULL>
+__global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     extern __shared__ unsigned long long H[]; // [NA][8][B][NS]
     const int tid = threadIdx.x, nthr = blockDim.x;
     const int lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
@@ -254,16 +260,17 @@ __global__ __launch_bounds__(MAXT) void k_hist_build16(HistArgs A) {
 
     const int sub = lane % NS, rloc = lane / NS;
     // byte offset of (t, bin 0) for this lane; bins are 1-based so bin*NS*8 is added on top
-    int coff[8];
+    // (32-bit unsigned arithmetic throughout: one 24-bit multiply-add per LDS address)
+    uint32_t coff[8];
     unsigned vmask = 0;
 #pragma unroll
     for (int t = 0; t < 8; t++) {
         const int f = sub * 8 + t;
         const bool ok = (f < A.F) && (A.jsmap[f] != 0xFFFF);
-        coff[t] = ((t * B - 1) * NS + sub) * 8;
+        coff[t] = (uint32_t)(((t * B - 1) * NS + sub) * 8);
         vmask |= ok ? (1u << t) : 0u;
     }
-    const int binmul = NS * 8;
+    const uint32_t binmul = (uint32_t)NS * 8u;
     const bool lane_on = vmask != 0;
     __syncthreads();
 
@@ -284,87 +291,106 @@ __global__ __launch_bounds__(MAXT) void k_hist_build16(HistArgs A) {
         const int64_t nxt = A.bprefix[i + 1];
         const int64_t nrows_end = nxt - A.seg_cost;
         const int64_t cend = end < nxt ? end : nxt;
-        const int64_t nend = cend < nrows_end ? cend : nrows_end;
-        if (start >= nend) { // only this node's padding lies in the span
+        const int64_t nend_all = cend < nrows_end ? cend : nrows_end;
+        if (start >= nend_all) { // only this node's padding lies in the span
             start = cend;
             i++;
             continue;
         }
+        // the packed row counter holds 16 bits: a longer run of one node is flushed in several parts
+        const int64_t nend = (PACK && nend_all - start > EVT_HIST_MAX_ROWS_PER_BLOCK) ? start + EVT_HIST_MAX_ROWS_PER_BLOCK : nend_all;
         const int64_t seg = A.bstart[i] - nbeg;
-        // software pipeline over U row groups per wave: the row ids of iteration k+2 and the records of
-        // iteration k+1 are in flight while the LDS atomics of iteration k are issued
+        // A wave takes SR = U * RPW consecutive positions of the run per iteration (U row groups of RPW rows).
+        // Row ids and gradient words are fetched one position per lane (one load instruction per SR rows instead of
+        // one per group): the number of load instructions in flight, not their bytes, is what a CU runs out of
+        // first.  Lane L holds position (L % 16) * RPW + rloc, i.e. lane u of every 16-lane DPP row holds what
+        // group u of that row's record needs, and a row broadcast (v_mov_dpp row_newbcast:u) hands it over.
+        // Rolling software pipeline: group u's atomics are issued as soon as its record (requested one iteration
+        // ago) is there, and the same registers are then reloaded with the group's record of the next iteration.
+        // Loads are unconditional (positions past the end are clamped to the run's last row, their groups are
+        // masked at the atomics) and the prologue issues its loads in the loop's order, so that the compiler's count
+        // of outstanding loads is exact and no wait drains the queue.
         {
-            constexpr uint32_t INV = 0xFFFFFFFFu;
-            const int64_t itstride = (int64_t)U * step;
-            uint32_t rc[U], rn[U];
-            uint2 vc[U], vn[U];
-            unsigned long long gc[U][NA], gn[U][NA];
-            int64_t b0 = start + (int64_t)wave * RPW;
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const int64_t p = b0 + (int64_t)u * step + rloc;
-                rc[u] = (lane_on && p < nend) ? A.is[seg + p] : INV;
+            const int SR = U * RPW; // positions per wave iteration (<= 64)
+            const int64_t itstride = (int64_t)nwaves * SR;
+            const uint32_t *isp = A.is + seg;
+            const int64_t lastp = nend - 1;          // >= start
+            int64_t pw = start + (int64_t)wave * SR; // first position of this wave's iteration
+            const int myu = lane & 15;
+            const int mypos = myu * RPW + rloc;      // position (within the iteration) whose id / gradient this lane fetches
+            const bool fetcher = myu < U;
+            uint32_t idc, idn;
+            unsigned long long gc[NA], gn[NA];
+            uint2 v[U];
+            {
+                const int64_t p = pw + mypos;
+                idc = isp[(fetcher && p < nend) ? p : lastp];
             }
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                vc[u] = make_uint2(0, 0);
-                if (rc[u] != INV) {
-                    vc[u] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)rc[u] * A.RS + sub * 8);
-#pragma unroll
-                    for (int a = 0; a < NA; a++) gc[u][a] = A.gq[(size_t)a * A.N + rc[u]];
-                }
+            for (int a = 0; a < NA; a++) gc[a] = A.gq[(size_t)a * A.N + idc];
+            {
+                const int64_t p = pw + itstride + mypos;
+                idn = isp[(fetcher && p < nend) ? p : lastp];
             }
+            __builtin_amdgcn_sched_barrier(0);
+#define EVT_H16_PRO(u_)                                                                                               \
+    if constexpr ((u_) < U) {                                                                                         \
+        const uint32_t row = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)idc, 0x150 + (u_), 0xF, 0xF, false);          \
+        v[(u_) < U ? (u_) : 0] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)row * A.RS + sub * 8);                 \
+        __builtin_amdgcn_sched_barrier(0);                                                                            \
+    }
+            EVT_H16_PRO(0) EVT_H16_PRO(1) EVT_H16_PRO(2) EVT_H16_PRO(3) EVT_H16_PRO(4) EVT_H16_PRO(5) EVT_H16_PRO(6) EVT_H16_PRO(7)
+            EVT_H16_PRO(8) EVT_H16_PRO(9) EVT_H16_PRO(10) EVT_H16_PRO(11) EVT_H16_PRO(12) EVT_H16_PRO(13) EVT_H16_PRO(14) EVT_H16_PRO(15)
+#undef EVT_H16_PRO
+            for (; pw < nend; pw += itstride) {
+                // next iteration's gradient words and the row ids of the one after: ahead of the records in issue order
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                const int64_t p = b0 + itstride + (int64_t)u * step + rloc;
-                rn[u] = (lane_on && p < nend) ? A.is[seg + p] : INV;
-            }
-            for (; b0 < nend; b0 += itstride) {
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    vn[u] = make_uint2(0, 0);
-                    if (rn[u] != INV) {
-                        vn[u] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)rn[u] * A.RS + sub * 8);
-#pragma unroll
-                        for (int a = 0; a < NA; a++) gn[u][a] = A.gq[(size_t)a * A.N + rn[u]];
-                    }
+                for (int a = 0; a < NA; a++) gn[a] = A.gq[(size_t)a * A.N + idn];
+                uint32_t idnn;
+                {
+                    const int64_t p = pw + 2 * itstride + mypos;
+                    idnn = isp[(fetcher && p < nend) ? p : lastp];
                 }
-                uint32_t rnn[U];
+                __builtin_amdgcn_sched_barrier(0);
+#define EVT_H16_STEP(u_)                                                                                              \
+    if constexpr ((u_) < U) {                                                                                         \
+        constexpr int ui = (u_) < U ? (u_) : 0;                                                                       \
+        {                                                                                                             \
+            unsigned long long gg[NA];                                                                                \
+            _Pragma("unroll") for (int a = 0; a < NA; a++) {                                                          \
+                const uint32_t glo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)gc[a], 0x150 + (u_), 0xF, 0xF, false); \
+                const uint32_t ghi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(gc[a] >> 32), 0x150 + (u_), 0xF, 0xF, false); \
+                gg[a] = ((unsigned long long)ghi << 32) | glo;                                                         \
+            }                                                                                                         \
+            if (lane_on && (pw + (u_) * RPW + rloc < nend)) {                                                          \
+                const uint32_t wds[2] = {v[ui].x, v[ui].y};                                                            \
+                _Pragma("unroll") for (int t = 0; t < 8; t++) {                                                        \
+                    if (FULL || (vmask & (1u << t))) {                                                                \
+                        const uint32_t bo = __umul24((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu, binmul) + coff[t];       \
+                        _Pragma("unroll") for (int a = 0; a < NA; a++)                                                 \
+                            atomicAdd(reinterpret_cast<unsigned long long *>(Hb + bo + (uint32_t)(a * plane * 8)), gg[a]); \
+                    }                                                                                                 \
+                }                                                                                                     \
+            }                                                                                                         \
+        }                                                                                                             \
+        const uint32_t row = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)idn, 0x150 + (u_), 0xF, 0xF, false);          \
+        v[ui] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)row * A.RS + sub * 8);                                \
+        __builtin_amdgcn_sched_barrier(0);                                                                            \
+    }
+                EVT_H16_STEP(0) EVT_H16_STEP(1) EVT_H16_STEP(2) EVT_H16_STEP(3) EVT_H16_STEP(4) EVT_H16_STEP(5) EVT_H16_STEP(6) EVT_H16_STEP(7)
+                EVT_H16_STEP(8) EVT_H16_STEP(9) EVT_H16_STEP(10) EVT_H16_STEP(11) EVT_H16_STEP(12) EVT_H16_STEP(13) EVT_H16_STEP(14) EVT_H16_STEP(15)
+#undef EVT_H16_STEP
 #pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const int64_t p = b0 + 2 * itstride + (int64_t)u * step + rloc;
-                    rnn[u] = (lane_on && p < nend) ? A.is[seg + p] : INV;
-                }
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    if (rc[u] != INV) {
-                        const uint32_t wds[2] = {vc[u].x, vc[u].y};
-#pragma unroll
-                        for (int t = 0; t < 8; t++) {
-                            if (vmask & (1u << t)) {
-                                const int bo = coff[t] + (int)((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu) * binmul;
-#pragma unroll
-                                for (int a = 0; a < NA; a++)
-                                    atomicAdd(reinterpret_cast<unsigned long long *>(Hb + bo + a * plane * 8), gc[u][a]);
-                            }
-                        }
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    rc[u] = rn[u];
-                    vc[u] = vn[u];
-#pragma unroll
-                    for (int a = 0; a < NA; a++) gc[u][a] = gn[u][a];
-                    rn[u] = rnn[u];
-                }
+                for (int a = 0; a < NA; a++) gc[a] = gn[a];
+                idc = idn;
+                idn = idnn;
             }
         }
         __syncthreads();
         // flush: a wave covers 8 consecutive bins x 8 consecutive pieces `sub` of one (channel, t): global
         // accesses are whole 64-byte runs of one feature's bins, LDS reads spread over 8 bank pairs.  Blocks
         // start at different items so that concurrent flushes of one node do not queue on the same addresses.
-        const bool sole = (nbeg >= blk_start) && (nrows_end <= blk_end);
+        const bool sole = (nbeg >= blk_start) && (nrows_end <= blk_end) && !(PACK && nrows_end - nbeg > EVT_HIST_MAX_ROWS_PER_BLOCK);
         long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
         const int nchunks = (B + 7) >> 3;
         const int nsg = NS >> 3;
@@ -382,11 +408,12 @@ __global__ __launch_bounds__(MAXT) void k_hist_build16(HistArgs A) {
             const int b = chunk * 8 + bl;
             const int sidx = sg * 8 + sl;
             const int f = sidx * 8 + t;
-            if (b >= B || f >= A.F) continue;
+            if (b >= B) continue;
             unsigned long long *hw = &H[(size_t)a * plane + ((size_t)t * B + b) * NS + sidx];
             const unsigned long long w = *hw;
             if (w == 0ull) continue;
             *hw = 0ull;
+            if (f >= A.F) continue; // a padding byte's word
             const int slot = A.jsmap[f];
             if (slot == 0xFFFF) continue;
             unsigned long long *base = reinterpret_cast<unsigned long long *>(hn) + ((int64_t)slot * A.NAg) * B + b;
@@ -407,14 +434,22 @@ __global__ __launch_bounds__(MAXT) void k_hist_build16(HistArgs A) {
             }
         }
         __syncthreads();
-        start = cend;
-        i++;
+        if (nend < nend_all) {
+            start = nend; // same node again
+        } else {
+            start = cend;
+            i++;
+        }
     }
 }
 
 template <int NA, bool PACK>
 static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
-    hipLaunchKernelGGL((k_hist_build16<NA, PACK, 4, 1024>), grid, dim3(threads), lds, c->stream, A);
+    constexpr int U = (NA <= 2) ? 16 : 8; // row groups (records) in flight per wave, bounded by registers
+    if (c->n_js_last == c->F)
+        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, true>), grid, dim3(threads), lds, c->stream, A);
+    else
+        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, false>), grid, dim3(threads), lds, c->stream, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -469,14 +504,11 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
     size_t lds = per_slot * slots_per_tile;
     int threads = c->hist_threads;
     int64_t blocks = c->hist_blocks;
-    // a block's span must stay below the row count the packed 16-bit counter can hold
-    int64_t need = (c->N + (int64_t)c->maxlvl * c->hist_seg_cost + EVT_HIST_MAX_ROWS_PER_BLOCK - 1) / EVT_HIST_MAX_ROWS_PER_BLOCK;
-    if (blocks < need) blocks = need;
     dim3 grid((unsigned)blocks, (unsigned)ntiles);
     const bool pack = c->unit_w;
-    // conflict-free variant: records of 128/256/512 bytes whose whole LDS histogram fits 64 KB
+    // conflict-free variant: records of 128, 256 or 512 bytes whose whole LDS histogram fits 64 KB
     const size_t lds16 = (size_t)c->NA * 8 * c->B * (c->RS / 8) * 8;
-    const bool can16 = (c->RS % 128 == 0) && c->RS <= 512 && lds16 <= 64 * 1024;
+    const bool can16 = (c->RS == 128 || c->RS == 256 || c->RS == 512) && lds16 <= 64 * 1024; // 16, 32 or 64 lanes per row
     const bool use16 = (c->hist_variant == 2) ? can16 : (c->hist_variant == 1 ? false : can16);
     if (use16) {
         dim3 grid16((unsigned)blocks, 1u);
