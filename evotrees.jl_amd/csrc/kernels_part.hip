@@ -71,14 +71,22 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
         const bool numeric = A.feattypes[f] != 0;
         const uint8_t *col = A.xcm + (size_t)f * A.N;
         int cnt = 0;
+        // all row ids, then all bin bytes, are requested before the first is used; positions past the end read the
+        // segment's last row (unconditional loads keep every request of the chunk in flight at once)
+        constexpr int NI = EVT_CHUNK / 256;
+        uint32_t rid[NI], xbv[NI];
 #pragma unroll
-        for (int it = 0; it < EVT_CHUNK / 256; it++) {
+        for (int it = 0; it < NI; it++) {
             const int64_t p = p0 + it * 256 + tid;
-            bool flag = false;
-            if (p < pend) {
-                const uint32_t xb = col[A.is_cur[p]];
-                flag = numeric ? (xb <= cb) : (xb == cb);
-            }
+            rid[it] = A.is_cur[p < pend ? p : pend - 1];
+        }
+#pragma unroll
+        for (int it = 0; it < NI; it++) xbv[it] = col[rid[it]];
+#pragma unroll
+        for (int it = 0; it < NI; it++) {
+            const int64_t p = p0 + it * 256 + tid;
+            const uint32_t xb = xbv[it];
+            const bool flag = (p < pend) && (numeric ? (xb <= cb) : (xb == cb));
             const unsigned long long bal = __ballot(flag);
             if (lane == 0) A.flagw[c * EVT_CHUNK_WORDS + it * 4 + wave] = bal;
             cnt += __popcll(bal);
@@ -116,8 +124,15 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
             const int64_t nl_node = A.seg_len[2 * n];
             const int64_t dstL = seg + lbase;
             const int64_t dstR = seg + nl_node + (cl * EVT_CHUNK - lbase);
+            constexpr int NI = EVT_CHUNK / 256;
+            uint32_t rid[NI];
 #pragma unroll
-            for (int it = 0; it < EVT_CHUNK / 256; it++) {
+            for (int it = 0; it < NI; it++) {
+                const int64_t p = p0 + it * 256 + tid;
+                rid[it] = A.is_cur[p < pend ? p : pend - 1];
+            }
+#pragma unroll
+            for (int it = 0; it < NI; it++) {
                 const int64_t p = p0 + it * 256 + tid;
                 if (p < pend) {
                     const int wi = it * 4 + wave;
@@ -125,9 +140,8 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
                     const int lrank = s_pre[wi] + __popcll(word & ((1ull << lane) - 1ull));
                     const bool flag = (word >> lane) & 1ull;
                     const int within = it * 256 + tid;
-                    const uint32_t row = A.is_cur[p];
                     const int64_t d = flag ? (dstL + lrank) : (dstR + (within - lrank));
-                    A.is_next[d] = row;
+                    A.is_next[d] = rid[it];
                 }
             }
             __syncthreads();
@@ -190,18 +204,40 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
             numeric = A.feattypes[f] != 0;
         }
         const uint8_t *col = A.xcm + (size_t)f * A.N;
+        // every request of the chunk goes out before the first result is used: row ids, then bin bytes, then (one
+        // output) the predictions; positions past the end read the segment's last row and are not written
+        constexpr int NI = EVT_CHUNK / 256;
+        uint32_t rid[NI], xbv[NI];
+        float prv[NI];
 #pragma unroll
-        for (int it = 0; it < EVT_CHUNK / 256; it++) {
+        for (int it = 0; it < NI; it++) {
+            const int64_t p = p0 + it * 256 + tid;
+            rid[it] = A.is_cur[p < pend ? p : pend - 1];
+        }
+#pragma unroll
+        for (int it = 0; it < NI; it++) xbv[it] = is_split ? (uint32_t)col[rid[it]] : 0u;
+        const bool fast1 = A.fuse_pred && K == 1;
+        if (fast1) {
+#pragma unroll
+            for (int it = 0; it < NI; it++) prv[it] = A.pred[rid[it]];
+        }
+#pragma unroll
+        for (int it = 0; it < NI; it++) {
             const int64_t p = p0 + it * 256 + tid;
             if (p < pend) {
-                const uint32_t row = A.is_cur[p];
+                const uint32_t row = rid[it];
                 int leaf = n;
                 if (is_split) {
-                    const uint32_t xb = col[row];
+                    const uint32_t xb = xbv[it];
                     const bool left = numeric ? (xb <= cb) : (xb == cb);
                     leaf = 2 * n + (left ? 0 : 1);
                 }
                 if (A.write_nidx) A.nidx[row] = (uint32_t)leaf;
+                if (fast1) {
+                    const float s = prv[it] + A.t_pred[leaf - 1];
+                    A.pred[row] = (A.loss == EVT_LOSS_LOGLOSS) ? fminf(fmaxf(s, -15.0f), 15.0f) : s;
+                    continue;
+                }
                 if (A.fuse_pred) {
                     float *pr = A.pred + (size_t)K * row;
                     const float *lp = A.t_pred + (size_t)K * (leaf - 1);
