@@ -17,15 +17,15 @@ import numpy as np
 from . import _lib
 from ._lib import EvtError, Handle, TreeArrays, make_params  # noqa: F401
 
-__all__ = ["EvoTreeRegressor", "EvoTreeCount", "EvoTreeMLE", "EvoTree", "Tree", "fit", "predict", "predict_leaf_idx", "init",
-           "grow_evotree", "get_edges", "check_args", "CallBack", "init_logger", "update_logger", "EvtError"]
+__all__ = ["EvoTreeRegressor", "EvoTreeCount", "EvoTreeClassifier", "EvoTreeMLE", "EvoTree", "Tree", "fit", "predict", "predict_leaf_idx", "init",
+           "grow_evotree", "update", "okay_to_continue", "get_edges", "check_args", "CallBack", "init_logger", "update_logger", "EvtError"]
 
 _GPU_DEVICES = ("gpu", "rocm", "amd", "hip")
 _LOSS_K = {"mse": 1, "logloss": 1, "gaussian_mle": 2, "poisson": 1, "gamma": 1, "tweedie": 1}
 _EXP_LINK = ("poisson", "gamma", "tweedie")
 # is_maximise, src/metrics.jl:195-207
 _MAXIMISE = {"mse": False, "rmse": False, "mae": False, "logloss": False, "poisson": False, "gamma": False, "tweedie": False,
-             "gaussian_mle": True}
+             "gaussian_mle": True, "mlogloss": False}
 
 
 def _device_check(device):
@@ -98,6 +98,13 @@ class EvoTreeCount(_Learner):
     _defaults = dict(_Learner._defaults, loss="poisson")
 
 
+class EvoTreeClassifier(_Learner):
+    """EvoTreeClassifier (src/learners.jl:207-290): multi-class log loss over the levels of the target."""
+    _losses = ("mlogloss",)
+    _metrics = ("mlogloss",)
+    _defaults = dict(_Learner._defaults, loss="mlogloss")
+
+
 class EvoTreeMLE(_Learner):
     """EvoTreeMLE (src/learners.jl:300-400), loss gaussian_mle; min_weight defaults to 8."""
     _losses = ("gaussian_mle",)
@@ -151,11 +158,37 @@ def _invsoftplus(x):
     return x + np.log(-np.expm1(-x))
 
 
+def _levelcode(y, levels):
+    """1-based position of every element of y in `levels` (eval_levelcode, src/callback.jl:11-19)."""
+    levels = np.asarray(levels)
+    order = np.argsort(levels, kind="stable")
+    pos = np.searchsorted(levels[order], y)
+    pos = np.clip(pos, 0, len(levels) - 1)
+    found = levels[order][pos] == y
+    if not found.all():
+        raise RuntimeError("`y_eval` contains levels absent from `y_train`: %s. Training levels are %s."
+                           % (sorted(set(np.asarray(y)[~found].tolist())), levels.tolist()))
+    return (order[pos] + 1).astype(np.float32)
+
+
 def _init_target(loss, y):
-    """_init_target, src/init.jl:10-146 (in-scope branches)."""
+    """_init_target, src/init.jl:10-146 (in-scope branches).  Returns K, y (Float32), mu, target levels."""
     y = np.asarray(y)
     if y.ndim != 1:
         raise ValueError("only vector targets are supported by this backend")
+    if loss == "mlogloss":  # src/init.jl:43-67: levels = sort(unique(y)), level codes, mu = log(proportions) - max
+        if y.dtype.kind == "f":
+            raise RuntimeError("Invalid target eltype: %s" % y.dtype)
+        levels = np.unique(y)
+        K = len(levels)
+        if K < 2:
+            raise RuntimeError("Classification requires a target with at least 2 levels, got %d: %s. "
+                               "A single-class problem is not meaningful." % (K, levels.tolist()))
+        codes = _levelcode(y, levels)
+        prop = np.bincount(codes.astype(np.int64) - 1, minlength=K) / float(len(y))
+        mu = np.log(prop).astype(np.float32)
+        mu = mu - mu.max()
+        return K, codes, mu.astype(np.float32), levels
     y32 = y.astype(np.float32)
     if loss == "logloss":
         if y32.min() < 0 or y32.max() > 1:
@@ -169,7 +202,7 @@ def _init_target(loss, y):
         mu = np.array([np.log(np.float32(y32.mean(dtype=np.float32)))], np.float32)
     else:
         mu = np.array([y32.mean(dtype=np.float32)], np.float32)
-    return _LOSS_K[loss], y32, mu.astype(np.float32)
+    return _LOSS_K[loss], y32, mu.astype(np.float32), None
 
 
 def _link_offset(loss, offset, N, K):
@@ -177,7 +210,7 @@ def _link_offset(loss, offset, N, K):
     offset = np.array(offset, np.float32).reshape(N, K)
     if loss == "logloss":
         offset = _logit(offset)
-    elif loss in _EXP_LINK:
+    elif loss in _EXP_LINK or loss == "mlogloss":
         offset = np.log(offset)
     elif loss == "gaussian_mle":
         offset[:, 1] = _invsoftplus(offset[:, 1])
@@ -187,8 +220,8 @@ def _link_offset(loss, offset, N, K):
 class Cache:
     """What CacheBaseGPU holds on the host side: the device handle plus RNG and sampling sizes."""
 
-    def __init__(self, handle, rng, nfs, params, N, F):
-        self.handle, self.rng, self.nfs, self.params, self.N, self.F = handle, rng, nfs, params, N, F
+    def __init__(self, handle, rng, nfs, params, N, F, config=None):
+        self.handle, self.rng, self.nfs, self.params, self.N, self.F, self.config = handle, rng, nfs, params, N, F, config
 
 
 def init(config, x_train, y_train, w_train=None, offset_train=None, feature_names=None, device=None):
@@ -203,7 +236,7 @@ def init(config, x_train, y_train, w_train=None, offset_train=None, feature_name
         raise AssertionError("length(feature_names) must equal size(x_train, 2)")
     rng = np.random.default_rng(config.seed)
     edges, featbins, feattypes = get_edges(x, config.nbins, rng)
-    K, y32, mu = _init_target(config.loss, y_train)
+    K, y32, mu, target_levels = _init_target(config.loss, y_train)
     if y32.shape[0] != N:
         raise AssertionError("target length must equal the number of rows")
     w = None
@@ -223,12 +256,12 @@ def init(config, x_train, y_train, w_train=None, offset_train=None, feature_name
         mono[int(k) - 1] = int(v)
     h.set_feature_meta(feattypes, mono)
     h.set_target(y32, w, mu, offset)
-    info = dict(nrounds=0, feature_names=feature_names, target_levels=None, target_isordered=False, edges=edges, featbins=featbins,
+    info = dict(nrounds=0, feature_names=feature_names, target_levels=target_levels, target_isordered=False, edges=edges, featbins=featbins,
                 feattypes=feattypes)
     m = EvoTree(config.loss, K, [Tree.bias(mu)], info)
     nfs = int(np.ceil(config.colsample * F))
     params = make_params(config.eta, config.L2, config.lambda_, config.gamma, config.min_weight, config.bagging_size, True)
-    return m, Cache(h, rng, nfs, params, N, F)
+    return m, Cache(h, rng, nfs, params, N, F, config)
 
 
 def grow_evotree(m, cache, config):
@@ -264,7 +297,10 @@ class CallBack:
         N, F = x.shape
         self.metric = config.metric
         self.maximise = _MAXIMISE[config.metric]
-        y32 = np.asarray(y_eval).astype(np.float32)
+        if m.loss_type == "mlogloss":
+            y32 = _levelcode(np.asarray(y_eval), m.info["target_levels"])
+        else:
+            y32 = np.asarray(y_eval).astype(np.float32)
         if y32.shape != (N,):
             raise AssertionError("y_eval length must equal the number of eval rows")
         w = None if w_eval is None else np.asarray(w_eval, np.float32)
@@ -344,6 +380,26 @@ def fit(config, x_train=None, y_train=None, w_train=None, offset_train=None, x_e
             cache.handle.close()  # post_fit_gc slot, src/fit.jl:340
     m.info["logger"] = logger
     return (m, cache) if return_cache else m
+
+
+def okay_to_continue(config, m, cache):
+    """okay_to_continue, src/MLJ.jl:30-33: only nrounds may differ, and it may not shrink below what is grown."""
+    a, b = dict(config.__dict__), dict(cache.config.__dict__)
+    a.pop("nrounds")
+    b.pop("nrounds")
+    return a == b and config.nrounds >= m.info["nrounds"]
+
+
+def update(config, m, cache, x_train=None, y_train=None, w_train=None):
+    """MMI.update, src/MLJ.jl:38-57: warm restart on the handle the first fit kept (`fit(..., return_cache=True)`);
+    any change other than a larger nrounds refits from scratch."""
+    if okay_to_continue(config, m, cache):
+        while m.info["nrounds"] < config.nrounds:
+            grow_evotree(m, cache, config)
+        cache.config = config
+        return m, cache
+    cache.handle.close()
+    return fit(config, x_train=x_train, y_train=y_train, w_train=w_train, return_cache=True)
 
 
 def binarize(x, edges):

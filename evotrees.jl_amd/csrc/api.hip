@@ -149,9 +149,10 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ARGCHK(nfeats >= 1 && nfeats <= 1024, "nfeats must be in [1, 1024]");
     ARGCHK(nbins >= 2 && nbins <= 255, "nbins must be in [2, 255]");
     ARGCHK(max_depth >= 1 && max_depth <= EVT_MAX_DEPTH, "max_depth must be in [1, 16]");
-    ARGCHK(loss >= 0 && loss <= EVT_LOSS_TWEEDIE, "loss must be one of mse (0), logloss (1), gaussian_mle (2), poisson (3), gamma (4), tweedie (5)");
+    ARGCHK(loss >= 0 && loss <= EVT_LOSS_MLOGLOSS, "loss must be one of mse (0), logloss (1), gaussian_mle (2), poisson (3), gamma (4), tweedie (5), mlogloss (6)");
     ARGCHK(tree_type == EVT_TREE_BINARY || tree_type == EVT_TREE_OBLIVIOUS, "tree_type must be binary (0) or oblivious (1)");
-    ARGCHK(K == (loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1), "K must be 2 for gaussian_mle and 1 for the other losses");
+    if (loss == EVT_LOSS_MLOGLOSS) ARGCHK(K >= 2 && K <= EVT_MAX_K, "mlogloss needs 2 <= K <= 16 classes");
+    else ARGCHK(K == (loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1), "K must be 2 for gaussian_mle and 1 for the other one-target losses");
     int ndev = 0;
     {
         int r = evt_device_count(&ndev);
@@ -264,10 +265,10 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->jsmap, c->RS);
     ALLOC(c->feattypes, c->F);
     ALLOC(c->mono, c->F);
-    ALLOC(c->absmax, 8);
-    ALLOC(c->qexp, 8);
-    ALLOC(c->qbits, 8);
-    ALLOC(c->qscale, 16);
+    ALLOC(c->absmax, EVT_MC_MAX_NK);
+    ALLOC(c->qexp, EVT_MC_MAX_NK);
+    ALLOC(c->qbits, EVT_MC_MAX_NK);
+    ALLOC(c->qscale, 2 * EVT_MC_MAX_NK);
     ALLOC(c->metric_partial, 2 * EVT_METRIC_BLOCKS + 1);
     ALLOC(c->errflag, 1);
     if (tree_type == EVT_TREE_OBLIVIOUS) ALLOC(c->ogains, (size_t)c->maxlvl * c->F * c->B);
@@ -288,7 +289,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
         std::vector<uint8_t> ft(c->F, 1);
         hipError_t e2 = hipMemcpy(c->feattypes, ft.data(), c->F, hipMemcpyHostToDevice);
         if (e2 == hipSuccess) e2 = hipMemset(c->mono, 0, sizeof(int32_t) * c->F);
-        if (e2 == hipSuccess) e2 = hipMemset(c->absmax, 0, sizeof(uint32_t) * 8);
+        if (e2 == hipSuccess) e2 = hipMemset(c->absmax, 0, sizeof(uint32_t) * EVT_MC_MAX_NK);
         if (e2 == hipSuccess) e2 = hipMemset(c->nidx, 0, sizeof(uint32_t) * N);
         if (e2 == hipSuccess) e2 = hipMemset(c->errflag, 0, sizeof(int32_t));
         if (e2 != hipSuccess) {
@@ -391,13 +392,13 @@ static void set_channels(evt_ctx *c) {
         if (!c->unit_w) c->chan_k[na++] = c->NK - 1;
     }
     c->NA = na;
-    for (int a = na; a < EVT_MAX_NA; a++) c->chan_k[a] = 0;
+    for (int a = na; a < EVT_MC_MAX_NK; a++) c->chan_k[a] = 0;
     c->NAg = (c->loss == EVT_LOSS_MSE) ? 2 : c->NK;
     int qbg = 62 - ceil_log2_i64(c->N);
     if (qbg > 40) qbg = 40;
     for (int k = 0; k < c->NK; k++) c->h_qbits[k] = qbg;
     if (c->unit_w) c->h_qbits[0] = EVT_PACK_QBITS;
-    for (int k = c->NK; k < 8; k++) c->h_qbits[k] = 0;
+    for (int k = c->NK; k < EVT_MC_MAX_NK; k++) c->h_qbits[k] = 0;
 }
 
 extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, const float *mu, const float *offset) {
@@ -408,7 +409,13 @@ extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, cons
     c->unit_w = (w == nullptr);
     set_channels(c);
     HIPCHK(hipMemcpyAsync(c->y, y, sizeof(float) * c->N, hipMemcpyDefault, c->stream));
-    HIPCHK(hipMemcpyAsync(c->qbits, c->h_qbits, sizeof(int32_t) * 8, hipMemcpyHostToDevice, c->stream));
+    if (c->loss == EVT_LOSS_MLOGLOSS) {
+        int r = launch_validate_classes(c);
+        if (r != EVT_OK) return r;
+        r = check_errflag(c, "mlogloss targets must be whole numbers in 1..K");
+        if (r != EVT_OK) return r;
+    }
+    HIPCHK(hipMemcpyAsync(c->qbits, c->h_qbits, sizeof(int32_t) * EVT_MC_MAX_NK, hipMemcpyHostToDevice, c->stream));
     // stage w / offset through the (not yet needed) fixed-point buffer
     float *tmp = reinterpret_cast<float *>(c->gq);
     if (w) {
@@ -448,6 +455,8 @@ extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, cons
     for (int j = 0; j < c->F; j++) {
         ft[j] = ft[j] ? 1 : 0;
         ARGCHK(mo[j] >= -1 && mo[j] <= 1, "monotone constraints must be -1, 0 or 1");
+        // the reference has no pred_scalar method for the multi-class loss (src/predict.jl:205-238): a constraint cannot be evaluated there
+        ARGCHK(mo[j] == 0 || c->loss != EVT_LOSS_MLOGLOSS, "monotone constraints are not defined for mlogloss");
     }
     HIPCHK(hipMemcpy(c->feattypes, ft.data(), c->F, hipMemcpyHostToDevice));
     HIPCHK(hipMemcpy(c->mono, mo.data(), sizeof(int32_t) * c->F, hipMemcpyHostToDevice));
@@ -740,8 +749,8 @@ extern "C" int evt_get_hist(evt_handle c, double *out) {
 extern "C" int evt_get_quant(evt_handle c, int32_t *qbits, int32_t *qexp) {
     CTXCHK(c);
     ARGCHK(qbits && qexp, "NULL argument");
-    int32_t e[8];
-    HIPCHK(hipMemcpyAsync(e, c->qexp, sizeof(int32_t) * 8, hipMemcpyDeviceToHost, c->stream));
+    int32_t e[EVT_MC_MAX_NK];
+    HIPCHK(hipMemcpyAsync(e, c->qexp, sizeof(int32_t) * EVT_MC_MAX_NK, hipMemcpyDeviceToHost, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     for (int k = 0; k < c->NK; k++) {
         qbits[k] = c->h_qbits[k];
@@ -754,9 +763,10 @@ extern "C" int evt_get_quant(evt_handle c, int32_t *qbits, int32_t *qexp) {
 extern "C" int evt_eval_metric(evt_handle c, int32_t metric, double *value_out) {
     CTXCHK(c);
     ARGCHK(value_out, "value_out is NULL");
-    ARGCHK(metric >= 0 && metric <= EVT_METRIC_TWEEDIE, "unknown metric");
+    ARGCHK(metric >= 0 && metric <= EVT_METRIC_MLOGLOSS, "unknown metric");
     ARGCHK((metric == EVT_METRIC_GAUSSIAN_MLE) == (c->loss == EVT_LOSS_GAUSSIAN_MLE),
            "gaussian_mle is the metric of the gaussian_mle loss and of no other");
+    ARGCHK((metric == EVT_METRIC_MLOGLOSS) == (c->loss == EVT_LOSS_MLOGLOSS), "mlogloss is the metric of the mlogloss loss and of no other");
     if (!c->have_target) {
         evt_set_error("evt_eval_metric: set the target first");
         return EVT_ERR_STATE;
@@ -781,7 +791,7 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
                           const int32_t *edge_off = nullptr) {
     ARGCHK(nobs >= 1 && nfeats >= 1 && ntrees >= 1, "nobs, nfeats, ntrees must be >= 1");
     ARGCHK((x_bin || x_f64) && tree_off && feat && cond_bin && split, "NULL argument");
-    ARGCHK(leaf_out || (pred && out && K >= 1 && K <= 4 && loss >= 0 && loss <= EVT_LOSS_TWEEDIE), "invalid prediction arguments");
+    ARGCHK(leaf_out || (pred && out && K >= 1 && K <= EVT_MAX_K && loss >= 0 && loss <= EVT_LOSS_MLOGLOSS), "invalid prediction arguments");
     std::vector<int32_t> eoff;
     if (x_f64) {
         ARGCHK(edges && edge_off, "NULL argument");

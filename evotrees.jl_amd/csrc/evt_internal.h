@@ -16,8 +16,11 @@
 
 #define EVT_CHUNK 2048        // rows per partition chunk (8 per thread of a 256-thread block)
 #define EVT_CHUNK_WORDS 32    // 64-bit ballot words per chunk
-#define EVT_MAX_NK 5
+#define EVT_MAX_NK 5  // gradient rows of the one- and two-output losses (register arrays of the specialised kernels)
 #define EVT_MAX_NA 5
+#define EVT_MAX_K 16     // classes of the multi-class loss
+#define EVT_MC_MAX_NK 40 // >= 2 * EVT_MAX_K + 1: sizes of the per-row quantisation tables and of the generic kernels' arrays
+#define EVT_HIST_GROUP 4 // accumulator channels one histogram launch handles; more channels take several launches
 #define EVT_METRIC_BLOCKS 1024 // partial sums of the evaluation metric
 #define EVT_MAX_DEPTH 16
 #define EVT_PACK_QBITS 30     // fixed-point bits of the gradient channel that shares a word with the row count
@@ -70,7 +73,7 @@ struct evt_ctx {
     bool unit_w;       // weights are all one (w == NULL at set_target)
     int32_t NA;        // LDS accumulator channels per bin
     int32_t NAg;       // global histogram channels per bin
-    int32_t chan_k[EVT_MAX_NA]; // gradient row of LDS channel a
+    int32_t chan_k[EVT_MC_MAX_NK]; // gradient row of accumulator channel a
     bool have_xbin, have_target, have_grads;
 
     // data
@@ -99,10 +102,10 @@ struct evt_ctx {
     uint16_t *jsmap;   // [RS] slot of feature f (0-based), 0xFFFF = not sampled / padding
     uint8_t *feattypes;
     int32_t *mono;
-    uint32_t *absmax;  // [8] float bits
-    int32_t *qexp;     // [8]
-    int32_t *qbits;    // [8]
-    double *qscale;    // [8] decode scale per global channel
+    uint32_t *absmax;  // [EVT_MC_MAX_NK] float bits
+    int32_t *qexp;     // [EVT_MC_MAX_NK]
+    int32_t *qbits;    // [EVT_MC_MAX_NK]
+    double *qscale;    // [2 * EVT_MC_MAX_NK]: decode scale per global channel, then encode multiplier per gradient row
     double *metric_partial; // [2 * EVT_METRIC_BLOCKS + 1] evaluation-metric partial sums, result last
     int64_t *stats;    // [D+1] rows built per level
     int32_t *errflag;  // device-side validation flag
@@ -113,7 +116,7 @@ struct evt_ctx {
     // host staging (pinned)
     uint8_t *h_stage;
     size_t h_stage_bytes;
-    int32_t h_qbits[8];
+    int32_t h_qbits[EVT_MC_MAX_NK];
     int32_t n_js_last;
     std::vector<uint32_t> js_last;
     bool last_all_rows;
@@ -153,11 +156,37 @@ void evt_set_error(const char *fmt, ...);
         }                                \
     } while (0)
 
+// predict!'s update of one row's K outputs with a leaf's values (src/predict.jl:1-62): plain sum (mse and the exp-link
+// losses), clamp to [-15, 15] (logloss), floor -15 on the scale outputs (gaussian_mle), shift by the row maximum and
+// floor -15 (mlogloss).  pr may point to registers or memory.
+#ifdef __HIPCC__
+__device__ __forceinline__ void evt_add_leaf(float *pr, const float *lp, int K, int loss) {
+    if (loss == EVT_LOSS_LOGLOSS) {
+        for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
+    } else if (loss == EVT_LOSS_GAUSSIAN_MLE) {
+        for (int t = 0; t < K / 2; t++) {
+            pr[2 * t] += lp[2 * t];
+            pr[2 * t + 1] = fmaxf(-15.0f, pr[2 * t + 1] + lp[2 * t + 1]);
+        }
+    } else if (loss == EVT_LOSS_MLOGLOSS) {
+        float m = -INFINITY;
+        for (int k = 0; k < K; k++) {
+            pr[k] += lp[k];
+            m = fmaxf(m, pr[k]);
+        }
+        for (int k = 0; k < K; k++) pr[k] = fmaxf(-15.0f, pr[k] - m);
+    } else {
+        for (int k = 0; k < K; k++) pr[k] += lp[k];
+    }
+}
+#endif
+
 // ---- kernel launchers (each only enqueues on c->stream) -----------------------------------
 // grad
 int launch_grads(evt_ctx *c);
 int launch_quantize(evt_ctx *c);
 int launch_set_weight_row(evt_ctx *c, const float *w_dev);
+int launch_validate_classes(evt_ctx *c);
 int launch_init_pred(evt_ctx *c, const float *mu_dev, const float *offset_dev);
 // data layout
 int launch_transpose_validate(evt_ctx *c);

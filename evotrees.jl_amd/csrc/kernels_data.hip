@@ -123,3 +123,20 @@ int launch_init_pred(evt_ctx *c, const float *mu_dev, const float *offset_dev) {
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
+
+// Multi-class targets are level codes 1..K stored as Float32; the gradient and metric kernels index with them.
+__global__ __launch_bounds__(256) void k_validate_classes(const float *__restrict__ y, int64_t N, int K, int32_t *errflag) {
+    bool bad = false;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
+        const float v = y[i];
+        bad |= !(v >= 1.0f && v <= (float)K && v == floorf(v));
+    }
+    if (bad) atomicOr(errflag, 1);
+}
+int launch_validate_classes(evt_ctx *c) {
+    int64_t nb = (c->N + 255) / 256;
+    if (nb > 2048) nb = 2048;
+    hipLaunchKernelGGL(k_validate_classes, dim3((unsigned)nb), dim3(256), 0, c->stream, c->y, c->N, c->K, c->errflag);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}

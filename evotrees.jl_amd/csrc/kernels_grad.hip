@@ -83,14 +83,66 @@ __global__ __launch_bounds__(256) void k_grads(const float *__restrict__ pred, c
     }
 }
 
+// Multi-class log loss (src/loss.jl:93-98, :113-128): prob_k = exp(p_k) / sum_j exp(p_j); g_k = (prob_k - [y == k]) w,
+// h_k = prob_k (1 - prob_k) w; y holds the 1-based class.  The row maxima are reduced one gradient row at a time.
+__global__ __launch_bounds__(256) void k_grads_mlogloss(const float *__restrict__ pred, const float *__restrict__ y,
+                                                       float *__restrict__ grad, int64_t N, int K, uint32_t *absmax) {
+    const int NK = 2 * K + 1;
+    __shared__ float s_m[4];
+    float mx[2 * EVT_MAX_K];
+#pragma unroll
+    for (int k = 0; k < 2 * EVT_MAX_K; k++) mx[k] = 0.0f;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
+        const float *pr = pred + (size_t)K * i;
+        float *g = grad + (size_t)NK * i;
+        const float w = g[NK - 1];
+        const int cls = (int)y[i];
+        float e[EVT_MAX_K];
+        float isum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < EVT_MAX_K; k++) {
+            if (k < K) {
+                e[k] = expf(pr[k]);
+                isum += e[k];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < EVT_MAX_K; k++) {
+            if (k < K) {
+                const float prob = e[k] / isum;
+                const float gg = ((cls == k + 1) ? prob - 1.0f : prob) * w;
+                const float hh = (prob * (1.0f - prob)) * w;
+                g[k] = gg;
+                g[K + k] = hh;
+                mx[k] = fmaxf(mx[k], fabsf(gg));
+                mx[EVT_MAX_K + k] = fmaxf(mx[EVT_MAX_K + k], fabsf(hh));
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 2 * EVT_MAX_K; k++) {
+        const int kk = k < EVT_MAX_K ? k : k - EVT_MAX_K;
+        if (kk < K) { // uniform
+            const float m = wave_max_f32(mx[k]);
+            __syncthreads();
+            if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                const float mm = fmaxf(fmaxf(s_m[0], s_m[1]), fmaxf(s_m[2], s_m[3]));
+                if (mm > 0.0f) atomicMax(&absmax[k < EVT_MAX_K ? kk : K + kk], __float_as_uint(mm));
+            }
+        }
+    }
+}
+
 // max |v| of every gradient row of an existing gradient matrix (injected gradients, weight row)
 __global__ __launch_bounds__(256) void k_absmax(const float *__restrict__ grad, int64_t N, int NK, int k0, int k1, uint32_t *absmax) {
-    float m[EVT_MAX_NK];
-    for (int k = 0; k < EVT_MAX_NK; k++) m[k] = 0.0f;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256)
-        for (int k = k0; k < k1; k++) m[k] = fmaxf(m[k], fabsf(grad[(size_t)NK * i + k]));
+    // one gradient row at a time: any number of rows without per-thread arrays
     for (int k = k0; k < k1; k++) {
-        float v = wave_max_f32(m[k]);
+        float m = 0.0f;
+        for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256)
+            m = fmaxf(m, fabsf(grad[(size_t)NK * i + k]));
+        const float v = wave_max_f32(m);
         if ((threadIdx.x & 63) == 0 && v > 0.0f) atomicMax(&absmax[k], __float_as_uint(v));
     }
 }
@@ -122,21 +174,18 @@ __global__ void k_quant_setup(const uint32_t *absmax, const int32_t *qbits, int3
 // Stages the fixed-point words the histogram kernel adds: plane a of gq holds, per row,
 // q = rint(v * 2^(qbits-qexp)) of gradient row chan_k[a]; with unit weights plane 0 also carries
 // the row count in its low 16 bits ((q << 16) + 1) so that one 64-bit LDS add serves both.
+// Channel a reads gradient row a, except for mse whose channels are {g, w} = rows {0, 2}.
 __global__ __launch_bounds__(256) void k_quantize(const float *__restrict__ grad, unsigned long long *__restrict__ gq, int64_t N,
-                                                 int NK, int NA, int4 chan03, int chan4, const double *__restrict__ qmul, int pack) {
+                                                 int NK, int NA, int mse, const double *__restrict__ qmul, int pack) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= N) return;
     const float *g = grad + (size_t)NK * i;
-    int chan[5] = {chan03.x, chan03.y, chan03.z, chan03.w, chan4};
-#pragma unroll
-    for (int a = 0; a < EVT_MAX_NA; a++) {
-        if (a < NA) {
-            int k = chan[a];
-            long long q = __double2ll_rn((double)g[k] * qmul[k]);
-            unsigned long long word = (unsigned long long)q;
-            if (a == 0 && pack) word = ((unsigned long long)q << EVT_PACK_CNT_BITS) + 1ull;
-            gq[(size_t)a * N + i] = word;
-        }
+    for (int a = 0; a < NA; a++) {
+        const int k = (mse && a == 1) ? 2 : a;
+        long long q = __double2ll_rn((double)g[k] * qmul[k]);
+        unsigned long long word = (unsigned long long)q;
+        if (a == 0 && pack) word = ((unsigned long long)q << EVT_PACK_CNT_BITS) + 1ull;
+        gq[(size_t)a * N + i] = word;
     }
 }
 
@@ -159,6 +208,8 @@ int launch_grads(evt_ctx *c) {
         hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
     else if (c->loss == EVT_LOSS_GAMMA)
         hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+    else if (c->loss == EVT_LOSS_MLOGLOSS)
+        hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax);
     else
         hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
     HIPCHK(hipGetLastError());
@@ -179,13 +230,12 @@ int launch_absmax_rows(evt_ctx *c, int k0, int k1) {
 }
 
 int launch_quantize(evt_ctx *c) {
-    double *qmul = c->qscale + 8; // qscale[0..7] decode scales per global channel, [8..15] encode multipliers per gradient row
+    double *qmul = c->qscale + EVT_MC_MAX_NK; // decode scales per global channel first, then encode multipliers per gradient row
     hipLaunchKernelGGL(k_quant_setup, dim3(1), dim3(64), 0, c->stream, c->absmax, c->qbits, c->qexp, qmul, c->qscale, c->NK, c->NAg,
                        c->loss, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
-    int4 c03 = make_int4(c->chan_k[0], c->chan_k[1], c->chan_k[2], c->chan_k[3]);
-    hipLaunchKernelGGL(k_quantize, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, c->gq, c->N, c->NK, c->NA, c03,
-                       c->chan_k[4], qmul, c->unit_w ? 1 : 0);
+    hipLaunchKernelGGL(k_quantize, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, c->gq, c->N, c->NK, c->NA,
+                       c->loss == EVT_LOSS_MSE ? 1 : 0, qmul, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -194,7 +244,12 @@ int launch_quantize(evt_ctx *c) {
 // Per row value of src/metrics.jl:1-28 (:88-91 for gaussian_mle) in Float32, weighted as eval[i] = w * v / K
 // (:43, :111), accumulated in Float64.  Two stages with a fixed shape (EVT_METRIC_BLOCKS partial sums, then one
 // block) keep the summation order, hence the result, independent of scheduling.
-__device__ __forceinline__ float metric_value(int metric, const float *__restrict__ pred, const float *__restrict__ y, int64_t i) {
+__device__ __forceinline__ float metric_value(int metric, int K, const float *__restrict__ pred, const float *__restrict__ y, int64_t i) {
+    if (metric == EVT_METRIC_MLOGLOSS) { // src/metrics.jl:59-77
+        float isum = 0.0f;
+        for (int k = 0; k < K; k++) isum += expf(pred[(size_t)K * i + k]);
+        return logf(isum) - pred[(size_t)K * i + (int)y[i] - 1];
+    }
     if (metric == EVT_METRIC_GAUSSIAN_MLE) {
         const float loc = pred[2 * i], scale = dev_softplus(pred[2 * i + 1]);
         const float d = y[i] - loc;
@@ -234,13 +289,13 @@ __device__ __forceinline__ double block_sum_f64(double v, double *s_red) {
 }
 
 __global__ __launch_bounds__(256) void k_metric_partial(const float *__restrict__ pred, const float *__restrict__ y,
-                                                       const float *__restrict__ grad, int64_t N, int NK, int metric, float kdiv,
+                                                       const float *__restrict__ grad, int64_t N, int NK, int K, int metric, float kdiv,
                                                        double *__restrict__ partial) {
     __shared__ double s_red[4];
     double num = 0.0, den = 0.0;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
         const float w = grad[(size_t)NK * i + NK - 1];
-        const float ev = w * metric_value(metric, pred, y, i) / kdiv;
+        const float ev = w * metric_value(metric, K, pred, y, i) / kdiv;
         num += (double)ev;
         den += (double)w;
     }
@@ -271,8 +326,8 @@ __global__ __launch_bounds__(256) void k_metric_final(const double *__restrict__
 int launch_eval_metric(evt_ctx *c, int metric, double *partial) {
     int64_t nb = (c->N + 255) / 256;
     if (nb > EVT_METRIC_BLOCKS) nb = EVT_METRIC_BLOCKS;
-    const float kdiv = (float)(metric == EVT_METRIC_GAUSSIAN_MLE ? c->K / 2 : c->K);
-    hipLaunchKernelGGL(k_metric_partial, dim3((unsigned)nb), dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->NK, metric, kdiv,
+    const float kdiv = (metric == EVT_METRIC_MLOGLOSS) ? 1.0f : (float)(metric == EVT_METRIC_GAUSSIAN_MLE ? c->K / 2 : c->K);
+    hipLaunchKernelGGL(k_metric_partial, dim3((unsigned)nb), dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->NK, c->K, metric, kdiv,
                        partial);
     HIPCHK(hipGetLastError());
     hipLaunchKernelGGL(k_metric_final, dim3(1), dim3(256), 0, c->stream, partial, (int)nb, metric, partial + 2 * EVT_METRIC_BLOCKS);

@@ -38,6 +38,7 @@ struct HistArgs {
     int slots_per_tile;
     int min_rows;
     int seg_cost;
+    int a0; // first global channel of this launch (channels beyond EVT_HIST_GROUP take further launches)
 };
 
 template <int NA, bool PACK>
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     const int n_build = (int)A.hdr[LH_N_BUILD];
     const int64_t total = A.hdr[LH_TOTAL_BUILD];
     if (n_build <= 0 || total <= 0) return;
-    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0 && A.a0 == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
 
     const int step = nwaves * A.RPW; // rows per block iteration
     // rows per block: an even share, but never so few that the flush of a whole LDS histogram
@@ -210,9 +211,9 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
                         atomicAdd(base + (int64_t)(A.NAg - 1) * A.B, cnt);
                     }
                 } else if (sole) {
-                    base[(int64_t)a * A.B] = w;
+                    base[(int64_t)(A.a0 + a) * A.B] = w;
                 } else {
-                    atomicAdd(base + (int64_t)a * A.B, w);
+                    atomicAdd(base + (int64_t)(A.a0 + a) * A.B, w);
                 }
             }
         }
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     const int n_build = (int)A.hdr[LH_N_BUILD];
     const int64_t total = A.hdr[LH_TOTAL_BUILD];
     if (n_build <= 0 || total <= 0) return;
-    if (blockIdx.x == 0 && tid == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
+    if (blockIdx.x == 0 && tid == 0 && A.a0 == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
 
     const int NS = A.RS >> 3;     // 8-byte pieces per record
     const int RPW = 64 / NS;      // rows per wave instruction
@@ -428,9 +429,9 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                     atomicAdd(base + (int64_t)(A.NAg - 1) * B, cnt);
                 }
             } else if (sole) {
-                base[(int64_t)a * B] = w;
+                base[(int64_t)(A.a0 + a) * B] = w;
             } else {
-                atomicAdd(base + (int64_t)a * B, w);
+                atomicAdd(base + (int64_t)(A.a0 + a) * B, w);
             }
         }
         __syncthreads();
@@ -490,51 +491,63 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
     A.B = c->B;
     A.NAg = c->NAg;
     A.level = level;
-    // feature tiling so that one block's LDS histogram stays within budget
-    const size_t budget = 64 * 1024;
-    size_t per_slot = (size_t)c->NA * c->B * 8;
-    int slots_per_tile = (int)(budget / per_slot);
-    if (slots_per_tile < 1) slots_per_tile = 1;
-    if (slots_per_tile > nfs) slots_per_tile = nfs;
-    int ntiles = (nfs + slots_per_tile - 1) / slots_per_tile;
-    slots_per_tile = (nfs + ntiles - 1) / ntiles;
-    A.slots_per_tile = slots_per_tile;
     A.min_rows = c->hist_min_rows;
     A.seg_cost = c->hist_seg_cost;
-    size_t lds = per_slot * slots_per_tile;
-    int threads = c->hist_threads;
-    int64_t blocks = c->hist_blocks;
-    dim3 grid((unsigned)blocks, (unsigned)ntiles);
-    const bool pack = c->unit_w;
-    // conflict-free variant: records of 128, 256 or 512 bytes whose whole LDS histogram fits 64 KB
-    const size_t lds16 = (size_t)c->NA * 8 * c->B * (c->RS / 8) * 8;
-    const bool can16 = (c->RS == 128 || c->RS == 256 || c->RS == 512) && lds16 <= 64 * 1024; // 16, 32 or 64 lanes per row
-    const bool use16 = (c->hist_variant == 2) ? can16 : (c->hist_variant == 1 ? false : can16);
-    if (use16) {
-        dim3 grid16((unsigned)blocks, 1u);
+    const int threads = c->hist_threads;
+    const int64_t blocks = c->hist_blocks;
+    // accumulator channels are taken EVT_HIST_GROUP at a time (one launch each; the one- and two-output losses need
+    // a single launch); the packed row counter rides on channel 0, i.e. in the first group only
+    for (int a0 = 0; a0 < c->NA; a0 += (c->NA <= EVT_MAX_NA ? EVT_MAX_NA : EVT_HIST_GROUP)) {
+        const int na = (c->NA <= EVT_MAX_NA) ? c->NA : (c->NA - a0 < EVT_HIST_GROUP ? c->NA - a0 : EVT_HIST_GROUP);
+        A.a0 = a0;
+        A.gq = c->gq + (size_t)a0 * c->N;
+        const bool pack = c->unit_w && a0 == 0;
+        // feature tiling so that one block's LDS histogram stays within budget
+        const size_t budget = 64 * 1024;
+        const size_t per_slot = (size_t)na * c->B * 8;
+        int slots_per_tile = (int)(budget / per_slot);
+        if (slots_per_tile < 1) slots_per_tile = 1;
+        if (slots_per_tile > nfs) slots_per_tile = nfs;
+        const int ntiles = (nfs + slots_per_tile - 1) / slots_per_tile;
+        slots_per_tile = (nfs + ntiles - 1) / ntiles;
+        A.slots_per_tile = slots_per_tile;
+        const size_t lds = per_slot * slots_per_tile;
+        dim3 grid((unsigned)blocks, (unsigned)ntiles);
+        // conflict-free variant: records of 128, 256 or 512 bytes whose whole LDS histogram fits 64 KB
+        const size_t lds16 = (size_t)na * 8 * c->B * (c->RS / 8) * 8;
+        const bool can16 = (c->RS == 128 || c->RS == 256 || c->RS == 512) && lds16 <= 64 * 1024; // 16, 32 or 64 lanes per row
+        const bool use16 = (c->hist_variant == 1) ? false : can16;
+        int r = EVT_ERR_ARG;
+        if (use16) {
+            dim3 grid16((unsigned)blocks, 1u);
 #define H16CASE(NA_) \
-    case NA_: return pack ? launch_hist16_t<NA_, true>(c, A, grid16, threads, lds16) : launch_hist16_t<NA_, false>(c, A, grid16, threads, lds16);
-        switch (c->NA) {
-            H16CASE(1)
-            H16CASE(2)
-            H16CASE(3)
-            H16CASE(4)
-            H16CASE(5)
-        }
+    case NA_: r = pack ? launch_hist16_t<NA_, true>(c, A, grid16, threads, lds16) : launch_hist16_t<NA_, false>(c, A, grid16, threads, lds16); break;
+            switch (na) {
+                H16CASE(1)
+                H16CASE(2)
+                H16CASE(3)
+                H16CASE(4)
+                H16CASE(5)
+            }
 #undef H16CASE
-    }
+        } else {
 #define HCASE(NA_) \
-    case NA_: return pack ? launch_hist_t<NA_, true>(c, A, grid, threads, lds) : launch_hist_t<NA_, false>(c, A, grid, threads, lds);
-    switch (c->NA) {
-        HCASE(1)
-        HCASE(2)
-        HCASE(3)
-        HCASE(4)
-        HCASE(5)
-    }
+    case NA_: r = pack ? launch_hist_t<NA_, true>(c, A, grid, threads, lds) : launch_hist_t<NA_, false>(c, A, grid, threads, lds); break;
+            switch (na) {
+                HCASE(1)
+                HCASE(2)
+                HCASE(3)
+                HCASE(4)
+                HCASE(5)
+            }
 #undef HCASE
-    evt_set_error("unsupported channel count %d", c->NA);
-    return EVT_ERR_ARG;
+        }
+        if (r != EVT_OK) {
+            if (r == EVT_ERR_ARG) evt_set_error("unsupported channel count %d", na);
+            return r;
+        }
+    }
+    return EVT_OK;
 }
 
 // Reference-layout export for parity checks: out[k, bin, feat, node] Float64 (src/init.jl:204).
@@ -549,7 +562,7 @@ __global__ __launch_bounds__(256) void k_hist_export(const long long *__restrict
     for (int idx = threadIdx.x; idx < nfs * B; idx += 256) {
         int jp = idx / B, b = idx - jp * B;
         int f = (int)js[jp] - 1;
-        double ch[EVT_MAX_NA];
+        double ch[EVT_MC_MAX_NK];
         for (int ag = 0; ag < NAg; ag++) ch[ag] = (double)hn[((int64_t)jp * NAg + ag) * B + b] * qscale[ag];
         double *o = out + (((int64_t)node * F + f) * B + b) * NK;
         if (loss == 0) {

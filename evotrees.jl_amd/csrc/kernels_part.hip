@@ -158,16 +158,7 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
                     if (A.fuse_pred) {
                         float *pr = A.pred + (size_t)K * row;
                         const float *lp = A.t_pred + (size_t)K * (n - 1);
-                        if (A.loss == EVT_LOSS_MSE) {
-                            for (int k = 0; k < K; k++) pr[k] += lp[k];
-                        } else if (A.loss == EVT_LOSS_LOGLOSS) {
-                            for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
-                        } else {
-                            for (int t = 0; t < K / 2; t++) {
-                                pr[2 * t] += lp[2 * t];
-                                pr[2 * t + 1] = fmaxf(-15.0f, pr[2 * t + 1] + lp[2 * t + 1]);
-                            }
-                        }
+                        evt_add_leaf(pr, lp, K, A.loss);
                     }
                 }
             }
@@ -241,16 +232,7 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
                 if (A.fuse_pred) {
                     float *pr = A.pred + (size_t)K * row;
                     const float *lp = A.t_pred + (size_t)K * (leaf - 1);
-                    if (A.loss == EVT_LOSS_MSE) {
-                        for (int k = 0; k < K; k++) pr[k] += lp[k];
-                    } else if (A.loss == EVT_LOSS_LOGLOSS) {
-                        for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
-                    } else {
-                        for (int t = 0; t < K / 2; t++) {
-                            pr[2 * t] += lp[2 * t];
-                            pr[2 * t + 1] = fmaxf(-15.0f, pr[2 * t + 1] + lp[2 * t + 1]);
-                        }
-                    }
+                    evt_add_leaf(pr, lp, K, A.loss);
                 }
             }
         }
@@ -553,7 +535,7 @@ static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32
     A.pred = c->pred;
     A.t_pred = c->tree.pred;
     A.K = c->K;
-    A.loss = (c->loss >= EVT_LOSS_POISSON) ? EVT_LOSS_MSE : c->loss; // only selects the leaf-add rule: plain sum like mse
+    A.loss = c->loss; // selects the leaf-add rule
     A.fuse_pred = fuse_pred ? 1 : 0;
     A.write_nidx = c->record_nidx ? 1 : 0;
 }

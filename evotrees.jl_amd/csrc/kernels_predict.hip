@@ -20,19 +20,6 @@ __device__ __forceinline__ int walk_packed(const uint32_t *__restrict__ nodes, c
     return nid;
 }
 
-__device__ __forceinline__ void add_leaf(float *pr, const float *lp, int K, int loss) {
-    if (loss == EVT_LOSS_MSE || loss >= EVT_LOSS_POISSON) { // every GradientRegression loss but logloss: plain sum
-        for (int k = 0; k < K; k++) pr[k] += lp[k];
-    } else if (loss == EVT_LOSS_LOGLOSS) {
-        for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
-    } else {
-        for (int t = 0; t < K / 2; t++) {
-            pr[2 * t] += lp[2 * t];
-            pr[2 * t + 1] = fmaxf(-15.0f, pr[2 * t + 1] + lp[2 * t + 1]);
-        }
-    }
-}
-
 // one tree added to pred (K x N), all rows
 __global__ __launch_bounds__(256) void k_predict_tree(const uint32_t *__restrict__ nodes, const float *__restrict__ leaf_pred,
                                                      const uint8_t *__restrict__ xcm, const uint8_t *__restrict__ feattypes, int64_t N,
@@ -40,7 +27,7 @@ __global__ __launch_bounds__(256) void k_predict_tree(const uint32_t *__restrict
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= N) return;
     const int nid = walk_packed(nodes, xcm, N, i, feattypes);
-    add_leaf(pred + (size_t)K * i, leaf_pred + (size_t)K * (nid - 1), K, loss);
+    evt_add_leaf(pred + (size_t)K * i, leaf_pred + (size_t)K * (nid - 1), K, loss);
 }
 
 // node each sampled row of the last tree ended in (0 outside the sample): the walk reproduces the
@@ -79,28 +66,60 @@ int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, const float
 // whole model: trees concatenated, tree t owns nodes [off[t], off[t+1]); the running prediction
 // stays in registers and is written once.  The per-tree clamps are applied after every tree, as
 // predict! does.
+template <int KMAX>
 __global__ __launch_bounds__(256) void k_predict_model(const uint32_t *__restrict__ nodes, const float *__restrict__ leaf_pred,
                                                       const int64_t *__restrict__ off, int ntrees, const uint8_t *__restrict__ xcm,
                                                       const uint8_t *__restrict__ feattypes, int64_t N, int K, int loss, int apply_link,
                                                       float *out) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= N) return;
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float acc[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; k++) acc[k] = 0.0f;
     for (int t = 0; t < ntrees; t++) {
         const int64_t o = off[t];
         const int nid = walk_packed(nodes + o, xcm, N, i, feattypes);
-        add_leaf(acc, leaf_pred + (size_t)K * (o + nid - 1), K, loss);
+        const float *lp = leaf_pred + (size_t)K * (o + nid - 1);
+        if (KMAX <= 4) {
+            evt_add_leaf(acc, lp, K, loss);
+        } else { // many outputs: constant trip counts keep the running prediction in registers
+            float m = -INFINITY;
+#pragma unroll
+            for (int k = 0; k < KMAX; k++) {
+                if (k < K) {
+                    acc[k] += lp[k];
+                    m = fmaxf(m, acc[k]);
+                }
+            }
+            if (loss == EVT_LOSS_MLOGLOSS) {
+#pragma unroll
+                for (int k = 0; k < KMAX; k++) acc[k] = fmaxf(-15.0f, acc[k] - m);
+            }
+        }
     }
     if (apply_link) { // apply_prediction_link!, src/predict.jl:105-116
         if (loss == EVT_LOSS_LOGLOSS) {
             for (int k = 0; k < K; k++) acc[k] = 1.0f / (1.0f + expf(-acc[k]));
         } else if (loss == EVT_LOSS_GAUSSIAN_MLE) {
             for (int k = 1; k < K; k += 2) acc[k] = fmaxf(acc[k], 0.0f) + log1pf(expf(-fabsf(acc[k])));
+        } else if (loss == EVT_LOSS_MLOGLOSS) { // softmax!, src/predict.jl:187-195
+            float isum = 0.0f;
+#pragma unroll
+            for (int k = 0; k < KMAX; k++) {
+                if (k < K) {
+                    acc[k] = expf(acc[k]);
+                    isum += acc[k];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < KMAX; k++) acc[k] /= isum;
         } else if (loss >= EVT_LOSS_POISSON) {
             for (int k = 0; k < K; k++) acc[k] = expf(acc[k]);
         }
     }
-    for (int k = 0; k < K; k++) out[(size_t)K * i + k] = acc[k];
+#pragma unroll
+    for (int k = 0; k < KMAX; k++)
+        if (k < K) out[(size_t)K * i + k] = acc[k];
 }
 
 __global__ __launch_bounds__(256) void k_leaf_idx_model(const uint32_t *__restrict__ nodes, const int64_t *__restrict__ off, int ntrees,
@@ -113,8 +132,12 @@ __global__ __launch_bounds__(256) void k_leaf_idx_model(const uint32_t *__restri
 
 int launch_predict_model(hipStream_t s, const uint32_t *nodes, const float *leaf_pred, const int64_t *off, int ntrees, const uint8_t *xcm,
                          const uint8_t *feattypes, int64_t N, int K, int loss, int apply_link, float *out) {
-    hipLaunchKernelGGL(k_predict_model, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, nodes, leaf_pred, off, ntrees, xcm, feattypes, N, K,
-                       loss, apply_link, out);
+    if (K <= 4)
+        hipLaunchKernelGGL(k_predict_model<4>, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, nodes, leaf_pred, off, ntrees, xcm, feattypes, N,
+                           K, loss, apply_link, out);
+    else
+        hipLaunchKernelGGL(k_predict_model<EVT_MAX_K>, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, nodes, leaf_pred, off, ntrees, xcm,
+                           feattypes, N, K, loss, apply_link, out);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

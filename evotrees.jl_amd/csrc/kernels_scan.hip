@@ -395,7 +395,7 @@ __global__ __launch_bounds__(1024) void k_obliv_select(OblivArgs A) {
     __shared__ int s_i[1024];
     __shared__ int s_dec[3];
     __shared__ double s_gain;
-    __shared__ double s_sc[EVT_MAX_NA];
+    __shared__ double s_sc[EVT_MC_MAX_NK];
     if (tid < NAG) s_sc[tid] = A.qscale[tid];
     // level matrix and its first maximum
     double bg = -INFINITY;
@@ -437,8 +437,8 @@ __global__ __launch_bounds__(1024) void k_obliv_select(OblivArgs A) {
     const double bgain = s_gain;
     for (int i = wave; i < n_act; i += nwaves) {
         const int n = A.act_node[i];
-        long long Sq[EVT_MAX_NA];
-        double S[EVT_MAX_NK];
+        long long Sq[EVT_MC_MAX_NK];
+        double S[EVT_MC_MAX_NK];
         for (int ag = 0; ag < NAG; ag++) Sq[ag] = A.node_sum[(int64_t)n * NAG + ag];
         decode_vals(Sq, s_sc, A.loss, NK, S);
         if (lane == 0) A.tree.w[n - 1] = (float)S[NK - 1];
@@ -481,6 +481,243 @@ __global__ __launch_bounds__(1024) void k_obliv_select(OblivArgs A) {
     }
 }
 
+// ---- any number of outputs (multi-class log loss) ------------------------------------------------
+// Same search as k_scan / k_scan_fin with the channel count a run-time value: the node statistics live in shared
+// memory and the candidate gain is accumulated output by output, gain += term(left_k) + term(right_k) in the
+// reference's order (split_gain, src/split.jl:108-117), from one prefix scan per channel.
+__device__ __forceinline__ void node_totals_mc(const ScanArgs &A, int n, const long long *hn, bool writer, long long *s_Sq, double *s_S,
+                                               double *s_sc) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int NAG = A.NAg;
+    if (tid < NAG) s_sc[tid] = A.qscale[tid];
+    if (A.level == 1) {
+        for (int ag = wave; ag < NAG; ag += (blockDim.x >> 6)) {
+            long long s = 0;
+            for (int b = lane; b < A.B; b += 64) s += hn[(int64_t)ag * A.B + b];
+            s = wave_sum_i64(s);
+            if (lane == 0) {
+                s_Sq[ag] = s;
+                if (writer) A.node_sum[(int64_t)n * NAG + ag] = s;
+            }
+        }
+    } else if (tid < NAG) {
+        s_Sq[tid] = A.node_sum[(int64_t)n * NAG + tid];
+    }
+    __syncthreads();
+    if (tid < NAG) s_S[tid] = (double)s_Sq[tid] * s_sc[tid];
+    __syncthreads();
+}
+
+// left-side sums of one channel for this lane's BPL bins (numeric: inclusive prefix; categorical: the bin alone);
+// subtract nodes materialise h[n] = h[parent] - h[sibling] on the way
+template <int BPL>
+__device__ __forceinline__ void left_sums(const ScanArgs &A, long long *hn, const long long *hp, const long long *hs, int64_t o, bool is_sub,
+                                          bool numeric, int lane, long long *left) {
+    long long val[BPL];
+    long long run = 0;
+#pragma unroll
+    for (int t = 0; t < BPL; t++) {
+        const int b = lane * BPL + t;
+        long long v = 0;
+        if (b < A.B) {
+            if (is_sub) {
+                v = hp[o + b] - hs[o + b];
+                hn[o + b] = v;
+            } else {
+                v = hn[o + b];
+            }
+        }
+        val[t] = v;
+        run += v;
+        left[t] = run;
+    }
+    const long long excl = wave_incl_scan_i64(run) - run;
+#pragma unroll
+    for (int t = 0; t < BPL; t++) left[t] = numeric ? left[t] + excl : val[t];
+}
+
+template <int BPL>
+__global__ __launch_bounds__(256) void k_scan_mc(ScanArgs A) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int n = (1 << (A.level - 1)) + blockIdx.x;
+    const int st = A.status[n];
+    if (st != ST_BUILD && st != ST_SUBTRACT) return;
+    const bool is_sub = (st == ST_SUBTRACT);
+    const int B = A.B, NK = A.NK, K = A.K, NAG = A.NAg;
+    long long *hn = A.hist + (int64_t)(n - 1) * A.node_stride;
+    const long long *hp = A.hist + (int64_t)((n >> 1) - 1) * A.node_stride;
+    const long long *hs = A.hist + (int64_t)((n ^ 1) - 1) * A.node_stride;
+
+    __shared__ long long s_Sq[EVT_MC_MAX_NK];
+    __shared__ double s_S[EVT_MC_MAX_NK];
+    __shared__ double s_sc[EVT_MC_MAX_NK];
+    __shared__ double s_wg[4];
+    __shared__ int s_wjp[4], s_wbin[4];
+
+    node_totals_mc(A, n, hn, blockIdx.y == 0, s_Sq, s_S, s_sc);
+    double gain_p = 0.0;
+    for (int k = 0; k < K; k++) gain_p += term_gh(s_S[k], s_S[K + k], s_S[2 * K], A.lambda, A.L2);
+    const double w_p = s_S[NK - 1];
+
+    double wbest = -INFINITY;
+    int wjp = NO_BIN, wbin = NO_BIN;
+    const int nodeidx = blockIdx.x;
+    const int jp = blockIdx.y * nwaves + wave;
+    if (jp < A.nfs) {
+        const int f = (int)A.js[jp] - 1;
+        const bool numeric = A.feattypes[f] != 0;
+        const int bmax = numeric ? B - 1 : B;
+        long long lq[BPL];
+        double w_l[BPL], w_r[BPL], sg[BPL];
+        bool ok[BPL];
+        left_sums<BPL>(A, hn, hp, hs, ((int64_t)jp * NAG + (NAG - 1)) * B, is_sub, numeric, lane, lq);
+#pragma unroll
+        for (int t = 0; t < BPL; t++) {
+            const int b = lane * BPL + t;
+            w_l[t] = (double)lq[t] * s_sc[NAG - 1];
+            w_r[t] = w_p - w_l[t];
+            ok[t] = (b < B) && (b + 1 <= bmax) && (w_l[t] > A.min_weight) && (w_r[t] > A.min_weight);
+            sg[t] = 0.0;
+        }
+        for (int k = 0; k < K; k++) {
+            long long gq[BPL], hq[BPL];
+            left_sums<BPL>(A, hn, hp, hs, ((int64_t)jp * NAG + k) * B, is_sub, numeric, lane, gq);
+            left_sums<BPL>(A, hn, hp, hs, ((int64_t)jp * NAG + K + k) * B, is_sub, numeric, lane, hq);
+            const double Sg = s_S[k], Sh = s_S[K + k];
+#pragma unroll
+            for (int t = 0; t < BPL; t++) {
+                const double g_l = (double)gq[t] * s_sc[k], h_l = (double)hq[t] * s_sc[K + k];
+                sg[t] += term_gh(g_l, h_l, w_l[t], A.lambda, A.L2) + term_gh(Sg - g_l, Sh - h_l, w_r[t], A.lambda, A.L2);
+            }
+        }
+        double lg = -INFINITY;
+        int lb = NO_BIN;
+#pragma unroll
+        for (int t = 0; t < BPL; t++) {
+            const int b = lane * BPL + t;
+            if (b < B) {
+                const double gain = sg[t] - gain_p;
+                if (A.oblivious) {
+                    A.ogains[((int64_t)nodeidx * A.nfs + jp) * B + b] = ok[t] ? gain : 0.0;
+                } else if (ok[t] && gain > lg) {
+                    lg = gain;
+                    lb = b + 1;
+                }
+            }
+        }
+        if (!A.oblivious) {
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const double og = shfl_xor_f64(lg, o);
+                const int ob = __shfl_xor(lb, o);
+                if (og > lg || (og == lg && ob < lb)) { lg = og; lb = ob; }
+            }
+            if (lg > wbest) { wbest = lg; wjp = jp; wbin = lb; }
+        }
+    }
+    if (A.oblivious) return;
+    if (lane == 0) { s_wg[wave] = wbest; s_wjp[wave] = wjp; s_wbin[wave] = wbin; }
+    __syncthreads();
+    if (tid == 0) {
+        double bg = -INFINITY;
+        int bj = NO_BIN, bb = NO_BIN;
+        for (int w = 0; w < nwaves; w++) {
+            if (s_wg[w] > bg || (s_wg[w] == bg && s_wjp[w] < bj)) { bg = s_wg[w]; bj = s_wjp[w]; bb = s_wbin[w]; }
+        }
+        ScanBest r;
+        r.gain = bg; r.jp = bj; r.bin = bb;
+        A.sbest[(int64_t)nodeidx * gridDim.y + blockIdx.y] = r;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_scan_fin_mc(ScanArgs A, int ngroups) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = (1 << (A.level - 1)) + blockIdx.x;
+    if (A.leaf_level) {
+        if (n > 1 && A.status[n >> 1] != ST_SPLIT) return;
+    } else {
+        const int st = A.status[n];
+        if (st != ST_BUILD && st != ST_SUBTRACT) return;
+    }
+    const int B = A.B, NK = A.NK, K = A.K, NAG = A.NAg;
+    long long *hn = A.hist + (int64_t)(n - 1) * A.node_stride;
+    __shared__ long long s_Sq[EVT_MC_MAX_NK];
+    __shared__ double s_S[EVT_MC_MAX_NK];
+    __shared__ double s_sc[EVT_MC_MAX_NK];
+    __shared__ double s_g[256];
+    __shared__ int s_j[256], s_b[256];
+    __shared__ int s_dec[3];
+    node_totals_mc(A, n, hn, true, s_Sq, s_S, s_sc);
+    if (tid == 0) A.tree.w[n - 1] = (float)s_S[NK - 1];
+    if (A.leaf_level) {
+        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(s_S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
+        if (tid == 0) A.status[n] = ST_LEAF;
+        return;
+    }
+    double bg = -INFINITY;
+    int bj = NO_BIN, bb = NO_BIN;
+    if (tid < ngroups) {
+        const ScanBest r = A.sbest[(int64_t)blockIdx.x * ngroups + tid];
+        bg = r.gain; bj = r.jp; bb = r.bin;
+    }
+    s_g[tid] = bg; s_j[tid] = bj; s_b[tid] = bb;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (tid < o) {
+            if (s_g[tid + o] > s_g[tid] || (s_g[tid + o] == s_g[tid] && s_j[tid + o] < s_j[tid])) {
+                s_g[tid] = s_g[tid + o]; s_j[tid] = s_j[tid + o]; s_b[tid] = s_b[tid + o];
+            }
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        bg = s_g[0]; bj = s_j[0]; bb = s_b[0];
+        const int found = (bb != NO_BIN && bg > A.gamma) ? 1 : 0;
+        s_dec[0] = found; s_dec[1] = bj; s_dec[2] = bb;
+        if (found) {
+            const int feat = (int)A.js[bj];
+            A.tree.feat[n - 1] = feat;
+            A.tree.cond_bin[n - 1] = (uint8_t)bb;
+            A.tree.gain[n - 1] = (float)bg;
+            A.tree.split[n - 1] = 1;
+            A.tree.packed[n - 1] = (uint32_t)feat | ((uint32_t)bb << 16) | (1u << 24);
+            A.status[n] = ST_SPLIT;
+        } else {
+            A.status[n] = ST_LEAF;
+        }
+    }
+    __syncthreads();
+    if (!s_dec[0]) {
+        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(s_S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
+        return;
+    }
+    bj = s_dec[1]; bb = s_dec[2];
+    {
+        const int f = (int)A.js[bj] - 1;
+        const bool numeric = A.feattypes[f] != 0;
+        for (int ag = wave; ag < NAG; ag += (blockDim.x >> 6)) {
+            const int64_t o = ((int64_t)bj * NAG + ag) * B;
+            long long s = 0;
+            for (int b = lane; b < B; b += 64) {
+                const bool in = numeric ? (b + 1 <= bb) : (b + 1 == bb);
+                if (in) s += hn[o + b];
+            }
+            s = wave_sum_i64(s);
+            if (lane == 0) {
+                A.node_sum[(int64_t)(2 * n) * NAG + ag] = s;
+                A.node_sum[(int64_t)(2 * n + 1) * NAG + ag] = s_Sq[ag] - s;
+            }
+        }
+    }
+    if (!A.zero_children) return;
+    long long *hc = A.hist + (int64_t)(2 * n - 1) * A.node_stride;
+    const int64_t used = (int64_t)A.nfs * NAG * B;
+    for (int64_t i = tid; i < used; i += blockDim.x) {
+        hc[i] = 0;
+        hc[A.node_stride + i] = 0;
+    }
+}
+
 int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     ScanArgs A;
     A.sbest = reinterpret_cast<ScanBest *>(c->sbest);
@@ -505,6 +742,16 @@ int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     const int ngroups = (A.nfs + 3) / 4; // 4 waves per block, one sampled feature each
     dim3 grid(nodes, (unsigned)ngroups);
     const int bpl = (c->B + 63) / 64;
+    if (c->loss == EVT_LOSS_MLOGLOSS) {
+        if (!leaf_level) {
+            if (bpl == 1) hipLaunchKernelGGL((k_scan_mc<1>), grid, dim3(256), 0, c->stream, A);
+            else if (bpl == 2) hipLaunchKernelGGL((k_scan_mc<2>), grid, dim3(256), 0, c->stream, A);
+            else hipLaunchKernelGGL((k_scan_mc<4>), grid, dim3(256), 0, c->stream, A);
+        }
+        if (!A.oblivious || leaf_level) hipLaunchKernelGGL(k_scan_fin_mc, dim3(nodes), dim3(256), 0, c->stream, A, ngroups);
+        HIPCHK(hipGetLastError());
+        return EVT_OK;
+    }
 #define SCASE(NAG_)                                                                                     \
     case NAG_:                                                                                          \
         if (!leaf_level) {                                                                              \

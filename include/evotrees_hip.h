@@ -48,7 +48,8 @@ enum {
     EVT_LOSS_GAUSSIAN_MLE = 2,
     EVT_LOSS_POISSON = 3,
     EVT_LOSS_GAMMA = 4,
-    EVT_LOSS_TWEEDIE = 5
+    EVT_LOSS_TWEEDIE = 5,
+    EVT_LOSS_MLOGLOSS = 6 /* K classes, y holds the 1-based class (level code) as a Float32 */
 };
 /* evaluation metrics, metric_dict of src/metrics.jl:209-224 (in-scope subset) */
 enum {
@@ -59,7 +60,8 @@ enum {
     EVT_METRIC_GAUSSIAN_MLE = 4,
     EVT_METRIC_POISSON = 5,
     EVT_METRIC_GAMMA = 6,
-    EVT_METRIC_TWEEDIE = 7
+    EVT_METRIC_TWEEDIE = 7,
+    EVT_METRIC_MLOGLOSS = 8
 };
 /* params.tree_type, src/learners.jl:45 */
 enum { EVT_TREE_BINARY = 0, EVT_TREE_OBLIVIOUS = 1 };
@@ -97,7 +99,8 @@ int evt_device_count(int32_t *count);
 /* ---- training cache ------------------------------------------------------------------
  * Replaces init_core(params, ::Type{<:GPU}, ...) device allocation
  * (ext/EvoTreesKernelAbstractionsExt/init.jl:1-151): sizes every device buffer.
- * nbins in [2,255] (src/learners.jl:527), K = 2 for gaussian_mle (one target), 1 for every other loss. */
+ * nbins in [2,255] (src/learners.jl:527), K = 2 for gaussian_mle (one target), the number of classes
+ * (2..16) for mlogloss, 1 for every other loss. */
 int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K, int32_t max_depth, int32_t loss,
                int32_t tree_type, evt_handle *out);
 /* Frees all device memory; the slot post_fit_gc has in the reference (src/fit.jl:340). */
@@ -113,7 +116,8 @@ int evt_set_xbin(evt_handle h, const uint8_t *x_bin_colmajor);
  * concatenated per feature, edge_off has nfeats+1 entries. */
 int evt_binarize_f64(evt_handle h, const double *x_colmajor, const double *edges, const int32_t *edge_off);
 
-/* Target, weights and initial prediction: y Float32[nobs]; w Float32[nobs] or NULL for ones
+/* Target, weights and initial prediction: y Float32[nobs] (for mlogloss the 1-based level code of each row,
+ * as _init_target builds it, src/init.jl:43-67); w Float32[nobs] or NULL for ones
  * (device_ones, src/init.jl:300); pred[:, i] = mu (+ offset[:, i] if offset != NULL), offset is
  * K x nobs (src/init.jl:168-174).  Writes the weight row of the gradient matrix. */
 int evt_set_target(evt_handle h, const float *y, const float *w, const float *mu, const float *offset);

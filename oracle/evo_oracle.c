@@ -45,6 +45,8 @@
 #define ORC_POISSON 3
 #define ORC_GAMMA 4
 #define ORC_TWEEDIE 5
+#define ORC_MLOGLOSS 6
+#define ORC_MAX_NK 40 /* 2K+1 with up to 16 classes, rounded up */
 
 typedef struct {
     int32_t loss;         /* ORC_MSE / ORC_LOGLOSS / ORC_GAUSSIAN_MLE                      */
@@ -73,8 +75,8 @@ typedef struct {
     int64_t *seg_off, *seg_len;  /* per node view into `is`                                */
     double *sum;   /* NK per node : TrainNode.∑                                            */
     int64_t *sumq; /* NK per node, fixed mode                                              */
-    int32_t qbits[8];
-    int32_t qexp[8];
+    int32_t qbits[ORC_MAX_NK];
+    int32_t qexp[ORC_MAX_NK];
     int nthreads;
 } orc_cache;
 
@@ -98,6 +100,18 @@ void orc_update_grads(const orc_params *p, int64_t N, const float *pred, const f
     for (int64_t i = 0; i < N; i++) {
         float w = grad[(int64_t)NK * i + NK - 1];
         float *g = grad + (int64_t)NK * i;
+        if (p->loss == ORC_MLOGLOSS) { /* src/loss.jl:93-98, :113-128; y holds the 1-based class */
+            const float *pr = pred + (int64_t)K * i;
+            float isum = 0.0f;
+            for (int k = 0; k < K; k++) isum += expf(pr[k]);
+            for (int k = 0; k < K; k++) {
+                float prob = expf(pr[k]) / isum;
+                float gg = ((int)y[i] == k + 1) ? prob - 1.0f : prob;
+                g[k] = gg * w;
+                g[K + k] = (prob * (1.0f - prob)) * w;
+            }
+            continue;
+        }
         if (p->loss == ORC_MSE) {
             float pk = pred[i], yk = y[i];
             float gg = 2.0f * (pk - yk), hh = 2.0f;
@@ -284,7 +298,7 @@ static void orc_update_hist(orc_cache *c, const int *build_nodes, int n_build, c
                     for (int k = 0; k < NK; k++) hh[k] += (double)g[k];
                 }
             } else {
-                int64_t q[8];
+                int64_t q[ORC_MAX_NK];
                 for (int k = 0; k < NK; k++) q[k] = orc_quant(g[k], c->qbits[k], c->qexp[k]);
                 for (int jj = j0; jj < j1; jj++) {
                     int j = (int)js[jj] - 1;
@@ -368,8 +382,8 @@ static void scan_node(orc_cache *c, int n, const uint32_t *js, int nj, int mode,
     const int NK = c->NK, K = p->K, B = p->nbins;
     const double eps = DBL_EPSILON;
     const double *S = c->sum + (size_t)n * NK;
-    double SL[8], SR[8];
-    int64_t SLq[8];
+    double SL[ORC_MAX_NK], SR[ORC_MAX_NK];
+    int64_t SLq[ORC_MAX_NK];
     double gain_p = node_gain(S, K, p->lambda, p->L2, eps);
     double w_p = S[NK - 1];
     for (int jj = 0; jj < nj; jj++) {
@@ -668,7 +682,11 @@ void orc_predict_tree(int32_t loss, int32_t K, int64_t N, const uint8_t *x_bin, 
         int nid = walk(x_bin, N, i, feattypes, t_feat, t_cond_bin, t_split);
         const float *lp = t_pred + (size_t)K * (nid - 1);
         float *pr = pred + (size_t)K * i;
-        if (loss == ORC_MSE || loss >= ORC_POISSON) {
+        if (loss == ORC_MLOGLOSS) { /* src/predict.jl:48-62: add, then shift by the row maximum, floor at -15 */
+            float m = -INFINITY;
+            for (int k = 0; k < K; k++) { pr[k] += lp[k]; if (pr[k] > m) m = pr[k]; }
+            for (int k = 0; k < K; k++) { float v = pr[k] - m; pr[k] = v > -15.0f ? v : -15.0f; }
+        } else if (loss == ORC_MSE || loss >= ORC_POISSON) {
             for (int k = 0; k < K; k++) pr[k] += lp[k];
         } else if (loss == ORC_LOGLOSS) {
             for (int k = 0; k < K; k++) {
@@ -700,6 +718,10 @@ void orc_apply_link(int32_t loss, int32_t K, int64_t N, float *pred) {
             for (int k = 0; k < K; k++) pred[(size_t)K * i + k] = orc_sigmoidf(pred[(size_t)K * i + k]);
         } else if (loss == ORC_GAUSSIAN_MLE) {
             for (int k = 1; k < K; k += 2) pred[(size_t)K * i + k] = orc_softplusf(pred[(size_t)K * i + k]);
+        } else if (loss == ORC_MLOGLOSS) { /* softmax!, src/predict.jl:187-195 */
+            float isum = 0.0f;
+            for (int k = 0; k < K; k++) { pred[(size_t)K * i + k] = expf(pred[(size_t)K * i + k]); isum += pred[(size_t)K * i + k]; }
+            for (int k = 0; k < K; k++) pred[(size_t)K * i + k] /= isum;
         } else if (loss >= ORC_POISSON) {
             for (int k = 0; k < K; k++) pred[(size_t)K * i + k] = expf(pred[(size_t)K * i + k]);
         }
@@ -709,13 +731,21 @@ void orc_apply_link(int32_t loss, int32_t K, int64_t N, float *pred) {
 /*
  * Evaluation metrics — src/metrics.jl:1-48 (_eval_metric: eval[i] = w[i] * value / K in Float32, result
  * sum(Float64, eval) / sum(Float64, w)) and :88-112 (gaussian_mle: mean log-likelihood).
- * metric: 0 mse, 1 rmse, 2 mae, 3 logloss, 4 gaussian_mle, 5 poisson, 6 gamma, 7 tweedie.
+ * metric: 0 mse, 1 rmse, 2 mae, 3 logloss, 4 gaussian_mle, 5 poisson, 6 gamma, 7 tweedie, 8 mlogloss (:59-77,
+ * eval[i] = w[i] * (log(sum_k exp(p[k,i])) - p[y[i], i]), not divided by K).
  */
 double orc_eval_metric(int32_t metric, int32_t K, int64_t N, const float *pred, const float *y, const float *w) {
     double num = 0.0, den = 0.0;
     for (int64_t i = 0; i < N; i++) {
         float wi = w ? w[i] : 1.0f;
         float v;
+        if (metric == 8) {
+            float isum = 0.0f;
+            for (int k = 0; k < K; k++) isum += expf(pred[(size_t)K * i + k]);
+            num += (double)(wi * (logf(isum) - pred[(size_t)K * i + (int)y[i] - 1]));
+            den += (double)wi;
+            continue;
+        }
         if (metric == 4) {
             float loc = pred[2 * i], scale = orc_softplusf(pred[2 * i + 1]);
             float d = y[i] - loc;

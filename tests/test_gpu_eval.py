@@ -16,11 +16,12 @@ METRICS_OF = {
     "poisson": ["poisson", "mae"],
     "gamma": ["gamma"],
     "tweedie": ["tweedie", "rmse"],
+    "mlogloss": ["mlogloss"],
 }
 
 
 @pytest.mark.parametrize("loss,weights", [("mse", True), ("logloss", False), ("gaussian_mle", True), ("poisson", True),
-                                          ("gamma", False), ("tweedie", True)])
+                                          ("gamma", False), ("tweedie", True), ("mlogloss", True)])
 def test_eval_metric_matches_oracle(evt, loss, weights):
     N, F, B, D = 70001, 6, 32, 4
     x_bin, y, w, mu = make_data(41, N, F, B, loss, weights)
@@ -39,9 +40,11 @@ def test_eval_metric_matches_oracle(evt, loss, weights):
             exact_rows = metric in ("mse", "rmse", "mae")  # per-row Float32 values identical, only the Float64 sum order differs
             np.testing.assert_allclose(got, want, rtol=1e-12 if exact_rows else RTOL)
             assert got == h.eval_metric(metric)  # fixed summation order: reproducible to the bit
-    if loss != "gaussian_mle":
+    if loss not in ("gaussian_mle", "mlogloss"):
         with pytest.raises(evt.EvtError):
             h.eval_metric("gaussian_mle")
+        with pytest.raises(evt.EvtError):
+            h.eval_metric("mlogloss")
     else:
         with pytest.raises(evt.EvtError):
             h.eval_metric("mse")
@@ -163,3 +166,70 @@ def test_predict_f64_equals_host_binarize_then_predict(evt):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     with pytest.raises(evt.EvtError):
         evt._lib.predict_model_f64(np.ascontiguousarray(X[:10].T), [np.zeros(0)] * F, ft, "mse", K, trees)
+
+
+def test_classifier_fit_levels_logger_and_errors(evt):
+    # three classes cut from a noisy function of two features; labels are strings, levels are sorted(unique)
+    rng = np.random.default_rng(10)
+    N = 3000
+    X = rng.random((N, 4))
+    score = X[:, 0] + 0.5 * X[:, 1] + 0.05 * rng.standard_normal(N)
+    lab = np.where(score < 0.5, "low", np.where(score < 0.95, "mid", "top"))
+    tr, ev = np.arange(2400), np.arange(2400, N)
+    cfg = evt.EvoTreeClassifier(nrounds=30, nbins=32, eta=0.3, max_depth=4)
+    m = evt.fit(cfg, x_train=X[tr], y_train=lab[tr], x_eval=X[ev], y_eval=lab[ev], verbosity=0)
+    assert m.K == 3 and list(m.info["target_levels"]) == ["low", "mid", "top"]
+    # bias: log(proportions) shifted by its maximum (src/init.jl:63-64)
+    prop = np.array([(lab[tr] == l).mean() for l in ("low", "mid", "top")])
+    np.testing.assert_allclose(m.trees[0].pred[0], np.log(prop) - np.log(prop).max(), rtol=1e-6, atol=1e-7)
+    p = m(X[ev])
+    assert p.shape == (len(ev), 3)
+    np.testing.assert_allclose(p.sum(axis=1), 1.0, rtol=1e-5)
+    acc = (np.array(["low", "mid", "top"])[p.argmax(axis=1)] == lab[ev]).mean()
+    assert acc > 0.8, acc
+    lg = m.info["logger"]
+    assert lg["name"] == "mlogloss" and lg["metrics"][-1] < 0.6 * lg["metrics"][0]
+    # the logged values equal the oracle's metric of the oracle's replay
+    xb = evt.binarize(X[ev], m.info["edges"])
+    codes = np.searchsorted(np.array(["low", "mid", "top"]), lab[ev]).astype(np.float32) + 1
+    pr = np.zeros((len(ev), 3), np.float32)
+    for i, t in enumerate(m.trees):
+        orc.predict_tree(orc.LOSS_IDS["mlogloss"], 3, xb, np.ones(4, np.uint8), t, pr)
+        np.testing.assert_allclose(lg["metrics"][i], orc.eval_metric("mlogloss", 3, pr, codes), rtol=RTOL)
+    # an eval set with a level the model never saw is an error, as is a single-class or a Float target
+    bad = lab[ev].copy()
+    bad[0] = "unseen"
+    with pytest.raises(RuntimeError, match="absent from `y_train`"):
+        evt.fit(evt.EvoTreeClassifier(nrounds=1), x_train=X[tr], y_train=lab[tr], x_eval=X[ev], y_eval=bad, verbosity=0)
+    with pytest.raises(RuntimeError, match="at least 2 levels"):
+        evt.fit(evt.EvoTreeClassifier(nrounds=1), x_train=X[:50], y_train=np.array(["a"] * 50))
+    with pytest.raises(RuntimeError, match="Invalid target eltype"):
+        evt.fit(evt.EvoTreeClassifier(nrounds=1), x_train=X[:50], y_train=X[:50, 0])
+    # class codes outside 1..K and monotone constraints are refused by the library itself
+    h = evt.Handle(10, 2, 8, 3, 2, "mlogloss")
+    with pytest.raises(evt.EvtError):
+        h.set_target(np.float32([1, 2, 3, 4, 1, 2, 3, 1, 2, 3]), None, np.zeros(3, np.float32))
+    with pytest.raises(evt.EvtError):
+        h.set_target(np.float32([1, 2, 2.5, 3, 1, 2, 3, 1, 2, 3]), None, np.zeros(3, np.float32))
+    with pytest.raises(evt.EvtError):
+        h.set_feature_meta(None, np.int32([1, 0]))
+    h.close()
+    with pytest.raises(evt.EvtError):
+        evt.Handle(10, 2, 8, 17, 2, "mlogloss")
+
+
+def test_update_continues_on_the_kept_handle(evt):
+    # MMI.update (src/MLJ.jl:38-57): only a larger nrounds continues; the result equals a single longer fit
+    rng = np.random.default_rng(11)
+    X, Y = _sinus(rng, 600)
+    kw = dict(nbins=16, eta=0.2, max_depth=4, rowsample=0.7, colsample=1.0, seed=5)
+    m, cache = evt.fit(evt.EvoTreeRegressor(nrounds=5, **kw), x_train=X, y_train=Y, return_cache=True)
+    m, cache = evt.update(evt.EvoTreeRegressor(nrounds=12, **kw), m, cache)
+    assert m.info["nrounds"] == 12 and len(m.trees) == 13
+    m_ref = evt.fit(evt.EvoTreeRegressor(nrounds=12, **kw), x_train=X, y_train=Y)
+    assert np.array_equal(m(X), m_ref(X))
+    assert not evt.okay_to_continue(evt.EvoTreeRegressor(nrounds=20, **dict(kw, eta=0.1)), m, cache)
+    assert not evt.okay_to_continue(evt.EvoTreeRegressor(nrounds=3, **kw), m, cache)
+    m2, cache2 = evt.update(evt.EvoTreeRegressor(nrounds=4, **dict(kw, eta=0.1)), m, cache, x_train=X, y_train=Y)
+    assert m2.info["nrounds"] == 4 and len(m2.trees) == 5
+    cache2.handle.close()

@@ -19,10 +19,14 @@ pytestmark = pytest.mark.gpu
 RTOL = 1e-5
 
 
-def make_data(seed, N, F, nbins, loss="mse", weights=False, signal=True):
+def n_outputs(loss, K=None):
+    return 2 if loss == "gaussian_mle" else ((K or 3) if loss == "mlogloss" else 1)
+
+
+def make_data(seed, N, F, nbins, loss="mse", weights=False, signal=True, K=None):
     rng = np.random.default_rng(seed)
     x_bin = rng.integers(1, nbins + 1, size=(F, N), dtype=np.uint8)
-    K = 2 if loss == "gaussian_mle" else 1
+    K = n_outputs(loss, K)
     y = rng.random(N).astype(np.float32)
     if signal:
         y = (y + 0.5 * (x_bin[0] / nbins) + 0.25 * (x_bin[F // 2] > nbins // 3)).astype(np.float32)
@@ -32,19 +36,23 @@ def make_data(seed, N, F, nbins, loss="mse", weights=False, signal=True):
         y = np.floor(y * 3).astype(np.float32)  # counts, zeros included
     elif loss in ("gamma", "tweedie"):
         y = (y + 0.1).astype(np.float32)  # strictly positive
+    elif loss == "mlogloss":
+        y = (np.minimum(np.floor(y / y.max() * K), K - 1) + 1).astype(np.float32)  # 1-based class, tied to the features
     w = (rng.random(N).astype(np.float32) + 0.5) if weights else None
     mu = (rng.standard_normal(K) * 0.1).astype(np.float32)
+    if loss == "mlogloss":
+        mu = mu - mu.max()  # as _init_target leaves it (src/init.jl:63-64): predict! of the bias tree then changes nothing
     return x_bin, y, w, mu
 
 
 def setup_pair(evt, loss, x_bin, y, w, mu, nbins, depth, tree_type="binary", feattypes=None, mono=None, **pk):
     F, N = x_bin.shape
-    K = 2 if loss == "gaussian_mle" else 1
+    K = mu.shape[0]
     h = evt.Handle(N, F, nbins, K, depth, loss, tree_type)
     h.set_xbin(x_bin)
     h.set_feature_meta(feattypes, mono)
     h.set_target(y, w, mu)
-    op = orc.make_params(loss, nbins=nbins, max_depth=depth, tree_type=tree_type, **pk)
+    op = orc.make_params(loss, nbins=nbins, max_depth=depth, tree_type=tree_type, K=K, **pk)
     o = orc.Oracle(op, x_bin, feattypes, mono)
     gp = evt.make_params(eta=op.eta, L2=op.L2, lambda_=op.lambda_, gamma=op.gamma, min_weight=op.min_weight,
                          bagging_size=op.bagging_size, update_pred=True)
@@ -74,7 +82,8 @@ def assert_tree_close(t_gpu, t_ref, pred_atol=1e-9):
 
 # --------------------------------------------------------------------------- gradients
 @pytest.mark.parametrize("loss,weights", [("mse", False), ("mse", True), ("logloss", True), ("gaussian_mle", False),
-                                          ("gaussian_mle", True), ("poisson", True), ("gamma", False), ("tweedie", True)])
+                                          ("gaussian_mle", True), ("poisson", True), ("gamma", False), ("tweedie", True),
+                                          ("mlogloss", False), ("mlogloss", True)])
 def test_gradient_kernel(evt, loss, weights):
     N, F, B = 70001, 5, 16
     x_bin, y, w, mu = make_data(1, N, F, B, loss, weights)
@@ -117,13 +126,19 @@ CASES = [
     ("poisson", True, 30000, 12, 32, 6, "binary", 9, 0.8, {}),
     ("gamma", False, 30000, 20, 64, 6, "binary", 20, 1.0, dict(lambda_=0.2)),
     ("tweedie", False, 30000, 12, 32, 5, "oblivious", 12, 1.0, {}),
+    ("mlogloss", False, 30000, 12, 32, 5, "binary", 12, 1.0, {}),
+    ("mlogloss", True, 20000, 100, 16, 5, "binary", 60, 0.7, dict(lambda_=0.1)),
+    ("mlogloss", False, 20000, 100, 16, 4, "binary", 100, 1.0, dict(K=2)),
+    ("mlogloss", False, 20000, 10, 32, 4, "oblivious", 10, 1.0, dict(K=5)),
+    ("mlogloss", True, 12000, 9, 128, 4, "binary", 9, 1.0, dict(K=16, min_weight=2.0)),
 ]
 
 
 @pytest.mark.parametrize("loss,weights,N,F,B,D,tt,n_js,rowsample,pk", CASES)
 def test_grow_tree_matches_oracle(evt, loss, weights, N, F, B, D, tt, n_js, rowsample, pk):
     print("case", loss, weights, N, F, B, D, tt, n_js, rowsample, pk, flush=True)
-    x_bin, y, w, mu = make_data(7, N, F, B, loss, weights)
+    pk = dict(pk)
+    x_bin, y, w, mu = make_data(7, N, F, B, loss, weights, K=pk.pop("K", None))
     h, o, op, gp, pred0, grad0 = setup_pair(evt, loss, x_bin, y, w, mu, B, D, tt, **pk)
     rng = np.random.default_rng(99)
     grad = grad0.copy()
@@ -286,7 +301,7 @@ def test_free_running_rounds_bit_exact_mse(evt, loss, tt, rowsample, colsample):
     o.close()
 
 
-@pytest.mark.parametrize("loss", ["logloss", "gaussian_mle", "poisson", "gamma", "tweedie"])
+@pytest.mark.parametrize("loss", ["logloss", "gaussian_mle", "poisson", "gamma", "tweedie", "mlogloss"])
 def test_free_running_rounds_tolerance(evt, loss):
     # device exp/log1p differ from the host's by an ulp: structure must still agree with the
     # reference arithmetic and predictions stay within 1e-5 over several rounds.
@@ -315,8 +330,8 @@ def test_free_running_rounds_tolerance(evt, loss):
 # --------------------------------------------------------------------------- inference
 def test_model_predict_and_leaf_idx(evt):
     N, F, B, D, R = 20000, 8, 32, 5, 6
-    for loss in ("mse", "logloss", "gaussian_mle", "poisson"):
-        x_bin, y, w, mu = make_data(31, N, F, B, loss, False)
+    for loss, Kc in (("mse", None), ("logloss", None), ("gaussian_mle", None), ("poisson", None), ("mlogloss", 3), ("mlogloss", 7)):
+        x_bin, y, w, mu = make_data(31, N, F, B, loss, False, K=Kc)
         pk = dict(min_weight=8.0) if loss == "gaussian_mle" else {}
         h, o, op, gp, pred0, grad0 = setup_pair(evt, loss, x_bin, y, w, mu, B, D, **pk)
         js = np.arange(1, F + 1, dtype=np.uint32)

@@ -16,11 +16,13 @@ from oracle import oracle as orc
 def make_data(seed, N, F, nbins, loss="mse", weights=False):
     rng = np.random.default_rng(seed)
     x_bin = rng.integers(1, nbins + 1, size=(F, N), dtype=np.uint8)
-    K = 2 if loss == "gaussian_mle" else 1
+    K = 2 if loss == "gaussian_mle" else (3 if loss == "mlogloss" else 1)
     NK = 2 * K + 1
     y = rng.random(N).astype(np.float32)
     if loss == "logloss":
         y = (y > 0.5).astype(np.float32)
+    elif loss == "mlogloss":
+        y = (np.floor(y * K) + 1).astype(np.float32)  # 1-based class
     pred = (rng.standard_normal((N, K)) * 0.3).astype(np.float32)
     grad = np.zeros((N, NK), np.float32)
     grad[:, NK - 1] = (rng.random(N).astype(np.float32) + 0.5) if weights else 1.0
@@ -167,11 +169,13 @@ def test_hist_against_dense_bruteforce_and_invariants(loss, weights):
     ("logloss", True, 0.3, 0.0, 1.0),
     ("gaussian_mle", False, 0.0, 0.0, 8.0),
     ("gaussian_mle", True, 0.2, 0.05, 4.0),
+    ("mlogloss", False, 0.0, 0.0, 1.0),
+    ("mlogloss", True, 0.4, 0.02, 2.0),
 ])
 def test_tree_against_bruteforce(loss, weights, lam, gamma, minw):
     N, F, B, D = 900, 6, 16, 5
     x_bin, y, pred, grad = make_data(20, N, F, B, loss, weights)
-    p = orc.make_params(loss, nbins=B, max_depth=D, lambda_=lam, gamma=gamma, min_weight=minw, eta=0.3)
+    p = orc.make_params(loss, nbins=B, max_depth=D, lambda_=lam, gamma=gamma, min_weight=minw, eta=0.3, K=pred.shape[1])
     orc.update_grads(p, pred, y, grad)
     rng = np.random.default_rng(21)
     rows = np.sort(rng.choice(N, 640, replace=False)).astype(np.uint32)
@@ -526,3 +530,56 @@ def test_exp_link_predict_and_apply_link():
     out = small.copy()
     orc.apply_link(orc.LOSS_IDS["gamma"], 1, out)
     np.testing.assert_allclose(out, np.exp(small.astype(np.float64)), rtol=2e-7)
+
+
+# ---------------------------------------------------------------- multi-class log loss
+def _softmax64(p):
+    e = np.exp(p.astype(np.float64) - p.astype(np.float64).max(axis=1, keepdims=True))
+    return e / e.sum(axis=1, keepdims=True)
+
+
+def test_mlogloss_grads_metric_and_link():
+    from scipy.special import softmax
+    from sklearn.metrics import log_loss
+    rng = np.random.default_rng(40)
+    N, K = 700, 4
+    pred = rng.standard_normal((N, K)).astype(np.float32)
+    y = rng.integers(1, K + 1, N).astype(np.float32)
+    grad = np.zeros((N, 2 * K + 1), np.float32)
+    grad[:, 2 * K] = rng.random(N).astype(np.float32) + 0.5
+    w = grad[:, 2 * K].astype(np.float64)
+    p = orc.make_params("mlogloss", K=K)
+    orc.update_grads(p, pred, y, grad)
+    P = _softmax64(pred)
+    onehot = np.eye(K)[y.astype(int) - 1]
+    np.testing.assert_allclose(grad[:, :K], (P - onehot) * w[:, None], rtol=0, atol=3e-7)   # softmax - onehot
+    np.testing.assert_allclose(grad[:, K:2 * K], P * (1 - P) * w[:, None], rtol=3e-6, atol=1e-9)
+    assert np.array_equal(grad[:, 2 * K], w.astype(np.float32))
+    # the metric is the weighted mean of -log softmax[y]; its derivative in every raw score is the gradient row
+    m = orc.eval_metric("mlogloss", K, pred, y, grad[:, 2 * K])
+    np.testing.assert_allclose(m, log_loss(y, P, sample_weight=w, labels=np.arange(1, K + 1)), rtol=2e-6)
+    i, k, e = 5, 2, 1e-2
+    pp, pm = pred.copy(), pred.copy()
+    pp[i, k] += e
+    pm[i, k] -= e
+    wsum = w.sum()
+    fd = (orc.eval_metric("mlogloss", K, pp, y, grad[:, 2 * K]) - orc.eval_metric("mlogloss", K, pm, y, grad[:, 2 * K])) / (2 * e) * wsum
+    np.testing.assert_allclose(fd, grad[i, k], rtol=2e-3, atol=2e-4)
+    # link: softmax of the raw scores
+    out = pred.copy()
+    orc.apply_link(orc.LOSS_IDS["mlogloss"], K, out)
+    np.testing.assert_allclose(out, softmax(pred.astype(np.float64), axis=1), rtol=2e-6)
+
+
+def test_mlogloss_predict_shifts_by_row_max_and_floors():
+    # src/predict.jl:48-62: after adding the leaf, each row is shifted so that its maximum is 0 and floored at -15
+    x_bin = np.array([[1, 2, 3]], np.uint8)
+    t = orc.Tree(3, 3)
+    t.feat[0], t.cond_bin[0], t.split[0] = 1, 1, 1
+    t.pred[1] = [1.0, 2.0, 4.0]
+    t.pred[2] = [0.0, -30.0, 3.0]
+    pred = np.float32([[0.5, 0.5, 0.5], [1.0, 0.0, 0.0], [0.0, 0.0, -1.0]])
+    orc.predict_tree(orc.LOSS_IDS["mlogloss"], 3, x_bin, np.ones(1, np.uint8), t, pred)
+    assert np.array_equal(pred[0], np.float32([-3.0, -2.0, 0.0]))
+    assert np.array_equal(pred[1], np.float32([-2.0, -15.0, 0.0]))
+    assert np.array_equal(pred[2], np.float32([-2.0, -15.0, 0.0]))
