@@ -151,30 +151,15 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     __shared__ double s_wg[4];
     __shared__ int s_wjp[4], s_wbin[4];
 
-    node_totals<NAG>(A, n, hn, blockIdx.y == 0, s_Sq, s_S, s_sc);
-    double S[EVT_MAX_NK];
-    for (int k = 0; k < NK; k++) S[k] = s_S[k];
-
-    double gain_p = 0.0;
-    for (int k = 0; k < K; k++) gain_p += term_gh(S[k], S[K + k], S[2 * K], A.lambda, A.L2);
-    const double w_p = S[NK - 1];
-
-    double wbest = -INFINITY;
-    int wjp = NO_BIN, wbin = NO_BIN;
-    const int nodeidx = blockIdx.x;
-
+    // the histogram slices are requested before the node totals are read and reduced: neither depends on the other,
+    // and the block would otherwise sit through two round trips to memory one after the other
     const int jp = blockIdx.y * nwaves + wave;
+    long long pre[NAG][BPL];
+    long long excl[NAG];
     if (jp < A.nfs) {
-        const int f = (int)A.js[jp] - 1;
-        const bool numeric = A.feattypes[f] != 0;
-        const int constraint = A.mono[f];
-        const int bmax = numeric ? B - 1 : B;
-        long long pre[NAG][BPL];
-        long long excl[NAG];
 #pragma unroll
         for (int ag = 0; ag < NAG; ag++) {
             const int64_t o = ((int64_t)jp * NAG + ag) * B;
-            long long run = 0;
 #pragma unroll
             for (int t = 0; t < BPL; t++) {
                 const int b = lane * BPL + t;
@@ -187,7 +172,35 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
                         v = hn[o + b];
                     }
                 }
-                run += v;
+                pre[ag][t] = v;
+            }
+        }
+    }
+
+    node_totals<NAG>(A, n, hn, blockIdx.y == 0, s_Sq, s_S, s_sc);
+    double S[EVT_MAX_NK];
+    for (int k = 0; k < NK; k++) S[k] = s_S[k];
+
+    double gain_p = 0.0;
+    for (int k = 0; k < K; k++) gain_p += term_gh(S[k], S[K + k], S[2 * K], A.lambda, A.L2);
+    const double w_p = S[NK - 1];
+
+    double wbest = -INFINITY;
+    int wjp = NO_BIN, wbin = NO_BIN;
+    const int nodeidx = blockIdx.x;
+
+    if (jp < A.nfs) {
+        const int f = (int)A.js[jp] - 1;
+        const bool numeric = A.feattypes[f] != 0;
+        const int constraint = A.mono[f];
+        const int bmax = numeric ? B - 1 : B;
+        // inclusive prefix over the bins: within the lane, then across the wavefront
+#pragma unroll
+        for (int ag = 0; ag < NAG; ag++) {
+            long long run = 0;
+#pragma unroll
+            for (int t = 0; t < BPL; t++) {
+                run += pre[ag][t];
                 pre[ag][t] = run;
             }
             const long long incl = wave_incl_scan_i64(run);
