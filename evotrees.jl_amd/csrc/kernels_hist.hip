@@ -397,41 +397,69 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         const int nsg = NS >> 3;
         const int nitems = NA * 8 * nchunks * nsg * 64;
         const int rot = (int)(((int64_t)blockIdx.x * 1031) % (nitems >> 6)) << 6;
-        for (int k0 = tid; k0 < nitems; k0 += nthr) {
-            int k = k0 + rot;
-            if (k >= nitems) k -= nitems;
-            const int bl = k & 7, sl = (k >> 3) & 7;
-            int rest = k >> 6;
-            const int chunk = rest % nchunks; rest /= nchunks;
-            const int sg = rest % nsg; rest /= nsg;
-            const int t = rest & 7;
-            const int a = rest >> 3;
-            const int b = chunk * 8 + bl;
-            const int sidx = sg * 8 + sl;
-            const int f = sidx * 8 + t;
-            if (b >= B) continue;
-            unsigned long long *hw = &H[(size_t)a * plane + ((size_t)t * B + b) * NS + sidx];
-            const unsigned long long w = *hw;
-            if (w == 0ull) continue;
-            *hw = 0ull;
-            if (f >= A.F) continue; // a padding byte's word
-            const int slot = A.jsmap[f];
-            if (slot == 0xFFFF) continue;
-            unsigned long long *base = reinterpret_cast<unsigned long long *>(hn) + ((int64_t)slot * A.NAg) * B + b;
-            if (PACK && a == 0) {
-                const long long gsum = (long long)w >> EVT_PACK_CNT_BITS;
-                const unsigned long long cnt = w & ((1ull << EVT_PACK_CNT_BITS) - 1ull);
-                if (sole) {
-                    base[0] = (unsigned long long)gsum;
-                    base[(int64_t)(A.NAg - 1) * B] = cnt;
-                } else {
-                    if (gsum != 0) atomicAdd(base, (unsigned long long)gsum);
-                    atomicAdd(base + (int64_t)(A.NAg - 1) * B, cnt);
+        // FU items per thread at a time: their LDS words (and, when features are sampled, their slots) are all
+        // requested before the first is used, so a flush costs one LDS and one memory round trip, not FU of each
+        constexpr int FU = 8;
+        const bool pow2 = (nchunks == 8) && (nsg == 2); // nbins in 57..64 with 128-byte records: decode with shifts
+        for (int k0 = tid; k0 < nitems; k0 += FU * nthr) {
+            unsigned long long wv[FU];
+            unsigned long long *hwv[FU];
+            int av[FU], bv[FU], slotv[FU];
+#pragma unroll
+            for (int j = 0; j < FU; j++) {
+                int k = k0 + j * nthr;
+                wv[j] = 0ull;
+                hwv[j] = H;
+                av[j] = 0; bv[j] = 0; slotv[j] = 0xFFFF;
+                if (k < nitems) {
+                    k += rot;
+                    if (k >= nitems) k -= nitems;
+                    const int bl = k & 7, sl = (k >> 3) & 7;
+                    int rest = k >> 6;
+                    int chunk, sg;
+                    if (pow2) {
+                        chunk = rest & 7; rest >>= 3;
+                        sg = rest & 1; rest >>= 1;
+                    } else {
+                        chunk = rest % nchunks; rest /= nchunks;
+                        sg = rest % nsg; rest /= nsg;
+                    }
+                    const int t = rest & 7;
+                    const int a = rest >> 3;
+                    const int b = chunk * 8 + bl;
+                    const int sidx = sg * 8 + sl;
+                    const int f = sidx * 8 + t;
+                    if (b < B) {
+                        hwv[j] = &H[(size_t)a * plane + ((size_t)t * B + b) * NS + sidx];
+                        wv[j] = *hwv[j];
+                        av[j] = a; bv[j] = b;
+                        if (f < A.F) slotv[j] = FULL ? f : (int)A.jsmap[f]; // a padding byte's word has no slot
+                    }
                 }
-            } else if (sole) {
-                base[(int64_t)(A.a0 + a) * B] = w;
-            } else {
-                atomicAdd(base + (int64_t)(A.a0 + a) * B, w);
+            }
+#pragma unroll
+            for (int j = 0; j < FU; j++) {
+                const unsigned long long w = wv[j];
+                if (w == 0ull) continue;
+                *hwv[j] = 0ull;
+                const int slot = slotv[j], a = av[j], b = bv[j];
+                if (slot == 0xFFFF) continue;
+                unsigned long long *base = reinterpret_cast<unsigned long long *>(hn) + ((int64_t)slot * A.NAg) * B + b;
+                if (PACK && a == 0) {
+                    const long long gsum = (long long)w >> EVT_PACK_CNT_BITS;
+                    const unsigned long long cnt = w & ((1ull << EVT_PACK_CNT_BITS) - 1ull);
+                    if (sole) {
+                        base[0] = (unsigned long long)gsum;
+                        base[(int64_t)(A.NAg - 1) * B] = cnt;
+                    } else {
+                        if (gsum != 0) atomicAdd(base, (unsigned long long)gsum);
+                        atomicAdd(base + (int64_t)(A.NAg - 1) * B, cnt);
+                    }
+                } else if (sole) {
+                    base[(int64_t)(A.a0 + a) * B] = w;
+                } else {
+                    atomicAdd(base + (int64_t)(A.a0 + a) * B, w);
+                }
             }
         }
         __syncthreads();
