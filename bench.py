@@ -247,6 +247,23 @@ def main():
     except Exception:  # measurement aid only
         out["copy_kernel_GBps"] = None
 
+    # predict!(pred, tree, x_bin) on the resident matrix (the eval CallBack's per-round work): 10 trees, HIP events
+    try:
+        h.set_profiling(["predict"])
+        h.reset_profile()
+        for _ in range(10):
+            h.predict_tree(tree)
+        h.synchronize()
+        pp = h.get_profile()["predict"]
+        h.set_profiling(False)
+        ms_tree = pp["ms"] / max(pp["launches"], 1)
+        depth_bytes = max(D - 1, 0)  # one bin byte per level walked
+        out["predict_tree"] = {"ms_per_tree": round(ms_tree, 4), "rows_per_s": round(N / (ms_tree * 1e-3), 1),
+                               "algorithmic_GBps": round(N * (8 * K + depth_bytes) / (ms_tree * 1e-3) / 1e9, 1),
+                               "bytes_per_row": 8 * K + depth_bytes}
+    except Exception as e:  # measurement aid only
+        out["predict_tree"] = {"error": str(e)}
+
     if args.predict:
         m_trees = []
         # a model of `steps` copies of the last tree has the same traversal cost as a trained one of that size
