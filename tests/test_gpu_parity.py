@@ -365,6 +365,40 @@ def test_model_predict_and_leaf_idx(evt):
         o.close()
 
 
+def _random_tree(rng, depth, F, B, K):
+    nn = (1 << depth) - 1
+    t = orc.Tree(K, nn)
+    for n in range(1, 1 << (depth - 1)):
+        if n == 1 or (t.split[(n >> 1) - 1] and rng.random() < 0.8):
+            t.feat[n - 1] = rng.integers(1, F + 1)
+            t.cond_bin[n - 1] = rng.integers(1, B)
+            t.split[n - 1] = 1
+    t.pred[:] = (rng.standard_normal((nn, K)) * 0.3).astype(np.float32)
+    return t
+
+
+@pytest.mark.parametrize("N,F,B,depths,K,loss", [
+    (3001, 700, 16, [3, 5, 1, 4], 1, "mse"),          # wide matrix
+    (70000, 9, 64, [15, 3, 15], 1, "logloss"),        # large trees, trees of different sizes in one model
+    (5000, 40, 255, [6, 6, 2], 6, "mlogloss"),        # many outputs
+    (1025, 3, 4, [2, 12], 2, "gaussian_mle"),         # odd row count
+    (64 * 512, 100, 64, [11] * 5, 1, "mse"),          # the benchmark's shape
+])
+def test_model_predict_random_trees(evt, N, F, B, depths, K, loss):
+    rng = np.random.default_rng(77)
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    ft = (rng.random(F) > 0.2).astype(np.uint8)
+    trees = [_random_tree(rng, d, F, B, K) for d in depths]
+    want = np.zeros((N, K), np.float32)
+    for t in trees:
+        orc.predict_tree(orc.LOSS_IDS[loss], K, x_bin, ft, t, want)
+    raw = evt._lib.predict_model(x_bin, ft, loss, K, trees, apply_link=False)
+    assert np.array_equal(raw.view(np.uint32), want.view(np.uint32))
+    linked = evt._lib.predict_model(x_bin, ft, loss, K, trees, apply_link=True)
+    orc.apply_link(orc.LOSS_IDS[loss], K, want)
+    np.testing.assert_allclose(linked, want, rtol=RTOL, atol=1e-7)
+
+
 def test_predict_tree_on_cache_and_clamps(evt):
     x_bin = np.array([[1, 2, 2]], np.uint8)
     t = orc.Tree(1, 3)
