@@ -235,6 +235,9 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
 // ((a*8 + t)*B + bin)*NS + sub for feature f = 8*sub + t, i.e. `sub` selects the bank pair, so the 16
 // lanes of a group always fall on 16 different bank pairs whatever their bins are.  Rows that share a
 // wave instruction sit in different groups and cannot collide inside one LDS pass either.
+// FULL: a lane adds all 8 bytes of its piece without testing which features are sampled.  A record's padding reads as
+// bin 1 and features outside the sample have LDS words of their own, so the extra adds land in words the flush clears
+// and never writes out; the per-feature test (FULL = false) only pays when most features are left out.
 template <int NA, bool PACK, int U, bool FULL>
 __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     extern __shared__ unsigned long long H[]; // [NA][8][B][NS]
@@ -400,6 +403,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         // FU items per thread at a time: their LDS words (and, when features are sampled, their slots) are all
         // requested before the first is used, so a flush costs one LDS and one memory round trip, not FU of each
         constexpr int FU = 8;
+        const bool all_feats = A.nfs == A.F; // slot of feature f is f itself
         const bool pow2 = (nchunks == 8) && (nsg == 2); // nbins in 57..64 with 128-byte records: decode with shifts
         for (int k0 = tid; k0 < nitems; k0 += FU * nthr) {
             unsigned long long wv[FU];
@@ -433,7 +437,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                         hwv[j] = &H[(size_t)a * plane + ((size_t)t * B + b) * NS + sidx];
                         wv[j] = *hwv[j];
                         av[j] = a; bv[j] = b;
-                        if (f < A.F) slotv[j] = FULL ? f : (int)A.jsmap[f]; // a padding byte's word has no slot
+                        if (f < A.F) slotv[j] = all_feats ? f : (int)A.jsmap[f]; // a padding byte's word has no slot
                     }
                 }
             }
@@ -475,7 +479,9 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
 template <int NA, bool PACK>
 static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
     constexpr int U = (NA <= 2) ? 16 : 8; // row groups (records) in flight per wave, bounded by registers
-    if (c->n_js_last == c->F)
+    // unpredicated atomics for every feature of the record pay off unless most features are left out: the words of
+    // features outside the sample are simply not flushed
+    if (2 * c->n_js_last >= c->F || c->n_js_last == c->F)
         hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, true>), grid, dim3(threads), lds, c->stream, A);
     else
         hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, false>), grid, dim3(threads), lds, c->stream, A);
