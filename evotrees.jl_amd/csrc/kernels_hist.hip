@@ -238,7 +238,25 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
 // FULL: a lane adds all 8 bytes of its piece without testing which features are sampled.  A record's padding reads as
 // bin 1 and features outside the sample have LDS words of their own, so the extra adds land in words the flush clears
 // and never writes out; the per-feature test (FULL = false) only pays when most features are left out.
-template <int NA, bool PACK, int U, bool FULL>
+// Q = record rows per 16-lane DPP row: 1 for records of 128 bytes and more, 2 for 64-byte records.  (32-byte records
+// were tried with Q = 4 and ran slower than the generic kernel: four broadcasts and three selects per value.)
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_row_bcast(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xF, 0xF, false);
+}
+// value held by the fetcher lane of (group u, this lane's record row) inside this lane's DPP row
+template <int Q, int u>
+__device__ __forceinline__ uint32_t grp_bcast(uint32_t x, int hh) {
+    if constexpr (Q == 1) {
+        return dpp_row_bcast<0x150 + u>(x);
+    } else {
+        static_assert(Q == 2, "records of 64 bytes and more");
+        const uint32_t a = dpp_row_bcast<0x150 + 2 * u>(x), b = dpp_row_bcast<0x150 + 2 * u + 1>(x);
+        return hh ? b : a;
+    }
+}
+
+template <int NA, bool PACK, int U, bool FULL, int Q>
 __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     extern __shared__ unsigned long long H[]; // [NA][8][B][NS]
     const int tid = threadIdx.x, nthr = blockDim.x;
@@ -320,9 +338,12 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             const uint32_t *isp = A.is + seg;
             const int64_t lastp = nend - 1;          // >= start
             int64_t pw = start + (int64_t)wave * SR; // first position of this wave's iteration
-            const int myu = lane & 15;
-            const int mypos = myu * RPW + rloc;      // position (within the iteration) whose id / gradient this lane fetches
+            // lane j of DPP row r fetches for group j / Q the record row r * Q + j % Q of that group
+            const int myu = (lane & 15) / Q;
+            // (a record wider than a DPP row, Q == 1, is fetched for by every DPP row it covers: its own row rloc)
+            const int mypos = myu * RPW + (Q == 1 ? rloc : (lane >> 4) * Q + (lane & 15) % Q); // position (within the iteration) this lane fetches
             const bool fetcher = myu < U;
+            const int hh = (lane & 15) / NS;         // this lane's record row inside its DPP row (0 when Q == 1)
             uint32_t idc, idn;
             unsigned long long gc[NA], gn[NA];
             uint2 v[U];
@@ -339,7 +360,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             __builtin_amdgcn_sched_barrier(0);
 #define EVT_H16_PRO(u_)                                                                                               \
     if constexpr ((u_) < U) {                                                                                         \
-        const uint32_t row = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)idc, 0x150 + (u_), 0xF, 0xF, false);          \
+        const uint32_t row = grp_bcast<Q, (u_) < U ? (u_) : 0>(idc, hh);                                               \
         v[(u_) < U ? (u_) : 0] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)row * A.RS + sub * 8);                 \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
@@ -362,8 +383,8 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         {                                                                                                             \
             unsigned long long gg[NA];                                                                                \
             _Pragma("unroll") for (int a = 0; a < NA; a++) {                                                          \
-                const uint32_t glo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)gc[a], 0x150 + (u_), 0xF, 0xF, false); \
-                const uint32_t ghi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(gc[a] >> 32), 0x150 + (u_), 0xF, 0xF, false); \
+                const uint32_t glo = grp_bcast<Q, ui>((uint32_t)gc[a], hh);                                            \
+                const uint32_t ghi = grp_bcast<Q, ui>((uint32_t)(gc[a] >> 32), hh);                                    \
                 gg[a] = ((unsigned long long)ghi << 32) | glo;                                                         \
             }                                                                                                         \
             if (lane_on && (pw + (u_) * RPW + rloc < nend)) {                                                          \
@@ -377,7 +398,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                 }                                                                                                     \
             }                                                                                                         \
         }                                                                                                             \
-        const uint32_t row = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)idn, 0x150 + (u_), 0xF, 0xF, false);          \
+        const uint32_t row = grp_bcast<Q, ui>(idn, hh);                                                                \
         v[ui] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)row * A.RS + sub * 8);                                \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
@@ -391,20 +412,20 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             }
         }
         __syncthreads();
-        // flush: a wave covers 8 consecutive bins x 8 consecutive pieces `sub` of one (channel, t): global
-        // accesses are whole 64-byte runs of one feature's bins, LDS reads spread over 8 bank pairs.  Blocks
-        // start at different items so that concurrent flushes of one node do not queue on the same addresses.
+        // flush: a wave covers 8 consecutive bins of 8 pieces `sub` (or of all NS pieces and 8 / NS bin chunks) of one
+        // (channel, t): global accesses are whole 64-byte runs of one feature's bins, LDS reads spread over the bank
+        // pairs.  Blocks start at different items so that concurrent flushes of one node do not queue on the same addresses.
         const bool sole = (nbeg >= blk_start) && (nrows_end <= blk_end) && !(PACK && nrows_end - nbeg > EVT_HIST_MAX_ROWS_PER_BLOCK);
         long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
         const int nchunks = (B + 7) >> 3;
-        const int nsg = NS >> 3;
-        const int nitems = NA * 8 * nchunks * nsg * 64;
+        const int nitems = NA * 8 * nchunks * NS * 8; // (channel, t, bin chunk, piece, bin in chunk), the last fastest
         const int rot = (int)(((int64_t)blockIdx.x * 1031) % (nitems >> 6)) << 6;
         // FU items per thread at a time: their LDS words (and, when features are sampled, their slots) are all
         // requested before the first is used, so a flush costs one LDS and one memory round trip, not FU of each
         constexpr int FU = 8;
         const bool all_feats = A.nfs == A.F; // slot of feature f is f itself
-        const bool pow2 = (nchunks == 8) && (nsg == 2); // nbins in 57..64 with 128-byte records: decode with shifts
+        const bool pow2 = (nchunks & (nchunks - 1)) == 0; // decode with shifts
+        const int ns_sh = __ffs(NS) - 1, nc_sh = __ffs(nchunks) - 1;
         for (int k0 = tid; k0 < nitems; k0 += FU * nthr) {
             unsigned long long wv[FU];
             unsigned long long *hwv[FU];
@@ -418,20 +439,21 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                 if (k < nitems) {
                     k += rot;
                     if (k >= nitems) k -= nitems;
-                    const int bl = k & 7, sl = (k >> 3) & 7;
-                    int rest = k >> 6;
-                    int chunk, sg;
+                    const int bl = k & 7;
+                    int rest = k >> 3;
+                    const int sidx = rest & (NS - 1);
+                    rest >>= ns_sh;
+                    int chunk;
                     if (pow2) {
-                        chunk = rest & 7; rest >>= 3;
-                        sg = rest & 1; rest >>= 1;
+                        chunk = rest & (nchunks - 1);
+                        rest >>= nc_sh;
                     } else {
-                        chunk = rest % nchunks; rest /= nchunks;
-                        sg = rest % nsg; rest /= nsg;
+                        chunk = rest % nchunks;
+                        rest /= nchunks;
                     }
                     const int t = rest & 7;
                     const int a = rest >> 3;
                     const int b = chunk * 8 + bl;
-                    const int sidx = sg * 8 + sl;
                     const int f = sidx * 8 + t;
                     if (b < B) {
                         hwv[j] = &H[(size_t)a * plane + ((size_t)t * B + b) * NS + sidx];
@@ -476,17 +498,32 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     }
 }
 
-template <int NA, bool PACK>
-static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
-    constexpr int U = (NA <= 2) ? 16 : 8; // row groups (records) in flight per wave, bounded by registers
+template <int NA, bool PACK, int U, int Q>
+static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
     // unpredicated atomics for every feature of the record pay off unless most features are left out: the words of
     // features outside the sample are simply not flushed
-    if (2 * c->n_js_last >= c->F || c->n_js_last == c->F)
-        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, true>), grid, dim3(threads), lds, c->stream, A);
+    const bool full = 2 * c->n_js_last >= c->F;
+    if (lds > 64 * 1024) { // one block per CU may take most of its 160 KB
+        static bool attr_set = false;
+        if (!attr_set) {
+            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, true, Q>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, false, Q>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            attr_set = true;
+        }
+    }
+    if (full)
+        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, true, Q>), grid, dim3(threads), lds, c->stream, A);
     else
-        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, false>), grid, dim3(threads), lds, c->stream, A);
+        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, false, Q>), grid, dim3(threads), lds, c->stream, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
+}
+
+template <int NA, bool PACK>
+static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
+    // row groups (records) in flight per wave: as many as a DPP row can address, fewer when registers run out
+    if (c->RS >= 128) return launch_hist16_q<NA, PACK, (NA <= 2) ? 16 : 8, 1>(c, A, grid, threads, lds);
+    return launch_hist16_q<NA, PACK, 8, 2>(c, A, grid, threads, lds); // 64-byte records
 }
 
 template <int NA, bool PACK>
@@ -547,9 +584,10 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
         A.slots_per_tile = slots_per_tile;
         const size_t lds = per_slot * slots_per_tile;
         dim3 grid((unsigned)blocks, (unsigned)ntiles);
-        // conflict-free variant: records of 128, 256 or 512 bytes whose whole LDS histogram fits 64 KB
+        // conflict-free variant: records of 64 to 512 bytes (8 to 64 lanes per row) whose whole LDS histogram fits
         const size_t lds16 = (size_t)na * 8 * c->B * (c->RS / 8) * 8;
-        const bool can16 = (c->RS == 128 || c->RS == 256 || c->RS == 512) && lds16 <= 64 * 1024; // 16, 32 or 64 lanes per row
+        const bool can16 = (c->RS == 64 || c->RS == 128 || c->RS == 256 || c->RS == 512) &&
+                           lds16 <= 128 * 1024;
         const bool use16 = (c->hist_variant == 1) ? false : can16;
         int r = EVT_ERR_ARG;
         if (use16) {
