@@ -131,6 +131,8 @@ CASES = [
     ("mlogloss", False, 20000, 100, 16, 4, "binary", 100, 1.0, dict(K=2)),
     ("mlogloss", False, 20000, 10, 32, 4, "oblivious", 10, 1.0, dict(K=5)),
     ("mlogloss", True, 12000, 9, 128, 4, "binary", 9, 1.0, dict(K=16, min_weight=2.0)),
+    ("mse", False, 60000, 5, 8, 14, "binary", 5, 1.0, dict(min_weight=0.0)),   # deep: most leaves hold a handful of rows
+    ("logloss", True, 3000, 4, 4, 16, "binary", 4, 0.9, dict(min_weight=0.0)),  # deepest supported tree, far more nodes than rows
 ]
 
 
