@@ -223,6 +223,8 @@ def main():
     kernels = {k: {"ms_per_round": round(v["ms"] / nb, 4), "launches_per_round": v["launches"] / nb} for k, v in prof_all.items()}
     if prof_all["grad"]["ms"] > 0:
         gb = N * (4 * K + 4 + 4 + 8 * K)
+        if cfg["rowsample"] >= 1.0:
+            gb += N * (4 + 4 * K)  # the last tree's leaf values are added in the same pass: node id read, prediction written
         kernels["grad"]["GBps"] = round(gb * nb / (prof_all["grad"]["ms"] * 1e-3) / 1e9, 1)
 
     out = {

@@ -121,7 +121,7 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->obest, c->sbest};
+                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->obest, c->sbest, c->pend_leaf};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -192,6 +192,10 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->hist_seg_cost = 2048;
     c->record_nidx = false;
     c->nidx_valid = false;
+    c->defer_pred = true;
+    c->write_nidx = false;
+    c->pend_pred = false;
+    c->pend_leaf = nullptr;
     c->last_cond = 255;
     c->profiling = 0;
     c->prof_open = false;
@@ -222,6 +226,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->is_a, N);
     ALLOC(c->is_b, N);
     ALLOC(c->nidx, N);
+    ALLOC(c->pend_leaf, (size_t)c->nnodes * K);
     ALLOC(c->mask, N);
     ALLOC(c->flagw, (size_t)c->max_chunks * EVT_CHUNK_WORDS);
     ALLOC(c->chunk_nleft, c->max_chunks + 1);
@@ -406,6 +411,7 @@ extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, cons
     ARGCHK(y && mu, "y and mu must not be NULL");
     c->have_target = false;
     c->have_grads = false;
+    c->pend_pred = false; // the predictions start again from mu
     c->unit_w = (w == nullptr);
     set_channels(c);
     HIPCHK(hipMemcpyAsync(c->y, y, sizeof(float) * c->N, hipMemcpyDefault, c->stream));
@@ -548,8 +554,16 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
         c->js_last = jsv;
     }
 
+    // With every row in the tree the leaf of each row is recorded while growing and its value is added later, in row
+    // order (fused into the next gradient pass): a scattered 4-byte write per row instead of a scattered read-modify-write.
+    const bool defer = p->update_pred && all_rows && c->defer_pred;
+    const bool fuse_pred = p->update_pred && all_rows && !defer;
+    c->write_nidx = c->record_nidx || defer;
+
     int r;
     prof_begin(c, EVT_K_OTHER, 0);
+    r = launch_apply_pending(c); // an earlier tree's values go in before its node ids are overwritten
+    if (r != EVT_OK) return r;
     if (all_rows) {
         r = launch_iota(c, c->is_a, c->N);
     } else {
@@ -561,7 +575,6 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     prof_end(c);
     if (r != EVT_OK) return r;
 
-    const bool fuse_pred = p->update_pred && all_rows;
     const bool obliv = (c->tree_type == EVT_TREE_OBLIVIOUS);
     uint32_t *is_cur = c->is_a, *is_next = c->is_b;
     // levels 1 .. D-1 split; the last of them sends its rows straight to the leaves of level D
@@ -601,7 +614,11 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
         if (r != EVT_OK) return r;
         if (c->profiling) c->prof_units[EVT_K_PREDICT] += c->N;
     }
-    if (c->profiling) {
+    if (defer) {
+        HIPCHK(hipMemcpyAsync(c->pend_leaf, c->tree_blob + c->blob_pred, sizeof(float) * (size_t)c->nnodes * c->K, hipMemcpyDeviceToDevice,
+                              c->stream));
+        c->pend_pred = true;
+        c->nidx_valid = true;
     }
 
     // read back the tree (and the per-level row counts) in one pinned transfer
@@ -658,6 +675,8 @@ extern "C" int evt_predict_tree(evt_handle c, int32_t nnodes_tree, const int64_t
     std::vector<uint32_t> nodes;
     int r = pack_tree(nnodes_tree, feat, cond_bin, split, c->F, nodes);
     if (r != EVT_OK) return r;
+    r = launch_apply_pending(c);
+    if (r != EVT_OK) return r;
     uint32_t *d_nodes = nullptr;
     float *d_pred = nullptr;
     HIPCHK(hipMalloc((void **)&d_nodes, sizeof(uint32_t) * nnodes_tree));
@@ -697,6 +716,10 @@ extern "C" int evt_get_xbin(evt_handle c, uint8_t *out) {
 extern "C" int evt_get_pred(evt_handle c, float *out) {
     CTXCHK(c);
     ARGCHK(out, "out is NULL");
+    {
+        int r = launch_apply_pending(c);
+        if (r != EVT_OK) return r;
+    }
     HIPCHK(hipMemcpyAsync(out, c->pred, sizeof(float) * (size_t)c->N * c->K, hipMemcpyDefault, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     return EVT_OK;
@@ -772,7 +795,8 @@ extern "C" int evt_eval_metric(evt_handle c, int32_t metric, double *value_out) 
         return EVT_ERR_STATE;
     }
     prof_begin(c, EVT_K_OTHER, 0);
-    int r = launch_eval_metric(c, metric, c->metric_partial);
+    int r = launch_apply_pending(c);
+    if (r == EVT_OK) r = launch_eval_metric(c, metric, c->metric_partial);
     prof_end(c);
     if (r != EVT_OK) return r;
     HIPCHK(hipMemcpyAsync(c->h_stage, c->metric_partial + 2 * EVT_METRIC_BLOCKS, sizeof(double), hipMemcpyDeviceToHost, c->stream));
@@ -938,6 +962,8 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
         c->hist_variant = (int)value;
     } else if (strcmp(name, "record_nidx") == 0) {
         c->record_nidx = value != 0;
+    } else if (strcmp(name, "defer_pred") == 0) {
+        c->defer_pred = value != 0;
     } else if (strcmp(name, "hist_threads") == 0) {
         ARGCHK(value == 256 || value == 512 || value == 1024, "hist_threads must be 256, 512 or 1024");
         c->hist_threads = (int)value;

@@ -126,6 +126,10 @@ struct evt_ctx {
     int hist_variant;  // 0 auto, 1 generic 16-byte-piece kernel, 2 conflict-free 8-byte-piece kernel where it applies
     bool record_nidx;  // leaf finalisation also writes the node id of every sampled row
     bool nidx_valid;   // nidx holds the last tree's node ids
+    bool defer_pred;   // a tree grown on every row records leaf ids and leaves the addition to the next row-order pass
+    bool write_nidx;   // the tree being grown records the node id of every row it places
+    bool pend_pred;    // pred lacks the leaf values pend_leaf[nidx[i] - 1] of the last tree
+    float *pend_leaf;  // [K * nnodes] leaf values of the tree whose addition is pending
     uint8_t last_cond;
 
     // profiling
@@ -185,6 +189,7 @@ __device__ __forceinline__ void evt_add_leaf(float *pr, const float *lp, int K, 
 // grad
 int launch_grads(evt_ctx *c);
 int launch_quantize(evt_ctx *c);
+int launch_apply_pending(evt_ctx *c);
 int launch_set_weight_row(evt_ctx *c, const float *w_dev);
 int launch_validate_classes(evt_ctx *c);
 int launch_init_pred(evt_ctx *c, const float *mu_dev, const float *offset_dev);

@@ -2,6 +2,11 @@
 //
 // Streaming work, HBM bound: per row the kernel reads pred (4K B), y (4 B) and the weight
 // (4 B, last row of the gradient matrix) and writes 8K B.
+//
+// A tree grown on every row leaves its leaf values pending: growing recorded the leaf of each row and
+// the addition to the prediction (predict!, src/predict.jl:1-46) happens here, in row order, as the
+// first thing the next gradient pass does (4 B of node id read and 4K B written more per row) - or in
+// k_apply_leaf when something else needs the predictions first.
 #include "evt_internal.h"
 
 __device__ __forceinline__ float wave_max_f32(float v) {
@@ -17,8 +22,9 @@ __device__ __forceinline__ float dev_softplus(float x) { return fmaxf(x, 0.0f) +
 // 4 gamma (:64-67), 5 tweedie with rho = 1.5 (:69-76).
 // grad rows: [g_1..g_K, h_1..h_K, w]; every written value is multiplied by w (src/loss.jl:104-108, :223-233).
 template <int LOSS>
-__global__ __launch_bounds__(256) void k_grads(const float *__restrict__ pred, const float *__restrict__ y,
-                                              float *__restrict__ grad, int64_t N, uint32_t *absmax) {
+__global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const float *__restrict__ y, float *__restrict__ grad, int64_t N,
+                                              uint32_t *absmax, const uint32_t *__restrict__ pend_nidx,
+                                              const float *__restrict__ pend_leaf) {
     constexpr int K = (LOSS == 2) ? 2 : 1;
     constexpr int NK = 2 * K + 1;
     float mx[2 * K];
@@ -28,6 +34,7 @@ __global__ __launch_bounds__(256) void k_grads(const float *__restrict__ pred, c
         float out[2 * K];
         float *g = grad + (size_t)NK * i;
         const float w = g[NK - 1];
+        if (pend_nidx) evt_add_leaf(pred + (size_t)K * i, pend_leaf + (size_t)K * (pend_nidx[i] - 1), K, LOSS);
         if (LOSS == 0) {
             const float gg = 2.0f * (pred[i] - y[i]);
             out[0] = gg * w;
@@ -85,18 +92,20 @@ __global__ __launch_bounds__(256) void k_grads(const float *__restrict__ pred, c
 
 // Multi-class log loss (src/loss.jl:93-98, :113-128): prob_k = exp(p_k) / sum_j exp(p_j); g_k = (prob_k - [y == k]) w,
 // h_k = prob_k (1 - prob_k) w; y holds the 1-based class.  The row maxima are reduced one gradient row at a time.
-__global__ __launch_bounds__(256) void k_grads_mlogloss(const float *__restrict__ pred, const float *__restrict__ y,
-                                                       float *__restrict__ grad, int64_t N, int K, uint32_t *absmax) {
+__global__ __launch_bounds__(256) void k_grads_mlogloss(float *__restrict__ pred, const float *__restrict__ y, float *__restrict__ grad,
+                                                       int64_t N, int K, uint32_t *absmax, const uint32_t *__restrict__ pend_nidx,
+                                                       const float *__restrict__ pend_leaf) {
     const int NK = 2 * K + 1;
     __shared__ float s_m[4];
     float mx[2 * EVT_MAX_K];
 #pragma unroll
     for (int k = 0; k < 2 * EVT_MAX_K; k++) mx[k] = 0.0f;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
-        const float *pr = pred + (size_t)K * i;
+        float *pr = pred + (size_t)K * i;
         float *g = grad + (size_t)NK * i;
         const float w = g[NK - 1];
         const int cls = (int)y[i];
+        if (pend_nidx) evt_add_leaf(pr, pend_leaf + (size_t)K * (pend_nidx[i] - 1), K, EVT_LOSS_MLOGLOSS);
         float e[EVT_MAX_K];
         float isum = 0.0f;
 #pragma unroll
@@ -198,21 +207,40 @@ int launch_grads(evt_ctx *c) {
     int64_t nb = (c->N + 255) / 256;
     if (nb > 2048) nb = 2048;
     dim3 grid((unsigned)nb);
+    const uint32_t *pn = c->pend_pred ? c->nidx : nullptr; // the last tree's leaf values are added on the way
+    c->pend_pred = false;
     if (c->loss == EVT_LOSS_MSE)
-        hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+        hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
     else if (c->loss == EVT_LOSS_LOGLOSS)
-        hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+        hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
     else if (c->loss == EVT_LOSS_GAUSSIAN_MLE)
-        hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+        hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
     else if (c->loss == EVT_LOSS_POISSON)
-        hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+        hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
     else if (c->loss == EVT_LOSS_GAMMA)
-        hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+        hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
     else if (c->loss == EVT_LOSS_MLOGLOSS)
-        hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax);
+        hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->pend_leaf);
     else
-        hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax);
+        hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
     HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
+// Adds the pending leaf values of the last tree to the predictions, row by row.
+__global__ __launch_bounds__(256) void k_apply_leaf(float *__restrict__ pred, const uint32_t *__restrict__ nidx,
+                                                   const float *__restrict__ leaf, int64_t N, int K, int loss) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256)
+        evt_add_leaf(pred + (size_t)K * i, leaf + (size_t)K * (nidx[i] - 1), K, loss);
+}
+
+int launch_apply_pending(evt_ctx *c) {
+    if (!c->pend_pred) return EVT_OK;
+    int64_t nb = (c->N + 255) / 256;
+    if (nb > 4096) nb = 4096;
+    hipLaunchKernelGGL(k_apply_leaf, dim3((unsigned)nb), dim3(256), 0, c->stream, c->pred, c->nidx, c->pend_leaf, c->N, c->K, c->loss);
+    HIPCHK(hipGetLastError());
+    c->pend_pred = false;
     return EVT_OK;
 }
 

@@ -283,20 +283,76 @@ struct NextArgs {
     int64_t seg_cost; // cost units added per build node in the histogram kernel's span space
 };
 
+// Two exclusive prefixes in one pass (same shape as block_excl_scan); s_tmp holds 34 values.
+__device__ void block_excl_scan2(long long va, long long vb, long long *pa, long long *pb, long long *ta, long long *tb, long long *s_tmp) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    long long xa = va, xb = vb;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int al = __shfl_up((int)(xa & 0xffffffffll), o), ah = __shfl_up((int)(xa >> 32), o);
+        const int bl = __shfl_up((int)(xb & 0xffffffffll), o), bh = __shfl_up((int)(xb >> 32), o);
+        if (lane >= o) {
+            xa += ((long long)ah << 32) | (unsigned int)al;
+            xb += ((long long)bh << 32) | (unsigned int)bl;
+        }
+    }
+    __syncthreads(); // s_tmp may still be read from a previous call
+    if (lane == 63) {
+        s_tmp[wave] = xa;
+        s_tmp[17 + wave] = xb;
+    }
+    __syncthreads();
+    if (tid < 2) {
+        long long *t = s_tmp + 17 * tid;
+        long long run = 0;
+        const int nw = blockDim.x >> 6;
+        for (int w = 0; w < nw; w++) { long long x = t[w]; t[w] = run; run += x; }
+        t[16] = run;
+    }
+    __syncthreads();
+    *ta = s_tmp[16];
+    *tb = s_tmp[33];
+    *pa = s_tmp[wave] + xa - va;
+    *pb = s_tmp[17 + wave] + xb - vb;
+}
+
+// One block turns the chunk counts of a level into the next level's tables.  It runs between two grid-wide kernels,
+// so its latency is what counts: loads that do not depend on each other are issued together (fixed-trip loops over
+// clamped indices instead of data-dependent ones) and values are kept in registers between the passes.
 __global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
     const int tid = threadIdx.x;
-    __shared__ long long s_tmp[17];
+    __shared__ long long s_tmp[34];
     const int n_act = (int)A.hdr[LH_N_ACT];
     const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
     long long total;
     // A: exclusive scan of the chunks' left counts
     {
+        constexpr int SP = 8;
         const int64_t span = (n_chunks + 1023) / 1024;
         const int64_t c0 = (int64_t)tid * span, c1 = (c0 + span < n_chunks) ? c0 + span : n_chunks;
-        long long s = 0;
-        for (int64_t c = c0; c < c1; c++) s += A.chunk_nleft[c];
-        long long pre = block_excl_scan(s, &total, s_tmp);
-        for (int64_t c = c0; c < c1; c++) { A.chunk_lpre[c] = pre; pre += A.chunk_nleft[c]; }
+        if (span <= SP) {
+            int v[SP];
+#pragma unroll
+            for (int k = 0; k < SP; k++) {
+                const int64_t c = c0 + k;
+                const int x = A.chunk_nleft[c < c1 ? c : 0];
+                v[k] = c < c1 ? x : 0;
+            }
+            long long s = 0;
+#pragma unroll
+            for (int k = 0; k < SP; k++) s += v[k];
+            long long pre = block_excl_scan(s, &total, s_tmp);
+#pragma unroll
+            for (int k = 0; k < SP; k++) {
+                if (c0 + k < c1) A.chunk_lpre[c0 + k] = pre;
+                pre += v[k];
+            }
+        } else {
+            long long s = 0;
+            for (int64_t c = c0; c < c1; c++) s += A.chunk_nleft[c];
+            long long pre = block_excl_scan(s, &total, s_tmp);
+            for (int64_t c = c0; c < c1; c++) { A.chunk_lpre[c] = pre; pre += A.chunk_nleft[c]; }
+        }
         if (tid == 0) A.chunk_lpre[n_chunks] = total;
     }
     __syncthreads();
@@ -306,9 +362,11 @@ __global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
     long long s_pos = 0, s_chunks = 0, s_brows = 0;
     for (int i = i0; i < i1; i++) {
         const int n = A.act_node[i];
-        if (A.status[n] != ST_SPLIT) continue;
-        const int64_t nl = A.chunk_lpre[A.cprefix[i + 1]] - A.chunk_lpre[A.cprefix[i]];
+        const int64_t cp0 = A.cprefix[i], cp1 = A.cprefix[i + 1];
+        const int st = A.status[n];
         const int64_t len = A.seg_len[n], start = A.seg_start[n];
+        const int64_t nl = A.chunk_lpre[cp1] - A.chunk_lpre[cp0];
+        if (st != ST_SPLIT) continue;
         const int64_t nr = len - nl;
         A.seg_start[2 * n] = start;
         A.seg_len[2 * n] = nl;
@@ -321,21 +379,23 @@ __global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
         s_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
         s_brows += (build_left ? nl : nr) + A.seg_cost;
     }
-    long long t_pos, t_chunks, t_brows;
-    long long p_pos = block_excl_scan(s_pos, &t_pos, s_tmp);
-    long long p_chunks = block_excl_scan(s_chunks, &t_chunks, s_tmp);
-    long long p_brows = block_excl_scan(s_brows, &t_brows, s_tmp);
+    // children count (low 24 bits) and chunk count share one scan; the build rows take the other
+    long long t_pc, t_brows, p_pc, p_brows;
+    block_excl_scan2((s_chunks << 24) | s_pos, s_brows, &p_pc, &p_brows, &t_pc, &t_brows, s_tmp);
+    long long p_pos = p_pc & 0xFFFFFF, p_chunks = p_pc >> 24;
+    const long long t_pos = t_pc & 0xFFFFFF, t_chunks = t_pc >> 24;
     for (int i = i0; i < i1; i++) {
         const int n = A.act_node[i];
         if (A.status[n] != ST_SPLIT) continue;
         const int64_t nl = A.seg_len[2 * n], nr = A.seg_len[2 * n + 1];
+        const int64_t start = A.seg_start[2 * n];
         const bool build_left = nr >= nl;
         A.n_act_node[2 * p_pos] = 2 * n;
         A.n_act_node[2 * p_pos + 1] = 2 * n + 1;
         A.n_cprefix[2 * p_pos] = p_chunks;
         A.n_cprefix[2 * p_pos + 1] = p_chunks + (nl + EVT_CHUNK - 1) / EVT_CHUNK;
         A.n_bnode[p_pos] = build_left ? 2 * n : 2 * n + 1;
-        A.n_bstart[p_pos] = build_left ? A.seg_start[2 * n] : A.seg_start[2 * n + 1];
+        A.n_bstart[p_pos] = build_left ? start : start + nl;
         A.n_bprefix[p_pos] = p_brows;
         p_pos += 1;
         p_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
@@ -537,7 +597,7 @@ static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32
     A.K = c->K;
     A.loss = c->loss; // selects the leaf-add rule
     A.fuse_pred = fuse_pred ? 1 : 0;
-    A.write_nidx = c->record_nidx ? 1 : 0;
+    A.write_nidx = c->write_nidx ? 1 : 0;
 }
 
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur) {
@@ -557,7 +617,7 @@ int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t 
 }
 
 int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred) {
-    if (!fuse_pred && !c->record_nidx) return EVT_OK;
+    if (!fuse_pred && !c->write_nidx) return EVT_OK;
     PartArgs A;
     fill_part_args(c, level, is_cur, nullptr, fuse_pred, A);
     hipLaunchKernelGGL(k_final_fused, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);

@@ -101,3 +101,48 @@ def test_calls_on_a_closed_or_null_handle_are_errors(evt):
     assert ei.value.code == evt._lib.EVT_ERR_STATE
     h.close()
     h.close()  # idempotent
+
+
+@pytest.mark.parametrize("loss,K,tt", [("mse", 1, "binary"), ("logloss", 1, "binary"), ("gaussian_mle", 2, "oblivious"), ("mlogloss", 3, "binary"),
+                                       ("poisson", 1, "binary")])
+def test_deferred_leaf_addition_equals_immediate(evt, loss, K, tt):
+    """A tree grown on every row leaves its leaf values pending until the next pass over the rows (the next gradient
+    update, or whatever reads the predictions first).  Every consumer must see them applied: predictions, metric,
+    node ids, gradients and the following trees are bit-identical to the path that adds the values while growing -
+    also with several trees per gradient update (bagging), a tree added from outside in between, and a subsampled
+    tree (not deferred) after a deferred one."""
+    N, F, B, D = 30000, 9, 32, 5
+    x_bin, y, w, mu = make_data(77, N, F, B, loss, weights=True, K=K if loss == "mlogloss" else None)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    gp = evt.make_params(eta=0.3, bagging_size=2)
+    metric = {"mse": "mse", "logloss": "logloss", "gaussian_mle": "gaussian_mle", "mlogloss": "mlogloss", "poisson": "poisson"}[loss]
+    mask = np.random.default_rng(5).integers(0, 256, N, dtype=np.uint8)
+    out = []
+    for defer in (1, 0):
+        h = evt.Handle(N, F, B, mu.shape[0], D, loss, tt)
+        h.set_option("defer_pred", defer)
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        rec = []
+        for r in range(3):
+            h.update_grads()
+            rec.append(h.get_grads())
+            t1 = h.grow_tree(js, gp)
+            t2 = h.grow_tree(js, gp)            # second tree of the bag: the first one's values are still pending
+            rec += [t1, t2, h.get_nidx(), h.eval_metric(metric)]
+            if r == 1:
+                h.predict_tree(t1)              # an outside tree on top of a pending one
+                t3 = h.grow_tree(js, gp, mask=mask, cond=128)
+                rec += [t3, h.get_pred()]
+        rec.append(h.get_pred())
+        h.set_target(y, w, mu)                  # a new target drops what is pending
+        rec.append(h.get_pred())
+        h.close()
+        out.append(rec)
+    for a, b in zip(*out):
+        if isinstance(a, np.ndarray):
+            assert a.tobytes() == b.tobytes()
+        elif isinstance(a, float):
+            assert a == b
+        else:
+            assert_tree_bits(a, b)
