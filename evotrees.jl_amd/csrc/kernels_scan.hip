@@ -136,7 +136,15 @@ template <int NAG, int BPL>
 __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const int n = (1 << (A.level - 1)) + blockIdx.x; // 1-based node id
+    // The block's time is a chain of round trips to memory, so requests go out in as few dependent steps as the data
+    // allows: node state and feature id first; then, in one batch of unconditional loads, the histogram slices, the
+    // feature's type and constraint, the node totals and the decode scales.
+    const int jp = blockIdx.y * nwaves + wave;
+    const bool have = jp < A.nfs; // wave-uniform; a wave past the last feature loads the last one's data and drops it
+    const int jpc = have ? jp : A.nfs - 1;
+    int f = (int)A.js[jpc] - 1;
     const int st = A.status[n];
+    asm volatile("" : "+v"(f)); // the feature id is requested ahead of the branch on the node state, not behind it
     if (st != ST_BUILD && st != ST_SUBTRACT) return;
     const bool is_sub = (st == ST_SUBTRACT);
     const int B = A.B, NK = A.NK, K = A.K;
@@ -151,33 +159,67 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     __shared__ double s_wg[4];
     __shared__ int s_wjp[4], s_wbin[4];
 
-    // the histogram slices are requested before the node totals are read and reduced: neither depends on the other,
-    // and the block would otherwise sit through two round trips to memory one after the other
-    const int jp = blockIdx.y * nwaves + wave;
     long long pre[NAG][BPL];
+    long long vb[NAG][BPL];
     long long excl[NAG];
-    if (jp < A.nfs) {
+    const int64_t o0 = (int64_t)jpc * NAG * B;
+    if (is_sub) {
 #pragma unroll
         for (int ag = 0; ag < NAG; ag++) {
-            const int64_t o = ((int64_t)jp * NAG + ag) * B;
 #pragma unroll
             for (int t = 0; t < BPL; t++) {
                 const int b = lane * BPL + t;
-                long long v = 0;
-                if (b < B) {
-                    if (is_sub) {
-                        v = hp[o + b] - hs[o + b];
-                        hn[o + b] = v; // subtract_hist!: h[n] = h[parent] - h[sibling]
-                    } else {
-                        v = hn[o + b];
-                    }
-                }
-                pre[ag][t] = v;
+                const int64_t o = o0 + (int64_t)ag * B + (b < B ? b : B - 1);
+                pre[ag][t] = hp[o];
+                vb[ag][t] = hs[o];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int ag = 0; ag < NAG; ag++) {
+#pragma unroll
+            for (int t = 0; t < BPL; t++) {
+                const int b = lane * BPL + t;
+                pre[ag][t] = hn[o0 + (int64_t)ag * B + (b < B ? b : B - 1)];
+                vb[ag][t] = 0;
             }
         }
     }
+    const bool numeric = A.feattypes[f] != 0;
+    const int constraint = A.mono[f];
+    const int tq = tid < NAG ? tid : 0;
+    const double qs = A.qscale[tq];
+    const long long nsq = A.node_sum[(int64_t)n * NAG + tq]; // not yet written at level 1, and not used there
 
-    node_totals<NAG>(A, n, hn, blockIdx.y == 0, s_Sq, s_S, s_sc);
+#pragma unroll
+    for (int ag = 0; ag < NAG; ag++) {
+#pragma unroll
+        for (int t = 0; t < BPL; t++) {
+            const int b = lane * BPL + t;
+            const long long v = (have && b < B) ? pre[ag][t] - vb[ag][t] : 0;
+            if (is_sub && have && b < B) hn[o0 + (int64_t)ag * B + b] = v; // subtract_hist!: h[n] = h[parent] - h[sibling]
+            pre[ag][t] = v;
+        }
+    }
+
+    // node totals -> Float64 statistics (as node_totals, with the values requested above)
+    if (A.level == 1) {
+        node_totals<NAG>(A, n, hn, blockIdx.y == 0, s_Sq, s_S, s_sc);
+    } else {
+        if (tid < NAG) {
+            s_sc[tid] = qs;
+            s_Sq[tid] = nsq;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            double v[EVT_MAX_NK];
+            long long q[NAG];
+            for (int ag = 0; ag < NAG; ag++) q[ag] = s_Sq[ag];
+            decode_vals(q, s_sc, A.loss, A.NK, v);
+            for (int k = 0; k < A.NK; k++) s_S[k] = v[k];
+        }
+        __syncthreads();
+    }
     double S[EVT_MAX_NK];
     for (int k = 0; k < NK; k++) S[k] = s_S[k];
 
@@ -189,10 +231,7 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     int wjp = NO_BIN, wbin = NO_BIN;
     const int nodeidx = blockIdx.x;
 
-    if (jp < A.nfs) {
-        const int f = (int)A.js[jp] - 1;
-        const bool numeric = A.feattypes[f] != 0;
-        const int constraint = A.mono[f];
+    if (have) {
         const int bmax = numeric ? B - 1 : B;
         // inclusive prefix over the bins: within the lane, then across the wavefront
 #pragma unroll
