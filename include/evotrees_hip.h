@@ -141,6 +141,11 @@ int evt_set_grads(evt_handle h, const float *grad);
  *  mask : UInt8[nobs] drawn by the host RNG, rows with mask[i] <= cond are kept; NULL keeps all.
  *  js   : sampled feature ids, 1-based, ascending, n_js of them (src/fit.jl:16).
  * Returns EVT_ERR_EMPTY when no row is kept.
+ * When every row is kept and params->update_pred is set, the tree's leaf values may still be pending on
+ * return: the library has recorded each row's leaf and adds the values in the next pass over the rows
+ * (evt_update_grads does it on the way; evt_get_pred, evt_eval_metric, evt_predict_tree and the next
+ * evt_grow_tree apply them first).  Every call sees the same predictions, bit for bit, as if predict! had
+ * run inside this call.
  */
 int evt_grow_tree(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js,
                   const evt_params *params, evt_tree_out *tree);
@@ -216,7 +221,9 @@ int evt_reset_profile(evt_handle h);
 /* Options: "hist_blocks", "hist_threads", "hist_min_rows", "hist_seg_cost", "hist_variant" (launch shape,
  * work split and kernel variant of the histogram builder, for sweeps; results do not depend on them);
  * "record_nidx" (1: the partition also records every sampled row's final node while the tree grows;
- * 0, default: evt_get_nidx derives it afterwards by walking the finished tree). */
+ * 0, default: evt_get_nidx derives it afterwards by walking the finished tree); "defer_pred" (1, default:
+ * leaf values of a tree grown on every row are added in row order by the next pass over the rows;
+ * 0: they are added while the tree's last level is partitioned; results do not depend on it). */
 int evt_set_option(evt_handle h, const char *name, int64_t value);
 /* Blocks until all work queued on the handle's stream is done. */
 int evt_synchronize(evt_handle h);
