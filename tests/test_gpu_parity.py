@@ -303,6 +303,34 @@ def test_free_running_rounds_bit_exact_mse(evt, loss, tt, rowsample, colsample):
     o.close()
 
 
+@pytest.mark.parametrize("weights", [False, True])
+def test_free_running_40_rounds_headline_shape(evt, weights):
+    # the headline workload's shape (100 features -> 128-byte records, 64 bins, deep trees) at a size the CPU side
+    # finishes in seconds: 40 free-running rounds, every tree and the final predictions bit identical
+    N, F, B, D, R = 300000, 100, 64, 9, 40
+    x_bin, y, w, mu = make_data(23, N, F, B, "mse", weights, signal=True)
+    h, o, op, gp, pred0, grad0 = setup_pair(evt, "mse", x_bin, y, w, mu, B, D, eta=0.3)
+    p_orc = pred0.copy()
+    grad = grad0.copy()
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    rows = np.arange(N, dtype=np.uint32)
+    nsplit = 0
+    for r in range(R):
+        h.update_grads()
+        orc.update_grads(op, p_orc, y, grad)
+        t_gpu = h.grow_tree(js, gp)
+        qb, qe = h.get_quant()
+        o.set_quant(grad, qb)
+        t_fx, _ = o.grow_tree(grad, rows, js, mode=1, want_nidx=False)
+        assert_tree_bits(t_gpu, t_fx)
+        nsplit += int(t_gpu.split.sum())
+        o.predict_tree(t_fx, p_orc)
+    assert nsplit > 40 * 100  # the trees are deep ones, not stumps
+    assert np.array_equal(h.get_pred().view(np.uint32), p_orc.view(np.uint32))
+    h.close()
+    o.close()
+
+
 @pytest.mark.parametrize("loss", ["logloss", "gaussian_mle", "poisson", "gamma", "tweedie", "mlogloss"])
 def test_free_running_rounds_tolerance(evt, loss):
     # device exp/log1p differ from the host's by an ulp: structure must still agree with the
