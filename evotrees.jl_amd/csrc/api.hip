@@ -121,7 +121,7 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->obest, c->sbest, c->pend_leaf};
+                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->obest, c->sbest, c->pend_leaf, c->is_id};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -196,6 +196,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->write_nidx = false;
     c->pend_pred = false;
     c->pend_leaf = nullptr;
+    c->is_id = nullptr;
     c->last_cond = 255;
     c->profiling = 0;
     c->prof_open = false;
@@ -225,6 +226,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->gq, (size_t)N * c->NK);
     ALLOC(c->is_a, N);
     ALLOC(c->is_b, N);
+    ALLOC(c->is_id, N);
     ALLOC(c->nidx, N);
     ALLOC(c->pend_leaf, (size_t)c->nnodes * K);
     ALLOC(c->mask, N);
@@ -301,6 +303,15 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
             evt_set_error("initial fills failed: %s", hipGetErrorString(e2));
             evt_destroy(c);
             return EVT_ERR_HIP;
+        }
+    }
+    {
+        int r = launch_iota(c, c->is_id, N);
+        hipError_t e3 = hipStreamSynchronize(c->stream);
+        if (r != EVT_OK || e3 != hipSuccess) {
+            if (r == EVT_OK) evt_set_error("initial fills failed: %s", hipGetErrorString(e3));
+            evt_destroy(c);
+            return r != EVT_OK ? r : EVT_ERR_HIP;
         }
     }
     *out = c;
@@ -564,9 +575,7 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     prof_begin(c, EVT_K_OTHER, 0);
     r = launch_apply_pending(c); // an earlier tree's values go in before its node ids are overwritten
     if (r != EVT_OK) return r;
-    if (all_rows) {
-        r = launch_iota(c, c->is_a, c->N);
-    } else {
+    if (!all_rows) {
         HIPCHK(hipMemcpyAsync(c->mask, mask, c->N, hipMemcpyDefault, c->stream));
         r = launch_compact_mask(c, cond);
         if (r == EVT_OK && c->record_nidx) r = launch_fill_u32(c, c->nidx, 0u, c->N);
@@ -576,7 +585,9 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     if (r != EVT_OK) return r;
 
     const bool obliv = (c->tree_type == EVT_TREE_OBLIVIOUS);
-    uint32_t *is_cur = c->is_a, *is_next = c->is_b;
+    // the root's list is the identity (kept, never written) or what the mask compaction left in is_a; the levels below
+    // alternate between is_a and is_b
+    uint32_t *is_cur = all_rows ? c->is_id : c->is_a, *is_next = all_rows ? c->is_a : c->is_b;
     // levels 1 .. D-1 split; the last of them sends its rows straight to the leaves of level D
     const int last_split = (c->D > 1) ? c->D - 1 : 1;
     for (int level = 1; level <= last_split; level++) {
@@ -604,7 +615,12 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
         }
         prof_end(c);
         if (r != EVT_OK) return r;
-        std::swap(is_cur, is_next);
+        if (is_cur == c->is_id) {
+            is_cur = is_next;
+            is_next = c->is_b;
+        } else {
+            std::swap(is_cur, is_next);
+        }
     }
     if (p->update_pred && !all_rows) {
         // rows outside the sample are predicted too (src/fit.jl:37): walk the new tree for all rows

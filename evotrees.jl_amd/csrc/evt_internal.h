@@ -84,6 +84,7 @@ struct evt_ctx {
     float *grad;    // NK x N
     unsigned long long *gq; // NA planes of N packed fixed-point words
     uint32_t *is_a, *is_b;
+    uint32_t *is_id;   // [N] 0..N-1, written once: the root's row list when every row is in the tree
     uint32_t *nidx;
     uint8_t *mask;
     unsigned long long *flagw;

@@ -157,7 +157,9 @@ __global__ __launch_bounds__(256) void k_absmax(const float *__restrict__ grad, 
 }
 
 // qexp[k] = ilogb(max) + 1 (0 for an all-zero row); qmul[k] = 2^(qbits-qexp) encodes, qscale decodes.
-__global__ void k_quant_setup(const uint32_t *absmax, const int32_t *qbits, int32_t *qexp, double *qmul, double *qscale_g,
+// The maxima of the rows the gradient kernel rewrites every round are cleared for its next pass once they are read;
+// the weight row (last) is written once and keeps its maximum.
+__global__ void k_quant_setup(uint32_t *absmax, const int32_t *qbits, int32_t *qexp, double *qmul, double *qscale_g,
                               int NK, int NAg, int loss, int unit_w) {
     int k = threadIdx.x;
     if (k < NK) {
@@ -170,6 +172,7 @@ __global__ void k_quant_setup(const uint32_t *absmax, const int32_t *qbits, int3
         }
         qexp[k] = e;
         qmul[k] = scalbn(1.0, qbits[k] - e);
+        if (k < NK - 1) absmax[k] = 0u;
     }
     __syncthreads();
     if (k < NAg) {
@@ -199,11 +202,7 @@ __global__ __launch_bounds__(256) void k_quantize(const float *__restrict__ grad
 }
 
 int launch_grads(evt_ctx *c) {
-    // absmax of the rows this kernel writes starts from zero; the weight row keeps its value
-    {
-        int r = launch_fill_u32(c, c->absmax, 0u, c->NK - 1);
-        if (r != EVT_OK) return r;
-    }
+    // absmax of the rows this kernel writes starts from zero (cleared at creation and by k_quant_setup after every use)
     int64_t nb = (c->N + 255) / 256;
     if (nb > 2048) nb = 2048;
     dim3 grid((unsigned)nb);
