@@ -303,7 +303,7 @@ def main():
             out["predict_model"] = {"trees": n_model, "s": round(best, 4), "rows_per_s": round(N / best, 1),
                                     "row_trees_per_s": round(N * n_model / best, 1),
                                     "lower_bound_GBps": round(N * (F + 4 * K) / best / 1e9, 1),
-                                    "note": "whole evt_predict call with device-resident x_bin and output (includes its device allocations and copies)"}
+                                    "note": "whole evt_predict call with device-resident x_bin and output, used in place (includes the host-side packing of the trees and their upload)"}
             hip.hipFree(d_x)
             hip.hipFree(d_out)
         except Exception as e:  # measurement aid only

@@ -10,10 +10,12 @@
 
 int launch_absmax_rows(evt_ctx *c, int k0, int k1);
 int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, const float *leaf_pred_dev);
-int launch_predict_model(hipStream_t s, const uint32_t *nodes, const float *leaf_pred, const int64_t *off, int ntrees, const uint8_t *xcm,
-                         const uint8_t *feattypes, int64_t N, int K, int loss, int apply_link, float *out);
-int launch_leaf_idx_model(hipStream_t s, const uint32_t *nodes, const int64_t *off, int ntrees, const uint8_t *xcm, const uint8_t *feattypes,
-                          int64_t N, uint32_t *out);
+int launch_predict_model(hipStream_t s, const uint32_t *nodes, const float *leaf_pred, const int64_t *off, int ntrees, const uint8_t *xcm, int64_t N,
+                         int K, int loss, int apply_link, float *out);
+int predict_lds_shape(int F, int max_int, int K, int hint);
+int launch_predict_model_lds(hipStream_t s, const uint32_t *cnodes, const float *cleaf, const void *meta, int ntrees, const uint8_t *xcm, int64_t N,
+                             int F, int max_int, int K, int loss, int apply_link, int all_numeric, int shape, float *out);
+int launch_leaf_idx_model(hipStream_t s, const uint32_t *nodes, const int64_t *off, int ntrees, const uint8_t *xcm, int64_t N, uint32_t *out);
 
 static thread_local char g_err[512] = "";
 
@@ -294,6 +296,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     // defaults: all numeric, no monotone constraint
     {
         std::vector<uint8_t> ft(c->F, 1);
+        c->h_feattypes = ft;
         hipError_t e2 = hipMemcpy(c->feattypes, ft.data(), c->F, hipMemcpyHostToDevice);
         if (e2 == hipSuccess) e2 = hipMemset(c->mono, 0, sizeof(int32_t) * c->F);
         if (e2 == hipSuccess) e2 = hipMemset(c->absmax, 0, sizeof(uint32_t) * EVT_MC_MAX_NK);
@@ -477,6 +480,7 @@ extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, cons
     }
     HIPCHK(hipMemcpy(c->feattypes, ft.data(), c->F, hipMemcpyHostToDevice));
     HIPCHK(hipMemcpy(c->mono, mo.data(), sizeof(int32_t) * c->F, hipMemcpyHostToDevice));
+    c->h_feattypes = ft;
     return EVT_OK;
 }
 
@@ -668,13 +672,14 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
 }
 
 // host tree -> packed device nodes; validates that every split node has both children in range
-static int pack_tree(int32_t nn, const int64_t *feat, const uint8_t *cond_bin, const uint8_t *split, int F, std::vector<uint32_t> &out) {
+static int pack_tree(int32_t nn, const int64_t *feat, const uint8_t *cond_bin, const uint8_t *split, int F, const uint8_t *feattypes,
+                     std::vector<uint32_t> &out) {
     out.assign(nn, 0u);
     for (int n = 1; n <= nn; n++) {
         if (split[n - 1]) {
             ARGCHK(2 * n + 1 <= nn, "split node without children inside the tree arrays");
             ARGCHK(feat[n - 1] >= 1 && feat[n - 1] <= F, "tree feature id outside 1..nfeats");
-            out[n - 1] = (uint32_t)feat[n - 1] | ((uint32_t)cond_bin[n - 1] << 16) | (1u << 24);
+            out[n - 1] = evt_pack_node((int)feat[n - 1], cond_bin[n - 1], feattypes == nullptr || feattypes[feat[n - 1] - 1] != 0);
         }
     }
     return EVT_OK;
@@ -689,7 +694,7 @@ extern "C" int evt_predict_tree(evt_handle c, int32_t nnodes_tree, const int64_t
         return EVT_ERR_STATE;
     }
     std::vector<uint32_t> nodes;
-    int r = pack_tree(nnodes_tree, feat, cond_bin, split, c->F, nodes);
+    int r = pack_tree(nnodes_tree, feat, cond_bin, split, c->F, c->h_feattypes.data(), nodes);
     if (r != EVT_OK) return r;
     r = launch_apply_pending(c);
     if (r != EVT_OK) return r;
@@ -822,6 +827,70 @@ extern "C" int evt_eval_metric(evt_handle c, int32_t metric, double *value_out) 
 }
 
 // ---- inference ------------------------------------------------------------------------------
+// Trees completed for the LDS kernel: every leaf above a tree's last level becomes a chain of always-left nodes that
+// carries its value down to that level, so that all rows walk depth - 1 levels.  Returns false when a tree's arrays are
+// not a full heap (2^depth - 1 entries) - the gather kernel takes such models.
+struct ModelTreeHost {
+    int32_t node_off, leaf_off, levels, n_int;
+};
+// EVT_PREDICT_SHAPE=1..4 in the environment picks the LDS kernel's launch shape when the model allows it (for sweeps)
+static int predict_shape_hint() {
+    const char *v = getenv("EVT_PREDICT_SHAPE");
+    return v ? atoi(v) : 0;
+}
+// Largest number of internal nodes over the model's trees; false when a tree's arrays are not a full heap
+// (2^depth - 1 entries): the gather kernel takes such models.
+static bool model_max_internal(int ntrees, const int64_t *tree_off, int &max_int) {
+    max_int = 0;
+    for (int t = 0; t < ntrees; t++) {
+        const int64_t nn = tree_off[t + 1] - tree_off[t];
+        if (nn < 1 || (nn & (nn + 1)) != 0 || nn > (1 << 20)) return false;
+        max_int = std::max(max_int, (int)((nn + 1) / 2 - 1));
+    }
+    return true;
+}
+// Every tree padded to `stride` node words and the list padded with trees of no levels to a multiple of `group`.
+static void complete_trees(int ntrees, const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const float *pred,
+                           const uint8_t *split, const uint8_t *feattypes, int K, int stride, int group, std::vector<uint32_t> &cnodes,
+                           std::vector<float> &cleaf, std::vector<ModelTreeHost> &meta, bool &all_numeric) {
+    const int npad = ((ntrees + group - 1) / group) * group;
+    cnodes.assign((size_t)npad * stride, 0u);
+    cleaf.clear();
+    meta.assign(npad, ModelTreeHost{0, 0, 0, 0});
+    all_numeric = true;
+    std::vector<int32_t> vsrc;
+    const uint32_t always_left = 0u | (255u << 16) | EVT_NODE_NUMERIC; // feature 1, bin <= 255
+    for (int t = 0; t < ntrees; t++) {
+        const int64_t o = tree_off[t];
+        const int64_t nn = tree_off[t + 1] - o;
+        int depth = 0;
+        while (((int64_t)1 << depth) - 1 < nn) depth++;
+        const int n_int = (1 << (depth - 1)) - 1, n_leaf = 1 << (depth - 1);
+        meta[t] = {(int32_t)((size_t)t * stride), (int32_t)(cleaf.size() / K), depth - 1, n_int};
+        // vsrc[n]: 0 = a split node of the tree; otherwise the leaf whose value node n carries
+        vsrc.assign(nn + 1, 0);
+        for (int64_t n = 1; n <= nn; n++) {
+            const int32_t up = (n == 1) ? 0 : vsrc[n >> 1];
+            vsrc[n] = up ? up : (split[o + n - 1] ? 0 : (int32_t)n);
+        }
+        uint32_t *cn = cnodes.data() + (size_t)t * stride;
+        for (int n = 1; n <= n_int; n++) {
+            uint32_t w = always_left;
+            if (vsrc[n] == 0) {
+                const int f0 = (int)feat[o + n - 1] - 1;
+                const bool numeric = feattypes == nullptr || feattypes[f0] != 0;
+                all_numeric = all_numeric && numeric;
+                w = (uint32_t)(((f0 >> 2) << 8) | (f0 & 3)) | ((uint32_t)cond_bin[o + n - 1] << 16) | (numeric ? EVT_NODE_NUMERIC : 0u);
+            }
+            cn[n - 1] = w;
+        }
+        for (int q = 0; q < n_leaf; q++) {
+            const int32_t src = vsrc[n_int + 1 + q]; // never 0: a split node's children lie inside the arrays (checked when packing)
+            for (int k = 0; k < K; k++) cleaf.push_back(pred[(size_t)K * (o + src - 1) + k]);
+        }
+    }
+}
+
 // Rows binned per pass of evt_predict_f64: bounds the Float64 staging buffer to chunk * nfeats * 8 bytes.
 static const int64_t PREDICT_F64_CHUNK = 1 << 20;
 
@@ -848,26 +917,57 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
         const int64_t o = tree_off[t];
         const int64_t nn = tree_off[t + 1] - o;
         ARGCHK(nn >= 1 && o >= 0, "tree_off must be ascending");
-        r = pack_tree((int32_t)nn, feat + o, cond_bin + o, split + o, nfeats, one);
+        r = pack_tree((int32_t)nn, feat + o, cond_bin + o, split + o, nfeats, feattypes, one);
         if (r != EVT_OK) return r;
         memcpy(nodes.data() + o, one.data(), sizeof(uint32_t) * nn);
     }
-    std::vector<uint8_t> ft(nfeats, 1);
-    if (feattypes)
-        for (int j = 0; j < nfeats; j++) ft[j] = feattypes[j] ? 1 : 0;
     hipStream_t s = nullptr;
-    uint8_t *d_x = nullptr, *d_ft = nullptr;
+    uint8_t *d_x = nullptr;
     uint32_t *d_nodes = nullptr, *d_leaf = nullptr;
     float *d_lp = nullptr, *d_out = nullptr;
     int64_t *d_off = nullptr;
-    hipError_t e = hipMalloc((void **)&d_x, (size_t)nobs * nfeats);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_ft, nfeats);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_nodes, sizeof(uint32_t) * total);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_off, sizeof(int64_t) * (ntrees + 1));
-    if (e == hipSuccess && !leaf_out) e = hipMalloc((void **)&d_lp, sizeof(float) * (size_t)total * K);
-    if (e == hipSuccess && !leaf_out) e = hipMalloc((void **)&d_out, sizeof(float) * (size_t)nobs * K);
+    // x_bin and the output are used in place when they already live on the device
+    auto on_device = [](const void *p) {
+        hipPointerAttribute_t attr;
+        const bool dev = p && hipPointerGetAttributes(&attr, p) == hipSuccess && attr.type == hipMemoryTypeDevice;
+        (void)hipGetLastError();
+        return dev;
+    };
+    const bool x_in_place = !x_f64 && on_device(x_bin);
+    const bool out_in_place = !leaf_out && on_device(out);
+    // models whose trees are full heaps of moderate depth go through the LDS kernel, on trees completed here
+    std::vector<uint32_t> cnodes;
+    std::vector<float> cleaf;
+    std::vector<ModelTreeHost> cmeta;
+    int max_int = 0, shape = 0;
+    bool all_numeric = true;
+    bool use_lds = !leaf_out && K <= 4 && ntrees >= 4 && !on_device(pred) && !on_device(feat) && model_max_internal(ntrees, tree_off, max_int);
+    if (use_lds) {
+        shape = predict_lds_shape(nfeats, max_int, K, predict_shape_hint());
+        use_lds = shape > 0;
+    }
+    if (use_lds)
+        complete_trees(ntrees, tree_off, feat, cond_bin, pred, split, feattypes, K, std::max(1, max_int), shape == 1 ? 4 : (shape == 2 ? 2 : 1), cnodes,
+                       cleaf, cmeta, all_numeric);
+    uint32_t *d_cn = nullptr;
+    float *d_cl = nullptr;
+    ModelTreeHost *d_cm = nullptr;
+    hipError_t e = hipSuccess;
+    if (x_in_place) d_x = const_cast<uint8_t *>(x_bin);
+    else e = hipMalloc((void **)&d_x, (size_t)nobs * nfeats);
+    if (use_lds) {
+        if (e == hipSuccess) e = hipMalloc((void **)&d_cn, sizeof(uint32_t) * std::max<size_t>(1, cnodes.size()));
+        if (e == hipSuccess) e = hipMalloc((void **)&d_cl, sizeof(float) * cleaf.size());
+        if (e == hipSuccess) e = hipMalloc((void **)&d_cm, sizeof(ModelTreeHost) * cmeta.size());
+    } else {
+        if (e == hipSuccess) e = hipMalloc((void **)&d_nodes, sizeof(uint32_t) * total);
+        if (e == hipSuccess) e = hipMalloc((void **)&d_off, sizeof(int64_t) * (ntrees + 1));
+        if (e == hipSuccess && !leaf_out) e = hipMalloc((void **)&d_lp, sizeof(float) * (size_t)total * K);
+    }
+    if (out_in_place) d_out = out;
+    else if (e == hipSuccess && !leaf_out) e = hipMalloc((void **)&d_out, sizeof(float) * (size_t)nobs * K);
     if (e == hipSuccess && leaf_out) e = hipMalloc((void **)&d_leaf, sizeof(uint32_t) * (size_t)nobs * ntrees);
-    if (e == hipSuccess && !x_f64) e = hipMemcpy(d_x, x_bin, (size_t)nobs * nfeats, hipMemcpyDefault);
+    if (e == hipSuccess && !x_f64 && !x_in_place) e = hipMemcpy(d_x, x_bin, (size_t)nobs * nfeats, hipMemcpyDefault);
     if (e == hipSuccess && x_f64) {
         // binarize on the device, PREDICT_F64_CHUNK rows at a time: each pass copies the rows' slice of every
         // column (a strided 2-D copy) and bins it into place
@@ -889,20 +989,26 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
         for (void *p : tmp)
             if (p) (void)hipFree(p);
     }
-    if (e == hipSuccess) e = hipMemcpy(d_ft, ft.data(), nfeats, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMemcpy(d_nodes, nodes.data(), sizeof(uint32_t) * total, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMemcpy(d_off, tree_off, sizeof(int64_t) * (ntrees + 1), hipMemcpyDefault);
-    if (e == hipSuccess && !leaf_out) e = hipMemcpy(d_lp, pred, sizeof(float) * (size_t)total * K, hipMemcpyDefault);
+    if (use_lds) {
+        if (e == hipSuccess && !cnodes.empty()) e = hipMemcpy(d_cn, cnodes.data(), sizeof(uint32_t) * cnodes.size(), hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = hipMemcpy(d_cl, cleaf.data(), sizeof(float) * cleaf.size(), hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = hipMemcpy(d_cm, cmeta.data(), sizeof(ModelTreeHost) * cmeta.size(), hipMemcpyHostToDevice);
+    } else {
+        if (e == hipSuccess) e = hipMemcpy(d_nodes, nodes.data(), sizeof(uint32_t) * total, hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = hipMemcpy(d_off, tree_off, sizeof(int64_t) * (ntrees + 1), hipMemcpyDefault);
+        if (e == hipSuccess && !leaf_out) e = hipMemcpy(d_lp, pred, sizeof(float) * (size_t)total * K, hipMemcpyDefault);
+    }
     if (e == hipSuccess && r == EVT_OK) {
-        if (leaf_out) r = launch_leaf_idx_model(s, d_nodes, d_off, ntrees, d_x, d_ft, nobs, d_leaf);
-        else r = launch_predict_model(s, d_nodes, d_lp, d_off, ntrees, d_x, d_ft, nobs, K, loss, apply_link, d_out);
+        if (leaf_out) r = launch_leaf_idx_model(s, d_nodes, d_off, ntrees, d_x, nobs, d_leaf);
+        else if (use_lds) r = launch_predict_model_lds(s, d_cn, d_cl, d_cm, ntrees, d_x, nobs, nfeats, max_int, K, loss, apply_link, all_numeric ? 1 : 0, shape, d_out);
+        else r = launch_predict_model(s, d_nodes, d_lp, d_off, ntrees, d_x, nobs, K, loss, apply_link, d_out);
         e = hipDeviceSynchronize();
     }
     if (e == hipSuccess && r == EVT_OK) {
         if (leaf_out) e = hipMemcpy(leaf_out, d_leaf, sizeof(uint32_t) * (size_t)nobs * ntrees, hipMemcpyDefault);
-        else e = hipMemcpy(out, d_out, sizeof(float) * (size_t)nobs * K, hipMemcpyDefault);
+        else if (!out_in_place) e = hipMemcpy(out, d_out, sizeof(float) * (size_t)nobs * K, hipMemcpyDefault);
     }
-    void *ptrs[] = {d_x, d_ft, d_nodes, d_off, d_lp, d_out, d_leaf};
+    void *ptrs[] = {x_in_place ? nullptr : d_x, d_nodes, d_off, d_lp, out_in_place ? nullptr : d_out, d_leaf, d_cn, d_cl, d_cm};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     if (e != hipSuccess) {

@@ -120,6 +120,7 @@ struct evt_ctx {
     int32_t h_qbits[EVT_MC_MAX_NK];
     int32_t n_js_last;
     std::vector<uint32_t> js_last;
+    std::vector<uint8_t> h_feattypes; // host copy: trees handed in from outside are packed with it
     bool last_all_rows;
 
     // tunables
@@ -164,7 +165,13 @@ void evt_set_error(const char *fmt, ...);
 // predict!'s update of one row's K outputs with a leaf's values (src/predict.jl:1-62): plain sum (mse and the exp-link
 // losses), clamp to [-15, 15] (logloss), floor -15 on the scale outputs (gaussian_mle), shift by the row maximum and
 // floor -15 (mlogloss).  pr may point to registers or memory.
+// A split node in one 32-bit word: feature id (1-based) | cond_bin << 16 | split << 24 | numeric << 25.  Leaves are 0.
+#define EVT_NODE_SPLIT (1u << 24)
+#define EVT_NODE_NUMERIC (1u << 25)
 #ifdef __HIPCC__
+__host__ __device__ __forceinline__ uint32_t evt_pack_node(int feat, int cond_bin, bool numeric) {
+    return (uint32_t)feat | ((uint32_t)cond_bin << 16) | EVT_NODE_SPLIT | (numeric ? EVT_NODE_NUMERIC : 0u);
+}
 __device__ __forceinline__ void evt_add_leaf(float *pr, const float *lp, int K, int loss) {
     if (loss == EVT_LOSS_LOGLOSS) {
         for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);

@@ -381,7 +381,7 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
             A.tree.cond_bin[n - 1] = (uint8_t)bb;
             A.tree.gain[n - 1] = (float)bg;
             A.tree.split[n - 1] = 1;
-            A.tree.packed[n - 1] = (uint32_t)feat | ((uint32_t)bb << 16) | (1u << 24);
+            A.tree.packed[n - 1] = evt_pack_node(feat, bb, A.feattypes[feat - 1] != 0);
             A.status[n] = ST_SPLIT;
         } else {
             for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (n - 1) + k] = (float)leaf_value(S, k, K, A.eta, A.bagging, A.lambda, A.L2);
@@ -520,7 +520,7 @@ __global__ __launch_bounds__(1024) void k_obliv_select(OblivArgs A) {
             A.tree.cond_bin[n - 1] = (uint8_t)bb;
             A.tree.gain[n - 1] = (float)bgain;
             A.tree.split[n - 1] = 1;
-            A.tree.packed[n - 1] = (uint32_t)feat | ((uint32_t)bb << 16) | (1u << 24);
+            A.tree.packed[n - 1] = evt_pack_node(feat, bb, A.feattypes[feat - 1] != 0);
             A.status[n] = ST_SPLIT;
         }
         if (!A.zero_children) continue;
@@ -732,7 +732,7 @@ __global__ __launch_bounds__(256) void k_scan_fin_mc(ScanArgs A, int ngroups) {
             A.tree.cond_bin[n - 1] = (uint8_t)bb;
             A.tree.gain[n - 1] = (float)bg;
             A.tree.split[n - 1] = 1;
-            A.tree.packed[n - 1] = (uint32_t)feat | ((uint32_t)bb << 16) | (1u << 24);
+            A.tree.packed[n - 1] = evt_pack_node(feat, bb, A.feattypes[feat - 1] != 0);
             A.status[n] = ST_SPLIT;
         } else {
             A.status[n] = ST_LEAF;

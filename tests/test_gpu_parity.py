@@ -413,11 +413,22 @@ def _random_tree(rng, depth, F, B, K):
     (5000, 40, 255, [6, 6, 2], 6, "mlogloss"),        # many outputs
     (1025, 3, 4, [2, 12], 2, "gaussian_mle"),         # odd row count
     (64 * 512, 100, 64, [11] * 5, 1, "mse"),          # the benchmark's shape
+    # models that take the kernel walking completed trees in LDS, in each of its launch shapes: 1024 rows x 4 trees side by
+    # side, 512 x 2, 512 x 1, 256 x 1; tree counts that do not fill the last group, stumps and bias trees in between,
+    # row counts that do not fill the last block, the deepest trees each shape takes
+    (4097, 150, 32, [7, 3, 7, 1, 6, 7], 1, "mse"),
+    (3000, 150, 32, [10, 10, 2, 10, 10], 2, "gaussian_mle"),
+    (2000, 250, 16, [5, 6, 6, 4], 1, "logloss"),
+    (100001, 20, 64, [12] * 7 + [1, 12], 1, "mse"),
+    (20000, 12, 64, [13, 2, 13, 13, 1], 1, "poisson"),
+    (777, 5, 8, [1, 1, 1, 1, 1], 1, "mse"),
+    (5000, 33, 16, [6] * 9, 2, "gaussian_mle"),
 ])
-def test_model_predict_random_trees(evt, N, F, B, depths, K, loss):
+@pytest.mark.parametrize("categorical", [True, False])
+def test_model_predict_random_trees(evt, N, F, B, depths, K, loss, categorical):
     rng = np.random.default_rng(77)
     x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
-    ft = (rng.random(F) > 0.2).astype(np.uint8)
+    ft = (rng.random(F) > 0.2).astype(np.uint8) if categorical else np.ones(F, np.uint8)
     trees = [_random_tree(rng, d, F, B, K) for d in depths]
     want = np.zeros((N, K), np.float32)
     for t in trees:
