@@ -184,7 +184,7 @@ int evt_get_quant(evt_handle h, int32_t *qbits /* 2K+1 */, int32_t *qexp /* 2K+1
  * [tree_off[t], tree_off[t+1]) of feat / cond_bin / split and K times that of pred.
  * out: K x nobs raw sums, link applied when apply_link != 0 (src/predict.jl:105-116).
  * The transposition to nobs x K (src/predict.jl:134) is left to the host.
- * x_bin and out may be host or device pointers (device memory is used in place); the tree arrays are host
+ * x_bin and out may be host or device pointers (device memory is used in place); feattypes and the tree arrays are host
  * arrays.  Models whose trees are full heaps (2^depth - 1 entries, as the reference stores them) of depth
  * <= 13 with K <= 4 and fewer than 1024 features are walked from LDS; others from global memory, with
  * identical results. */

@@ -72,3 +72,36 @@ def test_full_size_invariants(evt):
             assert np.array_equal(getattr(t1, a).view(np.uint32), getattr(t2, a).view(np.uint32))
         assert np.array_equal(h.get_nidx(), nidx_rec)  # derived by walking the tree this time
     h.close()
+
+
+def test_full_size_rounds_bit_exact_against_oracle(evt):
+    """Three free-running boosting rounds at the benchmark's full size against the fixed-point oracle: every tree array,
+    the node id of every row and the final predictions, bit for bit."""
+    from oracle import oracle as orc
+    from test_gpu_parity import assert_tree_bits, setup_pair
+    N, F, B, D, R = 10_000_000, 100, 64, 11, 3
+    rng = np.random.default_rng(99)
+    print("generating", N, "x", F, flush=True)
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    y = (rng.random(N, dtype=np.float32) + np.float32(0.3) * (x_bin[3] > 40) + np.float32(0.2) * (x_bin[70] / np.float32(B))).astype(np.float32)
+    mu = np.array([y.mean()], np.float32)
+    h, o, op, gp, pred0, grad0 = setup_pair(evt, "mse", x_bin, y, None, mu, B, D, eta=0.1)
+    p_orc = pred0.copy()
+    grad = grad0.copy()
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    rows = np.arange(N, dtype=np.uint32)
+    for r in range(R):
+        print("round", r + 1, flush=True)
+        h.update_grads()
+        orc.update_grads(op, p_orc, y, grad)
+        t_gpu = h.grow_tree(js, gp)
+        qb, qe = h.get_quant()
+        o.set_quant(grad, qb)
+        t_fx, nidx = o.grow_tree(grad, rows, js, mode=1)
+        assert_tree_bits(t_gpu, t_fx)
+        assert int(t_gpu.split.sum()) > 500
+        assert np.array_equal(h.get_nidx(), nidx)
+        o.predict_tree(t_fx, p_orc)
+    assert np.array_equal(h.get_pred().view(np.uint32), p_orc.view(np.uint32))
+    h.close()
+    o.close()
