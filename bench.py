@@ -265,7 +265,8 @@ def main():
         depth_bytes = max(D - 1, 0)  # one bin byte per level walked
         out["predict_tree"] = {"ms_per_tree": round(ms_tree, 4), "rows_per_s": round(N / (ms_tree * 1e-3), 1),
                                "algorithmic_GBps": round(N * (8 * K + depth_bytes) / (ms_tree * 1e-3) / 1e9, 1),
-                               "bytes_per_row": 8 * K + depth_bytes}
+                               "bytes_per_row": 8 * K + depth_bytes,
+                               "frac_of_hbm_peak": round(N * (8 * K + depth_bytes) / (ms_tree * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     except Exception as e:  # measurement aid only
         out["predict_tree"] = {"error": str(e)}
 
@@ -303,6 +304,7 @@ def main():
             out["predict_model"] = {"trees": n_model, "s": round(best, 4), "rows_per_s": round(N / best, 1),
                                     "row_trees_per_s": round(N * n_model / best, 1),
                                     "lower_bound_GBps": round(N * (F + 4 * K) / best / 1e9, 1),
+                                    "frac_of_hbm_peak": round(N * (F + 4 * K) / best / 1e9 / HBM_PEAK_GBS, 4),
                                     "note": "whole evt_predict call with device-resident x_bin and output, used in place (includes the host-side packing of the trees and their upload)"}
             hip.hipFree(d_x)
             hip.hipFree(d_out)
