@@ -41,6 +41,20 @@ struct HistArgs {
     int a0; // first global channel of this launch (channels beyond EVT_HIST_GROUP take further launches)
 };
 
+// First node of a block's span: the largest i with bprefix[i] <= start.  bprefix ascends from 0, so that is the number
+// of entries <= start, less one.  Every wavefront counts them for itself, 64 entries per step with all loads
+// independent: one trip to memory where a binary search makes log2(n_build) dependent ones.
+__device__ __forceinline__ int first_node_of_span(const int64_t *__restrict__ bprefix, int n_build, int64_t start) {
+    const int lane = threadIdx.x & 63;
+    int cnt = 0;
+    for (int k0 = 0; k0 < n_build; k0 += 64) {
+        const int k = k0 + lane;
+        const bool hit = (k < n_build) && (bprefix[k < n_build ? k : 0] <= start);
+        cnt += __popcll(__ballot(hit));
+    }
+    return cnt - 1;
+}
+
 template <int NA, bool PACK>
 __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     extern __shared__ unsigned long long H[]; // [NA][tile slots][B]
@@ -84,13 +98,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     const bool lane_on = (rloc < A.RPW) && vmask != 0;
     __syncthreads();
 
-    // first node of this block's span: largest i with bprefix[i] <= start
-    int lo = 0, hi = n_build;
-    while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (A.bprefix[mid] <= start) lo = mid; else hi = mid;
-    }
-    int i = lo;
+    int i = first_node_of_span(A.bprefix, n_build, start);
     const int64_t blk_start = start, blk_end = end;
 
     while (start < end) {
@@ -296,12 +304,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     const bool lane_on = vmask != 0;
     __syncthreads();
 
-    int lo = 0, hi = n_build;
-    while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (A.bprefix[mid] <= start) lo = mid; else hi = mid;
-    }
-    int i = lo;
+    int i = first_node_of_span(A.bprefix, n_build, start);
     const int64_t blk_start = start, blk_end = end;
     char *Hb = reinterpret_cast<char *>(H);
 
