@@ -16,14 +16,18 @@
 // No host round trip is needed between levels.
 #include "evt_internal.h"
 
-// largest i in [0, n) with pre[i] <= v   (pre ascending, pre[0] <= v)
-__device__ __forceinline__ int find_owner(const int64_t *pre, int n, int64_t v) {
-    int lo = 0, hi = n;
-    while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (pre[mid] <= v) lo = mid; else hi = mid;
+// largest i in [0, n) with pre[i] <= v   (pre ascending, pre[0] <= v): the number of such entries, less one.  Every
+// wavefront counts them for itself, 64 entries per step, all loads independent: one trip to memory where a binary
+// search makes log2(n) dependent ones - these blocks are short, so their chain of dependent loads is their run time.
+__device__ __forceinline__ int find_owner(const int64_t *__restrict__ pre, int n, int64_t v) {
+    const int lane = threadIdx.x & 63;
+    int cnt = 0;
+    for (int k0 = 0; k0 < n; k0 += 64) {
+        const int k = k0 + lane;
+        const bool hit = (k < n) && (pre[k < n ? k : 0] <= v);
+        cnt += __popcll(__ballot(hit));
     }
-    return lo;
+    return cnt - 1;
 }
 
 struct PartArgs {
@@ -33,9 +37,7 @@ struct PartArgs {
     const int32_t *status;
     const int64_t *seg_start;
     const int64_t *seg_len;
-    const int32_t *t_feat;
-    const uint8_t *t_bin;
-    const uint8_t *feattypes;
+    const uint32_t *t_packed; // split nodes as one word: feature | cond_bin << 16 | split << 24 | numeric << 25
     const uint8_t *xcm;
     int64_t N;
     const uint32_t *is_cur;
@@ -66,9 +68,10 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
         const int64_t seg = A.seg_start[n], len = A.seg_len[n];
         const int64_t p0 = seg + cl * EVT_CHUNK;
         const int64_t pend = seg + len;
-        const int f = A.t_feat[n - 1] - 1;
-        const uint32_t cb = A.t_bin[n - 1];
-        const bool numeric = A.feattypes[f] != 0;
+        const uint32_t nd = A.t_packed[n - 1];
+        const int f = (int)(nd & 0xFFFFu) - 1;
+        const uint32_t cb = (nd >> 16) & 0xFFu;
+        const bool numeric = (nd & EVT_NODE_NUMERIC) != 0;
         const uint8_t *col = A.xcm + (size_t)f * A.N;
         int cnt = 0;
         // all row ids, then all bin bytes, are requested before the first is used; positions past the end read the
@@ -190,9 +193,10 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
         uint32_t cb = 0;
         bool numeric = true;
         if (is_split) {
-            f = A.t_feat[n - 1] - 1;
-            cb = A.t_bin[n - 1];
-            numeric = A.feattypes[f] != 0;
+            const uint32_t nd = A.t_packed[n - 1];
+            f = (int)(nd & 0xFFFFu) - 1;
+            cb = (nd >> 16) & 0xFFu;
+            numeric = (nd & EVT_NODE_NUMERIC) != 0;
         }
         const uint8_t *col = A.xcm + (size_t)f * A.N;
         // every request of the chunk goes out before the first result is used: row ids, then bin bytes, then (one
@@ -581,9 +585,7 @@ static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32
     A.status = c->status;
     A.seg_start = c->seg_start;
     A.seg_len = c->seg_len;
-    A.t_feat = c->tree.feat;
-    A.t_bin = c->tree.cond_bin;
-    A.feattypes = c->feattypes;
+    A.t_packed = c->tree.packed;
     A.xcm = c->xcm;
     A.N = c->N;
     A.is_cur = is_cur;
