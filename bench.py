@@ -168,9 +168,12 @@ def main():
     tree = evt.Tree(K, h.nnodes)
     tree_out = tree.as_out()
 
+    # the host owns the row-sampling RNG (one uniform byte per row, drawn every round): raw 64-bit words viewed as bytes
+    mask_rng = np.random.default_rng(124)
+
     def one_round():
         h.update_grads()
-        mask = None if cond >= 255 else rng.integers(0, 256, N, dtype=np.uint8)
+        mask = None if cond >= 255 else mask_rng.bit_generator.random_raw((N + 7) // 8).view(np.uint8)[:N]
         js = np.arange(1, F + 1, dtype=np.uint32) if nfs >= F else (np.sort(rng.choice(F, nfs, replace=False)) + 1).astype(np.uint32)
         evt._lib.check(L.evt_grow_tree(h._h, evt._lib.ptr(mask), cond, evt._lib.ptr(js), js.shape[0], params, tree_out))
 
