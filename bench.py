@@ -171,11 +171,19 @@ def main():
     # the host owns the row-sampling RNG (one uniform byte per row, drawn every round): raw 64-bit words viewed as bytes
     mask_rng = np.random.default_rng(124)
 
+    def draw_mask():
+        return None if cond >= 255 else mask_rng.bit_generator.random_raw((N + 7) // 8).view(np.uint8)[:N]
+
+    nxt = [draw_mask()]
+
     def one_round():
         h.update_grads()
-        mask = None if cond >= 255 else mask_rng.bit_generator.random_raw((N + 7) // 8).view(np.uint8)[:N]
+        mask = nxt[0]
         js = np.arange(1, F + 1, dtype=np.uint32) if nfs >= F else (np.sort(rng.choice(F, nfs, replace=False)) + 1).astype(np.uint32)
-        evt._lib.check(L.evt_grow_tree(h._h, evt._lib.ptr(mask), cond, evt._lib.ptr(js), js.shape[0], params, tree_out))
+        # the next round's mask is drawn while the device grows this round's tree
+        evt._lib.check(L.evt_grow_tree_begin(h._h, evt._lib.ptr(mask), cond, evt._lib.ptr(js), js.shape[0], params))
+        nxt[0] = draw_mask()
+        evt._lib.check(L.evt_grow_tree_end(h._h, tree_out))
 
     for _ in range(args.warmup):
         one_round()

@@ -21,6 +21,7 @@ KERNEL_CLASSES = ["grad", "hist", "scan", "partition", "predict", "other"]
 EXPORTS = [
     "evt_last_error", "evt_device_count", "evt_create", "evt_destroy", "evt_set_xbin", "evt_binarize_f64",
     "evt_set_target", "evt_set_feature_meta", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
+    "evt_grow_tree_begin", "evt_grow_tree_end",
     "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
     "evt_predict", "evt_predict_f64", "evt_predict_leaf_idx", "evt_eval_metric", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
     "evt_set_option", "evt_synchronize", "evt_copy_bandwidth", "evt_read_bandwidth",
@@ -69,6 +70,8 @@ def load():
         "evt_update_grads": [vp],
         "evt_set_grads": [vp, vp],
         "evt_grow_tree": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams), C.POINTER(EvtTreeOut)],
+        "evt_grow_tree_begin": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams)],
+        "evt_grow_tree_end": [vp, C.POINTER(EvtTreeOut)],
         "evt_predict_tree": [vp, i32, vp, vp, vp, vp],
         "evt_get_xbin": [vp, vp],
         "evt_get_pred": [vp, vp],
@@ -205,6 +208,21 @@ class Handle:
         out = t.as_out() if want_tree else None
         check(load().evt_grow_tree(self._h, ptr(mask), int(cond), ptr(js), js.shape[0], C.byref(params),
                                    C.byref(out) if want_tree else None))
+        return t
+
+    def grow_tree_begin(self, js, params, mask=None, cond=255):
+        """Queues one tree and returns while the device grows it; grow_tree_end collects it.  Nothing else may be
+        called on the handle in between (the host is free to prepare the next round, e.g. draw the next row mask)."""
+        js = np.ascontiguousarray(js, np.uint32)
+        if mask is not None:
+            mask = np.ascontiguousarray(mask, np.uint8)
+            assert mask.shape == (self.N,)
+        check(load().evt_grow_tree_begin(self._h, ptr(mask), int(cond), ptr(js), js.shape[0], C.byref(params)))
+
+    def grow_tree_end(self, want_tree=True):
+        t = TreeArrays(self.K, self.nnodes) if want_tree else None
+        out = t.as_out() if want_tree else None
+        check(load().evt_grow_tree_end(self._h, C.byref(out) if want_tree else None))
         return t
 
     def predict_tree(self, tree):

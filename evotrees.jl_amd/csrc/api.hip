@@ -199,6 +199,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->pend_pred = false;
     c->pend_leaf = nullptr;
     c->is_id = nullptr;
+    c->tree_in_flight = false;
     c->last_cond = 255;
     c->profiling = 0;
     c->prof_open = false;
@@ -321,10 +322,16 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     return EVT_OK;
 }
 
-#define CTXCHK(c)                             \
-    do {                                      \
-        ARGCHK((c) != nullptr, "handle is NULL"); \
-        HIPCHK(hipSetDevice((c)->device));    \
+// every call on a handle but evt_grow_tree_end, evt_synchronize and evt_destroy waits for a tree begun with
+// evt_grow_tree_begin to be collected: its arrays sit in the handle's staging buffer until then
+#define CTXCHK(c)                                                                                      \
+    do {                                                                                               \
+        ARGCHK((c) != nullptr, "handle is NULL");                                                      \
+        HIPCHK(hipSetDevice((c)->device));                                                             \
+        if ((c)->tree_in_flight) {                                                                     \
+            evt_set_error("a tree begun with evt_grow_tree_begin has not been collected (evt_grow_tree_end)"); \
+            return EVT_ERR_STATE;                                                                      \
+        }                                                                                              \
     } while (0)
 
 static int check_errflag(evt_ctx *c, const char *what) {
@@ -520,8 +527,7 @@ extern "C" int evt_set_grads(evt_handle c, const float *grad) {
     return EVT_OK;
 }
 
-extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p,
-                             evt_tree_out *tree) {
+extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
     CTXCHK(c);
     ARGCHK(js && p, "js and params must not be NULL");
     ARGCHK(n_js >= 1 && n_js <= c->F, "n_js must be in [1, nfeats]");
@@ -581,6 +587,7 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
     if (r != EVT_OK) return r;
     if (!all_rows) {
         HIPCHK(hipMemcpyAsync(c->mask, mask, c->N, hipMemcpyDefault, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream)); // the caller may reuse its mask buffer as soon as this call returns
         r = launch_compact_mask(c, cond);
         if (r == EVT_OK && c->record_nidx) r = launch_fill_u32(c, c->nidx, 0u, c->N);
     }
@@ -641,12 +648,24 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
         c->nidx_valid = true;
     }
 
-    // read back the tree (and the per-level row counts) in one pinned transfer
+    // the tree (and the per-level row counts) comes back in one pinned transfer, queued behind the kernels
+    HIPCHK(hipMemcpyAsync(c->h_stage, c->tree_blob, c->blob_bytes, hipMemcpyDeviceToHost, c->stream));
+    c->tree_in_flight = true;
+    return EVT_OK;
+}
+
+extern "C" int evt_grow_tree_end(evt_handle c, evt_tree_out *tree) {
+    ARGCHK(c != nullptr, "handle is NULL");
+    HIPCHK(hipSetDevice(c->device));
+    if (!c->tree_in_flight) {
+        evt_set_error("evt_grow_tree_end without evt_grow_tree_begin");
+        return EVT_ERR_STATE;
+    }
+    c->tree_in_flight = false;
     const int nn = c->nnodes, K = c->K;
     uint8_t *hs = c->h_stage;
     const size_t o_feat = c->blob_feat, o_w = c->blob_w, o_gain = c->blob_gain, o_pred = c->blob_pred, o_stats = c->blob_stats,
                  o_bin = c->blob_bin, o_split = c->blob_split;
-    HIPCHK(hipMemcpyAsync(hs, c->tree_blob, c->blob_bytes, hipMemcpyDeviceToHost, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     const int64_t n_is = reinterpret_cast<const int64_t *>(hs + o_stats)[0];
     if (c->profiling) {
@@ -669,6 +688,13 @@ extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, co
         memcpy(tree->split, hs + o_split, nn);
     }
     return EVT_OK;
+}
+
+extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p,
+                             evt_tree_out *tree) {
+    const int r = evt_grow_tree_begin(c, mask, cond, js, n_js, p);
+    if (r != EVT_OK) return r;
+    return evt_grow_tree_end(c, tree);
 }
 
 // host tree -> packed device nodes; validates that every split node has both children in range
@@ -1096,7 +1122,8 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
     return EVT_OK;
 }
 extern "C" int evt_synchronize(evt_handle c) {
-    CTXCHK(c);
+    ARGCHK(c != nullptr, "handle is NULL");
+    HIPCHK(hipSetDevice(c->device));
     HIPCHK(hipStreamSynchronize(c->stream));
     return EVT_OK;
 }

@@ -130,6 +130,7 @@ struct evt_ctx {
     bool nidx_valid;   // nidx holds the last tree's node ids
     bool defer_pred;   // a tree grown on every row records leaf ids and leaves the addition to the next row-order pass
     bool write_nidx;   // the tree being grown records the node id of every row it places
+    bool tree_in_flight; // evt_grow_tree_begin has queued a tree that evt_grow_tree_end has not collected
     bool pend_pred;    // pred lacks the leaf values pend_leaf[nidx[i] - 1] of the last tree
     float *pend_leaf;  // [K * nnodes] leaf values of the tree whose addition is pending
     uint8_t last_cond;

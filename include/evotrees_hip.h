@@ -149,6 +149,15 @@ int evt_set_grads(evt_handle h, const float *grad);
  */
 int evt_grow_tree(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js,
                   const evt_params *params, evt_tree_out *tree);
+/* The same call in two halves, for a host that overlaps its own work of the next round (drawing the next row
+ * mask, src/subsample.jl:7; the reference's host does this between kernels of the device path,
+ * ext/.../subsample.jl:2-8) with the device growing this round's tree.  begin reads mask and js before it
+ * returns and queues all device work; end waits for it and fills the tree arrays (EVT_ERR_EMPTY when no row was
+ * kept).  Between the two, every other call on the handle except evt_synchronize and evt_destroy returns
+ * EVT_ERR_STATE.  evt_grow_tree is begin followed by end. */
+int evt_grow_tree_begin(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js,
+                        const evt_params *params);
+int evt_grow_tree_end(evt_handle h, evt_tree_out *tree);
 
 /* predict!(cache.pred, tree, cache.x_bin, feattypes): src/predict.jl:1-46; ext/.../predict.jl:60-75.
  * Adds one host tree (arrays of length nnodes_tree) to the cache's prediction. */

@@ -146,3 +146,51 @@ def test_deferred_leaf_addition_equals_immediate(evt, loss, K, tt):
             assert a == b
         else:
             assert_tree_bits(a, b)
+
+
+def test_grow_tree_in_two_halves(evt):
+    """evt_grow_tree_begin / evt_grow_tree_end give the trees and predictions of evt_grow_tree, bit for bit; between
+    the two halves the handle refuses every other call (and still answers afterwards); an end without a begin and an
+    empty subsample are reported by the half that knows."""
+    N, F, B, D = 40000, 11, 32, 6
+    x_bin, y, w, mu = make_data(91, N, F, B, "logloss", weights=True)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    gp = evt.make_params(eta=0.2)
+    rng_a, rng_b = np.random.default_rng(3), np.random.default_rng(3)
+
+    def make():
+        h = evt.Handle(N, F, B, 1, D, "logloss")
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        return h
+
+    ha, hb = make(), make()
+    for r in range(4):
+        sub = r % 2 == 1
+        ha.update_grads()
+        hb.update_grads()
+        ma = rng_a.integers(0, 256, N, dtype=np.uint8) if sub else None
+        mb = rng_b.integers(0, 256, N, dtype=np.uint8) if sub else None
+        ta = ha.grow_tree(js, gp, mask=ma, cond=140)
+        hb.grow_tree_begin(js, gp, mask=mb, cond=140)
+        if sub:
+            mb[:] = 0  # the mask has been read when begin returns
+        for call in (hb.update_grads, hb.get_pred, lambda: hb.eval_metric("logloss"), lambda: hb.grow_tree_begin(js, gp)):
+            with pytest.raises(evt.EvtError) as ei:
+                call()
+            assert ei.value.code == evt._lib.EVT_ERR_STATE
+        hb.synchronize()
+        tb = hb.grow_tree_end()
+        assert_tree_bits(ta, tb)
+    assert np.array_equal(ha.get_pred().view(np.uint32), hb.get_pred().view(np.uint32))
+    with pytest.raises(evt.EvtError) as ei:
+        hb.grow_tree_end()
+    assert ei.value.code == evt._lib.EVT_ERR_STATE
+    hb.update_grads()
+    hb.grow_tree_begin(js, gp, mask=np.full(N, 255, np.uint8), cond=10)  # keeps no row: the count is known at the end
+    with pytest.raises(evt.EvtError) as ei:
+        hb.grow_tree_end()
+    assert ei.value.code == evt._lib.EVT_ERR_EMPTY
+    hb.grow_tree(js, gp)  # the handle goes on working
+    ha.close()
+    hb.close()
