@@ -123,7 +123,7 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->obest, c->sbest, c->pend_leaf, c->is_id};
+                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->sbest, c->pend_leaf, c->is_id};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -181,7 +181,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->tree_blob = nullptr;
     memset(c->lvl, 0, sizeof(c->lvl));
     c->js = nullptr; c->jsmap = nullptr; c->feattypes = nullptr; c->mono = nullptr; c->absmax = nullptr; c->qexp = nullptr; c->qbits = nullptr;
-    c->qscale = nullptr; c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->obest = nullptr; c->sbest = nullptr;
+    c->qscale = nullptr; c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->sbest = nullptr;
     c->h_stage = nullptr; c->h_stage_bytes = 0;
     c->n_js_last = 0;
     c->last_all_rows = true;

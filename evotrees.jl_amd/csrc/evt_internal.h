@@ -111,7 +111,6 @@ struct evt_ctx {
     int64_t *stats;    // [D+1] rows built per level
     int32_t *errflag;  // device-side validation flag
     double *ogains;    // oblivious: [maxlvl][F][B]
-    double *obest;     // unused
     void *sbest;       // split search: best candidate per (node of the level, feature group), 16 B each
 
     // host staging (pinned)
