@@ -1106,7 +1106,7 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
         ARGCHK(value >= 0 && value <= 65536, "hist_seg_cost must be in [0, 65536]");
         c->hist_seg_cost = (int)value;
     } else if (strcmp(name, "hist_variant") == 0) {
-        ARGCHK(value >= 0 && value <= 2, "hist_variant must be 0 (auto), 1 (generic) or 2 (conflict-free)");
+        ARGCHK(value >= 0 && value <= 2, "hist_variant must be 0 (auto), 1 (generic) or 2 (conflict-free where it applies)");
         c->hist_variant = (int)value;
     } else if (strcmp(name, "record_nidx") == 0) {
         c->record_nidx = value != 0;

@@ -235,38 +235,45 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     }
 }
 
-// Bank-conflict-free variant for records of 128 / 256 / 512 bytes.
+// Bank-conflict-free variant for records of 32 / 64 / 128 / 256 / 512 bytes.
 //
-// A record is read as 8-byte pieces, NS = RS/8 lanes per row (a multiple of 16), so every group of
-// 16 consecutive lanes — the unit the LDS serves per cycle for 64-bit operations — holds 16 different
-// pieces `sub` of ONE row.  The LDS histogram is laid out as word(a, t, bin, sub) =
-// ((a*8 + t)*B + bin)*NS + sub for feature f = 8*sub + t, i.e. `sub` selects the bank pair, so the 16
-// lanes of a group always fall on 16 different bank pairs whatever their bins are.  Rows that share a
-// wave instruction sit in different groups and cannot collide inside one LDS pass either.
-// FULL: a lane adds all 8 bytes of its piece without testing which features are sampled.  A record's padding reads as
+// A record is read in pieces of PB bytes, one lane each, NS = RS/PB lanes per row with PB chosen so that NS is a
+// multiple of 16 (8-byte pieces from 128-byte records up, 4-byte pieces for 64-byte records, 2-byte pieces for
+// 32-byte ones): every group of 16 consecutive lanes - the unit the LDS serves per cycle for 64-bit operations -
+// holds 16 different pieces `sub` of ONE row.  The LDS histogram is laid out as word(a, t, bin, sub) =
+// ((a*PB + t)*B + bin)*NS + sub for feature f = PB*sub + t, i.e. `sub` selects the bank pair, so the 16 lanes of a
+// group always fall on 16 different bank pairs whatever their bins are.  Rows that share a wave instruction sit in
+// different groups and cannot collide inside one LDS pass either.  (Two 64-byte records per 16-lane group, 8 lanes of
+// 8-byte pieces each, collide whenever their bins' words share a bank half: cfg5's histograms took 0.64 ms per round
+// that way and take 0.41 ms with 4-byte pieces.)
+// FULL: a lane adds all PB bytes of its piece without testing which features are sampled.  A record's padding reads as
 // bin 1 and features outside the sample have LDS words of their own, so the extra adds land in words the flush clears
 // and never writes out; the per-feature test (FULL = false) only pays when most features are left out.
-// Q = record rows per 16-lane DPP row: 1 for records of 128 bytes and more, 2 for 64-byte records.  (32-byte records
-// were tried with Q = 4 and ran slower than the generic kernel: four broadcasts and three selects per value.)
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_row_bcast(uint32_t x) {
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xF, 0xF, false);
 }
-// value held by the fetcher lane of (group u, this lane's record row) inside this lane's DPP row
-template <int Q, int u>
-__device__ __forceinline__ uint32_t grp_bcast(uint32_t x, int hh) {
-    if constexpr (Q == 1) {
-        return dpp_row_bcast<0x150 + u>(x);
+// value held by lane u of this lane's DPP row: the fetcher of row group u
+template <int u>
+__device__ __forceinline__ uint32_t grp_bcast(uint32_t x) {
+    return dpp_row_bcast<0x150 + u>(x);
+}
+
+// A record piece of PB bytes in the low bytes of a register pair.
+template <int PB>
+__device__ __forceinline__ uint2 load_piece(const uint8_t *p) {
+    if constexpr (PB == 8) {
+        return *reinterpret_cast<const uint2 *>(p);
+    } else if constexpr (PB == 4) {
+        return make_uint2(*reinterpret_cast<const uint32_t *>(p), 0u);
     } else {
-        static_assert(Q == 2, "records of 64 bytes and more");
-        const uint32_t a = dpp_row_bcast<0x150 + 2 * u>(x), b = dpp_row_bcast<0x150 + 2 * u + 1>(x);
-        return hh ? b : a;
+        return make_uint2((uint32_t)*reinterpret_cast<const uint16_t *>(p), 0u);
     }
 }
 
-template <int NA, bool PACK, int U, bool FULL, int Q>
+template <int NA, bool PACK, int U, bool FULL, int PB>
 __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
-    extern __shared__ unsigned long long H[]; // [NA][8][B][NS]
+    extern __shared__ unsigned long long H[]; // [NA][PB][B][NS]
     const int tid = threadIdx.x, nthr = blockDim.x;
     const int lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
     const int n_build = (int)A.hdr[LH_N_BUILD];
@@ -274,7 +281,8 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     if (n_build <= 0 || total <= 0) return;
     if (blockIdx.x == 0 && tid == 0 && A.a0 == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
 
-    const int NS = A.RS >> 3;     // 8-byte pieces per record
+    static_assert(PB == 8 || PB == 4 || PB == 2, "a piece is 8, 4 or 2 bytes");
+    const int NS = A.RS / PB;     // pieces per record, one lane each
     const int RPW = 64 / NS;      // rows per wave instruction
     const int step = nwaves * RPW;
     int64_t T = (total + gridDim.x - 1) / gridDim.x;
@@ -285,17 +293,17 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     int64_t end = start + T < total ? start + T : total;
 
     const int B = A.B;
-    const int plane = 8 * B * NS; // words per channel
+    const int plane = PB * B * NS; // words per channel
     for (int i = tid; i < NA * plane; i += nthr) H[i] = 0ull;
 
     const int sub = lane % NS, rloc = lane / NS;
     // byte offset of (t, bin 0) for this lane; bins are 1-based so bin*NS*8 is added on top
     // (32-bit unsigned arithmetic throughout: one 24-bit multiply-add per LDS address)
-    uint32_t coff[8];
+    uint32_t coff[PB];
     unsigned vmask = 0;
 #pragma unroll
-    for (int t = 0; t < 8; t++) {
-        const int f = sub * 8 + t;
+    for (int t = 0; t < PB; t++) {
+        const int f = sub * PB + t;
         const bool ok = (f < A.F) && (A.jsmap[f] != 0xFFFF);
         coff[t] = (uint32_t)(((t * B - 1) * NS + sub) * 8);
         vmask |= ok ? (1u << t) : 0u;
@@ -341,12 +349,11 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             const uint32_t *isp = A.is + seg;
             const int64_t lastp = nend - 1;          // >= start
             int64_t pw = start + (int64_t)wave * SR; // first position of this wave's iteration
-            // lane j of DPP row r fetches for group j / Q the record row r * Q + j % Q of that group
-            const int myu = (lane & 15) / Q;
-            // (a record wider than a DPP row, Q == 1, is fetched for by every DPP row it covers: its own row rloc)
-            const int mypos = myu * RPW + (Q == 1 ? rloc : (lane >> 4) * Q + (lane & 15) % Q); // position (within the iteration) this lane fetches
+            // lane j of a DPP row fetches for row group j the row its DPP row belongs to (a record wider than a DPP row is
+            // fetched for by every DPP row it covers)
+            const int myu = lane & 15;
+            const int mypos = myu * RPW + rloc; // position (within the iteration) this lane fetches
             const bool fetcher = myu < U;
-            const int hh = (lane & 15) / NS;         // this lane's record row inside its DPP row (0 when Q == 1)
             uint32_t idc, idn;
             unsigned long long gc[NA], gn[NA];
             uint2 v[U];
@@ -363,8 +370,8 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             __builtin_amdgcn_sched_barrier(0);
 #define EVT_H16_PRO(u_)                                                                                               \
     if constexpr ((u_) < U) {                                                                                         \
-        const uint32_t row = grp_bcast<Q, (u_) < U ? (u_) : 0>(idc, hh);                                               \
-        v[(u_) < U ? (u_) : 0] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)row * A.RS + sub * 8);                 \
+        const uint32_t row = grp_bcast<(u_) < U ? (u_) : 0>(idc);                                               \
+        v[(u_) < U ? (u_) : 0] = load_piece<PB>(A.xrm + (size_t)row * A.RS + sub * PB);                 \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
             EVT_H16_PRO(0) EVT_H16_PRO(1) EVT_H16_PRO(2) EVT_H16_PRO(3) EVT_H16_PRO(4) EVT_H16_PRO(5) EVT_H16_PRO(6) EVT_H16_PRO(7)
@@ -386,13 +393,13 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         {                                                                                                             \
             unsigned long long gg[NA];                                                                                \
             _Pragma("unroll") for (int a = 0; a < NA; a++) {                                                          \
-                const uint32_t glo = grp_bcast<Q, ui>((uint32_t)gc[a], hh);                                            \
-                const uint32_t ghi = grp_bcast<Q, ui>((uint32_t)(gc[a] >> 32), hh);                                    \
+                const uint32_t glo = grp_bcast<ui>((uint32_t)gc[a]);                                            \
+                const uint32_t ghi = grp_bcast<ui>((uint32_t)(gc[a] >> 32));                                    \
                 gg[a] = ((unsigned long long)ghi << 32) | glo;                                                         \
             }                                                                                                         \
             if (lane_on && (pw + (u_) * RPW + rloc < nend)) {                                                          \
                 const uint32_t wds[2] = {v[ui].x, v[ui].y};                                                            \
-                _Pragma("unroll") for (int t = 0; t < 8; t++) {                                                        \
+                _Pragma("unroll") for (int t = 0; t < PB; t++) {                                                       \
                     if (FULL || (vmask & (1u << t))) {                                                                \
                         const uint32_t bo = __umul24((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu, binmul) + coff[t];       \
                         _Pragma("unroll") for (int a = 0; a < NA; a++)                                                 \
@@ -401,8 +408,8 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                 }                                                                                                     \
             }                                                                                                         \
         }                                                                                                             \
-        const uint32_t row = grp_bcast<Q, ui>(idn, hh);                                                                \
-        v[ui] = *reinterpret_cast<const uint2 *>(A.xrm + (size_t)row * A.RS + sub * 8);                                \
+        const uint32_t row = grp_bcast<ui>(idn);                                                                \
+        v[ui] = load_piece<PB>(A.xrm + (size_t)row * A.RS + sub * PB);                                \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
                 EVT_H16_STEP(0) EVT_H16_STEP(1) EVT_H16_STEP(2) EVT_H16_STEP(3) EVT_H16_STEP(4) EVT_H16_STEP(5) EVT_H16_STEP(6) EVT_H16_STEP(7)
@@ -421,7 +428,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         const bool sole = (nbeg >= blk_start) && (nrows_end <= blk_end) && !(PACK && nrows_end - nbeg > EVT_HIST_MAX_ROWS_PER_BLOCK);
         long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
         const int nchunks = (B + 7) >> 3;
-        const int nitems = NA * 8 * nchunks * NS * 8; // (channel, t, bin chunk, piece, bin in chunk), the last fastest
+        const int nitems = NA * PB * nchunks * NS * 8; // (channel, t, bin chunk, piece, bin in chunk), the last fastest
         const int rot = (int)(((int64_t)blockIdx.x * 1031) % (nitems >> 6)) << 6;
         // FU items per thread at a time: their LDS words (and, when features are sampled, their slots) are all
         // requested before the first is used, so a flush costs one LDS and one memory round trip, not FU of each
@@ -454,10 +461,10 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                         chunk = rest % nchunks;
                         rest /= nchunks;
                     }
-                    const int t = rest & 7;
-                    const int a = rest >> 3;
+                    const int t = rest & (PB - 1);
+                    const int a = rest / PB;
                     const int b = chunk * 8 + bl;
-                    const int f = sidx * 8 + t;
+                    const int f = sidx * PB + t;
                     if (b < B) {
                         hwv[j] = &H[(size_t)a * plane + ((size_t)t * B + b) * NS + sidx];
                         wv[j] = *hwv[j];
@@ -501,7 +508,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     }
 }
 
-template <int NA, bool PACK, int U, int Q>
+template <int NA, bool PACK, int U, int PB>
 static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
     // unpredicated atomics for every feature of the record pay off unless most features are left out: the words of
     // features outside the sample are simply not flushed
@@ -509,15 +516,15 @@ static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads
     if (lds > 64 * 1024) { // one block per CU may take most of its 160 KB
         static bool attr_set = false;
         if (!attr_set) {
-            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, true, Q>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, false, Q>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, true, PB>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, false, PB>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
             attr_set = true;
         }
     }
     if (full)
-        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, true, Q>), grid, dim3(threads), lds, c->stream, A);
+        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, true, PB>), grid, dim3(threads), lds, c->stream, A);
     else
-        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, false, Q>), grid, dim3(threads), lds, c->stream, A);
+        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, false, PB>), grid, dim3(threads), lds, c->stream, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -525,8 +532,10 @@ static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads
 template <int NA, bool PACK>
 static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
     // row groups (records) in flight per wave: as many as a DPP row can address, fewer when registers run out
-    if (c->RS >= 128) return launch_hist16_q<NA, PACK, (NA <= 2) ? 16 : 8, 1>(c, A, grid, threads, lds);
-    return launch_hist16_q<NA, PACK, 8, 2>(c, A, grid, threads, lds); // 64-byte records
+    constexpr int U = (NA <= 2) ? 16 : 8;
+    if (c->RS >= 128) return launch_hist16_q<NA, PACK, U, 8>(c, A, grid, threads, lds);
+    if (c->RS == 64) return launch_hist16_q<NA, PACK, U, 4>(c, A, grid, threads, lds);
+    return launch_hist16_q<NA, PACK, U, 2>(c, A, grid, threads, lds); // 32-byte records
 }
 
 template <int NA, bool PACK>
@@ -587,9 +596,10 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
         A.slots_per_tile = slots_per_tile;
         const size_t lds = per_slot * slots_per_tile;
         dim3 grid((unsigned)blocks, (unsigned)ntiles);
-        // conflict-free variant: records of 64 to 512 bytes (8 to 64 lanes per row) whose whole LDS histogram fits
-        const size_t lds16 = (size_t)na * 8 * c->B * (c->RS / 8) * 8;
-        const bool can16 = (c->RS == 64 || c->RS == 128 || c->RS == 256 || c->RS == 512) &&
+        // conflict-free variant: records of 32 to 512 bytes (16 to 64 lanes per row) whose whole LDS histogram fits
+        // (16-byte records as 1-byte pieces were measured: no faster than the generic kernel)
+        const size_t lds16 = (size_t)na * c->B * c->RS * 8; // channels x bins x (pieces x bytes per piece) words
+        const bool can16 = (c->RS == 32 || c->RS == 64 || c->RS == 128 || c->RS == 256 || c->RS == 512) &&
                            lds16 <= 128 * 1024;
         const bool use16 = (c->hist_variant == 1) ? false : can16;
         int r = EVT_ERR_ARG;
