@@ -35,6 +35,7 @@ struct HistArgs {
     int64_t N;
     int64_t node_stride;
     int RS, LPR, RPW, F, nfs, B, NAg, level;
+    int NSL; // conflict-free kernel: lanes per row, the power of two >= 16 that covers a record's pieces
     int slots_per_tile;
     int min_rows;
     int seg_cost;
@@ -282,7 +283,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     if (blockIdx.x == 0 && tid == 0 && A.a0 == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
 
     static_assert(PB == 8 || PB == 4 || PB == 2, "a piece is 8, 4 or 2 bytes");
-    const int NS = A.RS / PB;     // pieces per record, one lane each
+    const int NS = A.NSL;         // lanes per row: one per piece of the record, idle ones beyond its last piece
     const int RPW = 64 / NS;      // rows per wave instruction
     const int step = nwaves * RPW;
     int64_t T = (total + gridDim.x - 1) / gridDim.x;
@@ -297,6 +298,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     for (int i = tid; i < NA * plane; i += nthr) H[i] = 0ull;
 
     const int sub = lane % NS, rloc = lane / NS;
+    const int subl = (sub * PB < A.RS) ? sub : 0; // an idle lane loads the row's first piece and adds nothing (no feature: vmask 0)
     // byte offset of (t, bin 0) for this lane; bins are 1-based so bin*NS*8 is added on top
     // (32-bit unsigned arithmetic throughout: one 24-bit multiply-add per LDS address)
     uint32_t coff[PB];
@@ -371,7 +373,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
 #define EVT_H16_PRO(u_)                                                                                               \
     if constexpr ((u_) < U) {                                                                                         \
         const uint32_t row = grp_bcast<(u_) < U ? (u_) : 0>(idc);                                               \
-        v[(u_) < U ? (u_) : 0] = load_piece<PB>(A.xrm + (size_t)row * A.RS + sub * PB);                 \
+        v[(u_) < U ? (u_) : 0] = load_piece<PB>(A.xrm + (size_t)row * A.RS + subl * PB);                \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
             EVT_H16_PRO(0) EVT_H16_PRO(1) EVT_H16_PRO(2) EVT_H16_PRO(3) EVT_H16_PRO(4) EVT_H16_PRO(5) EVT_H16_PRO(6) EVT_H16_PRO(7)
@@ -409,7 +411,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             }                                                                                                         \
         }                                                                                                             \
         const uint32_t row = grp_bcast<ui>(idn);                                                                \
-        v[ui] = load_piece<PB>(A.xrm + (size_t)row * A.RS + sub * PB);                                \
+        v[ui] = load_piece<PB>(A.xrm + (size_t)row * A.RS + subl * PB);                               \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
                 EVT_H16_STEP(0) EVT_H16_STEP(1) EVT_H16_STEP(2) EVT_H16_STEP(3) EVT_H16_STEP(4) EVT_H16_STEP(5) EVT_H16_STEP(6) EVT_H16_STEP(7)
@@ -596,11 +598,15 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
         A.slots_per_tile = slots_per_tile;
         const size_t lds = per_slot * slots_per_tile;
         dim3 grid((unsigned)blocks, (unsigned)ntiles);
-        // conflict-free variant: records of 32 to 512 bytes (16 to 64 lanes per row) whose whole LDS histogram fits
+        // conflict-free variant: 16, 32 or 64 lanes per row - records of 32 to 512 bytes; a size that is not a power of two
+        // takes the next one's lanes and leaves the ones past its last piece idle - whose whole LDS histogram fits
         // (16-byte records as 1-byte pieces were measured: no faster than the generic kernel)
-        const size_t lds16 = (size_t)na * c->B * c->RS * 8; // channels x bins x (pieces x bytes per piece) words
-        const bool can16 = (c->RS == 32 || c->RS == 64 || c->RS == 128 || c->RS == 256 || c->RS == 512) &&
-                           lds16 <= 128 * 1024;
+        const int pb16 = c->RS >= 128 ? 8 : (c->RS == 64 ? 4 : 2);
+        int nsl = 16;
+        while (nsl * pb16 < c->RS) nsl <<= 1;
+        A.NSL = nsl;
+        const size_t lds16 = (size_t)na * c->B * pb16 * nsl * 8; // channels x bins x (lanes x bytes per piece) words
+        const bool can16 = c->RS >= 32 && nsl <= 64 && lds16 <= 128 * 1024;
         const bool use16 = (c->hist_variant == 1) ? false : can16;
         int r = EVT_ERR_ARG;
         if (use16) {
