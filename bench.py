@@ -233,7 +233,7 @@ def main():
     nb = max(1, extra)
     kernels = {k: {"ms_per_round": round(v["ms"] / nb, 4), "launches_per_round": v["launches"] / nb} for k, v in prof_all.items()}
     if prof_all["grad"]["ms"] > 0:
-        gb = N * (4 * K + 4 + 4 + 8 * K)
+        gb = N * (4 * K + 4 + 8 * K)  # pred, y read; g, h written (unit weights: the weight row is not read)
         if cfg["rowsample"] >= 1.0:
             gb += N * (4 + 4 * K)  # the last tree's leaf values are added in the same pass: node id read, prediction written
         kernels["grad"]["GBps"] = round(gb * nb / (prof_all["grad"]["ms"] * 1e-3) / 1e9, 1)

@@ -24,7 +24,7 @@ __device__ __forceinline__ float dev_softplus(float x) { return fmaxf(x, 0.0f) +
 template <int LOSS>
 __global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const float *__restrict__ y, float *__restrict__ grad, int64_t N,
                                               uint32_t *absmax, const uint32_t *__restrict__ pend_nidx,
-                                              const float *__restrict__ pend_leaf) {
+                                              const float *__restrict__ pend_leaf, int unit_w) {
     constexpr int K = (LOSS == 2) ? 2 : 1;
     constexpr int NK = 2 * K + 1;
     float mx[2 * K];
@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const f
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
         float out[2 * K];
         float *g = grad + (size_t)NK * i;
-        const float w = g[NK - 1];
+        const float w = unit_w ? 1.0f : g[NK - 1]; // unit weights: the weight row (all ones) is not read
         if (pend_nidx) evt_add_leaf(pred + (size_t)K * i, pend_leaf + (size_t)K * (pend_nidx[i] - 1), K, LOSS);
         if (LOSS == 0) {
             const float gg = 2.0f * (pred[i] - y[i]);
@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const f
 // h_k = prob_k (1 - prob_k) w; y holds the 1-based class.  The row maxima are reduced one gradient row at a time.
 __global__ __launch_bounds__(256) void k_grads_mlogloss(float *__restrict__ pred, const float *__restrict__ y, float *__restrict__ grad,
                                                        int64_t N, int K, uint32_t *absmax, const uint32_t *__restrict__ pend_nidx,
-                                                       const float *__restrict__ pend_leaf) {
+                                                       const float *__restrict__ pend_leaf, int unit_w) {
     const int NK = 2 * K + 1;
     __shared__ float s_m[4];
     float mx[2 * EVT_MAX_K];
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(256) void k_grads_mlogloss(float *__restrict__ pred
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
         float *pr = pred + (size_t)K * i;
         float *g = grad + (size_t)NK * i;
-        const float w = g[NK - 1];
+        const float w = unit_w ? 1.0f : g[NK - 1]; // unit weights: the weight row (all ones) is not read
         const int cls = (int)y[i];
         if (pend_nidx) evt_add_leaf(pr, pend_leaf + (size_t)K * (pend_nidx[i] - 1), K, EVT_LOSS_MLOGLOSS);
         float e[EVT_MAX_K];
@@ -209,19 +209,19 @@ int launch_grads(evt_ctx *c) {
     const uint32_t *pn = c->pend_pred ? c->nidx : nullptr; // the last tree's leaf values are added on the way
     c->pend_pred = false;
     if (c->loss == EVT_LOSS_MSE)
-        hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
+        hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_LOGLOSS)
-        hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
+        hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_GAUSSIAN_MLE)
-        hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
+        hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_POISSON)
-        hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
+        hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_GAMMA)
-        hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
+        hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_MLOGLOSS)
-        hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->pend_leaf);
+        hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
     else
-        hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf);
+        hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
