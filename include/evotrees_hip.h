@@ -131,7 +131,8 @@ int evt_set_feature_meta(evt_handle h, const uint8_t *feattypes, const int32_t *
 int evt_update_grads(evt_handle h);
 
 /* Overwrites the gradient matrix ((2K+1) x nobs Float32, weight row included) — used to feed
- * identical gradients to the library and to a CPU run. */
+ * identical gradients to the library and to a CPU run.  The weight row must agree with evt_set_target:
+ * all ones when that call got w == NULL (the row count then stands for the weight everywhere). */
 int evt_set_grads(evt_handle h, const float *grad);
 
 /*
