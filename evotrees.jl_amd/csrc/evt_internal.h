@@ -137,6 +137,7 @@ struct evt_ctx {
     // profiling
     int profiling;     // bit mask of kernel classes timed with events
     bool prof_open;
+    hipEvent_t launch_e0, launch_e1; // events the next histogram launch carries itself (nullptr: none)
     std::vector<ProfRec> recs;
     std::vector<hipEvent_t> free_events;
     int64_t prof_launches[EVT_K_COUNT];
@@ -227,4 +228,5 @@ int launch_nidx_from_tree(evt_ctx *c, bool use_mask, uint8_t cond);
 
 // profiling helpers
 void prof_begin(evt_ctx *c, int cls, int level);
+void prof_begin_launch(evt_ctx *c, int cls, int level);
 void prof_end(evt_ctx *c);

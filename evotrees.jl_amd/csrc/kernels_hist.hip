@@ -20,6 +20,7 @@
 //
 // Algorithmic HBM bytes per built row: RS-or-F bin bytes + 8*NA staged gradient bytes + 4 row-id bytes.
 #include "evt_internal.h"
+#include <hip/hip_ext.h>
 
 struct HistArgs {
     const uint8_t *xrm;
@@ -523,10 +524,11 @@ static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads
             attr_set = true;
         }
     }
+    // c->launch_e0 / launch_e1 (when profiling): the kernel's own dispatch records them
     if (full)
-        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, true, PB>), grid, dim3(threads), lds, c->stream, A);
+        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, true, PB>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
     else
-        hipLaunchKernelGGL((k_hist_build16<NA, PACK, U, false, PB>), grid, dim3(threads), lds, c->stream, A);
+        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, false, PB>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -547,7 +549,7 @@ static int launch_hist_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, 
         HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build<NA, PACK>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         attr_set = true;
     }
-    hipLaunchKernelGGL((k_hist_build<NA, PACK>), grid, dim3(threads), lds, c->stream, A);
+    hipExtLaunchKernelGGL((k_hist_build<NA, PACK>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -582,6 +584,13 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
     const int64_t blocks = c->hist_blocks;
     // accumulator channels are taken EVT_HIST_GROUP at a time (one launch each; the one- and two-output losses need
     // a single launch); the packed row counter rides on channel 0, i.e. in the first group only
+    // timing events: one launch carries them itself; several launches (channel groups) are bracketed by event records
+    const bool one_launch = c->NA <= EVT_MAX_NA;
+    hipEvent_t ev0 = c->launch_e0, ev1 = c->launch_e1;
+    if (!one_launch) {
+        c->launch_e0 = c->launch_e1 = nullptr;
+        if (ev0) (void)hipEventRecord(ev0, c->stream);
+    }
     for (int a0 = 0; a0 < c->NA; a0 += (c->NA <= EVT_MAX_NA ? EVT_MAX_NA : EVT_HIST_GROUP)) {
         const int na = (c->NA <= EVT_MAX_NA) ? c->NA : (c->NA - a0 < EVT_HIST_GROUP ? c->NA - a0 : EVT_HIST_GROUP);
         A.a0 = a0;
@@ -638,6 +647,7 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
             return r;
         }
     }
+    if (!one_launch && ev1) (void)hipEventRecord(ev1, c->stream);
     return EVT_OK;
 }
 
