@@ -186,6 +186,7 @@ def main():
         nxt[0] = draw_mask()
         evt._lib.check(L.evt_grow_tree_end(h._h, tree_out))
 
+    h.set_option("grads_ahead", 1)  # one tree per round: the next round's gradients are queued behind the tree
     for _ in range(args.warmup):
         one_round()
     h.synchronize()

@@ -262,6 +262,8 @@ def init(config, x_train, y_train, w_train=None, offset_train=None, feature_name
     m = EvoTree(config.loss, K, [Tree.bias(mu)], info)
     nfs = int(np.ceil(config.colsample * F))
     params = make_params(config.eta, config.L2, config.lambda_, config.gamma, config.min_weight, config.bagging_size, True)
+    if config.bagging_size == 1:
+        h.set_option("grads_ahead", 1)  # the next round's gradient update runs while the host collects the tree
     return m, Cache(h, rng, nfs, params, N, F, config)
 
 

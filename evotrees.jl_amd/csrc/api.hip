@@ -93,17 +93,26 @@ void prof_end(evt_ctx *c) {
 }
 // after a stream sync: fold finished event pairs into the per-class totals
 static void prof_collect(evt_ctx *c, const int64_t *stats_host) {
+    std::vector<ProfRec> later; // pairs whose kernels are still queued (work placed behind the point the host waited for)
     for (auto &r : c->recs) {
         float ms = 0.0f;
-        if (hipEventElapsedTime(&ms, r.e0, r.e1) == hipSuccess) {
+        const hipError_t e = hipEventElapsedTime(&ms, r.e0, r.e1);
+        if (e == hipErrorNotReady) {
+            (void)hipGetLastError();
+            later.push_back(r);
+            continue;
+        }
+        if (e == hipSuccess) {
             c->prof_launches[r.cls] += 1;
             c->prof_ms[r.cls] += (double)ms;
             if (r.cls == EVT_K_HIST && stats_host && r.level >= 1) c->prof_units[r.cls] += stats_host[r.level];
+        } else {
+            (void)hipGetLastError();
         }
         c->free_events.push_back(r.e0);
         c->free_events.push_back(r.e1);
     }
-    c->recs.clear();
+    c->recs.swap(later);
 }
 
 template <typename T>
@@ -145,7 +154,7 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->sbest, c->pend_leaf, c->is_id};
+                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -160,6 +169,7 @@ extern "C" int evt_destroy(evt_handle c) {
         (void)hipEventDestroy(r.e1);
     }
     for (auto e : c->free_events) (void)hipEventDestroy(e);
+    if (c->tree_ev) (void)hipEventDestroy(c->tree_ev);
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
     return EVT_OK;
@@ -204,7 +214,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     memset(c->lvl, 0, sizeof(c->lvl));
     c->js = nullptr; c->jsmap = nullptr; c->feattypes = nullptr; c->mono = nullptr; c->absmax = nullptr; c->qexp = nullptr; c->qbits = nullptr;
     c->qscale = nullptr; c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->sbest = nullptr;
-    c->h_stage = nullptr; c->h_stage_bytes = 0;
+    c->h_stage = nullptr; c->h_stage_dev = nullptr; c->h_stage_bytes = 0;
     c->n_js_last = 0;
     c->last_all_rows = true;
     // one block of 16 waves per CU: as many waves as two blocks of 8 (the LDS histogram caps a CU at 128 KB), half
@@ -219,9 +229,11 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->defer_pred = true;
     c->write_nidx = false;
     c->pend_pred = false;
-    c->pend_leaf = nullptr;
     c->is_id = nullptr;
     c->tree_in_flight = false;
+    c->tree_ev = nullptr;
+    c->grads_ahead = false;
+    c->grads_ready = false;
     c->last_cond = 255;
     c->profiling = 0;
     c->prof_open = false;
@@ -236,8 +248,10 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     }
     hipError_t e = hipGetDevice(&c->device);
     if (e == hipSuccess) e = hipStreamCreate(&c->stream);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->tree_ev, hipEventDisableTiming);
     if (e != hipSuccess) {
         evt_set_error("stream creation failed: %s", hipGetErrorString(e));
+        if (c->stream) (void)hipStreamDestroy(c->stream);
         delete c;
         return EVT_ERR_HIP;
     }
@@ -254,7 +268,6 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->is_b, N);
     ALLOC(c->is_id, N);
     ALLOC(c->nidx, N);
-    ALLOC(c->pend_leaf, (size_t)c->nnodes * K);
     ALLOC(c->mask, N);
     ALLOC(c->flagw, (size_t)c->max_chunks * EVT_CHUNK_WORDS);
     ALLOC(c->chunk_nleft, c->max_chunks + 1);
@@ -316,6 +329,11 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
         evt_set_error("hipHostMalloc failed");
         evt_destroy(c);
         return EVT_ERR_NOMEM;
+    }
+    if (hipHostGetDevicePointer((void **)&c->h_stage_dev, c->h_stage, 0) != hipSuccess) {
+        evt_set_error("pinned staging buffer is not addressable from the device");
+        evt_destroy(c);
+        return EVT_ERR_HIP;
     }
     // defaults: all numeric, no monotone constraint
     {
@@ -456,6 +474,7 @@ extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, cons
     c->have_target = false;
     c->have_grads = false;
     c->pend_pred = false; // the predictions start again from mu
+    c->grads_ready = false;
     c->unit_w = (w == nullptr);
     set_channels(c);
     HIPCHK(hipMemcpyAsync(c->y, y, sizeof(float) * c->N, hipMemcpyDefault, c->stream));
@@ -514,12 +533,7 @@ extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, cons
     return EVT_OK;
 }
 
-extern "C" int evt_update_grads(evt_handle c) {
-    CTXCHK(c);
-    if (!c->have_target) {
-        evt_set_error("evt_set_target must be called before evt_update_grads");
-        return EVT_ERR_STATE;
-    }
+static int queue_grads(evt_ctx *c) {
     prof_begin(c, EVT_K_GRAD, 0);
     int r = launch_grads(c);
     prof_end(c);
@@ -528,6 +542,21 @@ extern "C" int evt_update_grads(evt_handle c) {
     prof_begin(c, EVT_K_OTHER, 0);
     r = launch_quantize(c);
     prof_end(c);
+    return r;
+}
+
+extern "C" int evt_update_grads(evt_handle c) {
+    CTXCHK(c);
+    if (!c->have_target) {
+        evt_set_error("evt_set_target must be called before evt_update_grads");
+        return EVT_ERR_STATE;
+    }
+    if (c->grads_ready) { // queued behind the last tree ("grads_ahead"): the predictions have not changed since
+        c->grads_ready = false;
+        c->have_grads = true;
+        return EVT_OK;
+    }
+    const int r = queue_grads(c);
     if (r != EVT_OK) return r;
     c->have_grads = true;
     return EVT_OK;
@@ -540,6 +569,7 @@ extern "C" int evt_set_grads(evt_handle c, const float *grad) {
         evt_set_error("evt_set_target must be called before evt_set_grads");
         return EVT_ERR_STATE;
     }
+    c->grads_ready = false;
     HIPCHK(hipMemcpyAsync(c->grad, grad, sizeof(float) * (size_t)c->N * c->NK, hipMemcpyDefault, c->stream));
     int r = launch_absmax_rows(c, 0, c->NK);
     if (r != EVT_OK) return r;
@@ -579,6 +609,7 @@ extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t co
     // rows kept by the mask (the host owns the RNG; src/subsample.jl:7-9).  The threshold, the count and the
     // compaction run on the device; the count comes back with the finished tree.
     const bool all_rows = (mask == nullptr) || (cond == 255);
+    c->grads_ready = false; // this tree changes the predictions
     c->last_all_rows = all_rows;
     c->last_cond = cond;
     c->nidx_valid = c->record_nidx;
@@ -665,14 +696,20 @@ extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t co
         if (c->profiling) c->prof_units[EVT_K_PREDICT] += c->N;
     }
     if (defer) {
-        HIPCHK(hipMemcpyAsync(c->pend_leaf, c->tree_blob + c->blob_pred, sizeof(float) * (size_t)c->nnodes * c->K, hipMemcpyDeviceToDevice,
-                              c->stream));
         c->pend_pred = true;
         c->nidx_valid = true;
     }
 
     // the tree (and the per-level row counts) comes back in one pinned transfer, queued behind the kernels
-    HIPCHK(hipMemcpyAsync(c->h_stage, c->tree_blob, c->blob_bytes, hipMemcpyDeviceToHost, c->stream));
+    r = launch_copy_to_host(c, c->tree_blob, c->h_stage_dev, c->blob_bytes);
+    if (r != EVT_OK) return r;
+    HIPCHK(hipEventRecord(c->tree_ev, c->stream));
+    if (c->grads_ahead && p->update_pred) {
+        // the next round's gradient update runs while the host collects this tree and prepares the next call
+        r = queue_grads(c);
+        if (r != EVT_OK) return r;
+        c->grads_ready = true;
+    }
     c->tree_in_flight = true;
     return EVT_OK;
 }
@@ -689,7 +726,7 @@ extern "C" int evt_grow_tree_end(evt_handle c, evt_tree_out *tree) {
     uint8_t *hs = c->h_stage;
     const size_t o_feat = c->blob_feat, o_w = c->blob_w, o_gain = c->blob_gain, o_pred = c->blob_pred, o_stats = c->blob_stats,
                  o_bin = c->blob_bin, o_split = c->blob_split;
-    HIPCHK(hipStreamSynchronize(c->stream));
+    HIPCHK(hipEventSynchronize(c->tree_ev)); // the tree has arrived; work queued behind it may still be running
     const int64_t n_is = reinterpret_cast<const int64_t *>(hs + o_stats)[0];
     if (c->profiling) {
         c->prof_units[EVT_K_PARTITION] += n_is;
@@ -747,6 +784,7 @@ extern "C" int evt_predict_tree(evt_handle c, int32_t nnodes_tree, const int64_t
     if (r != EVT_OK) return r;
     r = launch_apply_pending(c);
     if (r != EVT_OK) return r;
+    c->grads_ready = false; // the predictions change
     uint32_t *d_nodes = nullptr;
     float *d_pred = nullptr;
     HIPCHK(hipMalloc((void **)&d_nodes, sizeof(uint32_t) * nnodes_tree));
@@ -1131,6 +1169,9 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
     } else if (strcmp(name, "hist_variant") == 0) {
         ARGCHK(value >= 0 && value <= 2, "hist_variant must be 0 (auto), 1 (generic) or 2 (conflict-free where it applies)");
         c->hist_variant = (int)value;
+    } else if (strcmp(name, "grads_ahead") == 0) {
+        c->grads_ahead = value != 0;
+        if (!c->grads_ahead) c->grads_ready = false;
     } else if (strcmp(name, "record_nidx") == 0) {
         c->record_nidx = value != 0;
     } else if (strcmp(name, "defer_pred") == 0) {

@@ -115,6 +115,7 @@ struct evt_ctx {
 
     // host staging (pinned)
     uint8_t *h_stage;
+    uint8_t *h_stage_dev; // the same pinned buffer as the device addresses it: the finished tree is written there by a kernel
     size_t h_stage_bytes;
     int32_t h_qbits[EVT_MC_MAX_NK];
     int32_t n_js_last;
@@ -129,9 +130,11 @@ struct evt_ctx {
     bool nidx_valid;   // nidx holds the last tree's node ids
     bool defer_pred;   // a tree grown on every row records leaf ids and leaves the addition to the next row-order pass
     bool write_nidx;   // the tree being grown records the node id of every row it places
+    bool grads_ahead;    // option: a tree with update_pred queues the next gradient update behind itself
+    bool grads_ready;    // the gradients of the predictions as they stand were computed ahead: evt_update_grads has nothing to do
+    hipEvent_t tree_ev;  // recorded behind the tree's transfer to the host: evt_grow_tree_end waits for this, not for the stream
     bool tree_in_flight; // evt_grow_tree_begin has queued a tree that evt_grow_tree_end has not collected
-    bool pend_pred;    // pred lacks the leaf values pend_leaf[nidx[i] - 1] of the last tree
-    float *pend_leaf;  // [K * nnodes] leaf values of the tree whose addition is pending
+    bool pend_pred;    // pred lacks the leaf values tree.pred[nidx[i] - 1] of the last tree (the device Tree arrays keep them until the next tree starts, and what is pending is applied before that)
     uint8_t last_cond;
 
     // profiling
@@ -219,6 +222,7 @@ int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_level_next(evt_ctx *c, int level);
 int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred);
 int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred);
+int launch_copy_to_host(evt_ctx *c, const void *src_dev, void *dst_host_dev, size_t nbytes);
 int launch_fill_u32(evt_ctx *c, uint32_t *dst, uint32_t v, int64_t n);
 int launch_fill_bytes(evt_ctx *c, void *dst, int64_t nbytes);
 // predict

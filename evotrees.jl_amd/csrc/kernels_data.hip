@@ -80,6 +80,23 @@ int launch_iota(evt_ctx *c, uint32_t *dst, int64_t n) {
     return EVT_OK;
 }
 
+// Small device -> pinned host copies by a kernel (16-byte words; nbytes is a multiple of 16).  A stream-ordered
+// hipMemcpyAsync goes through the copy engine, and handing the stream over to it and back stalls the kernels queued
+// behind it for tens of microseconds; a kernel's stores over the bus do not.
+__global__ __launch_bounds__(256) void k_copy_to_host(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = src[i];
+}
+int launch_copy_to_host(evt_ctx *c, const void *src_dev, void *dst_host_dev, size_t nbytes) {
+    const int64_t n = (int64_t)(nbytes / 16);
+    if (n <= 0) return EVT_OK;
+    int64_t nb = (n + 255) / 256;
+    if (nb > 64) nb = 64;
+    hipLaunchKernelGGL(k_copy_to_host, dim3((unsigned)nb), dim3(256), 0, c->stream, static_cast<const uint4 *>(src_dev),
+                       static_cast<uint4 *>(dst_host_dev), n);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
 __global__ __launch_bounds__(256) void k_fill_u32(uint32_t *dst, uint32_t v, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = v;
 }

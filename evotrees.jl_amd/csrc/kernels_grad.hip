@@ -209,19 +209,19 @@ int launch_grads(evt_ctx *c) {
     const uint32_t *pn = c->pend_pred ? c->nidx : nullptr; // the last tree's leaf values are added on the way
     c->pend_pred = false;
     if (c->loss == EVT_LOSS_MSE)
-        hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_LOGLOSS)
-        hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_GAUSSIAN_MLE)
-        hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_POISSON)
-        hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_GAMMA)
-        hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_MLOGLOSS)
-        hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else
-        hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->pend_leaf, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -237,7 +237,7 @@ int launch_apply_pending(evt_ctx *c) {
     if (!c->pend_pred) return EVT_OK;
     int64_t nb = (c->N + 255) / 256;
     if (nb > 4096) nb = 4096;
-    hipLaunchKernelGGL(k_apply_leaf, dim3((unsigned)nb), dim3(256), 0, c->stream, c->pred, c->nidx, c->pend_leaf, c->N, c->K, c->loss);
+    hipLaunchKernelGGL(k_apply_leaf, dim3((unsigned)nb), dim3(256), 0, c->stream, c->pred, c->nidx, c->tree.pred, c->N, c->K, c->loss);
     HIPCHK(hipGetLastError());
     c->pend_pred = false;
     return EVT_OK;

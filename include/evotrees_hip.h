@@ -237,7 +237,10 @@ int evt_reset_profile(evt_handle h);
  * "record_nidx" (1: the partition also records every sampled row's final node while the tree grows;
  * 0, default: evt_get_nidx derives it afterwards by walking the finished tree); "defer_pred" (1, default:
  * leaf values of a tree grown on every row are added in row order by the next pass over the rows;
- * 0: they are added while the tree's last level is partitioned; results do not depend on it). */
+ * 0: they are added while the tree's last level is partitioned; results do not depend on it); "grads_ahead"
+ * (1: a tree grown with update_pred queues the next evt_update_grads behind itself, so the device computes it
+ * while the host collects the tree, and that next call returns at once; meant for bagging_size 1 - with more
+ * trees per round only the last one's work is used; 0, default; results do not depend on it). */
 int evt_set_option(evt_handle h, const char *name, int64_t value);
 /* Blocks until all work queued on the handle's stream is done. */
 int evt_synchronize(evt_handle h);

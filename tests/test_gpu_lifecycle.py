@@ -194,3 +194,45 @@ def test_grow_tree_in_two_halves(evt):
     hb.grow_tree(js, gp)  # the handle goes on working
     ha.close()
     hb.close()
+
+
+@pytest.mark.parametrize("loss,tt", [("mse", "binary"), ("logloss", "oblivious"), ("gaussian_mle", "binary")])
+def test_gradients_queued_ahead_change_nothing(evt, loss, tt):
+    """With "grads_ahead" the gradient update of the next round is queued behind every tree and the next
+    evt_update_grads only takes note; trees, gradients and predictions stay bit-identical, also when the predictions
+    are changed from outside in between (evt_predict_tree, evt_set_target) or gradients are injected."""
+    N, F, B, D = 30000, 9, 32, 5
+    x_bin, y, w, mu = make_data(78, N, F, B, loss, weights=True)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    gp = evt.make_params(eta=0.3)
+    mask = np.random.default_rng(6).integers(0, 256, N, dtype=np.uint8)
+    out = []
+    for ahead in (1, 0):
+        h = evt.Handle(N, F, B, mu.shape[0], D, loss, tt)
+        h.set_option("grads_ahead", ahead)
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        rec = []
+        for r in range(5):
+            h.update_grads()
+            rec.append(h.get_grads())
+            t = h.grow_tree(js, gp, mask=mask if r == 2 else None, cond=128)
+            rec.append(t)
+            if r == 1:
+                h.predict_tree(t)            # the predictions change after the gradients were queued
+            if r == 3:
+                g = rec[0].copy()
+                h.set_grads(g)               # injected gradients replace the queued ones
+                rec.append(h.grow_tree(js, gp))
+        h.update_grads()
+        rec += [h.get_grads(), h.get_pred()]
+        h.set_target(y, w, mu)               # starts over: nothing queued survives
+        h.update_grads()
+        rec += [h.get_grads(), h.get_pred()]
+        h.close()
+        out.append(rec)
+    for a, b in zip(*out):
+        if isinstance(a, np.ndarray):
+            assert a.tobytes() == b.tobytes()
+        else:
+            assert_tree_bits(a, b)
