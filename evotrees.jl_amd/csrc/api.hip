@@ -623,8 +623,14 @@ extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t co
             h_js[i] = jsv[i];
             h_map[jsv[i] - 1] = (uint16_t)i;
         }
-        HIPCHK(hipMemcpyAsync(c->js, h_js, sizeof(uint32_t) * n_js, hipMemcpyHostToDevice, c->stream));
-        HIPCHK(hipMemcpyAsync(c->jsmap, h_map, sizeof(uint16_t) * c->RS, hipMemcpyHostToDevice, c->stream));
+        // read from the pinned buffer by a kernel (no trip through the copy engine); the buffer is not written again
+        // before the next tree, which starts after this one has been collected
+        {
+            const size_t o_js = c->blob_bytes, o_map = c->blob_bytes + (size_t)c->F * 4;
+            int rr = launch_copy_words(c, c->h_stage_dev + o_js, c->js, sizeof(uint32_t) * n_js);
+            if (rr == EVT_OK) rr = launch_copy_words(c, c->h_stage_dev + o_map, c->jsmap, sizeof(uint16_t) * c->RS);
+            if (rr != EVT_OK) return rr;
+        }
         c->n_js_last = n_js;
         c->js_last = jsv;
     }

@@ -223,6 +223,7 @@ int launch_level_next(evt_ctx *c, int level);
 int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred);
 int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred);
 int launch_copy_to_host(evt_ctx *c, const void *src_dev, void *dst_host_dev, size_t nbytes);
+int launch_copy_words(evt_ctx *c, const void *src, void *dst, size_t nbytes);
 int launch_fill_u32(evt_ctx *c, uint32_t *dst, uint32_t v, int64_t n);
 int launch_fill_bytes(evt_ctx *c, void *dst, int64_t nbytes);
 // predict

@@ -97,6 +97,20 @@ int launch_copy_to_host(evt_ctx *c, const void *src_dev, void *dst_host_dev, siz
     return EVT_OK;
 }
 
+// the same for small pinned host -> device uploads, in 4-byte words
+__global__ __launch_bounds__(256) void k_copy_words(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = src[i];
+}
+int launch_copy_words(evt_ctx *c, const void *src, void *dst, size_t nbytes) {
+    const int64_t n = (int64_t)(nbytes / 4);
+    if (n <= 0) return EVT_OK;
+    int64_t nb = (n + 255) / 256;
+    if (nb > 64) nb = 64;
+    hipLaunchKernelGGL(k_copy_words, dim3((unsigned)nb), dim3(256), 0, c->stream, static_cast<const uint32_t *>(src), static_cast<uint32_t *>(dst), n);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
 __global__ __launch_bounds__(256) void k_fill_u32(uint32_t *dst, uint32_t v, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = v;
 }
