@@ -154,7 +154,7 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id};
+                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id, c->pt_nodes, c->pt_pred};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -170,6 +170,7 @@ extern "C" int evt_destroy(evt_handle c) {
     }
     for (auto e : c->free_events) (void)hipEventDestroy(e);
     if (c->tree_ev) (void)hipEventDestroy(c->tree_ev);
+    if (c->pt_stage) (void)hipHostFree(c->pt_stage);
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
     return EVT_OK;
@@ -231,6 +232,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->pend_pred = false;
     c->is_id = nullptr;
     c->tree_in_flight = false;
+    c->pt_nodes = nullptr; c->pt_pred = nullptr; c->pt_stage = nullptr; c->pt_stage_dev = nullptr; c->pt_cap = 0; c->pt_busy = false;
     c->tree_ev = nullptr;
     c->grads_ahead = false;
     c->grads_ready = false;
@@ -791,29 +793,45 @@ extern "C" int evt_predict_tree(evt_handle c, int32_t nnodes_tree, const int64_t
     r = launch_apply_pending(c);
     if (r != EVT_OK) return r;
     c->grads_ready = false; // the predictions change
-    uint32_t *d_nodes = nullptr;
-    float *d_pred = nullptr;
-    HIPCHK(hipMalloc((void **)&d_nodes, sizeof(uint32_t) * nnodes_tree));
-    hipError_t e = hipMalloc((void **)&d_pred, sizeof(float) * (size_t)nnodes_tree * c->K);
-    if (e == hipSuccess) e = hipMemcpyAsync(d_nodes, nodes.data(), sizeof(uint32_t) * nnodes_tree, hipMemcpyHostToDevice, c->stream);
-    if (e == hipSuccess) e = hipMemcpyAsync(d_pred, pred, sizeof(float) * (size_t)nnodes_tree * c->K, hipMemcpyHostToDevice, c->stream);
-    if (e == hipSuccess) {
-        prof_begin(c, EVT_K_PREDICT, 0);
-        r = launch_predict_tree_nodes(c, d_nodes, d_pred);
-        prof_end(c);
-        e = hipStreamSynchronize(c->stream);
-        if (c->profiling) {
-            c->prof_units[EVT_K_PREDICT] += c->N;
-            prof_collect(c, nullptr);
+    const size_t nn = (size_t)nnodes_tree;
+    if (c->pt_busy) { // the last tree's upload must have been read before the pinned buffer is written again
+        HIPCHK(hipStreamSynchronize(c->stream));
+        c->pt_busy = false;
+    }
+    if (c->pt_cap < nn) { // device copies and upload buffer are kept between calls and grown on demand
+        HIPCHK(hipStreamSynchronize(c->stream));
+        if (c->pt_nodes) (void)hipFree(c->pt_nodes);
+        if (c->pt_pred) (void)hipFree(c->pt_pred);
+        if (c->pt_stage) (void)hipHostFree(c->pt_stage);
+        c->pt_nodes = nullptr; c->pt_pred = nullptr; c->pt_stage = nullptr; c->pt_stage_dev = nullptr; c->pt_cap = 0;
+        const size_t cap = std::max(nn, (size_t)2047);
+        hipError_t e = hipMalloc((void **)&c->pt_nodes, sizeof(uint32_t) * cap);
+        if (e == hipSuccess) e = hipMalloc((void **)&c->pt_pred, sizeof(float) * cap * c->K);
+        if (e == hipSuccess) e = hipHostMalloc((void **)&c->pt_stage, sizeof(uint32_t) * cap * (1 + c->K), hipHostMallocDefault);
+        if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&c->pt_stage_dev, c->pt_stage, 0);
+        if (e != hipSuccess) {
+            evt_set_error("predict_tree buffers: %s", hipGetErrorString(e));
+            return EVT_ERR_NOMEM;
         }
+        c->pt_cap = cap;
     }
-    if (d_nodes) (void)hipFree(d_nodes);
-    if (d_pred) (void)hipFree(d_pred);
-    if (e != hipSuccess) {
-        evt_set_error("predict_tree failed: %s", hipGetErrorString(e));
-        return EVT_ERR_HIP;
+    memcpy(c->pt_stage, nodes.data(), sizeof(uint32_t) * nn);
+    memcpy(c->pt_stage + sizeof(uint32_t) * nn, pred, sizeof(float) * nn * c->K);
+    r = launch_copy_words(c, c->pt_stage_dev, c->pt_nodes, sizeof(uint32_t) * nn);
+    if (r == EVT_OK) r = launch_copy_words(c, c->pt_stage_dev + sizeof(uint32_t) * nn, c->pt_pred, sizeof(float) * nn * c->K);
+    if (r != EVT_OK) return r;
+    c->pt_busy = true;
+    prof_begin(c, EVT_K_PREDICT, 0);
+    r = launch_predict_tree_nodes(c, c->pt_nodes, c->pt_pred);
+    prof_end(c);
+    if (r != EVT_OK) return r;
+    if (c->profiling) {
+        HIPCHK(hipStreamSynchronize(c->stream));
+        c->pt_busy = false;
+        c->prof_units[EVT_K_PREDICT] += c->N;
+        prof_collect(c, nullptr);
     }
-    return r;
+    return EVT_OK;
 }
 
 extern "C" int evt_get_xbin(evt_handle c, uint8_t *out) {
@@ -913,8 +931,10 @@ extern "C" int evt_eval_metric(evt_handle c, int32_t metric, double *value_out) 
     if (r == EVT_OK) r = launch_eval_metric(c, metric, c->metric_partial);
     prof_end(c);
     if (r != EVT_OK) return r;
-    HIPCHK(hipMemcpyAsync(c->h_stage, c->metric_partial + 2 * EVT_METRIC_BLOCKS, sizeof(double), hipMemcpyDeviceToHost, c->stream));
+    r = launch_copy_words(c, c->metric_partial + 2 * EVT_METRIC_BLOCKS, c->h_stage_dev, sizeof(double)); // a kernel's store, not the copy engine
+    if (r != EVT_OK) return r;
     HIPCHK(hipStreamSynchronize(c->stream));
+    c->pt_busy = false;
     memcpy(value_out, c->h_stage, sizeof(double));
     return EVT_OK;
 }

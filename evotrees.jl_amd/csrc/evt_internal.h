@@ -115,6 +115,13 @@ struct evt_ctx {
 
     // host staging (pinned)
     uint8_t *h_stage;
+    // evt_predict_tree: device copies of the tree handed in (packed nodes, leaf values) and the pinned buffer they are
+    // uploaded through; kept between calls and grown on demand
+    uint32_t *pt_nodes;
+    float *pt_pred;
+    uint8_t *pt_stage, *pt_stage_dev;
+    size_t pt_cap; // nodes
+    bool pt_busy;  // an upload from pt_stage has been queued since the stream was last drained here
     uint8_t *h_stage_dev; // the same pinned buffer as the device addresses it: the finished tree is written there by a kernel
     size_t h_stage_bytes;
     int32_t h_qbits[EVT_MC_MAX_NK];
