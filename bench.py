@@ -255,7 +255,7 @@ def main():
         else "train s/200 rounds (%s)" % args.workload,
         "value": round(value, 4), "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int64 fixed-point histograms, f64 gains, f32 gradients/predictions", "data": "synthetic",
+        "dtype": "int64", "arithmetic": "int64 fixed-point histograms, f64 gains, f32 gradients/predictions", "data": "synthetic",
         "config": {"workload": "%s: %s %dx%d nbins=%d max_depth=%d eta=%g rowsample=%g colsample=%g tree_type=%s" % (
             args.workload, loss, N, F, B, D, cfg["eta"], cfg["rowsample"], cfg["colsample"], cfg["tree_type"])},
         "roofline": roofline, "kernels_breakdown_%d_extra_rounds" % extra: kernels, "setup_s": round(t_setup, 2),
