@@ -328,6 +328,22 @@ template <int NAG>
 __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = (1 << (A.level - 1)) + blockIdx.x;
+    if (blockIdx.y > 0) {
+        // Blocks beyond the first of a node only clear the children's histogram slices (the build child accumulates
+        // into its own; a level with few nodes would otherwise leave 200 KB per node to one block).  They do not wait
+        // for the decision: the slices of a node that turns out a leaf are never read.  The node's state may already
+        // read SPLIT or LEAF here (the first block sets it), anything but INACTIVE means the level reached it.
+        if (A.status[n] == ST_INACTIVE) return;
+        long long *hc = A.hist + (int64_t)(2 * n - 1) * A.node_stride;
+        const int64_t used = (int64_t)A.nfs * NAG * A.B;
+        const int64_t zb = gridDim.y - 1, per = (used + zb - 1) / zb;
+        const int64_t i0 = (int64_t)(blockIdx.y - 1) * per, i1 = i0 + per < used ? i0 + per : used;
+        for (int64_t i = i0 + tid; i < i1; i += blockDim.x) {
+            hc[i] = 0;
+            hc[A.node_stride + i] = 0;
+        }
+        return;
+    }
     if (A.leaf_level) {
         // nodes of the last level are the children of the split nodes above them (the root when max_depth == 1)
         if (n > 1 && A.status[n >> 1] != ST_SPLIT) return;
@@ -408,8 +424,9 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
             }
         }
     }
-    // the children's histogram slices start from zero (the build child accumulates into it)
-    if (!A.zero_children) return;
+    // the children's histogram slices start from zero (the build child accumulates into it): with one block per node
+    // this block clears them, otherwise the node's other blocks have
+    if (!A.zero_children || gridDim.y > 1) return;
     long long *hc = A.hist + (int64_t)(2 * n - 1) * A.node_stride;
     const int64_t used = (int64_t)A.nfs * NAG * B;
     for (int64_t i = tid; i < used; i += blockDim.x) {
@@ -794,6 +811,9 @@ int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     const int ngroups = (A.nfs + 3) / 4; // 4 waves per block, one sampled feature each
     dim3 grid(nodes, (unsigned)ngroups);
     const int bpl = (c->B + 63) / 64;
+    // extra blocks per node that only clear the children's histogram slices, while a level has few nodes
+    unsigned zero_blocks = 0;
+    if (!leaf_level && A.zero_children && !A.oblivious && nodes < 64) zero_blocks = 64 / nodes < 16 ? 64 / nodes : 16;
     if (c->loss == EVT_LOSS_MLOGLOSS) {
         if (!leaf_level) {
             if (bpl == 1) hipLaunchKernelGGL((k_scan_mc<1>), grid, dim3(256), 0, c->stream, A);
@@ -811,7 +831,7 @@ int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
             else if (bpl == 2) hipLaunchKernelGGL((k_scan<NAG_, 2>), grid, dim3(256), 0, c->stream, A); \
             else hipLaunchKernelGGL((k_scan<NAG_, 4>), grid, dim3(256), 0, c->stream, A);               \
         }                                                                                               \
-        if (!A.oblivious || leaf_level) hipLaunchKernelGGL(k_scan_fin<NAG_>, dim3(nodes), dim3(256), 0, c->stream, A, ngroups); \
+        if (!A.oblivious || leaf_level) hipLaunchKernelGGL(k_scan_fin<NAG_>, dim3(nodes, 1 + zero_blocks), dim3(256), 0, c->stream, A, ngroups); \
         break;
     switch (c->NAg) {
         SCASE(2)
