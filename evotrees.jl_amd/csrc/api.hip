@@ -501,7 +501,7 @@ extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, cons
         int r = launch_absmax_rows(c, c->NK - 1, c->NK);
         if (r != EVT_OK) return r;
     }
-    float *mu_dev = reinterpret_cast<float *>(c->chunk_lpre); // small scratch
+    float *mu_dev = reinterpret_cast<float *>(c->metric_partial); // small scratch: thousands of doubles, K <= 16 floats needed
     HIPCHK(hipMemcpyAsync(mu_dev, mu, sizeof(float) * c->K, hipMemcpyDefault, c->stream));
     if (offset) {
         HIPCHK(hipStreamSynchronize(c->stream));
