@@ -36,7 +36,8 @@ struct HistArgs {
     int64_t N;
     int64_t node_stride;
     int RS, LPR, RPW, F, nfs, B, NAg, level;
-    int NSL; // conflict-free kernel: lanes per row, the power of two >= 16 that covers a record's pieces
+    int NSL; // conflict-free kernel: lanes per row, the power of two >= 16 that covers a column tile's pieces
+    int TW;  // conflict-free kernel: bytes of a record one block column (blockIdx.y) takes - a column tile
     int slots_per_tile;
     int min_rows;
     int seg_cost;
@@ -299,14 +300,17 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     for (int i = tid; i < NA * plane; i += nthr) H[i] = 0ull;
 
     const int sub = lane % NS, rloc = lane / NS;
-    const int subl = (sub * PB < A.RS) ? sub : 0; // an idle lane loads the row's first piece and adds nothing (no feature: vmask 0)
+    // column tile: block column y takes bytes [y * TW, (y + 1) * TW) of every record and keeps their histograms only -
+    // a record too wide for one LDS histogram is covered by several block columns, each reading its own bytes
+    const int tb = (int)blockIdx.y * A.TW;
+    const int subl = (tb + sub * PB < A.RS) ? sub : 0; // an idle lane loads the tile's first piece and adds nothing (no feature: vmask 0)
     // byte offset of (t, bin 0) for this lane; bins are 1-based so bin*NS*8 is added on top
     // (32-bit unsigned arithmetic throughout: one 24-bit multiply-add per LDS address)
     uint32_t coff[PB];
     unsigned vmask = 0;
 #pragma unroll
     for (int t = 0; t < PB; t++) {
-        const int f = sub * PB + t;
+        const int f = tb + sub * PB + t;
         const bool ok = (f < A.F) && (A.jsmap[f] != 0xFFFF);
         coff[t] = (uint32_t)(((t * B - 1) * NS + sub) * 8);
         vmask |= ok ? (1u << t) : 0u;
@@ -374,7 +378,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
 #define EVT_H16_PRO(u_)                                                                                               \
     if constexpr ((u_) < U) {                                                                                         \
         const uint32_t row = grp_bcast<(u_) < U ? (u_) : 0>(idc);                                               \
-        v[(u_) < U ? (u_) : 0] = load_piece<PB>(A.xrm + (size_t)row * A.RS + subl * PB);                \
+        v[(u_) < U ? (u_) : 0] = load_piece<PB>(A.xrm + (size_t)row * A.RS + tb + subl * PB);           \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
             EVT_H16_PRO(0) EVT_H16_PRO(1) EVT_H16_PRO(2) EVT_H16_PRO(3) EVT_H16_PRO(4) EVT_H16_PRO(5) EVT_H16_PRO(6) EVT_H16_PRO(7)
@@ -412,7 +416,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             }                                                                                                         \
         }                                                                                                             \
         const uint32_t row = grp_bcast<ui>(idn);                                                                \
-        v[ui] = load_piece<PB>(A.xrm + (size_t)row * A.RS + subl * PB);                               \
+        v[ui] = load_piece<PB>(A.xrm + (size_t)row * A.RS + tb + subl * PB);                          \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
                 EVT_H16_STEP(0) EVT_H16_STEP(1) EVT_H16_STEP(2) EVT_H16_STEP(3) EVT_H16_STEP(4) EVT_H16_STEP(5) EVT_H16_STEP(6) EVT_H16_STEP(7)
@@ -467,7 +471,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                     const int t = rest & (PB - 1);
                     const int a = rest / PB;
                     const int b = chunk * 8 + bl;
-                    const int f = sidx * PB + t;
+                    const int f = tb + sidx * PB + t;
                     if (b < B) {
                         hwv[j] = &H[(size_t)a * plane + ((size_t)t * B + b) * NS + sidx];
                         wv[j] = *hwv[j];
@@ -537,9 +541,9 @@ template <int NA, bool PACK>
 static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
     // row groups (records) in flight per wave: as many as a DPP row can address, fewer when registers run out
     constexpr int U = (NA <= 2) ? 16 : 8;
-    if (c->RS >= 128) return launch_hist16_q<NA, PACK, U, 8>(c, A, grid, threads, lds);
-    if (c->RS == 64) return launch_hist16_q<NA, PACK, U, 4>(c, A, grid, threads, lds);
-    return launch_hist16_q<NA, PACK, U, 2>(c, A, grid, threads, lds); // 32-byte records
+    if (A.TW >= 128) return launch_hist16_q<NA, PACK, U, 8>(c, A, grid, threads, lds);
+    if (A.TW == 64) return launch_hist16_q<NA, PACK, U, 4>(c, A, grid, threads, lds);
+    return launch_hist16_q<NA, PACK, U, 2>(c, A, grid, threads, lds); // 32-byte tiles
 }
 
 template <int NA, bool PACK>
@@ -607,19 +611,26 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
         A.slots_per_tile = slots_per_tile;
         const size_t lds = per_slot * slots_per_tile;
         dim3 grid((unsigned)blocks, (unsigned)ntiles);
-        // conflict-free variant: 16, 32 or 64 lanes per row - records of 32 to 512 bytes; a size that is not a power of two
-        // takes the next one's lanes and leaves the ones past its last piece idle - whose whole LDS histogram fits
-        // (16-byte records as 1-byte pieces were measured: no faster than the generic kernel)
-        const int pb16 = c->RS >= 128 ? 8 : (c->RS == 64 ? 4 : 2);
-        int nsl = 16;
-        while (nsl * pb16 < c->RS) nsl <<= 1;
-        A.NSL = nsl;
-        const size_t lds16 = (size_t)na * c->B * pb16 * nsl * 8; // channels x bins x (lanes x bytes per piece) words
-        const bool can16 = c->RS >= 32 && nsl <= 64 && lds16 <= 128 * 1024;
+        // conflict-free variant: a block column takes a tile of TW bytes of every record - the whole record when its LDS
+        // histogram fits, else the widest power of two that does (down to 32 bytes) - with 16, 32 or 64 lanes per row;
+        // lanes past the record's last piece idle.  (16-byte records as 1-byte pieces were measured: no faster than the
+        // generic kernel.)
+        int tw = 32;
+        while (tw < c->RS && tw < 512) tw <<= 1;
+        while (tw > 32 && (size_t)na * c->B * tw * 8 > 128 * 1024) tw >>= 1;
+        const int pb16 = tw >= 128 ? 8 : (tw == 64 ? 4 : 2);
+        A.TW = tw;
+        A.NSL = tw / pb16;
+        const int ntiles16 = (c->RS + tw - 1) / tw;
+        const size_t lds16 = (size_t)na * c->B * tw * 8; // channels x bins x tile bytes words
+        const bool can16 = c->RS >= 32 && lds16 <= 128 * 1024;
         const bool use16 = (c->hist_variant == 1) ? false : can16;
         int r = EVT_ERR_ARG;
         if (use16) {
-            dim3 grid16((unsigned)blocks, 1u);
+            // several block columns share the launch's blocks: the same number of LDS histograms is flushed per node
+            int64_t bx = blocks / ntiles16;
+            if (bx < 64) bx = blocks < 64 ? blocks : 64;
+            dim3 grid16((unsigned)bx, (unsigned)ntiles16);
 #define H16CASE(NA_) \
     case NA_: r = pack ? launch_hist16_t<NA_, true>(c, A, grid16, threads, lds16) : launch_hist16_t<NA_, false>(c, A, grid16, threads, lds16); break;
             switch (na) {

@@ -31,6 +31,14 @@ def _cases():
         tt = "oblivious" if rng.integers(0, 5) == 0 else "binary"
         cat = bool(rng.integers(0, 3) == 0)
         out.append((loss, weights, N, F, B, D, tt, n_js, rowsample, K, cat, i))
+    # histograms wider than one workgroup's LDS (several column tiles per launch), and many classes on very few rows
+    out += [
+        ("mse", False, 20000, 100, 255, 5, "binary", 100, 1.0, None, False, 100),
+        ("logloss", True, 15000, 300, 64, 4, "binary", 300, 0.5, None, True, 101),
+        ("gaussian_mle", True, 9000, 200, 128, 3, "binary", 77, 1.0, None, False, 102),
+        ("mse", False, 12000, 130, 255, 4, "oblivious", 130, 0.5, None, True, 103),
+        ("mlogloss", True, 1233, 578, 16, 1, "binary", 578, 0.5, 15, False, 104),
+    ]
     return out
 
 
