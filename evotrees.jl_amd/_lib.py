@@ -22,6 +22,7 @@ EXPORTS = [
     "evt_last_error", "evt_device_count", "evt_create", "evt_destroy", "evt_set_xbin", "evt_binarize_f64",
     "evt_set_target", "evt_set_feature_meta", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
     "evt_grow_tree_begin", "evt_grow_tree_end",
+    "evt_tree_open", "evt_hist_build", "evt_split_scan", "evt_update_nodes_idx", "evt_tree_close", "evt_peek_tree",
     "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
     "evt_predict", "evt_predict_f64", "evt_predict_leaf_idx", "evt_eval_metric", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
     "evt_set_option", "evt_synchronize", "evt_copy_bandwidth", "evt_read_bandwidth",
@@ -72,6 +73,12 @@ def load():
         "evt_grow_tree": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams), C.POINTER(EvtTreeOut)],
         "evt_grow_tree_begin": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams)],
         "evt_grow_tree_end": [vp, C.POINTER(EvtTreeOut)],
+        "evt_tree_open": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams)],
+        "evt_hist_build": [vp, i32],
+        "evt_split_scan": [vp, i32],
+        "evt_update_nodes_idx": [vp, i32],
+        "evt_tree_close": [vp],
+        "evt_peek_tree": [vp, C.POINTER(EvtTreeOut)],
         "evt_predict_tree": [vp, i32, vp, vp, vp, vp],
         "evt_get_xbin": [vp, vp],
         "evt_get_pred": [vp, vp],
@@ -223,6 +230,32 @@ class Handle:
         t = TreeArrays(self.K, self.nnodes) if want_tree else None
         out = t.as_out() if want_tree else None
         check(load().evt_grow_tree_end(self._h, C.byref(out) if want_tree else None))
+        return t
+
+    # one tree, one kernel stage at a time (update_hist!, the split search, update_nodes_idx! per level)
+    def tree_open(self, js, params, mask=None, cond=255):
+        js = np.ascontiguousarray(js, np.uint32)
+        if mask is not None:
+            mask = np.ascontiguousarray(mask, np.uint8)
+            assert mask.shape == (self.N,)
+        check(load().evt_tree_open(self._h, ptr(mask), int(cond), ptr(js), js.shape[0], C.byref(params)))
+
+    def hist_build(self, level):
+        check(load().evt_hist_build(self._h, int(level)))
+
+    def split_scan(self, level):
+        check(load().evt_split_scan(self._h, int(level)))
+
+    def update_nodes_idx(self, level):
+        check(load().evt_update_nodes_idx(self._h, int(level)))
+
+    def tree_close(self):
+        check(load().evt_tree_close(self._h))
+
+    def peek_tree(self):
+        t = TreeArrays(self.K, self.nnodes)
+        out = t.as_out()
+        check(load().evt_peek_tree(self._h, C.byref(out)))
         return t
 
     def predict_tree(self, tree):

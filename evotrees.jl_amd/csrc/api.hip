@@ -232,6 +232,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->pend_pred = false;
     c->is_id = nullptr;
     c->tree_in_flight = false;
+    c->step.phase = 0;
     c->pt_nodes = nullptr; c->pt_pred = nullptr; c->pt_stage = nullptr; c->pt_stage_dev = nullptr; c->pt_cap = 0; c->pt_busy = false;
     c->tree_ev = nullptr;
     c->grads_ahead = false;
@@ -368,6 +369,20 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
 // every call on a handle but evt_grow_tree_end, evt_synchronize and evt_destroy waits for a tree begun with
 // evt_grow_tree_begin to be collected: its arrays sit in the handle's staging buffer until then
 #define CTXCHK(c)                                                                                      \
+    do {                                                                                               \
+        ARGCHK((c) != nullptr, "handle is NULL");                                                      \
+        HIPCHK(hipSetDevice((c)->device));                                                             \
+        if ((c)->tree_in_flight) {                                                                     \
+            evt_set_error("a tree begun with evt_grow_tree_begin has not been collected (evt_grow_tree_end)"); \
+            return EVT_ERR_STATE;                                                                      \
+        }                                                                                              \
+        if ((c)->step.phase != 0) {                                                                    \
+            evt_set_error("a tree opened with evt_tree_open has not been closed (evt_tree_close)");    \
+            return EVT_ERR_STATE;                                                                      \
+        }                                                                                              \
+    } while (0)
+// calls that are also allowed between the stages of a tree opened with evt_tree_open
+#define CTXCHK_STEP(c)                                                                                 \
     do {                                                                                               \
         ARGCHK((c) != nullptr, "handle is NULL");                                                      \
         HIPCHK(hipSetDevice((c)->device));                                                             \
@@ -582,8 +597,7 @@ extern "C" int evt_set_grads(evt_handle c, const float *grad) {
     return EVT_OK;
 }
 
-extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
-    CTXCHK(c);
+static int tree_open(evt_ctx *c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p, bool staged) {
     ARGCHK(js && p, "js and params must not be NULL");
     ARGCHK(n_js >= 1 && n_js <= c->F, "n_js must be in [1, nfeats]");
     ARGCHK(p->bagging_size >= 1, "bagging_size must be >= 1");
@@ -614,7 +628,9 @@ extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t co
     c->grads_ready = false; // this tree changes the predictions
     c->last_all_rows = all_rows;
     c->last_cond = cond;
-    c->nidx_valid = c->record_nidx;
+    // a tree grown in stages records the node of every row on the way, so that evt_get_nidx can show it after each stage
+    const bool rec_nidx = c->record_nidx || staged;
+    c->nidx_valid = rec_nidx;
 
     // per-tree small uploads through pinned memory
     if (c->n_js_last != n_js || c->js_last != jsv) { // the column sample changed: refresh the device copies
@@ -641,7 +657,7 @@ extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t co
     // order (fused into the next gradient pass): a scattered 4-byte write per row instead of a scattered read-modify-write.
     const bool defer = p->update_pred && all_rows && c->defer_pred;
     const bool fuse_pred = p->update_pred && all_rows && !defer;
-    c->write_nidx = c->record_nidx || defer;
+    c->write_nidx = rec_nidx || defer;
 
     int r;
     prof_begin(c, EVT_K_OTHER, 0);
@@ -651,50 +667,96 @@ extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t co
         HIPCHK(hipMemcpyAsync(c->mask, mask, c->N, hipMemcpyDefault, c->stream));
         HIPCHK(hipStreamSynchronize(c->stream)); // the caller may reuse its mask buffer as soon as this call returns
         r = launch_compact_mask(c, cond);
-        if (r == EVT_OK && c->record_nidx) r = launch_fill_u32(c, c->nidx, 0u, c->N);
+        if (r == EVT_OK && rec_nidx) r = launch_fill_u32(c, c->nidx, 0u, c->N);
     }
     if (r == EVT_OK) r = launch_tree_begin(c, all_rows);
     prof_end(c);
     if (r != EVT_OK) return r;
 
-    const bool obliv = (c->tree_type == EVT_TREE_OBLIVIOUS);
+    c->step.all_rows = all_rows;
+    c->step.defer = defer;
+    c->step.fuse_pred = fuse_pred;
+    c->step.p = *p;
     // the root's list is the identity (kept, never written) or what the mask compaction left in is_a; the levels below
     // alternate between is_a and is_b
-    uint32_t *is_cur = all_rows ? c->is_id : c->is_a, *is_next = all_rows ? c->is_a : c->is_b;
-    // levels 1 .. D-1 split; the last of them sends its rows straight to the leaves of level D
-    const int last_split = (c->D > 1) ? c->D - 1 : 1;
-    for (int level = 1; level <= last_split; level++) {
-        prof_begin_launch(c, EVT_K_HIST, level);
-        r = launch_hist_build(c, level, is_cur);
-        c->launch_e0 = c->launch_e1 = nullptr;
-        if (r != EVT_OK) return r;
-        prof_begin(c, EVT_K_SCAN, level);
-        if (c->D == 1) {
-            r = launch_scan(c, 1, p, true); // a stump: the root is the only leaf
-        } else {
-            r = launch_scan(c, level, p, false);
-            if (r == EVT_OK && obliv) r = launch_obliv_select(c, level, p);
-            if (r == EVT_OK && level == last_split) r = launch_scan(c, c->D, p, true); // leaf values of level D
-        }
-        prof_end(c);
-        if (r != EVT_OK) return r;
-        prof_begin(c, EVT_K_PARTITION, level);
-        if (level < last_split) {
-            r = launch_part_count(c, level, is_cur);
-            if (r == EVT_OK) r = launch_level_next(c, level);
-            if (r == EVT_OK) r = launch_part_scatter(c, level, is_cur, is_next, fuse_pred);
-        } else {
-            r = launch_final_fused(c, level, is_cur, fuse_pred);
-        }
-        prof_end(c);
-        if (r != EVT_OK) return r;
-        if (is_cur == c->is_id) {
-            is_cur = is_next;
-            is_next = c->is_b;
-        } else {
-            std::swap(is_cur, is_next);
-        }
+    c->step.is_cur = all_rows ? c->is_id : c->is_a;
+    c->step.is_next = all_rows ? c->is_a : c->is_b;
+    c->step.level = 1;
+    c->step.phase = 1;
+    return EVT_OK;
+}
+
+// levels 1 .. D-1 split; the last of them sends its rows straight to the leaves of level D
+static inline int tree_last_split(const evt_ctx *c) { return (c->D > 1) ? c->D - 1 : 1; }
+
+// update_hist! for the build nodes of the level (src/fit-utils.jl:345-360)
+static int tree_stage_hist(evt_ctx *c) {
+    const int level = c->step.level;
+    prof_begin_launch(c, EVT_K_HIST, level);
+    int r = launch_hist_build(c, level, c->step.is_cur);
+    c->launch_e0 = c->launch_e1 = nullptr;
+    if (r != EVT_OK) return r;
+    c->step.phase = 2;
+    return EVT_OK;
+}
+
+// subtract_hist!, _scan_node!/get_best_split (update_gains! and the level's choice for oblivious trees), child sums and
+// leaf values for the active nodes of the level (src/fit-utils.jl:321-332, :403-486; src/fit.jl:190-217)
+static int tree_stage_scan(evt_ctx *c) {
+    const int level = c->step.level, last_split = tree_last_split(c);
+    const evt_params *p = &c->step.p;
+    const bool obliv = (c->tree_type == EVT_TREE_OBLIVIOUS);
+    int r;
+    prof_begin(c, EVT_K_SCAN, level);
+    if (c->D == 1) {
+        r = launch_scan(c, 1, p, true); // a stump: the root is the only leaf
+    } else {
+        r = launch_scan(c, level, p, false);
+        if (r == EVT_OK && obliv) r = launch_obliv_select(c, level, p);
+        if (r == EVT_OK && level == last_split) r = launch_scan(c, c->D, p, true); // leaf values of level D
     }
+    prof_end(c);
+    if (r != EVT_OK) return r;
+    c->step.phase = 3;
+    return EVT_OK;
+}
+
+// split_set! / update_nodes_idx!: the rows of every split node move to its children (src/fit-utils.jl:93-132,
+// ext/.../fit-utils.jl:9-31)
+static int tree_stage_partition(evt_ctx *c) {
+    const int level = c->step.level, last_split = tree_last_split(c);
+    uint32_t *is_cur = c->step.is_cur, *is_next = c->step.is_next;
+    int r;
+    prof_begin(c, EVT_K_PARTITION, level);
+    if (level < last_split) {
+        r = launch_part_count(c, level, is_cur);
+        if (r == EVT_OK) r = launch_level_next(c, level);
+        if (r == EVT_OK) r = launch_part_scatter(c, level, is_cur, is_next, c->step.fuse_pred);
+    } else {
+        r = launch_final_fused(c, level, is_cur, c->step.fuse_pred);
+    }
+    prof_end(c);
+    if (r != EVT_OK) return r;
+    if (is_cur == c->is_id) {
+        c->step.is_cur = is_next;
+        c->step.is_next = c->is_b;
+    } else {
+        std::swap(c->step.is_cur, c->step.is_next);
+    }
+    if (level < last_split) {
+        c->step.level = level + 1;
+        c->step.phase = 1;
+    } else {
+        c->step.phase = 4;
+    }
+    return EVT_OK;
+}
+
+static int tree_close(evt_ctx *c) {
+    const evt_params *p = &c->step.p;
+    const bool all_rows = c->step.all_rows, defer = c->step.defer;
+    int r;
+    c->step.phase = 0;
     if (p->update_pred && !all_rows) {
         // rows outside the sample are predicted too (src/fit.jl:37): walk the new tree for all rows
         prof_begin(c, EVT_K_PREDICT, 0);
@@ -722,6 +784,93 @@ extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t co
     return EVT_OK;
 }
 
+
+static int tree_fail(evt_ctx *c, int r) { // a failed stage leaves no tree open
+    c->step.phase = 0;
+    return r;
+}
+
+extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
+    CTXCHK(c);
+    int r = tree_open(c, mask, cond, js, n_js, p, false);
+    while (r == EVT_OK && c->step.phase != 4) {
+        r = tree_stage_hist(c);
+        if (r == EVT_OK) r = tree_stage_scan(c);
+        if (r == EVT_OK) r = tree_stage_partition(c);
+    }
+    if (r != EVT_OK) return tree_fail(c, r);
+    return tree_close(c);
+}
+
+extern "C" int evt_tree_open(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
+    CTXCHK(c);
+    int r = tree_open(c, mask, cond, js, n_js, p, true);
+    if (r != EVT_OK) return tree_fail(c, r);
+    return EVT_OK;
+}
+
+static int stage_check(evt_ctx *c, int phase, int32_t level, const char *name) {
+    if (c->step.phase == 0) {
+        evt_set_error("%s: no tree is open (evt_tree_open)", name);
+        return EVT_ERR_STATE;
+    }
+    if (c->step.phase != phase || c->step.level != level) {
+        static const char *const what[] = {"", "evt_hist_build", "evt_split_scan", "evt_update_nodes_idx", "evt_tree_close"};
+        evt_set_error("%s(level %d) out of order: the open tree expects %s%s%d%s", name, (int)level, what[c->step.phase],
+                      c->step.phase == 4 ? "" : "(level ", c->step.phase == 4 ? 0 : c->step.level, c->step.phase == 4 ? "" : ")");
+        return EVT_ERR_STATE;
+    }
+    return EVT_OK;
+}
+
+extern "C" int evt_hist_build(evt_handle c, int32_t level) {
+    CTXCHK_STEP(c);
+    int r = stage_check(c, 1, level, "evt_hist_build");
+    if (r != EVT_OK) return r;
+    r = tree_stage_hist(c);
+    return r == EVT_OK ? r : tree_fail(c, r);
+}
+
+extern "C" int evt_split_scan(evt_handle c, int32_t level) {
+    CTXCHK_STEP(c);
+    int r = stage_check(c, 2, level, "evt_split_scan");
+    if (r != EVT_OK) return r;
+    r = tree_stage_scan(c);
+    return r == EVT_OK ? r : tree_fail(c, r);
+}
+
+extern "C" int evt_update_nodes_idx(evt_handle c, int32_t level) {
+    CTXCHK_STEP(c);
+    int r = stage_check(c, 3, level, "evt_update_nodes_idx");
+    if (r != EVT_OK) return r;
+    r = tree_stage_partition(c);
+    return r == EVT_OK ? r : tree_fail(c, r);
+}
+
+extern "C" int evt_tree_close(evt_handle c) {
+    CTXCHK_STEP(c);
+    if (c->step.phase != 4) {
+        evt_set_error(c->step.phase == 0 ? "evt_tree_close: no tree is open" : "evt_tree_close before the last level was partitioned");
+        return EVT_ERR_STATE;
+    }
+    return tree_close(c);
+}
+
+// host copy of the device's tree arrays (in the pinned staging buffer) -> the caller's arrays
+static int fill_tree_out(evt_ctx *c, evt_tree_out *tree) {
+    ARGCHK(tree->feat && tree->cond_bin && tree->w && tree->gain && tree->pred && tree->split, "tree output arrays must not be NULL");
+    const int nn = c->nnodes, K = c->K;
+    const uint8_t *hs = c->h_stage;
+    const int32_t *f32 = reinterpret_cast<const int32_t *>(hs + c->blob_feat);
+    for (int n = 0; n < nn; n++) tree->feat[n] = (int64_t)f32[n];
+    memcpy(tree->w, hs + c->blob_w, (size_t)nn * 4);
+    memcpy(tree->gain, hs + c->blob_gain, (size_t)nn * 4);
+    memcpy(tree->pred, hs + c->blob_pred, (size_t)nn * 4 * K);
+    memcpy(tree->cond_bin, hs + c->blob_bin, nn);
+    memcpy(tree->split, hs + c->blob_split, nn);
+    return EVT_OK;
+}
+
 extern "C" int evt_grow_tree_end(evt_handle c, evt_tree_out *tree) {
     ARGCHK(c != nullptr, "handle is NULL");
     HIPCHK(hipSetDevice(c->device));
@@ -730,10 +879,8 @@ extern "C" int evt_grow_tree_end(evt_handle c, evt_tree_out *tree) {
         return EVT_ERR_STATE;
     }
     c->tree_in_flight = false;
-    const int nn = c->nnodes, K = c->K;
     uint8_t *hs = c->h_stage;
-    const size_t o_feat = c->blob_feat, o_w = c->blob_w, o_gain = c->blob_gain, o_pred = c->blob_pred, o_stats = c->blob_stats,
-                 o_bin = c->blob_bin, o_split = c->blob_split;
+    const size_t o_stats = c->blob_stats;
     HIPCHK(hipEventSynchronize(c->tree_ev)); // the tree has arrived; work queued behind it may still be running
     const int64_t n_is = reinterpret_cast<const int64_t *>(hs + o_stats)[0];
     if (c->profiling) {
@@ -745,17 +892,18 @@ extern "C" int evt_grow_tree_end(evt_handle c, evt_tree_out *tree) {
         evt_set_error("no subsample observation - choose larger rowsample");
         return EVT_ERR_EMPTY;
     }
-    if (tree) {
-        ARGCHK(tree->feat && tree->cond_bin && tree->w && tree->gain && tree->pred && tree->split, "tree output arrays must not be NULL");
-        const int32_t *f32 = reinterpret_cast<const int32_t *>(hs + o_feat);
-        for (int n = 0; n < nn; n++) tree->feat[n] = (int64_t)f32[n];
-        memcpy(tree->w, hs + o_w, (size_t)nn * 4);
-        memcpy(tree->gain, hs + o_gain, (size_t)nn * 4);
-        memcpy(tree->pred, hs + o_pred, (size_t)nn * 4 * K);
-        memcpy(tree->cond_bin, hs + o_bin, nn);
-        memcpy(tree->split, hs + o_split, nn);
-    }
+    if (tree) return fill_tree_out(c, tree);
     return EVT_OK;
+}
+
+// The tree arrays as they stand on the device, e.g. between the stages of a tree opened with evt_tree_open.
+extern "C" int evt_peek_tree(evt_handle c, evt_tree_out *tree) {
+    CTXCHK_STEP(c);
+    ARGCHK(tree, "tree is NULL");
+    int r = launch_copy_to_host(c, c->tree_blob, c->h_stage_dev, c->blob_bytes);
+    if (r != EVT_OK) return r;
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return fill_tree_out(c, tree);
 }
 
 extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p,
@@ -864,11 +1012,15 @@ extern "C" int evt_get_grads(evt_handle c, float *out) {
     return EVT_OK;
 }
 extern "C" int evt_get_nidx(evt_handle c, uint32_t *out) {
-    CTXCHK(c);
+    CTXCHK_STEP(c);
     ARGCHK(out, "out is NULL");
     if (c->n_js_last <= 0) {
         evt_set_error("no tree has been grown yet");
         return EVT_ERR_STATE;
+    }
+    if (c->step.phase >= 1 && c->step.phase <= 3) { // a tree in stages: rows still on their way down are in the level's row lists
+        int r = launch_nidx_from_segments(c, c->step.level, c->step.is_cur);
+        if (r != EVT_OK) return r;
     }
     if (!c->nidx_valid) { // not recorded while growing: walk the last tree (same decisions, row by row)
         int r = launch_nidx_from_tree(c, !c->last_all_rows, c->last_cond);
@@ -880,7 +1032,7 @@ extern "C" int evt_get_nidx(evt_handle c, uint32_t *out) {
     return EVT_OK;
 }
 extern "C" int evt_get_hist(evt_handle c, double *out) {
-    CTXCHK(c);
+    CTXCHK_STEP(c);
     ARGCHK(out, "out is NULL");
     if (c->n_js_last <= 0) {
         evt_set_error("no tree has been grown yet");

@@ -141,6 +141,14 @@ struct evt_ctx {
     bool grads_ready;    // the gradients of the predictions as they stand were computed ahead: evt_update_grads has nothing to do
     hipEvent_t tree_ev;  // recorded behind the tree's transfer to the host: evt_grow_tree_end waits for this, not for the stream
     bool tree_in_flight; // evt_grow_tree_begin has queued a tree that evt_grow_tree_end has not collected
+    // a tree grown one kernel stage at a time (evt_tree_open ... evt_tree_close); evt_grow_tree_begin drives the same stages
+    struct {
+        int phase; // 0 no tree open, 1 histogram next, 2 split search next, 3 partition next, 4 levels done
+        int level;
+        bool all_rows, defer, fuse_pred;
+        uint32_t *is_cur, *is_next; // row-id lists of the current level and of the one below
+        evt_params p;
+    } step;
     bool pend_pred;    // pred lacks the leaf values tree.pred[nidx[i] - 1] of the last tree (the device Tree arrays keep them until the next tree starts, and what is pending is applied before that)
     uint8_t last_cond;
 
@@ -229,6 +237,7 @@ int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_level_next(evt_ctx *c, int level);
 int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred);
 int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred);
+int launch_nidx_from_segments(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_copy_to_host(evt_ctx *c, const void *src_dev, void *dst_host_dev, size_t nbytes);
 int launch_copy_words(evt_ctx *c, const void *src, void *dst, size_t nbytes);
 int launch_fill_u32(evt_ctx *c, uint32_t *dst, uint32_t v, int64_t n);

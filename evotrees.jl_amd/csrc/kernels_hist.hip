@@ -669,7 +669,7 @@ __global__ __launch_bounds__(256) void k_hist_export(const long long *__restrict
     int node = blockIdx.x; // 0-based
     if (node + 1 >= last_level_first) return; // nodes of the last level never get a histogram
     int st = status[node + 1];
-    if (st != ST_SPLIT && st != ST_LEAF) return;
+    if (st != ST_SPLIT && st != ST_LEAF && st != ST_BUILD) return; // ST_BUILD: built from rows, not yet searched (a tree grown in stages)
     const long long *hn = hist + (int64_t)node * F * NAg * B;
     for (int idx = threadIdx.x; idx < nfs * B; idx += 256) {
         int jp = idx / B, b = idx - jp * B;

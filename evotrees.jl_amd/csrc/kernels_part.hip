@@ -627,6 +627,26 @@ int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_
     return EVT_OK;
 }
 
+// Node of every row that is still on its way down, read off the row lists: node n of the level owns
+// is[seg_start[n] .. +seg_len[n]).  Read-back for a tree grown in stages (rows that reached a leaf above this level
+// had their node recorded when they got there).
+__global__ __launch_bounds__(256) void k_nidx_from_segments(const uint32_t *__restrict__ is, const int64_t *__restrict__ seg_start,
+                                                           const int64_t *__restrict__ seg_len, const int32_t *__restrict__ status,
+                                                           int first_node, uint32_t *__restrict__ nidx) {
+    const int n = first_node + blockIdx.x;
+    if (status[n] == ST_INACTIVE) return;
+    const int64_t start = seg_start[n], len = seg_len[n];
+    for (int64_t i = (int64_t)blockIdx.y * 256 + threadIdx.x; i < len; i += (int64_t)gridDim.y * 256) nidx[is[start + i]] = (uint32_t)n;
+}
+
+int launch_nidx_from_segments(evt_ctx *c, int level, const uint32_t *is_cur) {
+    const int first = 1 << (level - 1), count = first; // nodes first .. 2 * first - 1
+    hipLaunchKernelGGL(k_nidx_from_segments, dim3((unsigned)count, 64), dim3(256), 0, c->stream, is_cur, c->seg_start, c->seg_len, c->status,
+                       first, c->nidx);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
 int launch_level_next(evt_ctx *c, int level) {
     const LevelTab &L = c->lvl[level & 1];
     const LevelTab &Nx = c->lvl[(level + 1) & 1];

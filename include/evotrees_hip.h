@@ -160,6 +160,36 @@ int evt_grow_tree_begin(evt_handle h, const uint8_t *mask, uint8_t cond, const u
                         const evt_params *params);
 int evt_grow_tree_end(evt_handle h, evt_tree_out *tree);
 
+/*
+ * The same tree, one kernel stage at a time: the stages are the reference's own per-level calls, so each can be
+ * checked (or timed) against its counterpart on its own.
+ *   evt_tree_open        subsample + root set-up, as evt_grow_tree_begin up to the first level (src/fit.jl:59-66)
+ *   evt_hist_build       update_hist! for the level's build nodes, i.e. the smaller child of every pair
+ *                        (src/fit-utils.jl:345-394; device twin ext/.../fit-utils.jl:148-226)
+ *   evt_split_scan       subtract_hist! for the larger children, then _scan_node!/get_best_split (update_gains! and
+ *                        the level's common choice for oblivious trees), _child_sums! and the leaf values of the
+ *                        nodes that end here (src/fit-utils.jl:321-332, :403-486; src/fit.jl:85-121, :190-217;
+ *                        src/predict.jl:198-234)
+ *   evt_update_nodes_idx split_set! / update_nodes_idx!: rows of split nodes move to the children, stably
+ *                        (src/fit-utils.jl:93-132; ext/.../fit-utils.jl:9-31)
+ *   evt_tree_close       the rest of evt_grow_tree_begin (predict! on rows outside the sample, the tree's way back);
+ *                        evt_grow_tree_end then collects the tree
+ * Levels run 1 .. max(1, max_depth - 1), each as hist_build, split_scan, update_nodes_idx in this order with the level
+ * passed along; a call out of order returns EVT_ERR_STATE and says which call the tree expects.  Between the
+ * stages evt_get_hist, evt_get_nidx (the node every sampled row has reached so far, read off the row lists the
+ * partition wrote), evt_peek_tree and evt_synchronize are allowed; every other call returns EVT_ERR_STATE
+ * until evt_tree_close.  A stage that fails closes the tree.  The stages queue exactly the kernels evt_grow_tree_begin
+ * queues: the finished tree is the same, bit for bit.
+ */
+int evt_tree_open(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js,
+                  const evt_params *params);
+int evt_hist_build(evt_handle h, int32_t level);
+int evt_split_scan(evt_handle h, int32_t level);
+int evt_update_nodes_idx(evt_handle h, int32_t level);
+int evt_tree_close(evt_handle h);
+/* The tree arrays as they stand on the device (nodes of levels not yet searched are zero). */
+int evt_peek_tree(evt_handle h, evt_tree_out *tree);
+
 /* predict!(cache.pred, tree, cache.x_bin, feattypes): src/predict.jl:1-46; ext/.../predict.jl:60-75.
  * Adds one host tree (arrays of length nnodes_tree) to the cache's prediction. */
 int evt_predict_tree(evt_handle h, int32_t nnodes_tree, const int64_t *feat, const uint8_t *cond_bin,
@@ -183,7 +213,8 @@ int evt_get_grads(evt_handle h, float *grad_out /* (2K+1) x nobs */);
 int evt_get_nidx(evt_handle h, uint32_t *nidx_out /* nobs */);
 /* Histogram of the last tree in the reference layout h∇[k, bin, feat, node] Float64
  * ((2K+1) x nbins x nfeats x (2^max_depth-1), src/init.jl:204); only slices of nodes that were
- * scanned and features in js are defined, the rest is zero. */
+ * scanned (or, inside a tree grown in stages, built from rows at the current level) and features in js are
+ * defined, the rest is zero. */
 int evt_get_hist(evt_handle h, double *hist_out);
 /* Fixed-point parameters of the last update: gradient row k is accumulated as
  * rint(v * 2^(qbits[k]-qexp[k])) in int64. */
