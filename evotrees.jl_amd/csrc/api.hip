@@ -619,8 +619,9 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, uint8_t cond, const uint32
         ARGCHK(jsv[i] >= 1 && jsv[i] <= (uint32_t)c->F, "js entries must be in 1..nfeats");
         ARGCHK(i == 0 || jsv[i] > jsv[i - 1], "js must be strictly ascending");
     }
-    // LDS budget of one block: channels x bins of a single feature must fit
-    ARGCHK((size_t)c->NA * c->B * 8 <= 64 * 1024, "histogram of one feature exceeds the LDS budget");
+    // LDS budget of one block: the channels of one launch x bins of a single feature must fit (more than EVT_MAX_NA
+    // channels go EVT_HIST_GROUP per launch)
+    ARGCHK((size_t)(c->NA <= EVT_MAX_NA ? c->NA : EVT_HIST_GROUP) * c->B * 8 <= 64 * 1024, "histogram of one feature exceeds the LDS budget");
 
     // rows kept by the mask (the host owns the RNG; src/subsample.jl:7-9).  The threshold, the count and the
     // compaction run on the device; the count comes back with the finished tree.

@@ -38,6 +38,7 @@ def _cases():
         ("gaussian_mle", True, 9000, 200, 128, 3, "binary", 77, 1.0, None, False, 102),
         ("mse", False, 12000, 130, 255, 4, "oblivious", 130, 0.5, None, True, 103),
         ("mlogloss", True, 1233, 578, 16, 1, "binary", 578, 0.5, 15, False, 104),
+        ("mlogloss", True, 112, 17, 255, 7, "binary", 13, 1.0, 16, True, 105),  # 33 channels x 255 bins
     ]
     return out
 
