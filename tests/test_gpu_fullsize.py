@@ -105,3 +105,45 @@ def test_full_size_rounds_bit_exact_against_oracle(evt):
     assert np.array_equal(h.get_pred().view(np.uint32), p_orc.view(np.uint32))
     h.close()
     o.close()
+
+
+@pytest.mark.parametrize("N,F", [(22_000_000, 100), (150_000_000, 8)])
+def test_offsets_past_two_to_the_31(evt, N, F):
+    """nobs x nfeats above 2^31 bytes (and nobs above 2^27 rows): every kernel's offsets are 64-bit.  The tree's node
+    ids, leaf weights, the updated prediction and whole-model inference are checked against an independent walk."""
+    B, D = 64, 6
+    rng = np.random.default_rng(1)
+    print("generating", N, "x", F, flush=True)
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    y = (rng.random(N, dtype=np.float32) + (x_bin[0] > 20) * 0.5 + (x_bin[F - 1] > 40) * 0.25).astype(np.float32)
+    mu = np.array([float(y[:1_000_000].mean())], np.float32)
+    h = evt.Handle(N, F, B, 1, D, "mse")
+    h.set_xbin(x_bin)
+    h.set_target(y, None, mu)
+    h.set_option("record_nidx", 1)
+    h.update_grads()
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    print("growing", flush=True)
+    t = h.grow_tree(js, evt.make_params(eta=0.5))
+    assert t.w[0] == np.float32(N)
+    assert t.feat[0] in (1, F)  # the two features the target depends on, the last one included
+    nidx = h.get_nidx()
+    pred = h.get_pred()[:, 0]
+    h.close()
+    print("walking", flush=True)
+    nid = np.ones(N, np.int64)
+    rows = np.arange(N)
+    for _ in range(D - 1):
+        sp = t.split[nid - 1].astype(bool)
+        f = np.where(sp, t.feat[nid - 1] - 1, 0)
+        nid = np.where(sp, 2 * nid + (x_bin[f, rows] > t.cond_bin[nid - 1]), nid)
+    assert np.array_equal(nidx, nid.astype(np.uint32))
+    cnt = np.bincount(nid, minlength=1 << D)
+    leaves = np.flatnonzero(cnt)
+    assert np.array_equal(t.w[leaves - 1], cnt[leaves].astype(np.float32))
+    assert np.array_equal(pred, (mu[0] + t.pred[nid - 1, 0]).astype(np.float32))
+    print("inference", flush=True)
+    ft = np.ones(F, np.uint8)
+    assert np.array_equal(evt._lib.predict_leaf_idx(x_bin, ft, [t]).reshape(-1), nid.astype(np.uint32))
+    raw = evt._lib.predict_model(x_bin, ft, "mse", 1, [t], apply_link=False)
+    assert np.array_equal(raw[:, 0], t.pred[nid - 1, 0])
