@@ -175,15 +175,19 @@ def main():
     def draw_mask():
         return None if cond >= 255 else mask_rng.bit_generator.random_raw((N + 7) // 8).view(np.uint8)[:N]
 
-    nxt = [draw_mask()]
+    staged = [False]
 
     def one_round():
         h.update_grads()
-        mask = nxt[0]
         js = np.arange(1, F + 1, dtype=np.uint32) if nfs >= F else (np.sort(rng.choice(F, nfs, replace=False)) + 1).astype(np.uint32)
-        # the next round's mask is drawn while the device grows this round's tree
-        evt._lib.check(L.evt_grow_tree_begin(h._h, evt._lib.ptr(mask), cond, evt._lib.ptr(js), js.shape[0], params))
-        nxt[0] = draw_mask()
+        if staged[0]:
+            evt._lib.check(L.evt_grow_tree_begin_staged(h._h, cond, evt._lib.ptr(js), js.shape[0], params))
+        else:
+            evt._lib.check(L.evt_grow_tree_begin(h._h, evt._lib.ptr(draw_mask()), cond, evt._lib.ptr(js), js.shape[0], params))
+        if cond < 255:
+            # the next round's mask is drawn and uploaded while the device grows this round's tree
+            h.stage_mask(draw_mask())
+            staged[0] = True
         evt._lib.check(L.evt_grow_tree_end(h._h, tree_out))
 
     h.set_option("grads_ahead", 1)  # one tree per round: the next round's gradients are queued behind the tree

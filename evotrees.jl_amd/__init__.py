@@ -222,7 +222,7 @@ class Cache:
 
     def __init__(self, handle, rng, nfs, params, N, F, config=None):
         self.handle, self.rng, self.nfs, self.params, self.N, self.F, self.config = handle, rng, nfs, params, N, F, config
-        self.next_mask = None  # the row mask of the next tree, drawn while the device grew the last one
+        self.mask_staged = False  # the row mask of the next tree has been drawn and uploaded while the device grew the last one
 
 
 def init(config, x_train, y_train, w_train=None, offset_train=None, feature_names=None, device=None):
@@ -275,9 +275,9 @@ def grow_evotree(m, cache, config):
     for _ in range(config.bagging_size):
         # all rows pass `mask <= 255`, so the draw is skipped when nothing can be dropped
         mask = None
-        if cond < 255:
-            mask = cache.next_mask if cache.next_mask is not None else cache.rng.integers(0, 256, cache.N, dtype=np.uint8)
-            cache.next_mask = None
+        staged = cache.mask_staged  # this tree's mask was drawn and uploaded while the device grew the last tree
+        if cond < 255 and not staged:
+            mask = cache.rng.integers(0, 256, cache.N, dtype=np.uint8)
         if cache.nfs >= cache.F:
             js = np.arange(1, cache.F + 1, dtype=np.uint32)
         else:
@@ -285,10 +285,15 @@ def grow_evotree(m, cache, config):
         t = Tree(m.K, h.nnodes)
         out = t.as_out()
         try:
-            _lib.check(_lib.load().evt_grow_tree_begin(h._h, _lib.ptr(mask), cond, _lib.ptr(js), js.shape[0], cache.params))
+            if staged:
+                cache.mask_staged = False
+                _lib.check(_lib.load().evt_grow_tree_begin_staged(h._h, cond, _lib.ptr(js), js.shape[0], cache.params))
+            else:
+                _lib.check(_lib.load().evt_grow_tree_begin(h._h, _lib.ptr(mask), cond, _lib.ptr(js), js.shape[0], cache.params))
             if cond < 255:
-                # the next draw of the RNG stream is the next tree's mask: made while the device grows this tree
-                cache.next_mask = cache.rng.integers(0, 256, cache.N, dtype=np.uint8)
+                # the next draw of the RNG stream is the next tree's mask: made and uploaded while the device grows this tree
+                h.stage_mask(cache.rng.integers(0, 256, cache.N, dtype=np.uint8))
+                cache.mask_staged = True
             _lib.check(_lib.load().evt_grow_tree_end(h._h, out))
         except EvtError as e:
             if e.code == _lib.EVT_ERR_EMPTY:

@@ -21,7 +21,7 @@ KERNEL_CLASSES = ["grad", "hist", "scan", "partition", "predict", "other"]
 EXPORTS = [
     "evt_last_error", "evt_device_count", "evt_create", "evt_destroy", "evt_set_xbin", "evt_binarize_f64",
     "evt_set_target", "evt_set_feature_meta", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
-    "evt_grow_tree_begin", "evt_grow_tree_end",
+    "evt_grow_tree_begin", "evt_grow_tree_end", "evt_stage_mask", "evt_grow_tree_begin_staged",
     "evt_tree_open", "evt_hist_build", "evt_split_scan", "evt_update_nodes_idx", "evt_tree_close", "evt_peek_tree",
     "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
     "evt_predict", "evt_predict_f64", "evt_predict_leaf_idx", "evt_eval_metric", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
@@ -73,6 +73,8 @@ def load():
         "evt_grow_tree": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams), C.POINTER(EvtTreeOut)],
         "evt_grow_tree_begin": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams)],
         "evt_grow_tree_end": [vp, C.POINTER(EvtTreeOut)],
+        "evt_stage_mask": [vp, vp],
+        "evt_grow_tree_begin_staged": [vp, C.c_uint8, vp, i32, C.POINTER(EvtParams)],
         "evt_tree_open": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams)],
         "evt_hist_build": [vp, i32],
         "evt_split_scan": [vp, i32],
@@ -225,6 +227,17 @@ class Handle:
             mask = np.ascontiguousarray(mask, np.uint8)
             assert mask.shape == (self.N,)
         check(load().evt_grow_tree_begin(self._h, ptr(mask), int(cond), ptr(js), js.shape[0], C.byref(params)))
+
+    def stage_mask(self, mask):
+        """Uploads the next tree's row mask while the tree begun with grow_tree_begin is still growing."""
+        mask = np.ascontiguousarray(mask, np.uint8)
+        assert mask.shape == (self.N,)
+        check(load().evt_stage_mask(self._h, ptr(mask)))
+
+    def grow_tree_begin_staged(self, js, params, cond):
+        """grow_tree_begin with the mask last given to stage_mask."""
+        js = np.ascontiguousarray(js, np.uint32)
+        check(load().evt_grow_tree_begin_staged(self._h, int(cond), ptr(js), js.shape[0], C.byref(params)))
 
     def grow_tree_end(self, want_tree=True):
         t = TreeArrays(self.K, self.nnodes) if want_tree else None

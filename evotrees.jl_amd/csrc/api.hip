@@ -154,7 +154,7 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id, c->pt_nodes, c->pt_pred};
+                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id, c->pt_nodes, c->pt_pred, c->mask_next};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -171,6 +171,10 @@ extern "C" int evt_destroy(evt_handle c) {
     for (auto e : c->free_events) (void)hipEventDestroy(e);
     if (c->tree_ev) (void)hipEventDestroy(c->tree_ev);
     if (c->pt_stage) (void)hipHostFree(c->pt_stage);
+    if (c->copy_stream) {
+        (void)hipStreamSynchronize(c->copy_stream);
+        (void)hipStreamDestroy(c->copy_stream);
+    }
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
     return EVT_OK;
@@ -235,6 +239,9 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->step.phase = 0;
     c->pt_nodes = nullptr; c->pt_pred = nullptr; c->pt_stage = nullptr; c->pt_stage_dev = nullptr; c->pt_cap = 0; c->pt_busy = false;
     c->tree_ev = nullptr;
+    c->mask_next = nullptr;
+    c->copy_stream = nullptr;
+    c->mask_next_valid = false;
     c->grads_ahead = false;
     c->grads_ready = false;
     c->last_cond = 255;
@@ -597,7 +604,8 @@ extern "C" int evt_set_grads(evt_handle c, const float *grad) {
     return EVT_OK;
 }
 
-static int tree_open(evt_ctx *c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p, bool staged) {
+static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p,
+                     bool staged) {
     ARGCHK(js && p, "js and params must not be NULL");
     ARGCHK(n_js >= 1 && n_js <= c->F, "n_js must be in [1, nfeats]");
     ARGCHK(p->bagging_size >= 1, "bagging_size must be >= 1");
@@ -625,7 +633,7 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, uint8_t cond, const uint32
 
     // rows kept by the mask (the host owns the RNG; src/subsample.jl:7-9).  The threshold, the count and the
     // compaction run on the device; the count comes back with the finished tree.
-    const bool all_rows = (mask == nullptr) || (cond == 255);
+    const bool all_rows = (mask == nullptr && !mask_staged) || (cond == 255);
     c->grads_ready = false; // this tree changes the predictions
     c->last_all_rows = all_rows;
     c->last_cond = cond;
@@ -664,9 +672,15 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, uint8_t cond, const uint32
     prof_begin(c, EVT_K_OTHER, 0);
     r = launch_apply_pending(c); // an earlier tree's values go in before its node ids are overwritten
     if (r != EVT_OK) return r;
+    if (mask_staged) { // uploaded by evt_stage_mask, which waited for the copy: the two buffers change places
+        std::swap(c->mask, c->mask_next);
+        c->mask_next_valid = false;
+    }
     if (!all_rows) {
-        HIPCHK(hipMemcpyAsync(c->mask, mask, c->N, hipMemcpyDefault, c->stream));
-        HIPCHK(hipStreamSynchronize(c->stream)); // the caller may reuse its mask buffer as soon as this call returns
+        if (!mask_staged) {
+            HIPCHK(hipMemcpyAsync(c->mask, mask, c->N, hipMemcpyDefault, c->stream));
+            HIPCHK(hipStreamSynchronize(c->stream)); // the caller may reuse its mask buffer as soon as this call returns
+        }
         r = launch_compact_mask(c, cond);
         if (r == EVT_OK && rec_nidx) r = launch_fill_u32(c, c->nidx, 0u, c->N);
     }
@@ -791,9 +805,8 @@ static int tree_fail(evt_ctx *c, int r) { // a failed stage leaves no tree open
     return r;
 }
 
-extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
-    CTXCHK(c);
-    int r = tree_open(c, mask, cond, js, n_js, p, false);
+// every stage of an opened tree, then the close: what evt_grow_tree_begin queues
+static int tree_run_stages(evt_ctx *c, int r) {
     while (r == EVT_OK && c->step.phase != 4) {
         r = tree_stage_hist(c);
         if (r == EVT_OK) r = tree_stage_scan(c);
@@ -803,9 +816,47 @@ extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t co
     return tree_close(c);
 }
 
+extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
+    CTXCHK(c);
+    int r = tree_open(c, mask, false, cond, js, n_js, p, false);
+    return tree_run_stages(c, r);
+}
+
+// The next tree's mask, uploaded while this one grows: the copy runs on a stream of its own, into the buffer the tree
+// in flight does not read.
+extern "C" int evt_stage_mask(evt_handle c, const uint8_t *mask) {
+    ARGCHK(c != nullptr, "handle is NULL");
+    ARGCHK(mask != nullptr, "mask is NULL");
+    HIPCHK(hipSetDevice(c->device));
+    if (c->step.phase != 0) {
+        evt_set_error("a tree opened with evt_tree_open has not been closed (evt_tree_close)");
+        return EVT_ERR_STATE;
+    }
+    if (!c->copy_stream) HIPCHK(hipStreamCreateWithFlags(&c->copy_stream, hipStreamNonBlocking));
+    if (!c->mask_next) {
+        int r = dev_alloc(&c->mask_next, (size_t)c->N);
+        if (r != EVT_OK) return r;
+    }
+    c->mask_next_valid = false;
+    HIPCHK(hipMemcpyAsync(c->mask_next, mask, c->N, hipMemcpyDefault, c->copy_stream));
+    HIPCHK(hipStreamSynchronize(c->copy_stream)); // the caller may reuse its buffer; the tree in flight keeps running
+    c->mask_next_valid = true;
+    return EVT_OK;
+}
+
+extern "C" int evt_grow_tree_begin_staged(evt_handle c, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
+    CTXCHK(c);
+    if (!c->mask_next_valid) {
+        evt_set_error("evt_grow_tree_begin_staged: no mask has been staged since the last tree (evt_stage_mask)");
+        return EVT_ERR_STATE;
+    }
+    int r = tree_open(c, nullptr, true, cond, js, n_js, p, false);
+    return tree_run_stages(c, r);
+}
+
 extern "C" int evt_tree_open(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
     CTXCHK(c);
-    int r = tree_open(c, mask, cond, js, n_js, p, true);
+    int r = tree_open(c, mask, false, cond, js, n_js, p, true);
     if (r != EVT_OK) return tree_fail(c, r);
     return EVT_OK;
 }

@@ -87,6 +87,10 @@ struct evt_ctx {
     uint32_t *is_id;   // [N] 0..N-1, written once: the root's row list when every row is in the tree
     uint32_t *nidx;
     uint8_t *mask;
+    // the next tree's row mask, uploaded on a stream of its own while the current tree grows (evt_stage_mask)
+    uint8_t *mask_next;
+    hipStream_t copy_stream;
+    bool mask_next_valid;
     unsigned long long *flagw;
     int32_t *chunk_nleft;
     int64_t *chunk_lpre;

@@ -159,6 +159,14 @@ int evt_grow_tree(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_
 int evt_grow_tree_begin(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js,
                         const evt_params *params);
 int evt_grow_tree_end(evt_handle h, evt_tree_out *tree);
+/* The upload of the next tree's mask (nobs bytes over PCIe, src/subsample.jl:7-9 / ext/.../subsample.jl:2-8) taken off
+ * the critical path: evt_stage_mask may be called while a tree begun with evt_grow_tree_begin is in flight; it copies
+ * the mask on a stream of its own into a second device buffer and returns when the copy is done (the caller's buffer
+ * is free again; the tree in flight keeps running).  evt_grow_tree_begin_staged is evt_grow_tree_begin with the mask
+ * staged last; EVT_ERR_STATE when none has been staged since the last tree.  Same trees, bit for bit. */
+int evt_stage_mask(evt_handle h, const uint8_t *mask);
+int evt_grow_tree_begin_staged(evt_handle h, uint8_t cond, const uint32_t *js, int32_t n_js,
+                               const evt_params *params);
 
 /*
  * The same tree, one kernel stage at a time: the stages are the reference's own per-level calls, so each can be

@@ -148,6 +148,51 @@ def test_deferred_leaf_addition_equals_immediate(evt, loss, K, tt):
             assert_tree_bits(a, b)
 
 
+def test_mask_staged_while_the_last_tree_grows(evt):
+    """evt_stage_mask + evt_grow_tree_begin_staged give the trees of evt_grow_tree with the same masks, bit for bit: the next
+    mask is uploaded while a tree is in flight (and the host buffer is free again on return); a staged begin without a
+    staged mask is refused; node ids derived afterwards use the mask of the tree they belong to."""
+    N, F, B, D = 60000, 9, 32, 6
+    x_bin, y, w, mu = make_data(17, N, F, B, "mse", weights=False)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    gp = evt.make_params(eta=0.3)
+    rng = np.random.default_rng(8)
+    masks = [rng.integers(0, 256, N, dtype=np.uint8) for _ in range(5)]
+    conds = [128, 40, 255, 200, 128]
+
+    def make():
+        h = evt.Handle(N, F, B, 1, D, "mse")
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        return h
+
+    ha, hb = make(), make()
+    with pytest.raises(evt.EvtError) as ei:
+        hb.grow_tree_begin_staged(js, gp, 128)
+    assert ei.value.code == evt._lib.EVT_ERR_STATE
+    hb.update_grads()
+    hb.stage_mask(masks[0].copy())
+    for r in range(5):
+        ha.update_grads()
+        ta = ha.grow_tree(js, gp, mask=masks[r], cond=conds[r])
+        if r > 0:
+            hb.update_grads()
+        hb.grow_tree_begin_staged(js, gp, conds[r])
+        if r + 1 < 5:
+            m = masks[r + 1].copy()
+            hb.stage_mask(m)  # while tree r is in flight
+            m[:] = 7          # the buffer is free again when the call returns
+        tb = hb.grow_tree_end()
+        assert_tree_bits(ta, tb)
+        assert np.array_equal(ha.get_nidx(), hb.get_nidx()), r  # walks the tree with the mask of tree r, not of tree r + 1
+    assert np.array_equal(ha.get_pred().view(np.uint32), hb.get_pred().view(np.uint32))
+    with pytest.raises(evt.EvtError) as ei:
+        hb.grow_tree_begin_staged(js, gp, 128)  # the last staged mask has been used
+    assert ei.value.code == evt._lib.EVT_ERR_STATE
+    ha.close()
+    hb.close()
+
+
 def test_grow_tree_in_two_halves(evt):
     """evt_grow_tree_begin / evt_grow_tree_end give the trees and predictions of evt_grow_tree, bit for bit; between
     the two halves the handle refuses every other call (and still answers afterwards); an end without a begin and an
