@@ -170,12 +170,15 @@ def main():
     tree_out = tree.as_out()
 
     # the host owns the row-sampling RNG (one uniform byte per row, drawn every round): raw 64-bit words viewed as bytes
-    mask_rng = np.random.default_rng(124)
+    mask_rng = np.random.Generator(np.random.SFC64(124))  # numpy's fastest bulk generator: the draw is host work inside the timed region
 
     def draw_mask():
         return None if cond >= 255 else mask_rng.bit_generator.random_raw((N + 7) // 8).view(np.uint8)[:N]
 
+    # below a few million rows a round is bound by the host's launches and the second stream's copy costs more than it hides
+    STAGE_MASK_MIN_ROWS = 4_000_000
     staged = [False]
+    nxt = [None]
 
     def one_round():
         h.update_grads()
@@ -183,11 +186,14 @@ def main():
         if staged[0]:
             evt._lib.check(L.evt_grow_tree_begin_staged(h._h, cond, evt._lib.ptr(js), js.shape[0], params))
         else:
-            evt._lib.check(L.evt_grow_tree_begin(h._h, evt._lib.ptr(draw_mask()), cond, evt._lib.ptr(js), js.shape[0], params))
+            mask = nxt[0] if nxt[0] is not None else draw_mask()
+            evt._lib.check(L.evt_grow_tree_begin(h._h, evt._lib.ptr(mask), cond, evt._lib.ptr(js), js.shape[0], params))
         if cond < 255:
-            # the next round's mask is drawn and uploaded while the device grows this round's tree
-            h.stage_mask(draw_mask())
-            staged[0] = True
+            # the next round's mask is drawn (and, for many rows, uploaded) while the device grows this round's tree
+            nxt[0] = draw_mask()
+            if N >= STAGE_MASK_MIN_ROWS:
+                h.stage_mask(nxt[0])
+                staged[0] = True
         evt._lib.check(L.evt_grow_tree_end(h._h, tree_out))
 
     h.set_option("grads_ahead", 1)  # one tree per round: the next round's gradients are queued behind the tree

@@ -223,6 +223,7 @@ class Cache:
     def __init__(self, handle, rng, nfs, params, N, F, config=None):
         self.handle, self.rng, self.nfs, self.params, self.N, self.F, self.config = handle, rng, nfs, params, N, F, config
         self.mask_staged = False  # the row mask of the next tree has been drawn and uploaded while the device grew the last one
+        self.next_mask = None  # ... or drawn only (few rows: the upload is not worth a second stream)
 
 
 def init(config, x_train, y_train, w_train=None, offset_train=None, feature_names=None, device=None):
@@ -267,6 +268,11 @@ def init(config, x_train, y_train, w_train=None, offset_train=None, feature_name
     return m, Cache(h, rng, nfs, params, N, F, config)
 
 
+# Rows from which the next tree's mask is drawn and uploaded while the current tree grows; below, a round is bound by the
+# host's launches and the second stream's copy costs more than it hides.
+STAGE_MASK_MIN_ROWS = 4_000_000
+
+
 def grow_evotree(m, cache, config):
     """grow_evotree!, src/fit.jl:6-42 (device twin ext/.../fit.jl:1-21): gradients, then bagging_size trees."""
     h = cache.handle
@@ -277,7 +283,8 @@ def grow_evotree(m, cache, config):
         mask = None
         staged = cache.mask_staged  # this tree's mask was drawn and uploaded while the device grew the last tree
         if cond < 255 and not staged:
-            mask = cache.rng.integers(0, 256, cache.N, dtype=np.uint8)
+            mask = cache.next_mask if cache.next_mask is not None else cache.rng.integers(0, 256, cache.N, dtype=np.uint8)
+            cache.next_mask = None
         if cache.nfs >= cache.F:
             js = np.arange(1, cache.F + 1, dtype=np.uint32)
         else:
@@ -291,9 +298,14 @@ def grow_evotree(m, cache, config):
             else:
                 _lib.check(_lib.load().evt_grow_tree_begin(h._h, _lib.ptr(mask), cond, _lib.ptr(js), js.shape[0], cache.params))
             if cond < 255:
-                # the next draw of the RNG stream is the next tree's mask: made and uploaded while the device grows this tree
-                h.stage_mask(cache.rng.integers(0, 256, cache.N, dtype=np.uint8))
-                cache.mask_staged = True
+                # the next draw of the RNG stream is the next tree's mask: made (and, for many rows, uploaded) while the
+                # device grows this tree
+                nm = cache.rng.integers(0, 256, cache.N, dtype=np.uint8)
+                if cache.N >= STAGE_MASK_MIN_ROWS:
+                    h.stage_mask(nm)
+                    cache.mask_staged = True
+                else:
+                    cache.next_mask = nm
             _lib.check(_lib.load().evt_grow_tree_end(h._h, out))
         except EvtError as e:
             if e.code == _lib.EVT_ERR_EMPTY:
