@@ -435,7 +435,14 @@ def binarize(x, edges):
     F = x.shape[1]
     out = np.empty((F, x.shape[0]), np.uint8)
     for j in range(F):
-        out[j] = np.searchsorted(edges[j], x[:, j], side="left") + 1
+        e = np.asarray(edges[j], np.float64)
+        col = np.asarray(x[:, j], np.float64)
+        idx = np.searchsorted(e, col, side="left")  # numpy orders NaN last, as isless does
+        # isless also puts -0.0 before 0.0: a +0.0 value passes the -0.0 edges that `<` treats as equal
+        pz = (col == 0) & ~np.signbit(col)
+        if pz.any() and (e == 0).any():
+            idx[pz] = np.searchsorted(e, 0.0, side="left") + int(((e == 0) & np.signbit(e)).sum())
+        out[j] = idx + 1
     return out
 
 

@@ -34,7 +34,16 @@ int launch_transpose_validate(evt_ctx *c) {
     return EVT_OK;
 }
 
-// searchsortedfirst(edges_j, x) = 1 + number of edges strictly below x.
+// Julia's isless on Float64 (the default order of searchsortedfirst): IEEE `<`, except that NaN sorts after everything and
+// -0.0 before 0.0.
+__device__ __forceinline__ bool jl_isless(double a, double b) {
+    if (a != a) return false;
+    if (b != b) return true;
+    if (a == 0.0 && b == 0.0) return (__double_as_longlong(a) < 0) && (__double_as_longlong(b) >= 0);
+    return a < b;
+}
+
+// searchsortedfirst(edges_j, x) = 1 + number of edges that are isless than x (src/fit-utils.jl:69); a NaN lands in the last bin.
 __global__ __launch_bounds__(256) void k_binarize(const double *__restrict__ x, const double *__restrict__ edges,
                                                  const int32_t *__restrict__ edge_off, uint8_t *__restrict__ xcm, int64_t N,
                                                  int64_t ldx, int64_t ldo) {
@@ -48,7 +57,7 @@ __global__ __launch_bounds__(256) void k_binarize(const double *__restrict__ x, 
         int lo = 0, hi = ne;
         while (lo < hi) {
             int mid = (lo + hi) >> 1;
-            if (s_edges[mid] < v) lo = mid + 1; else hi = mid;
+            if (jl_isless(s_edges[mid], v)) lo = mid + 1; else hi = mid;
         }
         xcm[(size_t)j * ldo + i] = (uint8_t)(lo + 1);
     }

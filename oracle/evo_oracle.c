@@ -154,7 +154,16 @@ void orc_update_grads(const orc_params *p, int64_t N, const float *pred, const f
     }
 }
 
-/* binarize — src/fit-utils.jl:66-72: searchsortedfirst(edges, x) = 1 + #(edges < x). */
+/* Julia's isless on Float64, the order searchsortedfirst uses by default: IEEE `<`, except that NaN sorts after
+ * everything (Inf included) and -0.0 before 0.0. */
+static inline int jl_isless(double a, double b) {
+    if (isnan(a)) return 0;
+    if (isnan(b)) return 1;
+    if (a == 0.0 && b == 0.0) return signbit(a) && !signbit(b);
+    return a < b;
+}
+
+/* binarize — src/fit-utils.jl:66-72: searchsortedfirst(edges, x) = 1 + #(edges isless x); a NaN lands in the last bin. */
 void orc_binarize(int64_t N, const double *x, const double *edges, int32_t nedges, uint8_t *out) {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < N; i++) {
@@ -162,7 +171,7 @@ void orc_binarize(int64_t N, const double *x, const double *edges, int32_t nedge
         int lo = 0, hi = nedges; /* first index with edges[idx] >= v */
         while (lo < hi) {
             int mid = (lo + hi) >> 1;
-            if (edges[mid] < v) lo = mid + 1; else hi = mid;
+            if (jl_isless(edges[mid], v)) lo = mid + 1; else hi = mid;
         }
         out[i] = (uint8_t)(lo + 1);
     }

@@ -472,8 +472,16 @@ def test_device_binarize(evt):
     edges = [np.sort(rng.random(B - 1)) for _ in range(F)]
     edges[2] = edges[2][:5]
     x[1, :63] = edges[1]  # values equal to an edge
+    # the order is Julia's isless: NaN after everything (the last bin), -0.0 before 0.0; infinities at the ends
+    edges[3] = np.sort(np.concatenate([-rng.random(30), [-0.0, 0.0], rng.random(31)]))
+    x[3] = rng.standard_normal(N)
+    x[3, :8] = [np.nan, -0.0, 0.0, np.inf, -np.inf, np.nan, 0.0, -0.0]
+    x[4, ::11] = np.nan
     h = evt.Handle(N, F, B, 1, 2, "mse")
     h.binarize(x, edges)
+    assert np.array_equal(h.get_xbin(), evt.binarize(x.T, edges))  # the host mirror's binarize (inference inputs) agrees
+    assert np.array_equal(h.get_xbin()[3, :8], orc.binarize(x[3, :8], edges[3]))
+    assert h.get_xbin()[3, 0] == 64 and h.get_xbin()[3, 2] == h.get_xbin()[3, 1] + 1
     # read the bins back through a one-split tree per feature: compare against the oracle's binarize
     h.set_target(np.zeros(N, np.float32), None, np.zeros(1, np.float32))
     for j in range(F):

@@ -106,6 +106,22 @@ def test_binarize_searchsortedfirst():
     assert got.min() >= 1 and got.max() <= 16
 
 
+def test_binarize_orders_values_as_julia_isless():
+    """searchsortedfirst's default order is isless (src/fit-utils.jl:69 passes none): NaN after everything, Inf included,
+    and -0.0 before 0.0.  Known answers worked by hand from that definition, and numpy's own NaN-last ordering."""
+    edges = np.array([-1.0, -0.0, 0.0, 1.0])
+    x = np.array([-np.inf, -1.0, -0.5, -0.0, 0.0, 0.5, 1.0, 2.0, np.inf, np.nan])
+    #             first index whose edge is not isless than x
+    want = np.array([1, 1, 2, 2, 3, 4, 4, 5, 5, 5], np.uint8)
+    assert np.array_equal(orc.binarize(x, edges), want)
+    rng = np.random.default_rng(5)
+    e2 = np.sort(rng.standard_normal(31))
+    x2 = rng.standard_normal(500)
+    x2[::7] = np.nan
+    assert np.array_equal(orc.binarize(x2, e2), (np.searchsorted(e2, x2, side="left") + 1).astype(np.uint8))
+    assert (orc.binarize(x2, e2)[::7] == 32).all()
+
+
 def test_subsample_threshold_rule():
     mask = np.arange(256, dtype=np.uint8)
     # src/subsample.jl:9: cond = round(UInt8, 255*rowsample), half-to-even: 0.5 -> 128
