@@ -21,7 +21,6 @@ __all__ = ["EvoTreeRegressor", "EvoTreeCount", "EvoTreeClassifier", "EvoTreeMLE"
            "grow_evotree", "update", "okay_to_continue", "get_edges", "check_args", "CallBack", "init_logger", "update_logger", "EvtError"]
 
 _GPU_DEVICES = ("gpu", "rocm", "amd", "hip")
-_LOSS_K = {"mse": 1, "logloss": 1, "gaussian_mle": 2, "poisson": 1, "gamma": 1, "tweedie": 1}
 _EXP_LINK = ("poisson", "gamma", "tweedie")
 # is_maximise, src/metrics.jl:195-207
 _MAXIMISE = {"mse": False, "rmse": False, "mae": False, "logloss": False, "poisson": False, "gamma": False, "tweedie": False,
@@ -171,12 +170,24 @@ def _levelcode(y, levels):
     return (order[pos] + 1).astype(np.float32)
 
 
-def _init_target(loss, y):
-    """_init_target, src/init.jl:10-146 (in-scope branches).  Returns K, y (Float32), mu, target levels."""
+def _target_rows(y):
+    """A vector target is one row; a matrix target holds one row per target (T x nobs, as the reference takes it)."""
     y = np.asarray(y)
-    if y.ndim != 1:
-        raise ValueError("only vector targets are supported by this backend")
+    if y.ndim == 1:
+        return y[None, :]
+    if y.ndim != 2:
+        raise ValueError("the target must be a vector or a targets x observations matrix")
+    return y
+
+
+def _init_target(loss, y):
+    """_init_target, src/init.jl:10-146 (in-scope branches).  Returns K, y (Float32; (N,) for one target, (N, T) for a
+    T x N matrix target), mu, target levels."""
+    y = np.asarray(y)
     if loss == "mlogloss":  # src/init.jl:43-67: levels = sort(unique(y)), level codes, mu = log(proportions) - max
+        if y.ndim != 1:  # src/init.jl:11-16
+            raise RuntimeError("Multi-target (matrix target) is supported for gradient-regression losses (mse, logloss, poisson, "
+                               "gamma, tweedie) and gaussian_mle. Got loss mlogloss.")
         if y.dtype.kind == "f":
             raise RuntimeError("Invalid target eltype: %s" % y.dtype)
         levels = np.unique(y)
@@ -189,20 +200,23 @@ def _init_target(loss, y):
         mu = np.log(prop).astype(np.float32)
         mu = mu - mu.max()
         return K, codes, mu.astype(np.float32), levels
-    y32 = y.astype(np.float32)
-    if loss == "logloss":
-        if y32.min() < 0 or y32.max() > 1:
-            raise AssertionError("logloss targets must be in [0, 1]")
-        mu = np.array([_logit(np.float32(y32.mean(dtype=np.float32)))], np.float32)
-    elif loss == "gaussian_mle":
-        m = np.float32(y32.mean(dtype=np.float32))
-        s = np.float32(y32.std(ddof=1, dtype=np.float32))
-        mu = np.array([m, _invsoftplus(s)], np.float32)
-    elif loss in _EXP_LINK:
-        mu = np.array([np.log(np.float32(y32.mean(dtype=np.float32)))], np.float32)
-    else:
-        mu = np.array([y32.mean(dtype=np.float32)], np.float32)
-    return _LOSS_K[loss], y32, mu.astype(np.float32), None
+    rows = _target_rows(y).astype(np.float32)  # T x N
+    if loss == "logloss" and (rows.min() < 0 or rows.max() > 1):
+        raise AssertionError("logloss targets must be in [0, 1]")
+    mu = []
+    for yt in rows:  # one bias per target (two for gaussian_mle), src/init.jl:24-31, :33-41, :68-83, :137-150
+        m = np.float32(yt.mean(dtype=np.float32))
+        if loss == "logloss":
+            mu.append(_logit(m))
+        elif loss == "gaussian_mle":
+            mu += [m, _invsoftplus(np.float32(yt.std(ddof=1, dtype=np.float32)))]
+        elif loss in _EXP_LINK:
+            mu.append(np.log(m))
+        else:
+            mu.append(m)
+    mu = np.array(mu, np.float32)
+    y32 = rows[0] if y.ndim == 1 else np.ascontiguousarray(rows.T)
+    return mu.shape[0], y32, mu, None
 
 
 def _link_offset(loss, offset, N, K):
@@ -213,7 +227,7 @@ def _link_offset(loss, offset, N, K):
     elif loss in _EXP_LINK or loss == "mlogloss":
         offset = np.log(offset)
     elif loss == "gaussian_mle":
-        offset[:, 1] = _invsoftplus(offset[:, 1])
+        offset[:, 1::2] = _invsoftplus(offset[:, 1::2])  # every scale column (unconstrain_mle_scale!)
     return offset.astype(np.float32)
 
 
@@ -327,8 +341,9 @@ class CallBack:
         if m.loss_type == "mlogloss":
             y32 = _levelcode(np.asarray(y_eval), m.info["target_levels"])
         else:
-            y32 = np.asarray(y_eval).astype(np.float32)
-        if y32.shape != (N,):
+            ye = np.asarray(y_eval).astype(np.float32)
+            y32 = ye if ye.ndim == 1 else np.ascontiguousarray(ye.T)  # a matrix target is targets x observations
+        if y32.shape[0] != N:
             raise AssertionError("y_eval length must equal the number of eval rows")
         w = None if w_eval is None else np.asarray(w_eval, np.float32)
         offset = None if offset_eval is None else _link_offset(m.loss_type, offset_eval, N, m.K)

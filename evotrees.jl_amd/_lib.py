@@ -192,7 +192,10 @@ class Handle:
         w = None if w is None else np.ascontiguousarray(w, np.float32)
         mu = np.ascontiguousarray(mu, np.float32)
         offset = None if offset is None else np.ascontiguousarray(offset, np.float32)
-        assert y.shape == (self.N,) and mu.shape == (self.K,)
+        # one value per row and target: (N,) for one target, (N, T) C-order (Julia's T x N) for several
+        T = 1 if self.loss == "mlogloss" else (self.K // 2 if self.loss == "gaussian_mle" else self.K)
+        assert (y.shape == (self.N,) and T == 1) or y.shape == (self.N, T)
+        assert mu.shape == (self.K,)
         check(load().evt_set_target(self._h, ptr(y), ptr(w), ptr(mu), ptr(offset)))
 
     def set_feature_meta(self, feattypes=None, monotone=None):

@@ -191,7 +191,8 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ARGCHK(loss >= 0 && loss <= EVT_LOSS_MLOGLOSS, "loss must be one of mse (0), logloss (1), gaussian_mle (2), poisson (3), gamma (4), tweedie (5), mlogloss (6)");
     ARGCHK(tree_type == EVT_TREE_BINARY || tree_type == EVT_TREE_OBLIVIOUS, "tree_type must be binary (0) or oblivious (1)");
     if (loss == EVT_LOSS_MLOGLOSS) ARGCHK(K >= 2 && K <= EVT_MAX_K, "mlogloss needs 2 <= K <= 16 classes");
-    else ARGCHK(K == (loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1), "K must be 2 for gaussian_mle and 1 for the other one-target losses");
+    else if (loss == EVT_LOSS_GAUSSIAN_MLE) ARGCHK(K >= 2 && K <= EVT_MAX_K && K % 2 == 0, "gaussian_mle needs K = 2 x targets, 2 <= K <= 16");
+    else ARGCHK(K >= 1 && K <= EVT_MAX_K, "K (targets) must be in [1, 16]");
     int ndev = 0;
     {
         int r = evt_device_count(&ndev);
@@ -205,6 +206,8 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     memset((void *)&c->device, 0, sizeof(int));
     c->stream = nullptr;
     c->N = nobs; c->F = nfeats; c->B = nbins; c->K = K; c->NK = 2 * K + 1; c->D = max_depth; c->loss = loss; c->tree_type = tree_type;
+    c->T = (loss == EVT_LOSS_MLOGLOSS) ? 1 : (loss == EVT_LOSS_GAUSSIAN_MLE ? K / 2 : K);
+    c->mc = (loss == EVT_LOSS_MLOGLOSS) || K > (loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1);
     c->nnodes = (1 << max_depth) - 1;
     c->maxlvl = 1 << (max_depth - 1);
     c->RS = record_stride(nfeats);
@@ -270,7 +273,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->max_chunks = (N + EVT_CHUNK - 1) / EVT_CHUNK + c->maxlvl + 2;
     ALLOC(c->xcm, (size_t)N * c->F);
     ALLOC(c->xrm, (size_t)N * c->RS);
-    ALLOC(c->y, N);
+    ALLOC(c->y, N * c->T);
     ALLOC(c->pred, (size_t)N * K);
     ALLOC(c->grad, (size_t)N * c->NK);
     ALLOC(c->gq, (size_t)N * c->NK);
@@ -475,7 +478,7 @@ extern "C" int evt_binarize_f64(evt_handle c, const double *x_colmajor, const do
 static void set_channels(evt_ctx *c) {
     // LDS channels (rows of the gradient matrix that need their own accumulator)
     int na = 0;
-    if (c->loss == EVT_LOSS_MSE) {
+    if (c->loss == EVT_LOSS_MSE && c->K == 1) {
         c->chan_k[na++] = 0;                   // g ; h == 2w is derived
         if (!c->unit_w) c->chan_k[na++] = 2;   // w
     } else {
@@ -484,7 +487,7 @@ static void set_channels(evt_ctx *c) {
     }
     c->NA = na;
     for (int a = na; a < EVT_MC_MAX_NK; a++) c->chan_k[a] = 0;
-    c->NAg = (c->loss == EVT_LOSS_MSE) ? 2 : c->NK;
+    c->NAg = (c->loss == EVT_LOSS_MSE && c->K == 1) ? 2 : c->NK;
     int qbg = 62 - ceil_log2_i64(c->N);
     if (qbg > 40) qbg = 40;
     for (int k = 0; k < c->NK; k++) c->h_qbits[k] = qbg;
@@ -501,7 +504,7 @@ extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, cons
     c->grads_ready = false;
     c->unit_w = (w == nullptr);
     set_channels(c);
-    HIPCHK(hipMemcpyAsync(c->y, y, sizeof(float) * c->N, hipMemcpyDefault, c->stream));
+    HIPCHK(hipMemcpyAsync(c->y, y, sizeof(float) * c->N * c->T, hipMemcpyDefault, c->stream));
     if (c->loss == EVT_LOSS_MLOGLOSS) {
         int r = launch_validate_classes(c);
         if (r != EVT_OK) return r;
@@ -550,6 +553,9 @@ extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, cons
         ARGCHK(mo[j] >= -1 && mo[j] <= 1, "monotone constraints must be -1, 0 or 1");
         // the reference has no pred_scalar method for the multi-class loss (src/predict.jl:205-238): a constraint cannot be evaluated there
         ARGCHK(mo[j] == 0 || c->loss != EVT_LOSS_MLOGLOSS, "monotone constraints are not defined for mlogloss");
+        // with several targets the reference's pred_scalar (src/predict.jl:205-208, :235-238) still reads the statistics at the
+        // one-target positions, i.e. another target's gradient as the hessian: refused rather than reproduced
+        ARGCHK(mo[j] == 0 || !c->mc, "monotone constraints are not defined for more than one target");
     }
     HIPCHK(hipMemcpy(c->feattypes, ft.data(), c->F, hipMemcpyHostToDevice));
     HIPCHK(hipMemcpy(c->mono, mo.data(), sizeof(int32_t) * c->F, hipMemcpyHostToDevice));

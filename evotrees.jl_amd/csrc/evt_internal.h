@@ -66,6 +66,8 @@ struct evt_ctx {
     hipStream_t stream;
     int64_t N;
     int32_t F, B, K, NK, D, loss, tree_type;
+    int32_t T;         // target columns of y: K for the gradient-regression losses, K / 2 for gaussian_mle, 1 (the class) for mlogloss
+    bool mc;           // more outputs than the specialised kernels take: run-time channel count (multi-class, several targets)
     int32_t nnodes;    // 2^D - 1
     int32_t maxlvl;    // 2^(D-1)
     int32_t RS;        // bytes per observation-major record

@@ -90,6 +90,100 @@ __global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const f
     }
 }
 
+// Several targets at once (y is T x N, one column per row of data; src/loss.jl:49-50, :100-111, :219-236): the same
+// per-target expressions as k_grads with K = T outputs (2T for gaussian_mle, whose rows are
+// [g_loc_1, g_scale_1, g_loc_2, ..., h_loc_1, h_scale_1, ..., w]).
+template <int LOSS>
+__device__ __forceinline__ void grad_hess_one(float pk, float yk, float &g, float &h) {
+    if (LOSS == 0) {
+        g = 2.0f * (pk - yk);
+        h = 2.0f;
+    } else if (LOSS == 1) {
+        const float s = dev_sigmoid(pk);
+        g = s - yk;
+        h = s * (1.0f - s);
+    } else if (LOSS == 3) {
+        const float e = expf(pk);
+        g = e - yk;
+        h = e;
+    } else if (LOSS == 4) {
+        const float e = expf(pk);
+        g = 2.0f * (1.0f - yk / e);
+        h = 2.0f * yk / e;
+    } else {
+        const float e = expf(pk);
+        const float a = powf(e, 0.5f), b = powf(e, -0.5f);
+        g = 2.0f * (a - yk * b);
+        h = 2.0f * (0.5f * a - (-0.5f) * yk * b);
+    }
+}
+
+template <int LOSS>
+__global__ __launch_bounds__(256) void k_grads_mt(float *__restrict__ pred, const float *__restrict__ y, float *__restrict__ grad, int64_t N,
+                                                 int K, uint32_t *absmax, const uint32_t *__restrict__ pend_nidx,
+                                                 const float *__restrict__ pend_leaf, int unit_w) {
+    const int NK = 2 * K + 1;
+    const int T = (LOSS == 2) ? K / 2 : K; // target columns
+    __shared__ float s_m[4];
+    float mx[2 * EVT_MAX_K];
+#pragma unroll
+    for (int k = 0; k < 2 * EVT_MAX_K; k++) mx[k] = 0.0f;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
+        float *pr = pred + (size_t)K * i;
+        float *g = grad + (size_t)NK * i;
+        const float *yi = y + (size_t)T * i;
+        const float w = unit_w ? 1.0f : g[NK - 1];
+        if (pend_nidx) evt_add_leaf(pr, pend_leaf + (size_t)K * (pend_nidx[i] - 1), K, LOSS);
+#pragma unroll
+        for (int k = 0; k < EVT_MAX_K; k++) {
+            if (k < K) {
+                float gg, hh;
+                if (LOSS == 2) {
+                    // output k of pair t = k / 2: even = location, odd = raw scale
+                    const int t = k >> 1;
+                    const float loc = pr[2 * t], raw = pr[2 * t + 1];
+                    const float scale = dev_softplus(raw);
+                    const float dscale = dev_sigmoid(raw);
+                    const float resid = loc - yi[t];
+                    const float s2 = scale * scale;
+                    const float ds = dscale / scale;
+                    if ((k & 1) == 0) {
+                        gg = (resid / s2) * w;
+                        hh = (1.0f / s2) * w;
+                    } else {
+                        gg = ((1.0f - (resid * resid) / s2) * dscale / scale) * w;
+                        hh = (2.0f * (ds * ds)) * w;
+                    }
+                } else {
+                    float g1, h1;
+                    grad_hess_one<LOSS>(pr[k], yi[k], g1, h1);
+                    gg = g1 * w;
+                    hh = h1 * w;
+                }
+                g[k] = gg;
+                g[K + k] = hh;
+                mx[k] = fmaxf(mx[k], fabsf(gg));
+                mx[EVT_MAX_K + k] = fmaxf(mx[EVT_MAX_K + k], fabsf(hh));
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 2 * EVT_MAX_K; k++) {
+        const int kk = k < EVT_MAX_K ? k : k - EVT_MAX_K;
+        if (kk < K) { // uniform
+            const float m = wave_max_f32(mx[k]);
+            __syncthreads();
+            if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                const float mm = fmaxf(fmaxf(s_m[0], s_m[1]), fmaxf(s_m[2], s_m[3]));
+                const int row = k < EVT_MAX_K ? k : K + kk;
+                if (mm > 0.0f) atomicMax(&absmax[row], __float_as_uint(mm));
+            }
+        }
+    }
+}
+
 // Multi-class log loss (src/loss.jl:93-98, :113-128): prob_k = exp(p_k) / sum_j exp(p_j); g_k = (prob_k - [y == k]) w,
 // h_k = prob_k (1 - prob_k) w; y holds the 1-based class.  The row maxima are reduced one gradient row at a time.
 __global__ __launch_bounds__(256) void k_grads_mlogloss(float *__restrict__ pred, const float *__restrict__ y, float *__restrict__ grad,
@@ -177,7 +271,7 @@ __global__ void k_quant_setup(uint32_t *absmax, const int32_t *qbits, int32_t *q
     __syncthreads();
     if (k < NAg) {
         // global channel ag -> gradient row: mse {g, w}; otherwise identity; last channel is w (or the row count)
-        int kk = (loss == 0) ? (k == 0 ? 0 : 2) : k;
+        int kk = (loss == 0 && NK == 3) ? (k == 0 ? 0 : 2) : k; // one-target mse: channels {g, w}
         if (k == NAg - 1 && unit_w) qscale_g[k] = 1.0;
         else qscale_g[k] = scalbn(1.0, qexp[kk] - qbits[kk]);
     }
@@ -208,6 +302,21 @@ int launch_grads(evt_ctx *c) {
     dim3 grid((unsigned)nb);
     const uint32_t *pn = c->pend_pred ? c->nidx : nullptr; // the last tree's leaf values are added on the way
     c->pend_pred = false;
+    const bool multi_target = c->loss != EVT_LOSS_MLOGLOSS && c->K > (c->loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1);
+    if (multi_target) {
+#define MT(L_) hipLaunchKernelGGL(k_grads_mt<L_>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0)
+        switch (c->loss) {
+        case EVT_LOSS_MSE: MT(0); break;
+        case EVT_LOSS_LOGLOSS: MT(1); break;
+        case EVT_LOSS_GAUSSIAN_MLE: MT(2); break;
+        case EVT_LOSS_POISSON: MT(3); break;
+        case EVT_LOSS_GAMMA: MT(4); break;
+        default: MT(5); break;
+        }
+#undef MT
+        HIPCHK(hipGetLastError());
+        return EVT_OK;
+    }
     if (c->loss == EVT_LOSS_MSE)
         hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_LOGLOSS)
@@ -262,7 +371,7 @@ int launch_quantize(evt_ctx *c) {
                        c->loss, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
     hipLaunchKernelGGL(k_quantize, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, c->gq, c->N, c->NK, c->NA,
-                       c->loss == EVT_LOSS_MSE ? 1 : 0, qmul, c->unit_w ? 1 : 0);
+                       (c->loss == EVT_LOSS_MSE && c->K == 1) ? 1 : 0, qmul, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -271,18 +380,29 @@ int launch_quantize(evt_ctx *c) {
 // Per row value of src/metrics.jl:1-28 (:88-91 for gaussian_mle) in Float32, weighted as eval[i] = w * v / K
 // (:43, :111), accumulated in Float64.  Two stages with a fixed shape (EVT_METRIC_BLOCKS partial sums, then one
 // block) keep the summation order, hence the result, independent of scheduling.
+__device__ __forceinline__ float metric_value_one(int metric, float pk, float yk);
 __device__ __forceinline__ float metric_value(int metric, int K, const float *__restrict__ pred, const float *__restrict__ y, int64_t i) {
     if (metric == EVT_METRIC_MLOGLOSS) { // src/metrics.jl:59-77
         float isum = 0.0f;
         for (int k = 0; k < K; k++) isum += expf(pred[(size_t)K * i + k]);
         return logf(isum) - pred[(size_t)K * i + (int)y[i] - 1];
     }
-    if (metric == EVT_METRIC_GAUSSIAN_MLE) {
-        const float loc = pred[2 * i], scale = dev_softplus(pred[2 * i + 1]);
-        const float d = y[i] - loc;
-        return -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+    if (metric == EVT_METRIC_GAUSSIAN_MLE) { // src/metrics.jl:88-91, :98-114: summed over the targets
+        const int T = K / 2;
+        float acc = 0.0f;
+        for (int t = 0; t < T; t++) {
+            const float loc = pred[(size_t)K * i + 2 * t], scale = dev_softplus(pred[(size_t)K * i + 2 * t + 1]);
+            const float d = y[(size_t)T * i + t] - loc;
+            acc += -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+        }
+        return acc;
     }
-    const float pk = pred[i], yk = y[i];
+    float acc = 0.0f; // src/metrics.jl:39-43: the per-target values are added in Float32, starting from zero
+    for (int k = 0; k < K; k++) acc += metric_value_one(metric, pred[(size_t)K * i + k], y[(size_t)K * i + k]);
+    return acc;
+}
+
+__device__ __forceinline__ float metric_value_one(int metric, float pk, float yk) {
     switch (metric) {
     case EVT_METRIC_MSE:
     case EVT_METRIC_RMSE: return (pk - yk) * (pk - yk);

@@ -677,7 +677,7 @@ __global__ __launch_bounds__(256) void k_hist_export(const long long *__restrict
         double ch[EVT_MC_MAX_NK];
         for (int ag = 0; ag < NAg; ag++) ch[ag] = (double)hn[((int64_t)jp * NAg + ag) * B + b] * qscale[ag];
         double *o = out + (((int64_t)node * F + f) * B + b) * NK;
-        if (loss == 0) {
+        if (loss == 0 && NK == 3) {
             o[0] = ch[0];
             o[1] = 2.0 * ch[1];
             o[2] = ch[1];

@@ -79,7 +79,7 @@ __device__ __forceinline__ double term_gh(double g, double h, double w, double l
 
 // fixed-point channel sums -> the 2K+1 Float64 statistics [g.., h.., w]
 __device__ __forceinline__ void decode_vals(const long long *q, const double *sc, int loss, int NK, double *out) {
-    if (loss == EVT_LOSS_MSE) {
+    if (loss == EVT_LOSS_MSE && NK == 3) { // one-target mse: channels {g, w}, h = 2w
         double w = (double)q[1] * sc[1];
         out[0] = (double)q[0] * sc[0];
         out[1] = 2.0 * w;
@@ -814,7 +814,7 @@ int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     // extra blocks per node that only clear the children's histogram slices, while a level has few nodes
     unsigned zero_blocks = 0;
     if (!leaf_level && A.zero_children && !A.oblivious && nodes < 64) zero_blocks = 64 / nodes < 16 ? 64 / nodes : 16;
-    if (c->loss == EVT_LOSS_MLOGLOSS) {
+    if (c->mc) { // any number of outputs: multi-class, several targets
         if (!leaf_level) {
             if (bpl == 1) hipLaunchKernelGGL((k_scan_mc<1>), grid, dim3(256), 0, c->stream, A);
             else if (bpl == 2) hipLaunchKernelGGL((k_scan_mc<2>), grid, dim3(256), 0, c->stream, A);

@@ -99,8 +99,10 @@ int evt_device_count(int32_t *count);
 /* ---- training cache ------------------------------------------------------------------
  * Replaces init_core(params, ::Type{<:GPU}, ...) device allocation
  * (ext/EvoTreesKernelAbstractionsExt/init.jl:1-151): sizes every device buffer.
- * nbins in [2,255] (src/learners.jl:527), K = 2 for gaussian_mle (one target), the number of classes
- * (2..16) for mlogloss, 1 for every other loss. */
+ * nbins in [2,255] (src/learners.jl:527).  K is the number of outputs (size(pred, 1) in the reference, at most 16):
+ * the number of targets for mse / logloss / poisson / gamma / tweedie (1, or more with a matrix target,
+ * src/init.jl:11-16, :142-150), twice the number of targets for gaussian_mle (src/init.jl:68-83), the number of
+ * classes (2..16) for mlogloss. */
 int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K, int32_t max_depth, int32_t loss,
                int32_t tree_type, evt_handle *out);
 /* Frees all device memory; the slot post_fit_gc has in the reference (src/fit.jl:340). */
@@ -117,13 +119,17 @@ int evt_set_xbin(evt_handle h, const uint8_t *x_bin_colmajor);
 int evt_binarize_f64(evt_handle h, const double *x_colmajor, const double *edges, const int32_t *edge_off);
 
 /* Target, weights and initial prediction: y Float32[nobs] (for mlogloss the 1-based level code of each row,
- * as _init_target builds it, src/init.jl:43-67); w Float32[nobs] or NULL for ones
+ * as _init_target builds it, src/init.jl:43-67) or, with T > 1 targets, the reference's T x nobs column-major matrix
+ * (the T values of a row side by side; _target(y, k, i), src/loss.jl:49-50); w Float32[nobs] or NULL for ones
  * (device_ones, src/init.jl:300); pred[:, i] = mu (+ offset[:, i] if offset != NULL), offset is
  * K x nobs (src/init.jl:168-174).  Writes the weight row of the gradient matrix. */
 int evt_set_target(evt_handle h, const float *y, const float *w, const float *mu, const float *offset);
 
 /* feattypes[j] != 0: numeric (<=), 0: categorical (==); monotone[j] in {-1,0,1}
- * (cache.feattypes / cache.monotone_constraints, src/init.jl:183-187).  NULL = all numeric / none. */
+ * (cache.feattypes / cache.monotone_constraints, src/init.jl:183-187).  NULL = all numeric / none.
+ * A constraint is refused (EVT_ERR_ARG) for mlogloss and for more than one target: the reference has no
+ * pred_scalar for the former, and for the latter its pred_scalar (src/predict.jl:205-208, :235-238) reads the
+ * statistics at the one-target positions. */
 int evt_set_feature_meta(evt_handle h, const uint8_t *feattypes, const int32_t *monotone);
 
 /* update_grads!(cache.∇, cache.pred, cache.y, L, params): src/loss.jl:100-111, :219-236;
@@ -204,7 +210,7 @@ int evt_predict_tree(evt_handle h, int32_t nnodes_tree, const int64_t *feat, con
                      const float *pred, const uint8_t *split);
 
 /* The eval CallBack's metric (src/callback.jl:130-135 -> src/metrics.jl:30-48, :100-116) on the
- * handle's own state: sum_i(Float32(w[i] * value(pred[:, i], y[i]) / K)) / sum_i(w[i]), both sums in
+ * handle's own state: sum_i(Float32(w[i] * sum_k value(pred[k, i], y[k, i]) / K)) / sum_i(w[i]), both sums in
  * Float64; rmse = sqrt(mse).  A handle created on the eval rows (evt_create + evt_set_xbin /
  * evt_binarize_f64 + evt_set_target with the eval y, w, offset and mu = 0) plays the CallBack: each
  * new tree is added with evt_predict_tree, then this call returns the metric.  The sum order is

@@ -92,7 +92,7 @@ static inline float orc_softplusf(float x) {
  * update_grads!  — src/loss.jl:100-111 (GradientRegression: mse :52, logloss :54-57) and
  * src/loss.jl:219-236 with mle2p_grad_hess(GaussianMLE) :194-203.
  * grad is (2K+1) x N Float32, k fastest; row 2K+1 holds the weight and is only read.
- * pred is K x N.  y has one value per row.
+ * pred is K x N.  y has one value per row and target (T x N: T = K targets, K / 2 for gaussian_mle; the class for mlogloss).
  */
 void orc_update_grads(const orc_params *p, int64_t N, const float *pred, const float *y, float *grad) {
     const int K = p->K, NK = 2 * K + 1;
@@ -112,44 +112,53 @@ void orc_update_grads(const orc_params *p, int64_t N, const float *pred, const f
             }
             continue;
         }
-        if (p->loss == ORC_MSE) {
-            float pk = pred[i], yk = y[i];
-            float gg = 2.0f * (pk - yk), hh = 2.0f;
-            g[0] = gg * w;
-            g[1] = hh * w;
-        } else if (p->loss == ORC_LOGLOSS) {
-            float s = orc_sigmoidf(pred[i]);
-            float gg = s - y[i], hh = s * (1.0f - s);
-            g[0] = gg * w;
-            g[1] = hh * w;
-        } else if (p->loss == ORC_POISSON) { /* src/loss.jl:59-62 */
-            float e = expf(pred[i]);
-            g[0] = (e - y[i]) * w;
-            g[1] = e * w;
-        } else if (p->loss == ORC_GAMMA) { /* src/loss.jl:64-67 */
-            float e = expf(pred[i]);
-            g[0] = (2.0f * (1.0f - y[i] / e)) * w;
-            g[1] = (2.0f * y[i] / e) * w;
-        } else if (p->loss == ORC_TWEEDIE) { /* src/loss.jl:69-76, rho = 1.5 */
-            float e = expf(pred[i]);
-            float a = powf(e, 0.5f), b = powf(e, -0.5f);
-            g[0] = (2.0f * (a - y[i] * b)) * w;
-            g[1] = (2.0f * (0.5f * a - (-0.5f) * y[i] * b)) * w;
-        } else { /* gaussian_mle, one target: rows [g_loc, g_scale, h_loc, h_scale, w] */
-            float loc = pred[2 * i], raw = pred[2 * i + 1];
-            float scale = orc_softplusf(raw);
-            float dscale = orc_sigmoidf(raw);
-            float resid = loc - y[i];
-            float s2 = scale * scale;
-            float g_loc = resid / s2;
-            float g_scale = (1.0f - (resid * resid) / s2) * dscale / scale;
-            float h_loc = 1.0f / s2;
-            float ds = dscale / scale;
-            float h_scale = 2.0f * (ds * ds);
-            g[0] = g_loc * w;
-            g[1] = g_scale * w;
-            g[2] = h_loc * w;
-            g[3] = h_scale * w;
+        if (p->loss == ORC_GAUSSIAN_MLE) { /* K = 2 x targets; rows [g_loc_1, g_scale_1, g_loc_2, ..., h_loc_1, h_scale_1, ..., w] */
+            const int Y = K / 2;
+            for (int t = 0; t < Y; t++) {
+                int gb = 2 * t, hb = 2 * Y + 2 * t; /* src/loss.jl:224-225 */
+                float loc = pred[(int64_t)K * i + 2 * t], raw = pred[(int64_t)K * i + 2 * t + 1];
+                float scale = orc_softplusf(raw);
+                float dscale = orc_sigmoidf(raw);
+                float resid = loc - y[(int64_t)Y * i + t];
+                float s2 = scale * scale;
+                float g_loc = resid / s2;
+                float g_scale = (1.0f - (resid * resid) / s2) * dscale / scale;
+                float h_loc = 1.0f / s2;
+                float ds = dscale / scale;
+                float h_scale = 2.0f * (ds * ds);
+                g[gb] = g_loc * w;
+                g[gb + 1] = g_scale * w;
+                g[hb] = h_loc * w;
+                g[hb + 1] = h_scale * w;
+            }
+            continue;
+        }
+        for (int k = 0; k < K; k++) { /* one column of y per target: _target(y, k, i), src/loss.jl:49-50 */
+            float pk = pred[(int64_t)K * i + k], yk = y[(int64_t)K * i + k];
+            float gg, hh;
+            if (p->loss == ORC_MSE) {
+                gg = 2.0f * (pk - yk);
+                hh = 2.0f;
+            } else if (p->loss == ORC_LOGLOSS) {
+                float s = orc_sigmoidf(pk);
+                gg = s - yk;
+                hh = s * (1.0f - s);
+            } else if (p->loss == ORC_POISSON) { /* src/loss.jl:59-62 */
+                float e = expf(pk);
+                gg = e - yk;
+                hh = e;
+            } else if (p->loss == ORC_GAMMA) { /* src/loss.jl:64-67 */
+                float e = expf(pk);
+                gg = 2.0f * (1.0f - yk / e);
+                hh = 2.0f * yk / e;
+            } else { /* tweedie, src/loss.jl:69-76, rho = 1.5 */
+                float e = expf(pk);
+                float a = powf(e, 0.5f), b = powf(e, -0.5f);
+                gg = 2.0f * (a - yk * b);
+                hh = 2.0f * (0.5f * a - (-0.5f) * yk * b);
+            }
+            g[k] = gg * w;
+            g[K + k] = hh * w;
         }
     }
 }
@@ -755,19 +764,26 @@ double orc_eval_metric(int32_t metric, int32_t K, int64_t N, const float *pred, 
             den += (double)wi;
             continue;
         }
+        v = 0.0f; /* acc = zero(T); acc += value per target, src/metrics.jl:39-43, :105-110 */
         if (metric == 4) {
-            float loc = pred[2 * i], scale = orc_softplusf(pred[2 * i + 1]);
-            float d = y[i] - loc;
-            v = -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+            const int Y = K / 2;
+            for (int t = 0; t < Y; t++) {
+                float loc = pred[(size_t)K * i + 2 * t], scale = orc_softplusf(pred[(size_t)K * i + 2 * t + 1]);
+                float d = y[(size_t)Y * i + t] - loc;
+                v += -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+            }
         } else {
-            float pk = pred[i], yk = y[i];
-            if (metric == 0 || metric == 1) v = (pk - yk) * (pk - yk);
-            else if (metric == 2) v = fabsf(pk - yk);
-            else if (metric == 3) { float s = orc_sigmoidf(pk); v = -yk * logf(s) + (yk - 1.0f) * logf(1.0f - s); }
-            else if (metric == 5) { float e = expf(pk); const float eps = 7.105427357601002e-15f; /* eps(Float32(1e-7)) = 2^-47 */
-                                    v = 2.0f * (yk * logf(yk / e + eps) + e - yk); }
-            else if (metric == 6) { float e = expf(pk); v = 2.0f * (logf(e / yk) + yk / e - 1.0f); }
-            else { float e = expf(pk); v = 2.0f * (powf(yk, 0.5f) / (-0.5f) / 0.5f - yk * powf(e, -0.5f) / (-0.5f) + powf(e, 0.5f) / 0.5f); }
+            for (int k = 0; k < K; k++) {
+                float pk = pred[(size_t)K * i + k], yk = y[(size_t)K * i + k], u;
+                if (metric == 0 || metric == 1) u = (pk - yk) * (pk - yk);
+                else if (metric == 2) u = fabsf(pk - yk);
+                else if (metric == 3) { float s = orc_sigmoidf(pk); u = -yk * logf(s) + (yk - 1.0f) * logf(1.0f - s); }
+                else if (metric == 5) { float e = expf(pk); const float eps = 7.105427357601002e-15f; /* eps(Float32(1e-7)) = 2^-47 */
+                                        u = 2.0f * (yk * logf(yk / e + eps) + e - yk); }
+                else if (metric == 6) { float e = expf(pk); u = 2.0f * (logf(e / yk) + yk / e - 1.0f); }
+                else { float e = expf(pk); u = 2.0f * (powf(yk, 0.5f) / (-0.5f) / 0.5f - yk * powf(e, -0.5f) / (-0.5f) + powf(e, 0.5f) / 0.5f); }
+                v += u;
+            }
         }
         float ev = wi * v / (float)((metric == 4) ? K / 2 : K);
         num += (double)ev;

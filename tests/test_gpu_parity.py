@@ -531,7 +531,8 @@ def test_error_paths(evt):
     assert t.split[0] == 1
     h.close()
     for args in [(0, 3, 8, 1, 3, "mse"), (10, 0, 8, 1, 3, "mse"), (10, 3, 1, 1, 3, "mse"), (10, 3, 256, 1, 3, "mse"),
-                 (10, 3, 8, 2, 3, "mse"), (10, 3, 8, 1, 0, "mse"), (10, 3, 8, 1, 17, "mse")]:
+                 (10, 3, 8, 17, 3, "mse"), (10, 3, 8, 3, 3, "gaussian_mle"), (10, 3, 8, 1, 3, "mlogloss"), (10, 3, 8, 1, 0, "mse"),
+                 (10, 3, 8, 1, 17, "mse")]:
         with pytest.raises(evt.EvtError):
             evt.Handle(*args)
 
