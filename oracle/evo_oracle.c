@@ -22,7 +22,10 @@
  * Parity status: pinned by tests/test_oracle_pins.py (brute-force dense histograms,
  * brute-force split search over all (feature, bin) pairs, closed-form gain for unit weights,
  * closed-form / finite-difference gradients, independent tree walk, stable
- * partition property, leaf-value closed form, tie and min_weight strictness cases).
+ * partition property, leaf-value closed form, tie and min_weight strictness cases; matrix
+ * targets by reduction to the one-target gradients and metrics, bit for bit, and by the brute-force
+ * search on multi-output gradients; binarize by numpy's searchsorted and hand-worked answers
+ * for NaN, signed zeros and infinities under Julia's isless).
  * Not pinned (needs a Julia run; stays host-side by design): exact quantile edges
  * from StatsBase.sample + Statistics.quantile, the Xoshiro row-mask / column-sample
  * streams, and Julia's pairwise Float32 mean/std for the bias.  -> "parity unpinned"

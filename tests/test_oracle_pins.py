@@ -599,3 +599,68 @@ def test_mlogloss_predict_shifts_by_row_max_and_floors():
     assert np.array_equal(pred[0], np.float32([-3.0, -2.0, 0.0]))
     assert np.array_equal(pred[1], np.float32([-2.0, -15.0, 0.0]))
     assert np.array_equal(pred[2], np.float32([-2.0, -15.0, 0.0]))
+
+
+# ---------------------------------------------------------------- matrix targets
+@pytest.mark.parametrize("loss", ["mse", "logloss", "poisson", "gamma", "tweedie", "gaussian_mle"])
+def test_matrix_target_grads_and_metric_reduce_to_the_one_target_case(loss):
+    """With T targets, output k sees only (pred[k, i], y[k, i]) (src/loss.jl:49-50, :100-111; :219-236 for gaussian_mle,
+    whose rows are [g_loc_1, g_scale_1, g_loc_2, ..., h_loc_1, h_scale_1, ..., w]): every gradient / hessian row must equal
+    the one-target gradients (pinned above by closed forms and finite differences) of that target alone, bit for bit,
+    and the metric is the mean over targets of the one-target metrics (src/metrics.jl:39-45, :105-112)."""
+    rng = np.random.default_rng(11)
+    N, T = 400, 3
+    K = 2 * T if loss == "gaussian_mle" else T
+    per = 2 if loss == "gaussian_mle" else 1  # outputs per target
+    y = (rng.random((N, T)) + 0.1).astype(np.float32)
+    if loss == "logloss":
+        y = (y > 0.6).astype(np.float32)
+    pred = (rng.standard_normal((N, K)) * 0.4).astype(np.float32)
+    w = (rng.random(N) + 0.5).astype(np.float32)
+    grad = np.zeros((N, 2 * K + 1), np.float32)
+    grad[:, 2 * K] = w
+    orc.update_grads(orc.make_params(loss, K=K), pred, y, grad)
+    assert np.array_equal(grad[:, 2 * K], w)
+    p1 = orc.make_params(loss)
+    metrics = []
+    for t in range(T):
+        pt = np.ascontiguousarray(pred[:, per * t:per * t + per])
+        yt = np.ascontiguousarray(y[:, t])
+        g1 = np.zeros((N, 2 * per + 1), np.float32)
+        g1[:, 2 * per] = w
+        orc.update_grads(p1, pt, yt, g1)
+        for q in range(per):
+            assert np.array_equal(grad[:, per * t + q], g1[:, q]), (t, q)              # gradient rows
+            assert np.array_equal(grad[:, K + per * t + q], g1[:, per + q]), (t, q)    # hessian rows
+        metrics.append(orc.eval_metric(loss, per, pt, yt, w))
+    got = orc.eval_metric(loss, K, pred, y, w)
+    assert abs(got - np.mean(metrics)) <= 2e-6 * abs(np.mean(metrics)) + 1e-9
+
+
+@pytest.mark.parametrize("loss,T", [("mse", 3), ("logloss", 2), ("gaussian_mle", 2)])
+def test_matrix_target_tree_against_bruteforce(loss, T):
+    """Gains and leaf values sum over the outputs (src/split.jl:58-66, :108-117; src/predict.jl:198-204, :224-234): the tree on
+    multi-target gradients against the brute-force search organised differently (node labels, no subtraction trick)."""
+    rng = np.random.default_rng(40)
+    N, F, B, D = 900, 6, 16, 5
+    K = 2 * T if loss == "gaussian_mle" else T
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    y = np.stack([rng.random(N) + 0.5 * (x_bin[t] / B) + 0.3 * (x_bin[(t + 3) % F] > B // 2) for t in range(T)], axis=1).astype(np.float32)
+    if loss == "logloss":
+        y = (y > np.median(y, axis=0)).astype(np.float32)
+    pred = (rng.standard_normal((N, K)) * 0.2).astype(np.float32)
+    grad = np.zeros((N, 2 * K + 1), np.float32)
+    grad[:, 2 * K] = (rng.random(N) + 0.5).astype(np.float32)
+    p = orc.make_params(loss, nbins=B, max_depth=D, lambda_=0.1, gamma=0.01, min_weight=2.0, eta=0.3, K=K)
+    orc.update_grads(p, pred, y, grad)
+    rows = np.sort(rng.choice(N, 700, replace=False)).astype(np.uint32)
+    js = np.array([1, 2, 4, 5, 6], np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t, nidx = o.grow_tree(grad, rows, js, mode=0)
+    Tb, label, hists, sums = brute.grow(x_bin, grad, rows, js, K, B, D, eta=0.3, lam=0.1, L2=1.0, gamma=0.01, min_weight=2.0)
+    assert trees_equal_struct(t, Tb)
+    assert t.split.sum() >= 3
+    np.testing.assert_allclose(t.gain, Tb["gain"], rtol=1e-5)
+    np.testing.assert_allclose(t.pred, Tb["pred"], rtol=1e-5, atol=1e-9)
+    assert np.array_equal(nidx.astype(np.int64), label)
+    o.close()
