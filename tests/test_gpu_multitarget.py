@@ -80,7 +80,9 @@ def test_multi_target_tree_against_the_oracle(evt, loss, T, weights, N, F, B, D,
     assert np.array_equal(o.get_quant()[1], qe)
     t_fx, nidx_fx = o.grow_tree(grad, rows, js, mode=1)
     assert_tree_bits(t_gpu, t_fx)
-    assert t_gpu.split[0] and t_gpu.pred.shape == (t_gpu.feat.shape[0], K)
+    assert t_gpu.pred.shape == (t_gpu.feat.shape[0], K)
+    if D > 1 and N >= 3000:
+        assert t_gpu.split[0]
     assert np.array_equal(h.get_nidx(), nidx_fx)
     p_orc = pred0.copy()
     o.predict_tree(t_fx, p_orc)
