@@ -24,7 +24,7 @@ _GPU_DEVICES = ("gpu", "rocm", "amd", "hip")
 _EXP_LINK = ("poisson", "gamma", "tweedie")
 # is_maximise, src/metrics.jl:195-207
 _MAXIMISE = {"mse": False, "rmse": False, "mae": False, "logloss": False, "poisson": False, "gamma": False, "tweedie": False,
-             "gaussian_mle": True, "mlogloss": False}
+             "gaussian_mle": True, "logistic_mle": True, "mlogloss": False}
 
 
 def _device_check(device):
@@ -105,9 +105,9 @@ class EvoTreeClassifier(_Learner):
 
 
 class EvoTreeMLE(_Learner):
-    """EvoTreeMLE (src/learners.jl:300-400), loss gaussian_mle; min_weight defaults to 8."""
-    _losses = ("gaussian_mle",)
-    _metrics = ("gaussian_mle",)
+    """EvoTreeMLE (src/learners.jl:300-400), losses gaussian_mle and logistic_mle; min_weight defaults to 8."""
+    _losses = ("gaussian_mle", "logistic_mle")
+    _metrics = ("gaussian_mle", "logistic_mle")
     _defaults = dict(_Learner._defaults, loss="gaussian_mle", min_weight=8.0)
 
 
@@ -210,6 +210,8 @@ def _init_target(loss, y):
             mu.append(_logit(m))
         elif loss == "gaussian_mle":
             mu += [m, _invsoftplus(np.float32(yt.std(ddof=1, dtype=np.float32)))]
+        elif loss == "logistic_mle":  # src/init.jl:84-100: scale = std * sqrt(3) / pi, evaluated in Float64
+            mu += [m, _invsoftplus(np.float64(np.float32(yt.std(ddof=1, dtype=np.float32))) * np.sqrt(3.0) / np.pi)]
         elif loss in _EXP_LINK:
             mu.append(np.log(m))
         else:
@@ -226,7 +228,7 @@ def _link_offset(loss, offset, N, K):
         offset = _logit(offset)
     elif loss in _EXP_LINK or loss == "mlogloss":
         offset = np.log(offset)
-    elif loss == "gaussian_mle":
+    elif loss in ("gaussian_mle", "logistic_mle"):
         offset[:, 1::2] = _invsoftplus(offset[:, 1::2])  # every scale column (unconstrain_mle_scale!)
     return offset.astype(np.float32)
 

@@ -12,8 +12,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libevotrees_hip.so")
 
 EVT_OK, EVT_ERR_ARG, EVT_ERR_HIP, EVT_ERR_STATE, EVT_ERR_EMPTY, EVT_ERR_NOMEM = 0, -1, -2, -3, -4, -5
-LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5, "mlogloss": 6}
-METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8}
+LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5, "mlogloss": 6, "logistic_mle": 7}
+METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8, "logistic_mle": 9}
 TREE_TYPES = {"binary": 0, "oblivious": 1}
 KERNEL_CLASSES = ["grad", "hist", "scan", "partition", "predict", "other"]
 
@@ -193,7 +193,7 @@ class Handle:
         mu = np.ascontiguousarray(mu, np.float32)
         offset = None if offset is None else np.ascontiguousarray(offset, np.float32)
         # one value per row and target: (N,) for one target, (N, T) C-order (Julia's T x N) for several
-        T = 1 if self.loss == "mlogloss" else (self.K // 2 if self.loss == "gaussian_mle" else self.K)
+        T = 1 if self.loss == "mlogloss" else (self.K // 2 if self.loss in ("gaussian_mle", "logistic_mle") else self.K)
         assert (y.shape == (self.N,) and T == 1) or y.shape == (self.N, T)
         assert mu.shape == (self.K,)
         check(load().evt_set_target(self._h, ptr(y), ptr(w), ptr(mu), ptr(offset)))

@@ -188,10 +188,11 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ARGCHK(nfeats >= 1 && nfeats <= 1024, "nfeats must be in [1, 1024]");
     ARGCHK(nbins >= 2 && nbins <= 255, "nbins must be in [2, 255]");
     ARGCHK(max_depth >= 1 && max_depth <= EVT_MAX_DEPTH, "max_depth must be in [1, 16]");
-    ARGCHK(loss >= 0 && loss <= EVT_LOSS_MLOGLOSS, "loss must be one of mse (0), logloss (1), gaussian_mle (2), poisson (3), gamma (4), tweedie (5), mlogloss (6)");
+    ARGCHK(loss >= 0 && loss <= EVT_LOSS_LOGISTIC_MLE,
+           "loss must be one of mse (0), logloss (1), gaussian_mle (2), poisson (3), gamma (4), tweedie (5), mlogloss (6), logistic_mle (7)");
     ARGCHK(tree_type == EVT_TREE_BINARY || tree_type == EVT_TREE_OBLIVIOUS, "tree_type must be binary (0) or oblivious (1)");
     if (loss == EVT_LOSS_MLOGLOSS) ARGCHK(K >= 2 && K <= EVT_MAX_K, "mlogloss needs 2 <= K <= 16 classes");
-    else if (loss == EVT_LOSS_GAUSSIAN_MLE) ARGCHK(K >= 2 && K <= EVT_MAX_K && K % 2 == 0, "gaussian_mle needs K = 2 x targets, 2 <= K <= 16");
+    else if (EVT_IS_MLE2P(loss)) ARGCHK(K >= 2 && K <= EVT_MAX_K && K % 2 == 0, "gaussian_mle / logistic_mle need K = 2 x targets, 2 <= K <= 16");
     else ARGCHK(K >= 1 && K <= EVT_MAX_K, "K (targets) must be in [1, 16]");
     int ndev = 0;
     {
@@ -206,8 +207,8 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     memset((void *)&c->device, 0, sizeof(int));
     c->stream = nullptr;
     c->N = nobs; c->F = nfeats; c->B = nbins; c->K = K; c->NK = 2 * K + 1; c->D = max_depth; c->loss = loss; c->tree_type = tree_type;
-    c->T = (loss == EVT_LOSS_MLOGLOSS) ? 1 : (loss == EVT_LOSS_GAUSSIAN_MLE ? K / 2 : K);
-    c->mc = (loss == EVT_LOSS_MLOGLOSS) || K > (loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1);
+    c->T = (loss == EVT_LOSS_MLOGLOSS) ? 1 : (EVT_IS_MLE2P(loss) ? K / 2 : K);
+    c->mc = (loss == EVT_LOSS_MLOGLOSS) || K > (EVT_IS_MLE2P(loss) ? 2 : 1);
     c->nnodes = (1 << max_depth) - 1;
     c->maxlvl = 1 << (max_depth - 1);
     c->RS = record_stride(nfeats);
@@ -1128,9 +1129,11 @@ extern "C" int evt_get_quant(evt_handle c, int32_t *qbits, int32_t *qexp) {
 extern "C" int evt_eval_metric(evt_handle c, int32_t metric, double *value_out) {
     CTXCHK(c);
     ARGCHK(value_out, "value_out is NULL");
-    ARGCHK(metric >= 0 && metric <= EVT_METRIC_MLOGLOSS, "unknown metric");
+    ARGCHK(metric >= 0 && metric <= EVT_METRIC_LOGISTIC_MLE, "unknown metric");
     ARGCHK((metric == EVT_METRIC_GAUSSIAN_MLE) == (c->loss == EVT_LOSS_GAUSSIAN_MLE),
            "gaussian_mle is the metric of the gaussian_mle loss and of no other");
+    ARGCHK((metric == EVT_METRIC_LOGISTIC_MLE) == (c->loss == EVT_LOSS_LOGISTIC_MLE),
+           "logistic_mle is the metric of the logistic_mle loss and of no other");
     ARGCHK((metric == EVT_METRIC_MLOGLOSS) == (c->loss == EVT_LOSS_MLOGLOSS), "mlogloss is the metric of the mlogloss loss and of no other");
     if (!c->have_target) {
         evt_set_error("evt_eval_metric: set the target first");
@@ -1223,7 +1226,7 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
                           const int32_t *edge_off = nullptr) {
     ARGCHK(nobs >= 1 && nfeats >= 1 && ntrees >= 1, "nobs, nfeats, ntrees must be >= 1");
     ARGCHK((x_bin || x_f64) && tree_off && feat && cond_bin && split, "NULL argument");
-    ARGCHK(leaf_out || (pred && out && K >= 1 && K <= EVT_MAX_K && loss >= 0 && loss <= EVT_LOSS_MLOGLOSS), "invalid prediction arguments");
+    ARGCHK(leaf_out || (pred && out && K >= 1 && K <= EVT_MAX_K && loss >= 0 && loss <= EVT_LOSS_LOGISTIC_MLE), "invalid prediction arguments");
     std::vector<int32_t> eoff;
     if (x_f64) {
         ARGCHK(edges && edge_off, "NULL argument");

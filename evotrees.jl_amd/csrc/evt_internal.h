@@ -191,6 +191,8 @@ void evt_set_error(const char *fmt, ...);
 // losses), clamp to [-15, 15] (logloss), floor -15 on the scale outputs (gaussian_mle), shift by the row maximum and
 // floor -15 (mlogloss).  pr may point to registers or memory.
 // A split node in one 32-bit word: feature id (1-based) | cond_bin << 16 | split << 24 | numeric << 25.  Leaves are 0.
+// the two-parameter MLE losses: outputs come in (location, raw scale) pairs
+#define EVT_IS_MLE2P(loss) ((loss) == EVT_LOSS_GAUSSIAN_MLE || (loss) == EVT_LOSS_LOGISTIC_MLE)
 #define EVT_NODE_SPLIT (1u << 24)
 #define EVT_NODE_NUMERIC (1u << 25)
 #ifdef __HIPCC__
@@ -200,7 +202,7 @@ __host__ __device__ __forceinline__ uint32_t evt_pack_node(int feat, int cond_bi
 __device__ __forceinline__ void evt_add_leaf(float *pr, const float *lp, int K, int loss) {
     if (loss == EVT_LOSS_LOGLOSS) {
         for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
-    } else if (loss == EVT_LOSS_GAUSSIAN_MLE) {
+    } else if (loss == EVT_LOSS_GAUSSIAN_MLE || loss == EVT_LOSS_LOGISTIC_MLE) {
         for (int t = 0; t < K / 2; t++) {
             pr[2 * t] += lp[2 * t];
             pr[2 * t + 1] = fmaxf(-15.0f, pr[2 * t + 1] + lp[2 * t + 1]);

@@ -18,6 +18,29 @@ __device__ __forceinline__ float wave_max_f32(float v) {
 __device__ __forceinline__ float dev_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float dev_softplus(float x) { return fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x))); }
 
+// mle2p_grad_hess, src/loss.jl:194-217: GaussianMLE (LOSS 2) and LogisticMLE (LOSS 7); raw is the unconstrained scale.
+template <int LOSS>
+__device__ __forceinline__ void mle2p_grad_hess(float loc, float raw, float y, float &g_loc, float &g_scale, float &h_loc, float &h_scale) {
+    const float scale = dev_softplus(raw);
+    const float dscale = dev_sigmoid(raw);
+    const float ds = dscale / scale;
+    if (LOSS == 2) {
+        const float resid = loc - y;
+        const float s2 = scale * scale;
+        g_loc = resid / s2;
+        g_scale = (1.0f - (resid * resid) / s2) * dscale / scale;
+        h_loc = 1.0f / s2;
+        h_scale = 2.0f * (ds * ds);
+    } else {
+        const float z = (y - loc) / scale;
+        const float th = tanhf(z / 2.0f);
+        g_loc = -th / scale;
+        g_scale = (1.0f - z * th) * dscale / scale;
+        h_loc = 1.0f / (3.0f * (scale * scale));
+        h_scale = (3.14159274f * 3.14159274f + 3.0f) / 9.0f * (ds * ds); // oftype(scale, pi)^2
+    }
+}
+
 // LOSS: 0 mse (src/loss.jl:52), 1 logloss (:54-57), 2 gaussian_mle (:194-203), 3 poisson (:59-62),
 // 4 gamma (:64-67), 5 tweedie with rho = 1.5 (:69-76).
 // grad rows: [g_1..g_K, h_1..h_K, w]; every written value is multiplied by w (src/loss.jl:104-108, :223-233).
@@ -25,7 +48,7 @@ template <int LOSS>
 __global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const float *__restrict__ y, float *__restrict__ grad, int64_t N,
                                               uint32_t *absmax, const uint32_t *__restrict__ pend_nidx,
                                               const float *__restrict__ pend_leaf, int unit_w) {
-    constexpr int K = (LOSS == 2) ? 2 : 1;
+    constexpr int K = (LOSS == 2 || LOSS == 7) ? 2 : 1;
     constexpr int NK = 2 * K + 1;
     float mx[2 * K];
 #pragma unroll
@@ -57,16 +80,12 @@ __global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const f
             out[0] = (2.0f * (a - y[i] * b)) * w;
             out[1] = (2.0f * (0.5f * a - (-0.5f) * y[i] * b)) * w;
         } else {
-            const float loc = pred[2 * i], raw = pred[2 * i + 1];
-            const float scale = dev_softplus(raw);
-            const float dscale = dev_sigmoid(raw);
-            const float resid = loc - y[i];
-            const float s2 = scale * scale;
-            const float ds = dscale / scale;
-            out[0] = (resid / s2) * w;
-            out[1] = ((1.0f - (resid * resid) / s2) * dscale / scale) * w;
-            out[2] = (1.0f / s2) * w;
-            out[3] = (2.0f * (ds * ds)) * w;
+            float g1, g2, h1, h2;
+            mle2p_grad_hess<LOSS>(pred[2 * i], pred[2 * i + 1], y[i], g1, g2, h1, h2);
+            out[0] = g1 * w;
+            out[1] = g2 * w;
+            out[2] = h1 * w;
+            out[3] = h2 * w;
         }
 #pragma unroll
         for (int k = 0; k < 2 * K; k++) {
@@ -123,7 +142,8 @@ __global__ __launch_bounds__(256) void k_grads_mt(float *__restrict__ pred, cons
                                                  int K, uint32_t *absmax, const uint32_t *__restrict__ pend_nidx,
                                                  const float *__restrict__ pend_leaf, int unit_w) {
     const int NK = 2 * K + 1;
-    const int T = (LOSS == 2) ? K / 2 : K; // target columns
+    constexpr bool MLE2P = (LOSS == 2 || LOSS == 7);
+    const int T = MLE2P ? K / 2 : K; // target columns
     __shared__ float s_m[4];
     float mx[2 * EVT_MAX_K];
 #pragma unroll
@@ -138,25 +158,16 @@ __global__ __launch_bounds__(256) void k_grads_mt(float *__restrict__ pred, cons
         for (int k = 0; k < EVT_MAX_K; k++) {
             if (k < K) {
                 float gg, hh;
-                if (LOSS == 2) {
+                if (MLE2P) {
                     // output k of pair t = k / 2: even = location, odd = raw scale
                     const int t = k >> 1;
-                    const float loc = pr[2 * t], raw = pr[2 * t + 1];
-                    const float scale = dev_softplus(raw);
-                    const float dscale = dev_sigmoid(raw);
-                    const float resid = loc - yi[t];
-                    const float s2 = scale * scale;
-                    const float ds = dscale / scale;
-                    if ((k & 1) == 0) {
-                        gg = (resid / s2) * w;
-                        hh = (1.0f / s2) * w;
-                    } else {
-                        gg = ((1.0f - (resid * resid) / s2) * dscale / scale) * w;
-                        hh = (2.0f * (ds * ds)) * w;
-                    }
+                    float g1, g2, h1, h2;
+                    mle2p_grad_hess<MLE2P ? LOSS : 2>(pr[2 * t], pr[2 * t + 1], yi[t], g1, g2, h1, h2);
+                    gg = (((k & 1) == 0) ? g1 : g2) * w;
+                    hh = (((k & 1) == 0) ? h1 : h2) * w;
                 } else {
                     float g1, h1;
-                    grad_hess_one<LOSS>(pr[k], yi[k], g1, h1);
+                    grad_hess_one<MLE2P ? 0 : LOSS>(pr[k], yi[k], g1, h1);
                     gg = g1 * w;
                     hh = h1 * w;
                 }
@@ -302,7 +313,7 @@ int launch_grads(evt_ctx *c) {
     dim3 grid((unsigned)nb);
     const uint32_t *pn = c->pend_pred ? c->nidx : nullptr; // the last tree's leaf values are added on the way
     c->pend_pred = false;
-    const bool multi_target = c->loss != EVT_LOSS_MLOGLOSS && c->K > (c->loss == EVT_LOSS_GAUSSIAN_MLE ? 2 : 1);
+    const bool multi_target = c->loss != EVT_LOSS_MLOGLOSS && c->K > (EVT_IS_MLE2P(c->loss) ? 2 : 1);
     if (multi_target) {
 #define MT(L_) hipLaunchKernelGGL(k_grads_mt<L_>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0)
         switch (c->loss) {
@@ -311,6 +322,7 @@ int launch_grads(evt_ctx *c) {
         case EVT_LOSS_GAUSSIAN_MLE: MT(2); break;
         case EVT_LOSS_POISSON: MT(3); break;
         case EVT_LOSS_GAMMA: MT(4); break;
+        case EVT_LOSS_LOGISTIC_MLE: MT(7); break;
         default: MT(5); break;
         }
 #undef MT
@@ -321,6 +333,8 @@ int launch_grads(evt_ctx *c) {
         hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_LOGLOSS)
         hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+    else if (c->loss == EVT_LOSS_LOGISTIC_MLE)
+        hipLaunchKernelGGL(k_grads<7>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_GAUSSIAN_MLE)
         hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_POISSON)
@@ -387,13 +401,18 @@ __device__ __forceinline__ float metric_value(int metric, int K, const float *__
         for (int k = 0; k < K; k++) isum += expf(pred[(size_t)K * i + k]);
         return logf(isum) - pred[(size_t)K * i + (int)y[i] - 1];
     }
-    if (metric == EVT_METRIC_GAUSSIAN_MLE) { // src/metrics.jl:88-91, :98-114: summed over the targets
+    if (metric == EVT_METRIC_GAUSSIAN_MLE || metric == EVT_METRIC_LOGISTIC_MLE) { // src/metrics.jl:84-114: summed over the targets
         const int T = K / 2;
         float acc = 0.0f;
         for (int t = 0; t < T; t++) {
             const float loc = pred[(size_t)K * i + 2 * t], scale = dev_softplus(pred[(size_t)K * i + 2 * t + 1]);
-            const float d = y[(size_t)T * i + t] - loc;
-            acc += -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+            if (metric == EVT_METRIC_GAUSSIAN_MLE) {
+                const float d = y[(size_t)T * i + t] - loc;
+                acc += -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+            } else {
+                const float az = fabsf((y[(size_t)T * i + t] - loc) / scale);
+                acc += -logf(scale) - az - 2.0f * log1pf(expf(-az));
+            }
         }
         return acc;
     }
@@ -473,7 +492,7 @@ __global__ __launch_bounds__(256) void k_metric_final(const double *__restrict__
 int launch_eval_metric(evt_ctx *c, int metric, double *partial) {
     int64_t nb = (c->N + 255) / 256;
     if (nb > EVT_METRIC_BLOCKS) nb = EVT_METRIC_BLOCKS;
-    const float kdiv = (metric == EVT_METRIC_MLOGLOSS) ? 1.0f : (float)(metric == EVT_METRIC_GAUSSIAN_MLE ? c->K / 2 : c->K);
+    const float kdiv = (metric == EVT_METRIC_MLOGLOSS) ? 1.0f : (float)((metric == EVT_METRIC_GAUSSIAN_MLE || metric == EVT_METRIC_LOGISTIC_MLE) ? c->K / 2 : c->K);
     hipLaunchKernelGGL(k_metric_partial, dim3((unsigned)nb), dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->NK, c->K, metric, kdiv,
                        partial);
     HIPCHK(hipGetLastError());

@@ -66,7 +66,7 @@ template <int KMAX>
 __device__ __forceinline__ void apply_link(float *acc, int K, int loss) {
     if (loss == EVT_LOSS_LOGLOSS) {
         for (int k = 0; k < K; k++) acc[k] = 1.0f / (1.0f + expf(-acc[k]));
-    } else if (loss == EVT_LOSS_GAUSSIAN_MLE) {
+    } else if (EVT_IS_MLE2P(loss)) {
         for (int k = 1; k < K; k += 2) acc[k] = fmaxf(acc[k], 0.0f) + log1pf(expf(-fabsf(acc[k])));
     } else if (loss == EVT_LOSS_MLOGLOSS) {
         float isum = 0.0f;
@@ -79,7 +79,7 @@ __device__ __forceinline__ void apply_link(float *acc, int K, int loss) {
         }
 #pragma unroll
         for (int k = 0; k < KMAX; k++) acc[k] /= isum;
-    } else if (loss >= EVT_LOSS_POISSON) {
+    } else if (loss >= EVT_LOSS_POISSON && loss <= EVT_LOSS_TWEEDIE) {
         for (int k = 0; k < K; k++) acc[k] = expf(acc[k]);
     }
 }

@@ -49,7 +49,8 @@ enum {
     EVT_LOSS_POISSON = 3,
     EVT_LOSS_GAMMA = 4,
     EVT_LOSS_TWEEDIE = 5,
-    EVT_LOSS_MLOGLOSS = 6 /* K classes, y holds the 1-based class (level code) as a Float32 */
+    EVT_LOSS_MLOGLOSS = 6, /* K classes, y holds the 1-based class (level code) as a Float32 */
+    EVT_LOSS_LOGISTIC_MLE = 7 /* the other two-parameter MLE loss (src/loss.jl:205-217): outputs and clamps as gaussian_mle */
 };
 /* evaluation metrics, metric_dict of src/metrics.jl:209-224 (in-scope subset) */
 enum {
@@ -61,7 +62,8 @@ enum {
     EVT_METRIC_POISSON = 5,
     EVT_METRIC_GAMMA = 6,
     EVT_METRIC_TWEEDIE = 7,
-    EVT_METRIC_MLOGLOSS = 8
+    EVT_METRIC_MLOGLOSS = 8,
+    EVT_METRIC_LOGISTIC_MLE = 9
 };
 /* params.tree_type, src/learners.jl:45 */
 enum { EVT_TREE_BINARY = 0, EVT_TREE_OBLIVIOUS = 1 };
@@ -101,7 +103,7 @@ int evt_device_count(int32_t *count);
  * (ext/EvoTreesKernelAbstractionsExt/init.jl:1-151): sizes every device buffer.
  * nbins in [2,255] (src/learners.jl:527).  K is the number of outputs (size(pred, 1) in the reference, at most 16):
  * the number of targets for mse / logloss / poisson / gamma / tweedie (1, or more with a matrix target,
- * src/init.jl:11-16, :142-150), twice the number of targets for gaussian_mle (src/init.jl:68-83), the number of
+ * src/init.jl:11-16, :142-150), twice the number of targets for gaussian_mle and logistic_mle (src/init.jl:68-100), the number of
  * classes (2..16) for mlogloss. */
 int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K, int32_t max_depth, int32_t loss,
                int32_t tree_type, evt_handle *out);

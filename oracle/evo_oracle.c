@@ -42,6 +42,8 @@
 #include <omp.h>
 #endif
 
+#define ORC_LOGISTIC_MLE 7
+#define ORC_IS_MLE2P(l) ((l) == ORC_GAUSSIAN_MLE || (l) == ORC_LOGISTIC_MLE)
 #define ORC_MSE 0
 #define ORC_LOGLOSS 1
 #define ORC_GAUSSIAN_MLE 2
@@ -115,20 +117,31 @@ void orc_update_grads(const orc_params *p, int64_t N, const float *pred, const f
             }
             continue;
         }
-        if (p->loss == ORC_GAUSSIAN_MLE) { /* K = 2 x targets; rows [g_loc_1, g_scale_1, g_loc_2, ..., h_loc_1, h_scale_1, ..., w] */
+        if (ORC_IS_MLE2P(p->loss)) { /* K = 2 x targets; rows [g_loc_1, g_scale_1, g_loc_2, ..., h_loc_1, h_scale_1, ..., w] */
             const int Y = K / 2;
             for (int t = 0; t < Y; t++) {
                 int gb = 2 * t, hb = 2 * Y + 2 * t; /* src/loss.jl:224-225 */
                 float loc = pred[(int64_t)K * i + 2 * t], raw = pred[(int64_t)K * i + 2 * t + 1];
                 float scale = orc_softplusf(raw);
                 float dscale = orc_sigmoidf(raw);
-                float resid = loc - y[(int64_t)Y * i + t];
-                float s2 = scale * scale;
-                float g_loc = resid / s2;
-                float g_scale = (1.0f - (resid * resid) / s2) * dscale / scale;
-                float h_loc = 1.0f / s2;
                 float ds = dscale / scale;
-                float h_scale = 2.0f * (ds * ds);
+                float g_loc, g_scale, h_loc, h_scale;
+                if (p->loss == ORC_GAUSSIAN_MLE) { /* src/loss.jl:194-203 */
+                    float resid = loc - y[(int64_t)Y * i + t];
+                    float s2 = scale * scale;
+                    g_loc = resid / s2;
+                    g_scale = (1.0f - (resid * resid) / s2) * dscale / scale;
+                    h_loc = 1.0f / s2;
+                    h_scale = 2.0f * (ds * ds);
+                } else { /* Logistic(loc, scale), src/loss.jl:205-217 */
+                    float z = (y[(int64_t)Y * i + t] - loc) / scale;
+                    float th = tanhf(z / 2.0f);
+                    const float pi32 = 3.14159274f;
+                    g_loc = -th / scale;
+                    g_scale = (1.0f - z * th) * dscale / scale;
+                    h_loc = 1.0f / (3.0f * (scale * scale));
+                    h_scale = (pi32 * pi32 + 3.0f) / 9.0f * (ds * ds);
+                }
                 g[gb] = g_loc * w;
                 g[gb + 1] = g_scale * w;
                 g[hb] = h_loc * w;
@@ -707,7 +720,7 @@ void orc_predict_tree(int32_t loss, int32_t K, int64_t N, const uint8_t *x_bin, 
             float m = -INFINITY;
             for (int k = 0; k < K; k++) { pr[k] += lp[k]; if (pr[k] > m) m = pr[k]; }
             for (int k = 0; k < K; k++) { float v = pr[k] - m; pr[k] = v > -15.0f ? v : -15.0f; }
-        } else if (loss == ORC_MSE || loss >= ORC_POISSON) {
+        } else if (loss == ORC_MSE || (loss >= ORC_POISSON && loss != ORC_LOGISTIC_MLE)) {
             for (int k = 0; k < K; k++) pr[k] += lp[k];
         } else if (loss == ORC_LOGLOSS) {
             for (int k = 0; k < K; k++) {
@@ -737,13 +750,13 @@ void orc_apply_link(int32_t loss, int32_t K, int64_t N, float *pred) {
     for (int64_t i = 0; i < N; i++) {
         if (loss == ORC_LOGLOSS) {
             for (int k = 0; k < K; k++) pred[(size_t)K * i + k] = orc_sigmoidf(pred[(size_t)K * i + k]);
-        } else if (loss == ORC_GAUSSIAN_MLE) {
+        } else if (ORC_IS_MLE2P(loss)) {
             for (int k = 1; k < K; k += 2) pred[(size_t)K * i + k] = orc_softplusf(pred[(size_t)K * i + k]);
         } else if (loss == ORC_MLOGLOSS) { /* softmax!, src/predict.jl:187-195 */
             float isum = 0.0f;
             for (int k = 0; k < K; k++) { pred[(size_t)K * i + k] = expf(pred[(size_t)K * i + k]); isum += pred[(size_t)K * i + k]; }
             for (int k = 0; k < K; k++) pred[(size_t)K * i + k] /= isum;
-        } else if (loss >= ORC_POISSON) {
+        } else if (loss >= ORC_POISSON && loss != ORC_LOGISTIC_MLE) {
             for (int k = 0; k < K; k++) pred[(size_t)K * i + k] = expf(pred[(size_t)K * i + k]);
         }
     }
@@ -752,7 +765,7 @@ void orc_apply_link(int32_t loss, int32_t K, int64_t N, float *pred) {
 /*
  * Evaluation metrics — src/metrics.jl:1-48 (_eval_metric: eval[i] = w[i] * value / K in Float32, result
  * sum(Float64, eval) / sum(Float64, w)) and :88-112 (gaussian_mle: mean log-likelihood).
- * metric: 0 mse, 1 rmse, 2 mae, 3 logloss, 4 gaussian_mle, 5 poisson, 6 gamma, 7 tweedie, 8 mlogloss (:59-77,
+ * metric: 0 mse, 1 rmse, 2 mae, 3 logloss, 4 gaussian_mle, 5 poisson, 6 gamma, 7 tweedie, 9 logistic_mle, 8 mlogloss (:59-77,
  * eval[i] = w[i] * (log(sum_k exp(p[k,i])) - p[y[i], i]), not divided by K).
  */
 double orc_eval_metric(int32_t metric, int32_t K, int64_t N, const float *pred, const float *y, const float *w) {
@@ -768,12 +781,17 @@ double orc_eval_metric(int32_t metric, int32_t K, int64_t N, const float *pred, 
             continue;
         }
         v = 0.0f; /* acc = zero(T); acc += value per target, src/metrics.jl:39-43, :105-110 */
-        if (metric == 4) {
+        if (metric == 4 || metric == 9) {
             const int Y = K / 2;
             for (int t = 0; t < Y; t++) {
                 float loc = pred[(size_t)K * i + 2 * t], scale = orc_softplusf(pred[(size_t)K * i + 2 * t + 1]);
-                float d = y[(size_t)Y * i + t] - loc;
-                v += -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+                if (metric == 4) {
+                    float d = y[(size_t)Y * i + t] - loc;
+                    v += -(logf(scale) + (d * d) / (2.0f * (scale * scale)));
+                } else { /* logistic_mle, src/metrics.jl:92-97 */
+                    float az = fabsf((y[(size_t)Y * i + t] - loc) / scale);
+                    v += -logf(scale) - az - 2.0f * log1pf(expf(-az));
+                }
             }
         } else {
             for (int k = 0; k < K; k++) {
@@ -788,7 +806,7 @@ double orc_eval_metric(int32_t metric, int32_t K, int64_t N, const float *pred, 
                 v += u;
             }
         }
-        float ev = wi * v / (float)((metric == 4) ? K / 2 : K);
+        float ev = wi * v / (float)((metric == 4 || metric == 9) ? K / 2 : K);
         num += (double)ev;
         den += (double)wi;
     }

@@ -12,8 +12,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libevo_oracle.so")
 
-LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5, "mlogloss": 6}
-METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8}
+LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5, "mlogloss": 6, "logistic_mle": 7}
+METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8, "logistic_mle": 9}
 TREE_TYPES = {"binary": 0, "oblivious": 1}
 
 
@@ -94,7 +94,7 @@ def _p(a):
 def make_params(loss="mse", nbins=64, max_depth=6, tree_type="binary", bagging_size=1, eta=0.1, L2=1.0,
                 lambda_=0.0, gamma=0.0, min_weight=1.0, K=None):
     if K is None:
-        K = 2 if loss == "gaussian_mle" else 1
+        K = 2 if loss in ("gaussian_mle", "logistic_mle") else 1
     return OrcParams(LOSS_IDS[loss], K, nbins, max_depth, TREE_TYPES[tree_type], bagging_size, eta, L2, lambda_,
                      gamma, min_weight)
 

@@ -13,6 +13,7 @@ METRICS_OF = {
     "mse": ["mse", "rmse", "mae"],
     "logloss": ["logloss", "mse"],
     "gaussian_mle": ["gaussian_mle"],
+    "logistic_mle": ["logistic_mle"],
     "poisson": ["poisson", "mae"],
     "gamma": ["gamma"],
     "tweedie": ["tweedie", "rmse"],
@@ -21,13 +22,13 @@ METRICS_OF = {
 
 
 @pytest.mark.parametrize("loss,weights", [("mse", True), ("logloss", False), ("gaussian_mle", True), ("poisson", True),
-                                          ("gamma", False), ("tweedie", True), ("mlogloss", True)])
+                                          ("gamma", False), ("tweedie", True), ("mlogloss", True), ("logistic_mle", True)])
 def test_eval_metric_matches_oracle(evt, loss, weights):
     N, F, B, D = 70001, 6, 32, 4
     x_bin, y, w, mu = make_data(41, N, F, B, loss, weights)
     if loss == "poisson":
         y = y + 1.0  # the metric's log(y / pred + eps) amplifies ulp differences of exp at y = 0; covered separately below
-    pk = dict(min_weight=8.0) if loss == "gaussian_mle" else {}
+    pk = dict(min_weight=8.0) if loss in ("gaussian_mle", "logistic_mle") else {}
     h, o, op, gp, pred0, grad0 = setup_pair(evt, loss, x_bin, y, w, mu, B, D, **pk)
     js = np.arange(1, F + 1, dtype=np.uint32)
     for r in range(3):
@@ -40,9 +41,11 @@ def test_eval_metric_matches_oracle(evt, loss, weights):
             exact_rows = metric in ("mse", "rmse", "mae")  # per-row Float32 values identical, only the Float64 sum order differs
             np.testing.assert_allclose(got, want, rtol=1e-12 if exact_rows else RTOL)
             assert got == h.eval_metric(metric)  # fixed summation order: reproducible to the bit
-    if loss not in ("gaussian_mle", "mlogloss"):
+    if loss not in ("gaussian_mle", "mlogloss", "logistic_mle"):
         with pytest.raises(evt.EvtError):
             h.eval_metric("gaussian_mle")
+        with pytest.raises(evt.EvtError):
+            h.eval_metric("logistic_mle")
         with pytest.raises(evt.EvtError):
             h.eval_metric("mlogloss")
     else:
@@ -84,7 +87,8 @@ def _sinus(rng, n):
 
 
 @pytest.mark.parametrize("cfg_kw", [dict(loss="mse", metric="mae"), dict(loss="logloss"), dict(loss="gamma"), dict(loss="tweedie"),
-                                    dict(loss="poisson", learner="count"), dict(loss="gaussian_mle", learner="mle")])
+                                    dict(loss="poisson", learner="count"), dict(loss="gaussian_mle", learner="mle"),
+                                    dict(loss="logistic_mle", learner="mle")])
 def test_fit_with_eval_logger_matches_oracle_replay(evt, cfg_kw):
     # every logged value equals the oracle's metric of the oracle's own replay of the model on the eval rows
     rng = np.random.default_rng(7)
@@ -99,14 +103,15 @@ def test_fit_with_eval_logger_matches_oracle_replay(evt, cfg_kw):
     m = evt.fit(cfg, x_train=X[tr], y_train=Y[tr], x_eval=X[ev], y_eval=Y[ev], w_eval=w_ev, verbosity=0)
     lg = m.info["logger"]
     assert lg["name"] == cfg.metric and lg["iter"] == list(range(13)) and lg["nrounds"] == 12
-    assert lg["maximise"] == (cfg.loss == "gaussian_mle")
+    assert lg["maximise"] == (cfg.loss in ("gaussian_mle", "logistic_mle"))
     xb = evt.binarize(X[ev], m.info["edges"])
     ft = np.ones(1, np.uint8)
     p = np.zeros((len(ev), m.K), np.float32)
     y32 = Y[ev].astype(np.float32)
     for i, t in enumerate(m.trees):
         orc.predict_tree(orc.LOSS_IDS[cfg.loss], m.K, xb, ft, t, p)
-        np.testing.assert_allclose(lg["metrics"][i], orc.eval_metric(cfg.metric, m.K, p, y32, w_ev), rtol=RTOL)
+        # a mean log-likelihood can pass through zero: the absolute bound is 1e-6 of the per-row values' scale (~1)
+        np.testing.assert_allclose(lg["metrics"][i], orc.eval_metric(cfg.metric, m.K, p, y32, w_ev), rtol=RTOL, atol=1e-6)
     best = int(np.argmax(lg["metrics"]) if lg["maximise"] else np.argmin(lg["metrics"]))
     assert lg["best_iter"] == best and lg["best_metric"] == lg["metrics"][best]
     better = lg["metrics"][-1] > lg["metrics"][0] if lg["maximise"] else lg["metrics"][-1] < lg["metrics"][0]

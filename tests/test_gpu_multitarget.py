@@ -24,7 +24,7 @@ def make_targets(seed, N, F, B, loss, T, weights):
         y = np.floor(y * 3).astype(np.float32)
     elif loss in ("gamma", "tweedie"):
         y = (y + 0.1).astype(np.float32)
-    K = 2 * T if loss == "gaussian_mle" else T
+    K = 2 * T if loss in ("gaussian_mle", "logistic_mle") else T
     w = (rng.random(N).astype(np.float32) + 0.5) if weights else None
     mu = (rng.standard_normal(K) * 0.1).astype(np.float32)
     return x_bin, y, w, mu
@@ -42,6 +42,8 @@ CASES = [
     ("gaussian_mle", 3, False, 9000, 50, 64, 4, "oblivious", 30, 0.5, False),
     ("mse", 16, False, 3000, 6, 16, 3, "binary", 6, 1.0, False),
     ("gaussian_mle", 8, True, 3000, 6, 255, 3, "binary", 6, 1.0, False),
+    ("logistic_mle", 2, True, 12000, 14, 32, 5, "binary", 14, 1.0, False),
+    ("logistic_mle", 3, False, 9000, 40, 64, 4, "oblivious", 25, 0.5, True),
 ]
 
 
@@ -51,7 +53,7 @@ def test_multi_target_tree_against_the_oracle(evt, loss, T, weights, N, F, B, D,
     x_bin, y, w, mu = make_targets(900, N, F, B, loss, T, weights)
     K = mu.shape[0]
     feattypes = (rng.random(F) > 0.3).astype(np.uint8) if cat else None
-    min_weight = 8.0 if loss == "gaussian_mle" else 1.0
+    min_weight = 8.0 if loss in ("gaussian_mle", "logistic_mle") else 1.0
     h, o, op, gp, pred0, grad0 = setup_pair(evt, loss, x_bin, y, w, mu, B, D, tt, feattypes=feattypes, min_weight=min_weight, L2=0.1)
     # gradients: the kernel against the oracle (mse is exact Float32 arithmetic)
     grad = grad0.copy()
@@ -103,7 +105,7 @@ def test_multi_target_tree_against_the_oracle(evt, loss, T, weights, N, F, B, D,
         assert abs(float(t_gpu.gain[n0]) - float(t_ref.gain[n0])) <= 1e-6 * abs(float(t_ref.gain[n0])) + 1e-12
     # the evaluation metric on the updated prediction
     metric = {"mse": "mse", "logloss": "logloss", "poisson": "poisson", "gamma": "gamma", "tweedie": "tweedie",
-              "gaussian_mle": "gaussian_mle"}[loss]
+              "gaussian_mle": "gaussian_mle", "logistic_mle": "logistic_mle"}[loss]
     got = h.eval_metric(metric)
     want = orc.eval_metric(metric, K, p_orc, y, w)
     assert abs(got - want) <= 1e-5 * abs(want) + 1e-9

@@ -10,7 +10,7 @@ from test_gpu_parity import assert_tree_bits, make_data, setup_pair
 
 pytestmark = pytest.mark.gpu
 
-LOSSES = ["mse", "logloss", "gaussian_mle", "poisson", "gamma", "tweedie", "mlogloss"]
+LOSSES = ["mse", "logloss", "gaussian_mle", "poisson", "gamma", "tweedie", "mlogloss", "logistic_mle"]
 
 
 def _cases():

@@ -664,3 +664,69 @@ def test_matrix_target_tree_against_bruteforce(loss, T):
     np.testing.assert_allclose(t.pred, Tb["pred"], rtol=1e-5, atol=1e-9)
     assert np.array_equal(nidx.astype(np.int64), label)
     o.close()
+
+
+# ---------------------------------------------------------------- logistic_mle
+def test_logistic_mle_grads_are_derivatives_of_the_logpdf_and_fisher_hessians():
+    """mle2p_grad_hess(LogisticMLE), src/loss.jl:205-217: g = -d logpdf / d(loc, raw) of the Logistic(loc, softplus(raw))
+    density (scipy's logistic.logpdf, central differences in Float64); the hessians are the Fisher information
+    1 / (3 s^2) and (pi^2 + 3) / 9 * (sigmoid(raw) / s)^2, which do not depend on the residual."""
+    from scipy.stats import logistic
+    rng = np.random.default_rng(12)
+    N = 300
+    pred = np.stack([rng.standard_normal(N), rng.standard_normal(N) * 0.7], axis=1).astype(np.float32)
+    y = (rng.standard_normal(N) * 1.5).astype(np.float32)
+    w = (rng.random(N) + 0.5).astype(np.float32)
+    grad = np.zeros((N, 5), np.float32)
+    grad[:, 4] = w
+    orc.update_grads(orc.make_params("logistic_mle"), pred, y, grad)
+    loc, raw, yy = pred[:, 0].astype(np.float64), pred[:, 1].astype(np.float64), y.astype(np.float64)
+    sp = lambda r: np.logaddexp(0.0, r)
+    f = lambda l, r: logistic.logpdf(yy, loc=l, scale=sp(r))
+    eps = 1e-5
+    d_loc = (f(loc + eps, raw) - f(loc - eps, raw)) / (2 * eps)
+    d_raw = (f(loc, raw + eps) - f(loc, raw - eps)) / (2 * eps)
+    np.testing.assert_allclose(grad[:, 0], -d_loc * w, rtol=2e-5, atol=2e-6)
+    np.testing.assert_allclose(grad[:, 1], -d_raw * w, rtol=2e-5, atol=2e-6)
+    s = sp(raw)
+    dsc = 1 / (1 + np.exp(-raw))
+    np.testing.assert_allclose(grad[:, 2], w / (3 * s ** 2), rtol=2e-6)
+    np.testing.assert_allclose(grad[:, 3], w * (np.pi ** 2 + 3) / 9 * (dsc / s) ** 2, rtol=2e-6)
+    # Fisher information = E[score^2] under the model: checked by quadrature for one parameter pair
+    l0, r0 = 0.3, -0.2
+    s0 = sp(r0)
+    grid = np.linspace(l0 - 40 * s0, l0 + 40 * s0, 400001)
+    pdf = logistic.pdf(grid, loc=l0, scale=s0)
+    z = (grid - l0) / s0
+    th = np.tanh(z / 2)
+    score_loc = th / s0
+    score_raw = -(1 - z * th) * (1 / (1 + np.exp(-r0))) / s0
+    dx = grid[1] - grid[0]
+    assert abs((pdf * score_loc ** 2).sum() * dx - 1 / (3 * s0 ** 2)) < 1e-6
+    assert abs((pdf * score_raw ** 2).sum() * dx - (np.pi ** 2 + 3) / 9 * ((1 / (1 + np.exp(-r0))) / s0) ** 2) < 1e-6
+
+
+def test_logistic_mle_metric_link_and_predict():
+    from scipy.stats import logistic
+    rng = np.random.default_rng(13)
+    N = 500
+    pred = np.stack([rng.standard_normal(N), rng.standard_normal(N)], axis=1).astype(np.float32)
+    y = rng.standard_normal(N).astype(np.float32)
+    w = (rng.random(N) + 0.5).astype(np.float32)
+    got = orc.eval_metric("logistic_mle", 2, pred, y, w)
+    s = np.logaddexp(0.0, pred[:, 1].astype(np.float64))
+    want = (w * logistic.logpdf(y.astype(np.float64), loc=pred[:, 0].astype(np.float64), scale=s)).sum() / w.astype(np.float64).sum()
+    assert abs(got - want) < 2e-6 * abs(want) + 1e-7  # the metric is the weighted mean log-likelihood (src/metrics.jl:92-97)
+    linked = pred.copy()
+    orc.apply_link(orc.LOSS_IDS["logistic_mle"], 2, linked)
+    assert np.array_equal(linked[:, 0], pred[:, 0])
+    np.testing.assert_allclose(linked[:, 1], s, rtol=2e-6)
+    # predict!: location adds, the raw scale is floored at -15 (src/predict.jl:31-46, the MLE2P method)
+    x_bin = np.array([[1, 2]], np.uint8)
+    t = orc.Tree(2, 3)
+    t.feat[0], t.cond_bin[0], t.split[0] = 1, 1, 1
+    t.pred[1] = [2.0, -40.0]
+    t.pred[2] = [-3.0, 1.0]
+    p = np.zeros((2, 2), np.float32)
+    orc.predict_tree(orc.LOSS_IDS["logistic_mle"], 2, x_bin, np.ones(1, np.uint8), t, p)
+    assert p.tolist() == [[2.0, -15.0], [-3.0, 1.0]]
