@@ -281,3 +281,48 @@ def test_gradients_queued_ahead_change_nothing(evt, loss, tt):
             assert a.tobytes() == b.tobytes()
         else:
             assert_tree_bits(a, b)
+
+
+def test_two_handles_on_two_threads(evt):
+    """Different handles may be driven from different threads at once (each has its own stream; the error message is
+    per thread): two threads boost different problems concurrently and get, bit for bit, what a single thread gets."""
+    import threading
+    specs = [("mse", 60000, 20, 32, 6, 11), ("logloss", 45000, 9, 64, 5, 12)]
+
+    def run(spec, out, k, barrier=None):
+        loss, N, F, B, D, seed = spec
+        x_bin, y, w, mu = make_data(seed, N, F, B, loss, weights=True)
+        h = evt.Handle(N, F, B, 1, D, loss)
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        gp = evt.make_params(eta=0.2)
+        js = np.arange(1, F + 1, dtype=np.uint32)
+        rng = np.random.default_rng(seed)
+        trees = []
+        if barrier is not None:
+            barrier.wait()
+        for r in range(12):
+            h.update_grads()
+            mask = rng.integers(0, 256, N, dtype=np.uint8) if r % 3 == 1 else None
+            trees.append(h.grow_tree(js, gp, mask=mask, cond=150))
+        try:
+            h.grow_tree(np.array([F + 5], np.uint32), gp)  # an error on this thread: its message stays on this thread
+        except evt.EvtError as e:
+            out[k] = (trees, h.get_pred(), str(e))
+        h.close()
+
+    seq, par = {}, {}
+    for k, s in enumerate(specs):
+        run(s, seq, k)
+    barrier = threading.Barrier(2)
+    ths = [threading.Thread(target=run, args=(s, par, k, barrier)) for k, s in enumerate(specs)]
+    for t in ths:
+        t.start()
+    for t in ths:
+        t.join()
+    for k in range(2):
+        assert k in par, "thread %d did not finish" % k
+        for ta, tb in zip(seq[k][0], par[k][0]):
+            assert_tree_bits(ta, tb)
+        assert np.array_equal(seq[k][1].view(np.uint32), par[k][1].view(np.uint32))
+        assert "js entries" in par[k][2]
