@@ -63,8 +63,9 @@ def test_multi_target_tree_against_the_oracle(evt, loss, T, weights, N, F, B, D,
     if loss == "mse":
         assert np.array_equal(g_dev.view(np.uint32), grad.view(np.uint32))
     else:
-        # (1 - r^2 / s^2) cancels near r = s: the absolute bound scales with the largest gradient
-        np.testing.assert_allclose(g_dev, grad, rtol=2e-6, atol=2e-7 * float(np.abs(grad[:, :2 * K]).max()))
+        # (1 - r^2 / s^2) and (1 - z tanh(z / 2)) cancel, which magnifies the last-bit differences between two libm's exp / tanh:
+        # the absolute bound scales with the largest gradient
+        np.testing.assert_allclose(g_dev, grad, rtol=2e-6, atol=1e-6 * float(np.abs(grad[:, :2 * K]).max()))
     assert np.array_equal(g_dev[:, 2 * K], grad[:, 2 * K])
     # one tree on identical gradients
     h.set_grads(grad)
