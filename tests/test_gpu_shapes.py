@@ -39,6 +39,10 @@ def _cases():
         ("mse", False, 12000, 130, 255, 4, "oblivious", 130, 0.5, None, True, 103),
         ("mlogloss", True, 1233, 578, 16, 1, "binary", 578, 0.5, 15, False, 104),
         ("mlogloss", True, 112, 17, 255, 7, "binary", 13, 1.0, 16, True, 105),  # 33 channels x 255 bins
+        # the widest matrix the library takes, 255 bins: 32 column tiles, or the generic kernel when one tile's channels do not fit
+        ("mse", False, 3000, 1024, 255, 3, "binary", 1024, 1.0, None, False, 106),
+        ("gaussian_mle", True, 4000, 512, 255, 3, "oblivious", 512, 1.0, None, False, 107),
+        ("logistic_mle", False, 5000, 1000, 128, 3, "binary", 999, 0.5, None, True, 108),
     ]
     return out
 
