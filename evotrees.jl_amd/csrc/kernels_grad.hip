@@ -300,9 +300,11 @@ __global__ __launch_bounds__(256) void k_quantize(const float *__restrict__ grad
     for (int a = 0; a < NA; a++) {
         const int k = (mse && a == 1) ? 2 : a;
         long long q = __double2ll_rn((double)g[k] * qmul[k]);
-        unsigned long long word = (unsigned long long)q;
-        if (a == 0 && pack) word = ((unsigned long long)q << EVT_PACK_CNT_BITS) + 1ull;
-        gq[(size_t)a * N + i] = word;
+        if (a == 0 && pack) { // 30 bits: staged as a 32-bit word, widened to (q << 16) + 1 (the row count) by the histogram kernel
+            reinterpret_cast<int32_t *>(gq)[i] = (int32_t)q;
+            continue;
+        }
+        gq[(size_t)a * N + i] = (unsigned long long)q;
     }
 }
 

@@ -58,6 +58,17 @@ __device__ __forceinline__ int first_node_of_span(const int64_t *__restrict__ bp
     return cnt - 1;
 }
 
+// The fixed-point word of channel a for one row.  The channel that shares its word with the row count holds 30 bits:
+// it is staged as a 32-bit word (half the plane to gather from) and widened here to (q << 16) + 1.
+template <bool PACK>
+__device__ __forceinline__ unsigned long long load_gq(const unsigned long long *__restrict__ gq, int64_t N, int a, uint32_t id) {
+    if (PACK && a == 0) {
+        const long long q = (long long)reinterpret_cast<const int32_t *>(gq)[id];
+        return ((unsigned long long)q << EVT_PACK_CNT_BITS) + 1ull;
+    }
+    return gq[(size_t)a * N + id];
+}
+
 template <int NA, bool PACK>
 __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     extern __shared__ unsigned long long H[]; // [NA][tile slots][B]
@@ -142,7 +153,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
                 if (rc[u] != INV) {
                     vc[u] = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)rc[u] * A.RS + sub * 16);
 #pragma unroll
-                    for (int a = 0; a < NA; a++) gc[u][a] = A.gq[(size_t)a * A.N + rc[u]];
+                    for (int a = 0; a < NA; a++) gc[u][a] = load_gq<PACK>(A.gq, A.N, a, rc[u]);
                 }
             }
 #pragma unroll
@@ -157,7 +168,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
                     if (rn[u] != INV) {
                         vn[u] = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)rn[u] * A.RS + sub * 16);
 #pragma unroll
-                        for (int a = 0; a < NA; a++) gn[u][a] = A.gq[(size_t)a * A.N + rn[u]];
+                        for (int a = 0; a < NA; a++) gn[u][a] = load_gq<PACK>(A.gq, A.N, a, rn[u]);
                     }
                 }
                 uint32_t rnn[U];
@@ -369,7 +380,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                 idc = isp[(fetcher && p < nend) ? p : lastp];
             }
 #pragma unroll
-            for (int a = 0; a < NA; a++) gc[a] = A.gq[(size_t)a * A.N + idc];
+            for (int a = 0; a < NA; a++) gc[a] = load_gq<PACK>(A.gq, A.N, a, idc);
             {
                 const int64_t p = pw + itstride + mypos;
                 idn = isp[(fetcher && p < nend) ? p : lastp];
@@ -387,7 +398,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             for (; pw < nend; pw += itstride) {
                 // next iteration's gradient words and the row ids of the one after: ahead of the records in issue order
 #pragma unroll
-                for (int a = 0; a < NA; a++) gn[a] = A.gq[(size_t)a * A.N + idn];
+                for (int a = 0; a < NA; a++) gn[a] = load_gq<PACK>(A.gq, A.N, a, idn);
                 uint32_t idnn;
                 {
                     const int64_t p = pw + 2 * itstride + mypos;
