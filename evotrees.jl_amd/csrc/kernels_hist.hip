@@ -277,11 +277,14 @@ __device__ __forceinline__ uint32_t grp_bcast(uint32_t x) {
 template <int PB>
 __device__ __forceinline__ uint2 load_piece(const uint8_t *p) {
     if constexpr (PB == 8) {
-        return *reinterpret_cast<const uint2 *>(p);
+        // a record is read once per level: the streaming hint keeps it from displacing the gradient words, which neighbouring
+        // rows of other nodes will gather again
+        const unsigned long long v = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(p));
+        return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
     } else if constexpr (PB == 4) {
-        return make_uint2(*reinterpret_cast<const uint32_t *>(p), 0u);
+        return make_uint2(__builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p)), 0u);
     } else {
-        return make_uint2((uint32_t)*reinterpret_cast<const uint16_t *>(p), 0u);
+        return make_uint2((uint32_t)__builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(p)), 0u);
     }
 }
 
@@ -377,13 +380,13 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             uint2 v[U];
             {
                 const int64_t p = pw + mypos;
-                idc = isp[(fetcher && p < nend) ? p : lastp];
+                idc = __builtin_nontemporal_load(isp + ((fetcher && p < nend) ? p : lastp));
             }
 #pragma unroll
             for (int a = 0; a < NA; a++) gc[a] = load_gq<PACK>(A.gq, A.N, a, idc);
             {
                 const int64_t p = pw + itstride + mypos;
-                idn = isp[(fetcher && p < nend) ? p : lastp];
+                idn = __builtin_nontemporal_load(isp + ((fetcher && p < nend) ? p : lastp));
             }
             __builtin_amdgcn_sched_barrier(0);
 #define EVT_H16_PRO(u_)                                                                                               \
@@ -402,7 +405,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                 uint32_t idnn;
                 {
                     const int64_t p = pw + 2 * itstride + mypos;
-                    idnn = isp[(fetcher && p < nend) ? p : lastp];
+                    idnn = __builtin_nontemporal_load(isp + ((fetcher && p < nend) ? p : lastp));
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #define EVT_H16_STEP(u_)                                                                                              \
