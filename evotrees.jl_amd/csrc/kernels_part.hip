@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
             rid[it] = A.is_cur[p < pend ? p : pend - 1];
         }
 #pragma unroll
-        for (int it = 0; it < NI; it++) xbv[it] = col[rid[it]];
+        for (int it = 0; it < NI; it++) xbv[it] = __builtin_nontemporal_load(col + rid[it]);
 #pragma unroll
         for (int it = 0; it < NI; it++) {
             const int64_t p = p0 + it * 256 + tid;
@@ -210,7 +210,7 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
             rid[it] = A.is_cur[p < pend ? p : pend - 1];
         }
 #pragma unroll
-        for (int it = 0; it < NI; it++) xbv[it] = is_split ? (uint32_t)col[rid[it]] : 0u;
+        for (int it = 0; it < NI; it++) xbv[it] = is_split ? (uint32_t)__builtin_nontemporal_load(col + rid[it]) : 0u;
         const bool fast1 = A.fuse_pred && K == 1;
         if (fast1) {
 #pragma unroll
