@@ -274,21 +274,32 @@ __device__ __forceinline__ uint32_t grp_bcast(uint32_t x) {
 }
 
 // A record piece of PB bytes in the low bytes of a register pair.
-template <int PB>
+// NT: the streaming hint.  A record is read once per level; when the record array is larger than the last-level cache the
+// hint keeps it from displacing the gradient words, which neighbouring rows of other nodes will gather again.  A smaller
+// array is better left to the caches: it is still there at the next level.
+template <int PB, bool NT>
 __device__ __forceinline__ uint2 load_piece(const uint8_t *p) {
     if constexpr (PB == 8) {
-        // a record is read once per level: the streaming hint keeps it from displacing the gradient words, which neighbouring
-        // rows of other nodes will gather again
-        const unsigned long long v = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(p));
-        return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
+        if constexpr (NT) {
+            const unsigned long long v = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(p));
+            return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
+        } else {
+            return *reinterpret_cast<const uint2 *>(p);
+        }
     } else if constexpr (PB == 4) {
-        return make_uint2(__builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p)), 0u);
+        const uint32_t *q = reinterpret_cast<const uint32_t *>(p);
+        return make_uint2(NT ? __builtin_nontemporal_load(q) : *q, 0u);
     } else {
-        return make_uint2((uint32_t)__builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(p)), 0u);
+        const uint16_t *q = reinterpret_cast<const uint16_t *>(p);
+        return make_uint2((uint32_t)(NT ? __builtin_nontemporal_load(q) : *q), 0u);
     }
 }
+template <bool NT>
+__device__ __forceinline__ uint32_t load_id(const uint32_t *p) {
+    return NT ? __builtin_nontemporal_load(p) : *p;
+}
 
-template <int NA, bool PACK, int U, bool FULL, int PB>
+template <int NA, bool PACK, int U, bool FULL, int PB, bool NT>
 __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     extern __shared__ unsigned long long H[]; // [NA][PB][B][NS]
     const int tid = threadIdx.x, nthr = blockDim.x;
@@ -380,19 +391,19 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             uint2 v[U];
             {
                 const int64_t p = pw + mypos;
-                idc = __builtin_nontemporal_load(isp + ((fetcher && p < nend) ? p : lastp));
+                idc = load_id<NT>(isp + ((fetcher && p < nend) ? p : lastp));
             }
 #pragma unroll
             for (int a = 0; a < NA; a++) gc[a] = load_gq<PACK>(A.gq, A.N, a, idc);
             {
                 const int64_t p = pw + itstride + mypos;
-                idn = __builtin_nontemporal_load(isp + ((fetcher && p < nend) ? p : lastp));
+                idn = load_id<NT>(isp + ((fetcher && p < nend) ? p : lastp));
             }
             __builtin_amdgcn_sched_barrier(0);
 #define EVT_H16_PRO(u_)                                                                                               \
     if constexpr ((u_) < U) {                                                                                         \
         const uint32_t row = grp_bcast<(u_) < U ? (u_) : 0>(idc);                                               \
-        v[(u_) < U ? (u_) : 0] = load_piece<PB>(A.xrm + (size_t)row * A.RS + tb + subl * PB);           \
+        v[(u_) < U ? (u_) : 0] = load_piece<PB, NT>(A.xrm + (size_t)row * A.RS + tb + subl * PB);           \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
             EVT_H16_PRO(0) EVT_H16_PRO(1) EVT_H16_PRO(2) EVT_H16_PRO(3) EVT_H16_PRO(4) EVT_H16_PRO(5) EVT_H16_PRO(6) EVT_H16_PRO(7)
@@ -405,7 +416,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                 uint32_t idnn;
                 {
                     const int64_t p = pw + 2 * itstride + mypos;
-                    idnn = __builtin_nontemporal_load(isp + ((fetcher && p < nend) ? p : lastp));
+                    idnn = load_id<NT>(isp + ((fetcher && p < nend) ? p : lastp));
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #define EVT_H16_STEP(u_)                                                                                              \
@@ -430,7 +441,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             }                                                                                                         \
         }                                                                                                             \
         const uint32_t row = grp_bcast<ui>(idn);                                                                \
-        v[ui] = load_piece<PB>(A.xrm + (size_t)row * A.RS + tb + subl * PB);                          \
+        v[ui] = load_piece<PB, NT>(A.xrm + (size_t)row * A.RS + tb + subl * PB);                          \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
                 EVT_H16_STEP(0) EVT_H16_STEP(1) EVT_H16_STEP(2) EVT_H16_STEP(3) EVT_H16_STEP(4) EVT_H16_STEP(5) EVT_H16_STEP(6) EVT_H16_STEP(7)
@@ -529,7 +540,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     }
 }
 
-template <int NA, bool PACK, int U, int PB>
+template <int NA, bool PACK, int U, int PB, bool NT>
 static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
     // unpredicated atomics for every feature of the record pay off unless most features are left out: the words of
     // features outside the sample are simply not flushed
@@ -537,16 +548,16 @@ static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads
     if (lds > 64 * 1024) { // one block per CU may take most of its 160 KB
         static bool attr_set = false;
         if (!attr_set) {
-            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, true, PB>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, false, PB>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, true, PB, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, false, PB, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
             attr_set = true;
         }
     }
     // c->launch_e0 / launch_e1 (when profiling): the kernel's own dispatch records them
     if (full)
-        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, true, PB>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
+        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, true, PB, NT>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
     else
-        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, false, PB>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
+        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, false, PB, NT>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -555,9 +566,11 @@ template <int NA, bool PACK>
 static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
     // row groups (records) in flight per wave: as many as a DPP row can address, fewer when registers run out
     constexpr int U = (NA <= 2) ? 16 : 8;
-    if (A.TW >= 128) return launch_hist16_q<NA, PACK, U, 8>(c, A, grid, threads, lds);
-    if (A.TW == 64) return launch_hist16_q<NA, PACK, U, 4>(c, A, grid, threads, lds);
-    return launch_hist16_q<NA, PACK, U, 2>(c, A, grid, threads, lds); // 32-byte tiles
+    // records larger in total than the last-level cache (256 MB) are streamed past it
+    const bool nt = (size_t)c->N * c->RS > ((size_t)256 << 20);
+    if (A.TW >= 128) return nt ? launch_hist16_q<NA, PACK, U, 8, true>(c, A, grid, threads, lds) : launch_hist16_q<NA, PACK, U, 8, false>(c, A, grid, threads, lds);
+    if (A.TW == 64) return nt ? launch_hist16_q<NA, PACK, U, 4, true>(c, A, grid, threads, lds) : launch_hist16_q<NA, PACK, U, 4, false>(c, A, grid, threads, lds);
+    return nt ? launch_hist16_q<NA, PACK, U, 2, true>(c, A, grid, threads, lds) : launch_hist16_q<NA, PACK, U, 2, false>(c, A, grid, threads, lds); // 32-byte tiles
 }
 
 template <int NA, bool PACK>

@@ -50,8 +50,12 @@ struct PartArgs {
     float *pred;
     const float *t_pred;
     int K, loss, fuse_pred, write_nidx;
+    int stream_hint; // the binned matrix does not fit the last-level cache
 };
 
+// NT: the streaming hint on the gathered bin bytes (a template parameter: a run-time branch between two otherwise
+// identical loads is merged by the compiler, which drops the hint)
+template <bool NT>
 __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n_act = (int)A.hdr[LH_N_ACT];
@@ -83,8 +87,10 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
             const int64_t p = p0 + it * 256 + tid;
             rid[it] = A.is_cur[p < pend ? p : pend - 1];
         }
+        // a binned matrix larger than the last-level cache is gathered with the streaming hint: each byte's line would
+        // displace data that is read again (row lists, gradient words) and is rarely hit a second time itself
 #pragma unroll
-        for (int it = 0; it < NI; it++) xbv[it] = __builtin_nontemporal_load(col + rid[it]);
+        for (int it = 0; it < NI; it++) xbv[it] = NT ? __builtin_nontemporal_load(col + rid[it]) : col[rid[it]];
 #pragma unroll
         for (int it = 0; it < NI; it++) {
             const int64_t p = p0 + it * 256 + tid;
@@ -174,6 +180,7 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
 // for a categorical feature) but the row list is not rewritten: nothing reads it afterwards.  Each row
 // gets its leaf's value added to the prediction (predict!, src/predict.jl:1-46) and, on request, its
 // node id recorded.
+template <bool NT>
 __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
     const int tid = threadIdx.x;
     const int n_act = (int)A.hdr[LH_N_ACT];
@@ -210,7 +217,7 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
             rid[it] = A.is_cur[p < pend ? p : pend - 1];
         }
 #pragma unroll
-        for (int it = 0; it < NI; it++) xbv[it] = is_split ? (uint32_t)__builtin_nontemporal_load(col + rid[it]) : 0u;
+        for (int it = 0; it < NI; it++) xbv[it] = is_split ? (uint32_t)(NT ? __builtin_nontemporal_load(col + rid[it]) : col[rid[it]]) : 0u;
         const bool fast1 = A.fuse_pred && K == 1;
         if (fast1) {
 #pragma unroll
@@ -600,12 +607,14 @@ static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32
     A.loss = c->loss; // selects the leaf-add rule
     A.fuse_pred = fuse_pred ? 1 : 0;
     A.write_nidx = c->write_nidx ? 1 : 0;
+    A.stream_hint = ((size_t)c->N * c->F > ((size_t)256 << 20)) ? 1 : 0;
 }
 
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur) {
     PartArgs A;
     fill_part_args(c, level, is_cur, nullptr, false, A);
-    hipLaunchKernelGGL(k_part_count, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
+    if (A.stream_hint) hipLaunchKernelGGL(k_part_count<true>, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
+    else hipLaunchKernelGGL(k_part_count<false>, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -622,7 +631,8 @@ int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_
     if (!fuse_pred && !c->write_nidx) return EVT_OK;
     PartArgs A;
     fill_part_args(c, level, is_cur, nullptr, fuse_pred, A);
-    hipLaunchKernelGGL(k_final_fused, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
+    if (A.stream_hint) hipLaunchKernelGGL(k_final_fused<true>, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
+    else hipLaunchKernelGGL(k_final_fused<false>, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
