@@ -9,6 +9,7 @@
 #include <new>
 
 int launch_absmax_rows(evt_ctx *c, int k0, int k1);
+int launch_check_unit_weight(evt_ctx *c);
 int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, const float *leaf_pred_dev);
 int launch_predict_model(hipStream_t s, const uint32_t *nodes, const float *leaf_pred, const int64_t *off, int ntrees, const uint8_t *xcm, int64_t N,
                          int K, int loss, int apply_link, float *out);
@@ -28,7 +29,25 @@ void evt_set_error(const char *fmt, ...) {
 
 extern "C" const char *evt_last_error(void) { return g_err; }
 
+// No C++ exception crosses the C ABI: every entry point that returns a status runs inside this guard.
+template <typename F>
+static int guarded(F &&f) {
+    try {
+        return f();
+    } catch (const std::bad_alloc &) {
+        evt_set_error("out of host memory");
+        return EVT_ERR_NOMEM;
+    } catch (const std::exception &e) {
+        evt_set_error("internal error: %s", e.what());
+        return EVT_ERR_NOMEM;
+    } catch (...) {
+        evt_set_error("internal error");
+        return EVT_ERR_NOMEM;
+    }
+}
+
 extern "C" int evt_device_count(int32_t *count) {
+    return guarded([&]() -> int {
     ARGCHK(count, "count is NULL");
     int n = 0;
     hipError_t e = hipGetDeviceCount(&n);
@@ -39,6 +58,7 @@ extern "C" int evt_device_count(int32_t *count) {
     }
     *count = n;
     return EVT_OK;
+    });
 }
 
 // ---- profiling ------------------------------------------------------------------------------
@@ -149,12 +169,13 @@ static int ceil_log2_i64(int64_t v) {
 }
 
 extern "C" int evt_destroy(evt_handle c) {
+    return guarded([&]() -> int {
     if (!c) return EVT_OK;
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
-                    c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp, c->qbits,
-                    c->qscale, c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id, c->pt_nodes, c->pt_pred, c->mask_next};
+                    c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp_buf[0], c->qexp_buf[1], c->qbits,
+                    c->qscale_buf[0], c->qscale_buf[1], c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id, c->pt_nodes, c->pt_pred, c->mask_next};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -178,10 +199,12 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
     return EVT_OK;
+    });
 }
 
 extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K, int32_t max_depth, int32_t loss, int32_t tree_type,
                           evt_handle *out) {
+    return guarded([&]() -> int {
     ARGCHK(out, "out handle is NULL");
     *out = nullptr;
     ARGCHK(nobs >= 1 && nobs <= (int64_t)0xFFFFFFFFll, "nobs must be in [1, 2^32-1]");
@@ -222,7 +245,8 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->tree_blob = nullptr;
     memset(c->lvl, 0, sizeof(c->lvl));
     c->js = nullptr; c->jsmap = nullptr; c->feattypes = nullptr; c->mono = nullptr; c->absmax = nullptr; c->qexp = nullptr; c->qbits = nullptr;
-    c->qscale = nullptr; c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->sbest = nullptr;
+    c->qscale = nullptr; c->qexp_buf[0] = c->qexp_buf[1] = nullptr; c->qscale_buf[0] = c->qscale_buf[1] = nullptr; c->q_cur = c->q_tree = 0;
+    c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->sbest = nullptr;
     c->h_stage = nullptr; c->h_stage_dev = nullptr; c->h_stage_bytes = 0;
     c->n_js_last = 0;
     c->last_all_rows = true;
@@ -326,9 +350,13 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->feattypes, c->F);
     ALLOC(c->mono, c->F);
     ALLOC(c->absmax, EVT_MC_MAX_NK);
-    ALLOC(c->qexp, EVT_MC_MAX_NK);
+    for (int s = 0; s < 2; s++) {
+        ALLOC(c->qexp_buf[s], EVT_MC_MAX_NK);
+        ALLOC(c->qscale_buf[s], 2 * EVT_MC_MAX_NK);
+    }
+    c->qexp = c->qexp_buf[0];
+    c->qscale = c->qscale_buf[0];
     ALLOC(c->qbits, EVT_MC_MAX_NK);
-    ALLOC(c->qscale, 2 * EVT_MC_MAX_NK);
     ALLOC(c->metric_partial, 2 * EVT_METRIC_BLOCKS + 1);
     ALLOC(c->errflag, 1);
     if (tree_type == EVT_TREE_OBLIVIOUS) ALLOC(c->ogains, (size_t)c->maxlvl * c->F * c->B);
@@ -375,6 +403,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     }
     *out = c;
     return EVT_OK;
+    });
 }
 
 // every call on a handle but evt_grow_tree_end, evt_synchronize and evt_destroy waits for a tree begun with
@@ -417,6 +446,7 @@ static int check_errflag(evt_ctx *c, const char *what) {
 }
 
 extern "C" int evt_set_xbin(evt_handle c, const uint8_t *x_bin_colmajor) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(x_bin_colmajor, "x_bin is NULL");
     c->have_xbin = false;
@@ -427,9 +457,11 @@ extern "C" int evt_set_xbin(evt_handle c, const uint8_t *x_bin_colmajor) {
     if (r != EVT_OK) return r;
     c->have_xbin = true;
     return EVT_OK;
+    });
 }
 
 extern "C" int evt_binarize_f64(evt_handle c, const double *x_colmajor, const double *edges, const int32_t *edge_off) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(x_colmajor && edges && edge_off, "NULL argument");
     c->have_xbin = false;
@@ -474,6 +506,7 @@ extern "C" int evt_binarize_f64(evt_handle c, const double *x_colmajor, const do
     if (r != EVT_OK) return r;
     c->have_xbin = true;
     return EVT_OK;
+    });
 }
 
 static void set_channels(evt_ctx *c) {
@@ -497,6 +530,7 @@ static void set_channels(evt_ctx *c) {
 }
 
 extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, const float *mu, const float *offset) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(y && mu, "y and mu must not be NULL");
     c->have_target = false;
@@ -541,9 +575,11 @@ extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, cons
     HIPCHK(hipStreamSynchronize(c->stream));
     c->have_target = true;
     return EVT_OK;
+    });
 }
 
 extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, const int32_t *monotone) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     std::vector<uint8_t> ft(c->F, 1);
     std::vector<int32_t> mo(c->F, 0);
@@ -562,6 +598,7 @@ extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, cons
     HIPCHK(hipMemcpy(c->mono, mo.data(), sizeof(int32_t) * c->F, hipMemcpyHostToDevice));
     c->h_feattypes = ft;
     return EVT_OK;
+    });
 }
 
 static int queue_grads(evt_ctx *c) {
@@ -577,6 +614,7 @@ static int queue_grads(evt_ctx *c) {
 }
 
 extern "C" int evt_update_grads(evt_handle c) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     if (!c->have_target) {
         evt_set_error("evt_set_target must be called before evt_update_grads");
@@ -591,9 +629,11 @@ extern "C" int evt_update_grads(evt_handle c) {
     if (r != EVT_OK) return r;
     c->have_grads = true;
     return EVT_OK;
+    });
 }
 
 extern "C" int evt_set_grads(evt_handle c, const float *grad) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(grad, "grad is NULL");
     if (!c->have_target) {
@@ -601,14 +641,22 @@ extern "C" int evt_set_grads(evt_handle c, const float *grad) {
         return EVT_ERR_STATE;
     }
     c->grads_ready = false;
+    c->have_grads = false;
     HIPCHK(hipMemcpyAsync(c->grad, grad, sizeof(float) * (size_t)c->N * c->NK, hipMemcpyDefault, c->stream));
-    int r = launch_absmax_rows(c, 0, c->NK);
+    int r = EVT_OK;
+    if (c->unit_w) { // the target was set without weights: the row count stands for the weight, the weight row must say so
+        r = launch_check_unit_weight(c);
+        if (r == EVT_OK) r = check_errflag(c, "evt_set_grads: the weight row must be all ones when evt_set_target was given no weights");
+        if (r != EVT_OK) return r;
+    }
+    r = launch_absmax_rows(c, 0, c->NK);
     if (r != EVT_OK) return r;
     r = launch_quantize(c);
     if (r != EVT_OK) return r;
     HIPCHK(hipStreamSynchronize(c->stream));
     c->have_grads = true;
     return EVT_OK;
+    });
 }
 
 static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p,
@@ -644,6 +692,7 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
     c->grads_ready = false; // this tree changes the predictions
     c->last_all_rows = all_rows;
     c->last_cond = cond;
+    c->q_tree = c->q_cur; // this tree is grown on (and decoded with) the tables of the gradients quantised last
     // a tree grown in stages records the node of every row on the way, so that evt_get_nidx can show it after each stage
     const bool rec_nidx = c->record_nidx || staged;
     c->nidx_valid = rec_nidx;
@@ -796,8 +845,10 @@ static int tree_close(evt_ctx *c) {
     r = launch_copy_to_host(c, c->tree_blob, c->h_stage_dev, c->blob_bytes);
     if (r != EVT_OK) return r;
     HIPCHK(hipEventRecord(c->tree_ev, c->stream));
-    if (c->grads_ahead && p->update_pred) {
-        // the next round's gradient update runs while the host collects this tree and prepares the next call
+    if (c->grads_ahead && p->update_pred && p->bagging_size == 1) {
+        // the next round's gradient update runs while the host collects this tree and prepares the next call.  Not with
+        // bagging: the trees of one round are all grown on the same gradients (src/fit.jl:9-11), and the library cannot
+        // tell which call is the round's last.
         r = queue_grads(c);
         if (r != EVT_OK) return r;
         c->grads_ready = true;
@@ -824,14 +875,17 @@ static int tree_run_stages(evt_ctx *c, int r) {
 }
 
 extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     int r = tree_open(c, mask, false, cond, js, n_js, p, false);
     return tree_run_stages(c, r);
+    });
 }
 
 // The next tree's mask, uploaded while this one grows: the copy runs on a stream of its own, into the buffer the tree
 // in flight does not read.
 extern "C" int evt_stage_mask(evt_handle c, const uint8_t *mask) {
+    return guarded([&]() -> int {
     ARGCHK(c != nullptr, "handle is NULL");
     ARGCHK(mask != nullptr, "mask is NULL");
     HIPCHK(hipSetDevice(c->device));
@@ -849,9 +903,11 @@ extern "C" int evt_stage_mask(evt_handle c, const uint8_t *mask) {
     HIPCHK(hipStreamSynchronize(c->copy_stream)); // the caller may reuse its buffer; the tree in flight keeps running
     c->mask_next_valid = true;
     return EVT_OK;
+    });
 }
 
 extern "C" int evt_grow_tree_begin_staged(evt_handle c, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     if (!c->mask_next_valid) {
         evt_set_error("evt_grow_tree_begin_staged: no mask has been staged since the last tree (evt_stage_mask)");
@@ -859,13 +915,16 @@ extern "C" int evt_grow_tree_begin_staged(evt_handle c, uint8_t cond, const uint
     }
     int r = tree_open(c, nullptr, true, cond, js, n_js, p, false);
     return tree_run_stages(c, r);
+    });
 }
 
 extern "C" int evt_tree_open(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     int r = tree_open(c, mask, false, cond, js, n_js, p, true);
     if (r != EVT_OK) return tree_fail(c, r);
     return EVT_OK;
+    });
 }
 
 static int stage_check(evt_ctx *c, int phase, int32_t level, const char *name) {
@@ -883,36 +942,44 @@ static int stage_check(evt_ctx *c, int phase, int32_t level, const char *name) {
 }
 
 extern "C" int evt_hist_build(evt_handle c, int32_t level) {
+    return guarded([&]() -> int {
     CTXCHK_STEP(c);
     int r = stage_check(c, 1, level, "evt_hist_build");
     if (r != EVT_OK) return r;
     r = tree_stage_hist(c);
     return r == EVT_OK ? r : tree_fail(c, r);
+    });
 }
 
 extern "C" int evt_split_scan(evt_handle c, int32_t level) {
+    return guarded([&]() -> int {
     CTXCHK_STEP(c);
     int r = stage_check(c, 2, level, "evt_split_scan");
     if (r != EVT_OK) return r;
     r = tree_stage_scan(c);
     return r == EVT_OK ? r : tree_fail(c, r);
+    });
 }
 
 extern "C" int evt_update_nodes_idx(evt_handle c, int32_t level) {
+    return guarded([&]() -> int {
     CTXCHK_STEP(c);
     int r = stage_check(c, 3, level, "evt_update_nodes_idx");
     if (r != EVT_OK) return r;
     r = tree_stage_partition(c);
     return r == EVT_OK ? r : tree_fail(c, r);
+    });
 }
 
 extern "C" int evt_tree_close(evt_handle c) {
+    return guarded([&]() -> int {
     CTXCHK_STEP(c);
     if (c->step.phase != 4) {
         evt_set_error(c->step.phase == 0 ? "evt_tree_close: no tree is open" : "evt_tree_close before the last level was partitioned");
         return EVT_ERR_STATE;
     }
     return tree_close(c);
+    });
 }
 
 // host copy of the device's tree arrays (in the pinned staging buffer) -> the caller's arrays
@@ -931,6 +998,7 @@ static int fill_tree_out(evt_ctx *c, evt_tree_out *tree) {
 }
 
 extern "C" int evt_grow_tree_end(evt_handle c, evt_tree_out *tree) {
+    return guarded([&]() -> int {
     ARGCHK(c != nullptr, "handle is NULL");
     HIPCHK(hipSetDevice(c->device));
     if (!c->tree_in_flight) {
@@ -953,23 +1021,28 @@ extern "C" int evt_grow_tree_end(evt_handle c, evt_tree_out *tree) {
     }
     if (tree) return fill_tree_out(c, tree);
     return EVT_OK;
+    });
 }
 
 // The tree arrays as they stand on the device, e.g. between the stages of a tree opened with evt_tree_open.
 extern "C" int evt_peek_tree(evt_handle c, evt_tree_out *tree) {
+    return guarded([&]() -> int {
     CTXCHK_STEP(c);
     ARGCHK(tree, "tree is NULL");
     int r = launch_copy_to_host(c, c->tree_blob, c->h_stage_dev, c->blob_bytes);
     if (r != EVT_OK) return r;
     HIPCHK(hipStreamSynchronize(c->stream));
     return fill_tree_out(c, tree);
+    });
 }
 
 extern "C" int evt_grow_tree(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p,
                              evt_tree_out *tree) {
+    return guarded([&]() -> int {
     const int r = evt_grow_tree_begin(c, mask, cond, js, n_js, p);
     if (r != EVT_OK) return r;
     return evt_grow_tree_end(c, tree);
+    });
 }
 
 // host tree -> packed device nodes; validates that every split node has both children in range
@@ -988,6 +1061,7 @@ static int pack_tree(int32_t nn, const int64_t *feat, const uint8_t *cond_bin, c
 
 extern "C" int evt_predict_tree(evt_handle c, int32_t nnodes_tree, const int64_t *feat, const uint8_t *cond_bin, const float *pred,
                                 const uint8_t *split) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(feat && cond_bin && pred && split && nnodes_tree >= 1, "NULL tree arrays");
     if (!c->have_xbin || !c->have_target) {
@@ -1039,9 +1113,11 @@ extern "C" int evt_predict_tree(evt_handle c, int32_t nnodes_tree, const int64_t
         prof_collect(c, nullptr);
     }
     return EVT_OK;
+    });
 }
 
 extern "C" int evt_get_xbin(evt_handle c, uint8_t *out) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(out, "out is NULL");
     if (!c->have_xbin) {
@@ -1051,8 +1127,10 @@ extern "C" int evt_get_xbin(evt_handle c, uint8_t *out) {
     HIPCHK(hipMemcpyAsync(out, c->xcm, (size_t)c->N * c->F, hipMemcpyDefault, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     return EVT_OK;
+    });
 }
 extern "C" int evt_get_pred(evt_handle c, float *out) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(out, "out is NULL");
     {
@@ -1062,15 +1140,19 @@ extern "C" int evt_get_pred(evt_handle c, float *out) {
     HIPCHK(hipMemcpyAsync(out, c->pred, sizeof(float) * (size_t)c->N * c->K, hipMemcpyDefault, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     return EVT_OK;
+    });
 }
 extern "C" int evt_get_grads(evt_handle c, float *out) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(out, "out is NULL");
     HIPCHK(hipMemcpyAsync(out, c->grad, sizeof(float) * (size_t)c->N * c->NK, hipMemcpyDefault, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     return EVT_OK;
+    });
 }
 extern "C" int evt_get_nidx(evt_handle c, uint32_t *out) {
+    return guarded([&]() -> int {
     CTXCHK_STEP(c);
     ARGCHK(out, "out is NULL");
     if (c->n_js_last <= 0) {
@@ -1089,8 +1171,10 @@ extern "C" int evt_get_nidx(evt_handle c, uint32_t *out) {
     HIPCHK(hipMemcpyAsync(out, c->nidx, sizeof(uint32_t) * (size_t)c->N, hipMemcpyDefault, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     return EVT_OK;
+    });
 }
 extern "C" int evt_get_hist(evt_handle c, double *out) {
+    return guarded([&]() -> int {
     CTXCHK_STEP(c);
     ARGCHK(out, "out is NULL");
     if (c->n_js_last <= 0) {
@@ -1111,22 +1195,27 @@ extern "C" int evt_get_hist(evt_handle c, double *out) {
         return EVT_ERR_HIP;
     }
     return r;
+    });
 }
 extern "C" int evt_get_quant(evt_handle c, int32_t *qbits, int32_t *qexp) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(qbits && qexp, "NULL argument");
     int32_t e[EVT_MC_MAX_NK];
-    HIPCHK(hipMemcpyAsync(e, c->qexp, sizeof(int32_t) * EVT_MC_MAX_NK, hipMemcpyDeviceToHost, c->stream));
+    // the tables of the last tree's gradients, also when the next round's have been quantised behind it
+    HIPCHK(hipMemcpyAsync(e, c->n_js_last > 0 ? c->qexp_buf[c->q_tree] : c->qexp, sizeof(int32_t) * EVT_MC_MAX_NK, hipMemcpyDeviceToHost, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     for (int k = 0; k < c->NK; k++) {
         qbits[k] = c->h_qbits[k];
         qexp[k] = e[k];
     }
     return EVT_OK;
+    });
 }
 
 // ---- evaluation metric ------------------------------------------------------------------------
 extern "C" int evt_eval_metric(evt_handle c, int32_t metric, double *value_out) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(value_out, "value_out is NULL");
     ARGCHK(metric >= 0 && metric <= EVT_METRIC_LOGISTIC_MLE, "unknown metric");
@@ -1150,6 +1239,7 @@ extern "C" int evt_eval_metric(evt_handle c, int32_t metric, double *value_out) 
     c->pt_busy = false;
     memcpy(value_out, c->h_stage, sizeof(double));
     return EVT_OK;
+    });
 }
 
 // ---- inference ------------------------------------------------------------------------------
@@ -1237,12 +1327,16 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
     int ndev = 0;
     int r = evt_device_count(&ndev);
     if (r != EVT_OK) return r;
+    // the offsets are checked before anything is sized by them
+    ARGCHK(tree_off[0] == 0, "tree_off must start at 0");
+    for (int t = 0; t < ntrees; t++)
+        ARGCHK(tree_off[t + 1] > tree_off[t] && tree_off[t + 1] - tree_off[t] <= ((int64_t)1 << 24), "tree_off must be strictly ascending, at most 2^24 nodes per tree");
     const int64_t total = tree_off[ntrees];
+    ARGCHK(total <= ((int64_t)1 << 31), "the model holds more than 2^31 nodes");
     std::vector<uint32_t> nodes((size_t)total, 0u), one;
     for (int t = 0; t < ntrees; t++) {
         const int64_t o = tree_off[t];
         const int64_t nn = tree_off[t + 1] - o;
-        ARGCHK(nn >= 1 && o >= 0, "tree_off must be ascending");
         r = pack_tree((int32_t)nn, feat + o, cond_bin + o, split + o, nfeats, feattypes, one);
         if (r != EVT_OK) return r;
         memcpy(nodes.data() + o, one.data(), sizeof(uint32_t) * nn);
@@ -1347,32 +1441,41 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
 extern "C" int evt_predict(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, const uint8_t *feattypes, int32_t loss, int32_t K, int32_t ntrees,
                            const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const float *pred, const uint8_t *split,
                            int32_t apply_link, float *out) {
+    return guarded([&]() -> int {
     return predict_common(nobs, nfeats, x_bin, feattypes, loss, K, ntrees, tree_off, feat, cond_bin, pred, split, apply_link, out, nullptr);
+    });
 }
 
 extern "C" int evt_predict_f64(int64_t nobs, int32_t nfeats, const double *x_colmajor, const double *edges, const int32_t *edge_off,
                                const uint8_t *feattypes, int32_t loss, int32_t K, int32_t ntrees, const int64_t *tree_off, const int64_t *feat,
                                const uint8_t *cond_bin, const float *pred, const uint8_t *split, int32_t apply_link, float *out) {
+    return guarded([&]() -> int {
     ARGCHK(x_colmajor, "x is NULL");
     return predict_common(nobs, nfeats, nullptr, feattypes, loss, K, ntrees, tree_off, feat, cond_bin, pred, split, apply_link, out, nullptr,
                           x_colmajor, edges, edge_off);
+    });
 }
 
 extern "C" int evt_predict_leaf_idx(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, const uint8_t *feattypes, int32_t ntrees,
                                     const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const uint8_t *split, uint32_t *out) {
+    return guarded([&]() -> int {
     ARGCHK(out, "out is NULL");
     return predict_common(nobs, nfeats, x_bin, feattypes, 0, 1, ntrees, tree_off, feat, cond_bin, nullptr, split, 0, nullptr, out);
+    });
 }
 
 // ---- measurement ----------------------------------------------------------------------------
 extern "C" int evt_set_profiling(evt_handle c, int32_t on) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     HIPCHK(hipStreamSynchronize(c->stream));
     prof_collect(c, nullptr);
     c->profiling = (on == 1) ? 0x7fffffff : on; // 1: every class; otherwise a bit mask of EVT_K_* classes
     return EVT_OK;
+    });
 }
 extern "C" int evt_get_profile(evt_handle c, int64_t *launches, double *ms, int64_t *units) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(launches && ms && units, "NULL argument");
     HIPCHK(hipStreamSynchronize(c->stream));
@@ -1383,8 +1486,10 @@ extern "C" int evt_get_profile(evt_handle c, int64_t *launches, double *ms, int6
         units[k] = c->prof_units[k];
     }
     return EVT_OK;
+    });
 }
 extern "C" int evt_reset_profile(evt_handle c) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     HIPCHK(hipStreamSynchronize(c->stream));
     prof_collect(c, nullptr);
@@ -1392,8 +1497,10 @@ extern "C" int evt_reset_profile(evt_handle c) {
     memset(c->prof_ms, 0, sizeof(c->prof_ms));
     memset(c->prof_units, 0, sizeof(c->prof_units));
     return EVT_OK;
+    });
 }
 extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
+    return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(name, "name is NULL");
     if (strcmp(name, "hist_blocks") == 0) {
@@ -1423,12 +1530,15 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
         return EVT_ERR_ARG;
     }
     return EVT_OK;
+    });
 }
 extern "C" int evt_synchronize(evt_handle c) {
+    return guarded([&]() -> int {
     ARGCHK(c != nullptr, "handle is NULL");
     HIPCHK(hipSetDevice(c->device));
     HIPCHK(hipStreamSynchronize(c->stream));
     return EVT_OK;
+    });
 }
 
 __global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t n) {
@@ -1445,6 +1555,7 @@ __global__ __launch_bounds__(256) void k_read16(const uint4 *__restrict__ src, i
 }
 
 extern "C" int evt_read_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out) {
+    return guarded([&]() -> int {
     ARGCHK(gbps_out && nbytes >= 4096 && iters >= 1, "invalid arguments");
     int ndev = 0;
     int r = evt_device_count(&ndev);
@@ -1477,9 +1588,11 @@ extern "C" int evt_read_bandwidth(int64_t nbytes, int32_t iters, double *gbps_ou
     }
     *gbps_out = (double)(n * 16) * iters / ((double)ms * 1e-3) / 1e9;
     return EVT_OK;
+    });
 }
 
 extern "C" int evt_copy_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out) {
+    return guarded([&]() -> int {
     ARGCHK(gbps_out && nbytes >= 4096 && iters >= 1, "invalid arguments");
     int ndev = 0;
     int r = evt_device_count(&ndev);
@@ -1511,4 +1624,5 @@ extern "C" int evt_copy_bandwidth(int64_t nbytes, int32_t iters, double *gbps_ou
     }
     *gbps_out = 2.0 * (double)(n * 16) * iters / ((double)ms * 1e-3) / 1e9;
     return EVT_OK;
+    });
 }

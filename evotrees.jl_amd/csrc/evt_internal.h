@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include <string>
 #include <vector>
 
@@ -110,9 +111,15 @@ struct evt_ctx {
     uint8_t *feattypes;
     int32_t *mono;
     uint32_t *absmax;  // [EVT_MC_MAX_NK] float bits
-    int32_t *qexp;     // [EVT_MC_MAX_NK]
+    int32_t *qexp;     // [EVT_MC_MAX_NK]; points into qexp_buf: the tables of the gradients quantised last
     int32_t *qbits;    // [EVT_MC_MAX_NK]
     double *qscale;    // [2 * EVT_MC_MAX_NK]: decode scale per global channel, then encode multiplier per gradient row
+    // The fixed-point tables exist twice: a gradient update writes the set the last grown tree does NOT use, so that the
+    // tree's histogram can still be decoded (evt_get_hist, evt_get_quant) after the next round's gradients were
+    // quantised behind it.  q_cur: set of the gradients quantised last; q_tree: set the last tree was grown on.
+    int32_t *qexp_buf[2];
+    double *qscale_buf[2];
+    int q_cur, q_tree;
     double *metric_partial; // [2 * EVT_METRIC_BLOCKS + 1] evaluation-metric partial sums, result last
     int64_t *stats;    // [D+1] rows built per level
     int32_t *errflag;  // device-side validation flag
@@ -167,6 +174,22 @@ struct evt_ctx {
     int64_t prof_launches[EVT_K_COUNT];
     double prof_ms[EVT_K_COUNT];
     int64_t prof_units[EVT_K_COUNT];
+};
+
+// A set-up step that has to run once per device (hipFuncSetAttribute applies to the current device), from whichever
+// thread gets there first.  The step itself is idempotent, so two threads that both find it pending may both run it;
+// the flag is an atomic bit per device.
+struct EvtDevOnce {
+    std::atomic<uint64_t> done{0};
+    static int current() {
+        int d = -1;
+        if (hipGetDevice(&d) != hipSuccess) d = -1;
+        return d;
+    }
+    bool pending(int device) const { return device < 0 || device >= 64 || !((done.load(std::memory_order_acquire) >> device) & 1ull); }
+    void mark(int device) {
+        if (device >= 0 && device < 64) done.fetch_or(1ull << device, std::memory_order_release);
+    }
 };
 
 // ---- error plumbing ---------------------------------------------------------------------

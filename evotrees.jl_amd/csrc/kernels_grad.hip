@@ -368,6 +368,21 @@ int launch_apply_pending(evt_ctx *c) {
     return EVT_OK;
 }
 
+// Unit weights: the row count stands for the weight in every histogram, so a gradient matrix handed in from outside
+// must carry ones in its weight row.  Flags the first kind of violation it sees.
+__global__ __launch_bounds__(256) void k_check_unit_weight(const float *__restrict__ grad, int64_t N, int NK, int32_t *errflag) {
+    bool bad = false;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) bad |= grad[(size_t)NK * i + NK - 1] != 1.0f;
+    if (__ballot(bad) != 0ull && (threadIdx.x & 63) == 0) *errflag = 1;
+}
+int launch_check_unit_weight(evt_ctx *c) {
+    int64_t nb = (c->N + 255) / 256;
+    if (nb > 4096) nb = 4096;
+    hipLaunchKernelGGL(k_check_unit_weight, dim3((unsigned)nb), dim3(256), 0, c->stream, c->grad, c->N, c->NK, c->errflag);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
 // absmax over rows [k0, k1) of the current gradient matrix
 int launch_absmax_rows(evt_ctx *c, int k0, int k1) {
     {
@@ -382,6 +397,10 @@ int launch_absmax_rows(evt_ctx *c, int k0, int k1) {
 }
 
 int launch_quantize(evt_ctx *c) {
+    // write the set of tables the last grown tree does not use: its histogram stays decodable
+    c->q_cur = c->q_tree ^ 1;
+    c->qexp = c->qexp_buf[c->q_cur];
+    c->qscale = c->qscale_buf[c->q_cur];
     double *qmul = c->qscale + EVT_MC_MAX_NK; // decode scales per global channel first, then encode multipliers per gradient row
     hipLaunchKernelGGL(k_quant_setup, dim3(1), dim3(64), 0, c->stream, c->absmax, c->qbits, c->qexp, qmul, c->qscale, c->NK, c->NAg,
                        c->loss, c->unit_w ? 1 : 0);

@@ -546,11 +546,11 @@ static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads
     // features outside the sample are simply not flushed
     const bool full = 2 * c->n_js_last >= c->F;
     if (lds > 64 * 1024) { // one block per CU may take most of its 160 KB
-        static bool attr_set = false;
-        if (!attr_set) {
+        static EvtDevOnce once;
+        if (once.pending(c->device)) {
             HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, true, PB, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
             HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, false, PB, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-            attr_set = true;
+            once.mark(c->device);
         }
     }
     // c->launch_e0 / launch_e1 (when profiling): the kernel's own dispatch records them
@@ -575,10 +575,10 @@ static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads
 
 template <int NA, bool PACK>
 static int launch_hist_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
-    static bool attr_set = false;
-    if (!attr_set && lds > 64 * 1024) {
+    static EvtDevOnce once;
+    if (lds > 64 * 1024 && once.pending(c->device)) {
         HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build<NA, PACK>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_set = true;
+        once.mark(c->device);
     }
     hipExtLaunchKernelGGL((k_hist_build<NA, PACK>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
     HIPCHK(hipGetLastError());
@@ -716,7 +716,7 @@ __global__ __launch_bounds__(256) void k_hist_export(const long long *__restrict
 
 int launch_hist_export(evt_ctx *c, double *out_dev) {
     hipLaunchKernelGGL(k_hist_export, dim3((unsigned)c->nnodes), dim3(256), 0, c->stream, c->hist, c->js, c->n_js_last, c->F, c->B, c->NK,
-                       c->NAg, c->loss, c->qscale, c->status, c->nnodes, 1 << (c->D - 1), out_dev);
+                       c->NAg, c->loss, c->qscale_buf[c->q_tree], c->status, c->nnodes, 1 << (c->D - 1), out_dev);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

@@ -286,11 +286,12 @@ __global__ __launch_bounds__(256) void k_leaf_idx_model(const uint32_t *__restri
 template <int RB, int NT, int PRE, bool ALLNUM>
 static int launch_model_lds(hipStream_t s, const uint32_t *cnodes, const float *cleaf, const void *meta, int ntrees, const uint8_t *xcm, int64_t N,
                             int F, int max_int, int K, int loss, int apply_link, float *out) {
-    static bool attr_set = false;
-    if (!attr_set) {
+    static EvtDevOnce once;
+    const int dev = EvtDevOnce::current();
+    if (once.pending(dev)) {
         HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_predict_model_lds<4, RB, NT, PRE, ALLNUM>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_set = true;
+        once.mark(dev);
     }
     const int S4 = (F + 3) >> 2;
     const size_t lds = (size_t)RB * S4 * 4 + 8 * (size_t)NT * max_int;

@@ -107,6 +107,49 @@ def test_full_size_rounds_bit_exact_against_oracle(evt):
     o.close()
 
 
+@pytest.mark.parametrize("N,F,D,R", [(100_000, 10, 6, 3), (10_000_000, 100, 11, 1)])
+def test_reference_arithmetic_on_pure_noise_target(evt, N, F, D, R):
+    """The benchmark workloads' own target, y ~ U(0,1) independent of x (gains are tiny and close), against the
+    oracle's Float64 REFERENCE arithmetic (mode 0: Float32 gradients added into Float64 bins in row order,
+    src/fit-utils.jl:388, src/init.jl:204) at full size, teacher forced: every split (feature, bin), the split flags and
+    the node of every row must be equal; gains, weights and leaf values within 1e-5.  A node that differs is examined
+    exactly, from the device's integer histogram: only candidates that tie in real arithmetic may differ."""
+    from exact_tie import is_exact_tie
+    from oracle import oracle as orc
+    from test_gpu_parity import assert_tree_close, setup_pair
+    B = 64
+    rng = np.random.default_rng(123)
+    print("generating", N, "x", F, flush=True)
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    y = rng.random(N, dtype=np.float32)
+    mu = np.array([y.mean()], np.float32)
+    h, o, op, gp, pred0, grad0 = setup_pair(evt, "mse", x_bin, y, None, mu, B, D, eta=0.1)
+    p_orc = pred0.copy()
+    grad = grad0.copy()
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    rows = np.arange(N, dtype=np.uint32)
+    for r in range(R):
+        print("round", r + 1, flush=True)
+        orc.update_grads(op, p_orc, y, grad)
+        h.set_grads(grad)
+        t_gpu = h.grow_tree(js, gp)
+        nidx_gpu = h.get_nidx()
+        t_ref, nidx_ref = o.grow_tree(grad, rows, js, mode=0)
+        print("split nodes:", int(t_gpu.split.sum()), "smallest gain of a split:", float(t_gpu.gain[t_gpu.split.astype(bool)].min()), flush=True)
+        same = np.array_equal(t_gpu.feat, t_ref.feat) and np.array_equal(t_gpu.cond_bin, t_ref.cond_bin) and np.array_equal(t_gpu.split, t_ref.split)
+        if not same:
+            tie, text = is_exact_tie(h.get_hist(), t_gpu, t_ref, None, 1, op.lambda_, op.L2)
+            print("structure differs from the Float64 oracle:", text, "-> exact tie" if tie else "-> NOT a tie", flush=True)
+        assert same
+        assert int(t_gpu.split.sum()) > (500 if D == 11 else 20)
+        assert_tree_close(t_gpu, t_ref)
+        assert np.array_equal(nidx_gpu, nidx_ref)
+        o.predict_tree(t_ref, p_orc)
+        np.testing.assert_allclose(h.get_pred(), p_orc, rtol=1e-5, atol=1e-7)
+    h.close()
+    o.close()
+
+
 @pytest.mark.parametrize("N,F", [(22_000_000, 100), (150_000_000, 8)])
 def test_offsets_past_two_to_the_31(evt, N, F):
     """nobs x nfeats above 2^31 bytes (and nobs above 2^27 rows): every kernel's offsets are 64-bit.  The tree's node

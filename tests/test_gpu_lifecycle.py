@@ -283,6 +283,41 @@ def test_gradients_queued_ahead_change_nothing(evt, loss, tt):
             assert_tree_bits(a, b)
 
 
+@pytest.mark.parametrize("bagging", [1, 2])
+def test_gradients_queued_ahead_with_bagging_and_read_back(evt, bagging):
+    """A round of bagging_size trees is grown on ONE set of gradients (src/fit.jl:9-11): "grads_ahead" must not refresh
+    them between the trees of a round.  And what describes the tree just grown - its histogram and its fixed-point
+    tables - reads the same right after evt_grow_tree whether or not the next round's gradients were queued behind it."""
+    N, F, B, D = 30000, 9, 32, 5
+    x_bin, y, w, mu = make_data(79, N, F, B, "logloss", weights=True)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    gp = evt.make_params(eta=0.3, bagging_size=bagging)
+    rng = np.random.default_rng(8)
+    masks = [rng.integers(0, 256, N, dtype=np.uint8) for _ in range(8)]
+    out = []
+    for ahead in (1, 0):
+        h = evt.Handle(N, F, B, 1, D, "logloss")
+        h.set_option("grads_ahead", ahead)
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        rec = []
+        for r in range(3):
+            h.update_grads()
+            for b in range(bagging):
+                t = h.grow_tree(js, gp, mask=masks[2 * r + b], cond=200)
+                qb, qe = h.get_quant()
+                rec += [t, h.get_hist(), qb, qe]
+        rec.append(h.get_pred())
+        h.close()
+        out.append(rec)
+    for a, b in zip(*out):
+        if isinstance(a, np.ndarray):
+            assert a.tobytes() == b.tobytes()
+        else:
+            assert_tree_bits(a, b)
+    assert out[0][0].split.sum() >= 3
+
+
 def test_two_handles_on_two_threads(evt):
     """Different handles may be driven from different threads at once (each has its own stream; the error message is
     per thread): two threads boost different problems concurrently and get, bit for bit, what a single thread gets."""

@@ -534,7 +534,30 @@ def test_error_paths(evt):
     # the handle is still usable afterwards
     t = h.grow_tree(np.array([1, 2, 3], np.uint32), gp)
     assert t.split[0] == 1
+    # gradients handed in from outside: with no weights given to evt_set_target the weight row must be all ones
+    g = h.get_grads()
+    g[17, 2] = 0.5
+    with pytest.raises(evt.EvtError) as e:
+        h.set_grads(g)
+    assert e.value.code == evt._lib.EVT_ERR_ARG and "weight row" in str(e.value)
+    with pytest.raises(evt.EvtError) as e:  # ... and leaves no gradients behind
+        h.grow_tree(np.array([1, 2, 3], np.uint32), gp)
+    assert e.value.code == evt._lib.EVT_ERR_STATE
+    g[17, 2] = 1.0
+    h.set_grads(g)
+    assert h.grow_tree(np.array([1, 2, 3], np.uint32), gp).split[0] == 1
     h.close()
+    # model offsets are checked before anything is sized by them: no exception crosses the C ABI
+    import ctypes as C
+    L = evt._lib.load()
+    P = evt._lib.ptr
+    feat = np.zeros(3, np.int64); cb = np.zeros(3, np.uint8); sp = np.zeros(3, np.uint8); pr = np.zeros(3, np.float32)
+    out = np.zeros(N, np.float32)
+    for off in ([0, -5], [2, 3], [0, 0], [0, 1 << 40], [-(1 << 62), 3]):
+        off = np.array(off, np.int64)
+        rc = L.evt_predict(N, F, P(x_bin), None, 0, 1, 1, P(off), P(feat), P(cb), P(pr), P(sp), 0, P(out))
+        assert rc == evt._lib.EVT_ERR_ARG, (off, rc)
+        assert b"tree_off" in L.evt_last_error() or b"2^31" in L.evt_last_error()
     for args in [(0, 3, 8, 1, 3, "mse"), (10, 0, 8, 1, 3, "mse"), (10, 3, 1, 1, 3, "mse"), (10, 3, 256, 1, 3, "mse"),
                  (10, 3, 8, 17, 3, "mse"), (10, 3, 8, 3, 3, "gaussian_mle"), (10, 3, 8, 1, 3, "mlogloss"), (10, 3, 8, 1, 0, "mse"),
                  (10, 3, 8, 1, 17, "mse")]:

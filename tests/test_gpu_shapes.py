@@ -6,10 +6,12 @@ import numpy as np
 import pytest
 
 from oracle import oracle as orc
+from exact_tie import is_exact_tie
 from test_gpu_parity import assert_tree_bits, make_data, setup_pair
 
 pytestmark = pytest.mark.gpu
 
+TIES = []  # (case, text) of every case whose structure differs from the Float64 oracle by an exact tie
 LOSSES = ["mse", "logloss", "gaussian_mle", "poisson", "gamma", "tweedie", "mlogloss", "logistic_mle"]
 
 
@@ -88,14 +90,26 @@ def test_shape_sweep(evt, loss, weights, N, F, B, D, tt, n_js, rowsample, K, cat
     assert_tree_bits(h.grow_tree(js, evt.make_params(eta=op.eta, L2=op.L2, lambda_=op.lambda_, gamma=op.gamma, min_weight=op.min_weight,
                                                      update_pred=False), mask=mask, cond=cond), t_fx)
     assert np.array_equal(h.get_pred(), pr)  # update_pred = 0 leaves the prediction alone
-    # Float64 reference arithmetic: same structure unless two candidates tie within rounding noise
+    # Float64 reference arithmetic: same structure.  The one difference a case may show is a tie in REAL arithmetic
+    # between the two chosen candidates (the device resolves it by position, the reference by rounding noise); it is
+    # established exactly, from the device's integer histogram, and counted.
     t_ref, _ = o.grow_tree(grad, rows, js, mode=0)
     same = np.array_equal(t_gpu.feat, t_ref.feat) and np.array_equal(t_gpu.cond_bin, t_ref.cond_bin)
     if same:
         np.testing.assert_allclose(t_gpu.pred, t_ref.pred, rtol=1e-5, atol=1e-7)
     else:
-        # a different choice is only acceptable between candidates whose gains agree to Float64 rounding
-        n0 = int(np.flatnonzero((t_gpu.feat != t_ref.feat) | (t_gpu.cond_bin != t_ref.cond_bin))[0])
-        assert abs(float(t_gpu.gain[n0]) - float(t_ref.gain[n0])) <= 1e-6 * abs(float(t_ref.gain[n0])) + 1e-12, (n0, t_gpu.gain[n0], t_ref.gain[n0])
+        h.set_option("hist_variant", 0)
+        h.grow_tree(js, gp, mask=mask, cond=cond)
+        tie, text = is_exact_tie(h.get_hist(), t_gpu, t_ref, feattypes, op.K, op.lambda_, op.L2, oblivious=(tt == "oblivious"))
+        TIES.append((seed, text))
+        print("structure differs from the Float64 oracle:", text, "-> exact tie" if tie else "-> NOT a tie", flush=True)
+        assert tie, text
     h.close()
     o.close()
+
+
+def test_shape_sweep_tie_report():
+    """Says how many cases of the sweep differed from the Float64 oracle (each one asserted above to be an exact tie)."""
+    print("cases resolved as exact ties:", len(TIES), flush=True)
+    for seed, text in TIES:
+        print("  case", seed, text, flush=True)
