@@ -25,7 +25,7 @@ EXPORTS = [
     "evt_tree_open", "evt_hist_build", "evt_split_scan", "evt_update_nodes_idx", "evt_tree_close", "evt_peek_tree",
     "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
     "evt_predict", "evt_predict_f64", "evt_predict_leaf_idx", "evt_eval_metric", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
-    "evt_set_option", "evt_synchronize", "evt_copy_bandwidth", "evt_read_bandwidth",
+    "evt_set_option", "evt_synchronize", "evt_copy_bandwidth", "evt_read_bandwidth", "evt_predict_static",
 ]
 
 
@@ -99,6 +99,7 @@ def load():
         "evt_synchronize": [vp],
         "evt_copy_bandwidth": [i64, i32, vp],
         "evt_read_bandwidth": [i64, i32, vp],
+        "evt_predict_static": [vp, i64, i32, vp, vp, i32, i32, i32, i64, vp, vp, vp, vp, vp, i32, vp, vp],
     }
     for name, args in sigs.items():
         f = getattr(L, name)

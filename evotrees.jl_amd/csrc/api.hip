@@ -12,7 +12,7 @@ int launch_absmax_rows(evt_ctx *c, int k0, int k1);
 int launch_check_unit_weight(evt_ctx *c);
 int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, const float *leaf_pred_dev);
 int launch_predict_model(hipStream_t s, const uint32_t *nodes, const float *leaf_pred, const int64_t *off, int ntrees, const uint8_t *xcm, int64_t N,
-                         int K, int loss, int apply_link, float *out);
+                         int K, int loss, int apply_link, float *out, const int32_t *skip_flag);
 int predict_lds_shape(int F, int max_int, int K, int hint);
 int launch_predict_model_lds(hipStream_t s, const uint32_t *cnodes, const float *cleaf, const void *meta, int ntrees, const uint8_t *xcm, int64_t N,
                              int F, int max_int, int K, int loss, int apply_link, int all_numeric, int shape, float *out);
@@ -1421,7 +1421,7 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
     if (e == hipSuccess && r == EVT_OK) {
         if (leaf_out) r = launch_leaf_idx_model(s, d_nodes, d_off, ntrees, d_x, nobs, d_leaf);
         else if (use_lds) r = launch_predict_model_lds(s, d_cn, d_cl, d_cm, ntrees, d_x, nobs, nfeats, max_int, K, loss, apply_link, all_numeric ? 1 : 0, shape, d_out);
-        else r = launch_predict_model(s, d_nodes, d_lp, d_off, ntrees, d_x, nobs, K, loss, apply_link, d_out);
+        else r = launch_predict_model(s, d_nodes, d_lp, d_off, ntrees, d_x, nobs, K, loss, apply_link, d_out, nullptr);
         e = hipDeviceSynchronize();
     }
     if (e == hipSuccess && r == EVT_OK) {

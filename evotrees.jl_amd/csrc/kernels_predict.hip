@@ -111,9 +111,10 @@ __device__ __forceinline__ void add_tree(float *acc, const float *lp, int K, int
 template <int KMAX>
 __global__ __launch_bounds__(256) void k_predict_model(const uint32_t *__restrict__ nodes, const float *__restrict__ leaf_pred,
                                                       const int64_t *__restrict__ off, int ntrees, const uint8_t *__restrict__ xcm, int64_t N,
-                                                      int K, int loss, int link, float *out) {
+                                                      int K, int loss, int link, float *out, const int32_t *__restrict__ skip_flag) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= N) return;
+    if (skip_flag && *skip_flag) return; // the model was packed on the device and found invalid: nothing is walked
     float acc[KMAX];
 #pragma unroll
     for (int k = 0; k < KMAX; k++) acc[k] = 0.0f;
@@ -332,13 +333,13 @@ int launch_predict_model_lds(hipStream_t s, const uint32_t *cnodes, const float 
 }
 
 int launch_predict_model(hipStream_t s, const uint32_t *nodes, const float *leaf_pred, const int64_t *off, int ntrees, const uint8_t *xcm, int64_t N,
-                         int K, int loss, int apply_link, float *out) {
+                         int K, int loss, int apply_link, float *out, const int32_t *skip_flag) {
     if (K <= 4)
         hipLaunchKernelGGL(k_predict_model<4>, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, nodes, leaf_pred, off, ntrees, xcm, N, K, loss,
-                           apply_link, out);
+                           apply_link, out, skip_flag);
     else
         hipLaunchKernelGGL(k_predict_model<EVT_MAX_K>, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, nodes, leaf_pred, off, ntrees, xcm, N, K,
-                           loss, apply_link, out);
+                           loss, apply_link, out, skip_flag);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

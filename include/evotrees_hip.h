@@ -262,6 +262,24 @@ int evt_predict_leaf_idx(int64_t nobs, int32_t nfeats, const uint8_t *x_bin_colm
                          int32_t ntrees, const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin,
                          const uint8_t *split, uint32_t *out);
 
+/* No counterpart in the reference: evt_predict for callers that cannot allocate - code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  Every pointer is device memory: x_bin (nobs x nfeats column-major),
+ * the model in the reference's arrays, concatenated as for evt_predict (tree_off has ntrees + 1 entries and ends at
+ * total_nodes), feattypes (or NULL: all numeric), out (K x nobs).  Three kernels are queued on `stream` (a hipStream_t;
+ * NULL = the default stream) and the call returns without waiting: it allocates nothing, copies nothing and
+ * synchronises nothing.  The packed node words evt_predict allocates per call live in a file-scope device array of
+ * EVT_STATIC_MAX_NODES words (4 MiB + a 256-byte header, held by each GPU the call has run on until the process ends);
+ * a model with more nodes is refused with EVT_ERR_ARG.  The model is checked on the device by the rules evt_predict
+ * applies on the host; a model that breaks them leaves `out` unwritten and EVT_ERR_ARG in *status (a device int32,
+ * EVT_OK otherwise; may be NULL).  Results equal evt_predict's, bit for bit.  The device that is current on the calling
+ * thread must be the one the pointers live on.  All calls on one GPU share the one array: calls that overlap on a GPU
+ * (two streams, two threads) race, and a call must have finished before the next one is queued on another stream. */
+#define EVT_STATIC_MAX_NODES (1 << 20)
+int evt_predict_static(void *stream, int64_t nobs, int32_t nfeats, const uint8_t *x_bin_dev, const uint8_t *feattypes_dev,
+                       int32_t loss, int32_t K, int32_t ntrees, int64_t total_nodes, const int64_t *tree_off_dev,
+                       const int64_t *feat_dev, const uint8_t *cond_bin_dev, const float *pred_dev, const uint8_t *split_dev,
+                       int32_t apply_link, float *out_dev, int32_t *status_dev);
+
 /* ---- measurement ---------------------------------------------------------------------
  * Kernel classes timed with HIP events on the handle's stream when profiling is on. */
 enum {
