@@ -8,7 +8,8 @@ row and column sampling, 200 rounds).
 
 Prints one JSON line.  `value` = seconds per 200 rounds (lower is better), scaled from the K timed
 rounds.  `roofline` = histogram kernel: algorithmic bytes rows_built*(Fs + 4*(2K+1) + 4) over the
-HIP-event time of its launches inside the timed region, against 8 TB/s.  `cpu_baseline` = the CPU
+HIP-event time of its launches inside the timed region, against 8 TB/s.  `workloads` = the other BASELINE
+configurations (a few dozen rounds each), `fit_total_s` = init + 200 rounds of the headline workload.  `cpu_baseline` = the CPU
 oracle (a restatement of the reference's CPU algorithm, OpenMP over node x feature tiles) timed
 on this box's host cores on a few rounds of the same workload.
 """
@@ -110,6 +111,131 @@ def measured_traffic_per_launch(path):
         return None
 
 
+def prepare(evt, cfg, opts=None):
+    """Synthetic data of the configuration, quantile edges, handle creation, upload + device binarize, target.
+    Returns the handle and the seconds spent in each part (data generation apart: it is not part of a fit)."""
+    N, F, B, D, loss = cfg["N"], cfg["F"], cfg["nbins"], cfg["depth"], cfg["loss"]
+    K = 2 if loss == "gaussian_mle" else 1
+    t0 = time.time()
+    x, y, rng = synth(cfg)
+    t1 = time.time()
+    edges = edges_from_sample(x, B, rng)
+    t2 = time.time()
+    h = evt.Handle(N, F, B, K, D, loss, cfg["tree_type"])
+    h.binarize(x, edges)
+    del x
+    mu = bias(loss, y)
+    h.set_target(y, None, mu)
+    for name, v in (opts or {}).items():
+        h.set_option(name, v)
+    t3 = time.time()
+    return h, y, mu, rng, {"generate_s": round(t1 - t0, 2), "edges_s": round(t2 - t1, 2), "upload_binarize_target_s": round(t3 - t2, 2)}
+
+
+class Rounds:
+    """Boosting rounds on a prepared handle, as the host mirror's grow_evotree drives them: gradients, the column sample,
+    the tree in two halves with the next round's mask drawn (and for many rows uploaded) in between."""
+
+    # below a few million rows a round is bound by the host's launches and the second stream's copy costs more than it hides
+    STAGE_MASK_MIN_ROWS = 4_000_000
+
+    def __init__(self, evt, h, cfg, rng):
+        self.evt, self.h, self.cfg, self.rng = evt, h, cfg, rng
+        self.N, self.F = cfg["N"], cfg["F"]
+        self.K = 2 if cfg["loss"] == "gaussian_mle" else 1
+        self.params = evt.make_params(eta=cfg["eta"], min_weight=cfg["min_weight"], update_pred=True)
+        self.cond = int(np.rint(255 * cfg["rowsample"]))
+        self.nfs = int(np.ceil(cfg["colsample"] * self.F))
+        self.L = evt._lib.load()
+        self.tree = evt.Tree(self.K, h.nnodes)
+        self.tree_out = self.tree.as_out()
+        # the host owns the row-sampling RNG (one uniform byte per row, drawn every round): raw 64-bit words viewed as bytes;
+        # numpy's fastest bulk generator: the draw is host work inside the timed region
+        self.mask_rng = np.random.Generator(np.random.SFC64(124))
+        self.staged = False
+        self.nxt = None
+        h.set_option("grads_ahead", 1)  # one tree per round: the next round's gradients are queued behind the tree
+
+    def draw_mask(self):
+        return None if self.cond >= 255 else self.mask_rng.bit_generator.random_raw((self.N + 7) // 8).view(np.uint8)[:self.N]
+
+    def one_round(self):
+        evt, h, L, F = self.evt, self.h, self.L, self.F
+        h.update_grads()
+        js = np.arange(1, F + 1, dtype=np.uint32) if self.nfs >= F else (np.sort(self.rng.choice(F, self.nfs, replace=False)) + 1).astype(np.uint32)
+        if self.staged:
+            evt._lib.check(L.evt_grow_tree_begin_staged(h._h, self.cond, evt._lib.ptr(js), js.shape[0], self.params))
+        else:
+            mask = self.nxt if self.nxt is not None else self.draw_mask()
+            evt._lib.check(L.evt_grow_tree_begin(h._h, evt._lib.ptr(mask), self.cond, evt._lib.ptr(js), js.shape[0], self.params))
+        if self.cond < 255:
+            # the next round's mask is drawn (and, for many rows, uploaded) while the device grows this round's tree
+            self.nxt = self.draw_mask()
+            if self.N >= self.STAGE_MASK_MIN_ROWS:
+                h.stage_mask(self.nxt)
+                self.staged = True
+        evt._lib.check(L.evt_grow_tree_end(h._h, self.tree_out))
+
+    def timed(self, steps, warmup, profile_every=4, no_profile=False):
+        """`warmup` untimed rounds, then `steps` timed ones.  HIP events around the histogram launches only (the kernel
+        the roofline is quoted on), and only in every profile_every-th round: an event costs the stream about 4.5 us on
+        either side of the kernel it times (measured with rocprofv3 --kernel-trace), 90 us per round if every launch
+        carried a pair.  Returns (ms per round, histogram profile, rounds sampled)."""
+        h = self.h
+        for _ in range(warmup):
+            self.one_round()
+        h.synchronize()
+        pe = max(1, profile_every)
+        h.set_profiling(False)
+        h.reset_profile()
+        sampled = 0
+        t1 = time.perf_counter()
+        for step in range(steps):
+            on = (not no_profile) and step % pe == 0
+            if on:
+                h.set_profiling(["hist"])
+                sampled += 1
+            self.one_round()
+            if on:
+                h.set_profiling(False)
+        h.synchronize()
+        t2 = time.perf_counter()
+        return (t2 - t1) * 1e3 / steps, h.get_profile()["hist"], sampled
+
+
+def hist_roofline(cfg, prof_hist, nfs, NK):
+    """Algorithmic bytes of the histogram launches that carried events over their HIP-event time."""
+    if prof_hist["ms"] <= 0:
+        return None, None
+    bytes_per_row = nfs + 4 * NK + 4
+    achieved = prof_hist["units"] * bytes_per_row / (prof_hist["ms"] * 1e-3) / 1e9
+    return achieved, bytes_per_row
+
+
+def side_workload(evt, name, steps, h=None, y=None, mu=None, rng=None):
+    """One of BASELINE.json's other configurations, a few dozen rounds: ms per round, seconds per 200 rounds and the
+    histogram kernel's fraction of the HBM peak.  cfg3s runs on the headline workload's own handle (same matrix)."""
+    cfg = dict(WORKLOADS[name])
+    own = h is None
+    t_init = None
+    if own:
+        h, y, mu, rng, t_init = prepare(evt, cfg)
+    r = Rounds(evt, h, cfg, rng)
+    ms, ph, sampled = r.timed(steps, 3)
+    K = r.K
+    ach, _ = hist_roofline(cfg, ph, r.nfs, 2 * K + 1)
+    out = {"ms_per_step": round(ms, 4), "s_per_200": round(ms * 0.2, 4), "steps": steps,
+           "hist_frac": None if ach is None else round(ach / HBM_PEAK_GBS, 4),
+           "hist_ms_per_round": round(ph["ms"] / max(1, sampled), 4), "rows_built_per_round": ph["units"] // max(1, sampled),
+           "workload": "%s %dx%d nbins=%d max_depth=%d rowsample=%g colsample=%g %s" % (
+               cfg["loss"], cfg["N"], cfg["F"], cfg["nbins"], cfg["depth"], cfg["rowsample"], cfg["colsample"], cfg["tree_type"])}
+    if t_init is not None:
+        out["init_s"] = round(t_init["edges_s"] + t_init["upload_binarize_target_s"], 2)
+    if own:
+        h.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -125,8 +251,10 @@ def main():
     ap.add_argument("--hist-min-rows", type=int, default=0)
     ap.add_argument("--hist-variant", type=int, default=0)
     ap.add_argument("--hist-seg-cost", type=int, default=-1)
+    ap.add_argument("--option", action="append", default=[], help="name=value passed to evt_set_option (sweeps)")
     ap.add_argument("--predict", action="store_true", help="also time model inference on the training rows")
     ap.add_argument("--no-model-predict", action="store_true", help="skip the resident whole-model prediction figure")
+    ap.add_argument("--side-steps", type=int, default=40, help="timed rounds of each of the other BASELINE configurations (0: skip them)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no multi-GPU path is built)" % args.gpus,
@@ -142,83 +270,29 @@ def main():
     K = 2 if loss == "gaussian_mle" else 1
     NK = 2 * K + 1
 
-    t0 = time.time()
-    x, y, rng = synth(cfg)
-    edges = edges_from_sample(x, B, rng)
-    h = evt.Handle(N, F, B, K, D, loss, cfg["tree_type"])
-    h.binarize(x, edges)
-    del x
-    mu = bias(loss, y)
-    h.set_target(y, None, mu)
+    opts = {}
     if args.hist_blocks:
-        h.set_option("hist_blocks", args.hist_blocks)
+        opts["hist_blocks"] = args.hist_blocks
     if args.hist_threads:
-        h.set_option("hist_threads", args.hist_threads)
+        opts["hist_threads"] = args.hist_threads
     if args.hist_min_rows:
-        h.set_option("hist_min_rows", args.hist_min_rows)
+        opts["hist_min_rows"] = args.hist_min_rows
     if args.hist_variant:
-        h.set_option("hist_variant", args.hist_variant)
+        opts["hist_variant"] = args.hist_variant
     if args.hist_seg_cost >= 0:
-        h.set_option("hist_seg_cost", args.hist_seg_cost)
-    t_setup = time.time() - t0
+        opts["hist_seg_cost"] = args.hist_seg_cost
+    for o in args.option:
+        k, v = o.split("=")
+        opts[k] = int(v)
+    h, y, mu, rng, t_init = prepare(evt, cfg, opts)
+    t_setup = t_init["edges_s"] + t_init["upload_binarize_target_s"]
 
-    params = evt.make_params(eta=cfg["eta"], min_weight=cfg["min_weight"], update_pred=True)
-    cond = int(np.rint(255 * cfg["rowsample"]))
-    nfs = int(np.ceil(cfg["colsample"] * F))
-    L = evt._lib.load()
-    tree = evt.Tree(K, h.nnodes)
-    tree_out = tree.as_out()
-
-    # the host owns the row-sampling RNG (one uniform byte per row, drawn every round): raw 64-bit words viewed as bytes
-    mask_rng = np.random.Generator(np.random.SFC64(124))  # numpy's fastest bulk generator: the draw is host work inside the timed region
-
-    def draw_mask():
-        return None if cond >= 255 else mask_rng.bit_generator.random_raw((N + 7) // 8).view(np.uint8)[:N]
-
-    # below a few million rows a round is bound by the host's launches and the second stream's copy costs more than it hides
-    STAGE_MASK_MIN_ROWS = 4_000_000
-    staged = [False]
-    nxt = [None]
-
-    def one_round():
-        h.update_grads()
-        js = np.arange(1, F + 1, dtype=np.uint32) if nfs >= F else (np.sort(rng.choice(F, nfs, replace=False)) + 1).astype(np.uint32)
-        if staged[0]:
-            evt._lib.check(L.evt_grow_tree_begin_staged(h._h, cond, evt._lib.ptr(js), js.shape[0], params))
-        else:
-            mask = nxt[0] if nxt[0] is not None else draw_mask()
-            evt._lib.check(L.evt_grow_tree_begin(h._h, evt._lib.ptr(mask), cond, evt._lib.ptr(js), js.shape[0], params))
-        if cond < 255:
-            # the next round's mask is drawn (and, for many rows, uploaded) while the device grows this round's tree
-            nxt[0] = draw_mask()
-            if N >= STAGE_MASK_MIN_ROWS:
-                h.stage_mask(nxt[0])
-                staged[0] = True
-        evt._lib.check(L.evt_grow_tree_end(h._h, tree_out))
-
-    h.set_option("grads_ahead", 1)  # one tree per round: the next round's gradients are queued behind the tree
-    for _ in range(args.warmup):
-        one_round()
-    h.synchronize()
-    # timed region: HIP events around the histogram launches only (the kernel the roofline is quoted on), and only in
-    # every args.profile_every-th round: an event costs the stream about 4.5 us on either side of the kernel it times
-    # (measured with rocprofv3 --kernel-trace), 90 us per round if every launch carried a pair
+    R = Rounds(evt, h, cfg, rng)
+    cond, nfs, L, tree = R.cond, R.nfs, R.L, R.tree
+    one_round = R.one_round
+    ms_per_step, prof_hist, sampled = R.timed(args.steps, args.warmup, args.profile_every, args.no_profile)
+    prof = {"hist": prof_hist}
     pe = max(1, args.profile_every)
-    h.set_profiling(False)
-    h.reset_profile()
-    sampled = 0
-    t1 = time.perf_counter()
-    for step in range(args.steps):
-        on = (not args.no_profile) and step % pe == 0
-        if on:
-            h.set_profiling(["hist"])
-            sampled += 1
-        one_round()
-        if on:
-            h.set_profiling(False)
-    h.synchronize()
-    t2 = time.perf_counter()
-    prof = h.get_profile()
     # per-class breakdown from a few extra rounds with events around every kernel (outside the timed region)
     extra = 0 if args.no_profile else min(10, args.steps)
     if extra:
@@ -230,9 +304,7 @@ def main():
         prof_all = h.get_profile()
         h.set_profiling(False)
     else:
-        prof_all = prof
-    elapsed = t2 - t1
-    ms_per_step = elapsed * 1e3 / args.steps
+        prof_all = h.get_profile()
     value = ms_per_step * 200 / 1e3
 
     # roofline of the dominant kernel (histogram build)
@@ -269,6 +341,9 @@ def main():
         "config": {"workload": "%s: %s %dx%d nbins=%d max_depth=%d eta=%g rowsample=%g colsample=%g tree_type=%s" % (
             args.workload, loss, N, F, B, D, cfg["eta"], cfg["rowsample"], cfg["colsample"], cfg["tree_type"])},
         "roofline": roofline, "kernels_breakdown_%d_extra_rounds" % extra: kernels, "setup_s": round(t_setup, 2),
+        # what a whole fit of this workload costs: quantile edges on the host, upload of the Float64 matrix, device
+        # binarize, target upload (init, once), then the 200 rounds; the synthetic data's generation is not part of a fit
+        "init_s": t_init, "fit_total_s": round(t_setup + value, 2),
     }
     # rows built per level of the last tree (unit weights: Tree.w holds row counts): the smaller child of every split
     per_level = [int(N if cond >= 255 else tree.w[0])]
@@ -354,6 +429,24 @@ def main():
         evt._lib.predict_model(xb, None, loss, K, m_trees, apply_link=True)
         out["predict"] = {"rows_per_s_incl_transfers": round(N / (time.perf_counter() - tp), 1), "trees": len(m_trees)}
 
+    # BASELINE.json's other configurations, a few dozen rounds each (cfg3s = the headline matrix with the sampling the
+    # reference's published 10M x 100 table was run with, on the same handle)
+    if args.side_steps > 0 and args.workload == "cfg3" and not args.rows:
+        side = {}
+        try:
+            side["cfg3s"] = side_workload(evt, "cfg3s", args.side_steps, h, y, mu, rng)
+        except Exception as e:  # measurement aid only
+            side["cfg3s"] = {"error": str(e)}
+        out["workloads"] = side
+        if "s_per_200" in side["cfg3s"]:
+            # context only: other hardware, Float32 inputs, eta 0.05, and the reference's figure includes a per-round
+            # evaluation pass over the training set (benchmarks/regressor.jl:72-80)
+            out["published_reference_context"] = {
+                "workload": "mse 10Mx100 depth 11 rowsample=colsample=0.5, 200 rounds, init included",
+                "this_fit_total_s": round(t_setup + side["cfg3s"]["s_per_200"], 2),
+                "reference_cpu_s": 192.58, "reference_cpu_hw": "Ryzen 5900X, 12 threads (README.md:69)",
+                "reference_gpu_s": 37.25, "reference_gpu_hw": "RTX A4000, KernelAbstractions/CUDA path (README.md:86)"}
+
     if args.cpu_rounds > 0:
         from oracle import oracle as orc
         xb = h.get_xbin()
@@ -378,6 +471,12 @@ def main():
         out["speedup_vs_cpu_baseline"] = round(cpu_s * 200 / value, 1)
         o.close()
     h.close()
+    if "workloads" in out:
+        for name in ("cfg1", "cfg2", "cfg4", "cfg5", "cfg5o"):
+            try:
+                out["workloads"][name] = side_workload(evt, name, args.side_steps)
+            except Exception as e:  # measurement aid only
+                out["workloads"][name] = {"error": str(e)}
     print(json.dumps(out))
 
 

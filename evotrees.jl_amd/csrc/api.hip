@@ -175,7 +175,7 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp_buf[0], c->qexp_buf[1], c->qbits,
-                    c->qscale_buf[0], c->qscale_buf[1], c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id, c->pt_nodes, c->pt_pred, c->mask_next};
+                    c->qscale_buf[0], c->qscale_buf[1], c->planes, c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id, c->pt_nodes, c->pt_pred, c->mask_next};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -238,6 +238,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->LPR = c->RS / 16;
     c->unit_w = true;
     c->have_xbin = c->have_target = c->have_grads = false;
+    c->planes = nullptr; c->plane_words = 0; c->planes_ready = false; c->use_planes = 1;
     c->xcm = nullptr; c->xrm = nullptr; c->y = nullptr; c->pred = nullptr; c->grad = nullptr; c->gq = nullptr;
     c->is_a = c->is_b = nullptr; c->nidx = nullptr; c->mask = nullptr; c->flagw = nullptr; c->chunk_nleft = nullptr; c->chunk_lpre = nullptr;
     c->hist = nullptr; c->seg_start = c->seg_len = nullptr; c->status = nullptr; c->node_sum = nullptr;
@@ -450,6 +451,7 @@ extern "C" int evt_set_xbin(evt_handle c, const uint8_t *x_bin_colmajor) {
     CTXCHK(c);
     ARGCHK(x_bin_colmajor, "x_bin is NULL");
     c->have_xbin = false;
+    c->planes_ready = false;
     HIPCHK(hipMemcpyAsync(c->xcm, x_bin_colmajor, (size_t)c->N * c->F, hipMemcpyDefault, c->stream));
     int r = launch_transpose_validate(c);
     if (r != EVT_OK) return r;
@@ -465,6 +467,7 @@ extern "C" int evt_binarize_f64(evt_handle c, const double *x_colmajor, const do
     CTXCHK(c);
     ARGCHK(x_colmajor && edges && edge_off, "NULL argument");
     c->have_xbin = false;
+    c->planes_ready = false;
     hipPointerAttribute_t attr;
     bool on_dev = (hipPointerGetAttributes(&attr, x_colmajor) == hipSuccess) && attr.type == hipMemoryTypeDevice;
     (void)hipGetLastError();
@@ -601,6 +604,32 @@ extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, cons
     });
 }
 
+// Threshold bit planes for the partition, built before the first tree grown on the current x_bin.  They cost
+// F * (B - 1) * N / 8 bytes: taken when that is at most 16 GiB and a third of the memory still free, skipped otherwise
+// (the partition then gathers bin bytes).  A failed allocation is not an error.
+static int ensure_planes(evt_ctx *c) {
+    if (c->planes_ready || c->use_planes == 0 || c->D < 2) return EVT_OK;
+    if (!c->planes) {
+        if (c->use_planes < 0) return EVT_OK; // tried before, did not fit
+        const int64_t W = (((c->N + 31) / 32) + 31) / 32 * 32;
+        const size_t bytes = (size_t)c->F * (size_t)(c->B - 1) * (size_t)W * 4;
+        size_t free_b = 0, total_b = 0;
+        if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) free_b = 0;
+        (void)hipGetLastError();
+        if (bytes > ((size_t)16 << 30) || bytes > free_b / 3 || hipMalloc((void **)&c->planes, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            c->planes = nullptr;
+            c->use_planes = -1;
+            return EVT_OK;
+        }
+        c->plane_words = W;
+    }
+    const int r = launch_build_planes(c);
+    if (r != EVT_OK) return r;
+    c->planes_ready = true;
+    return EVT_OK;
+}
+
 static int queue_grads(evt_ctx *c) {
     prof_begin(c, EVT_K_GRAD, 0);
     int r = launch_grads(c);
@@ -724,7 +753,8 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
     const bool fuse_pred = p->update_pred && all_rows && !defer;
     c->write_nidx = rec_nidx || defer;
 
-    int r;
+    int r = ensure_planes(c);
+    if (r != EVT_OK) return r;
     prof_begin(c, EVT_K_OTHER, 0);
     r = launch_apply_pending(c); // an earlier tree's values go in before its node ids are overwritten
     if (r != EVT_OK) return r;
@@ -1361,7 +1391,7 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
     std::vector<ModelTreeHost> cmeta;
     int max_int = 0, shape = 0;
     bool all_numeric = true;
-    bool use_lds = !leaf_out && K <= 4 && ntrees >= 4 && !on_device(pred) && !on_device(feat) && model_max_internal(ntrees, tree_off, max_int);
+    bool use_lds = !leaf_out && ntrees >= 4 && !on_device(pred) && !on_device(feat) && model_max_internal(ntrees, tree_off, max_int);
     if (use_lds) {
         shape = predict_lds_shape(nfeats, max_int, K, predict_shape_hint());
         use_lds = shape > 0;
@@ -1515,6 +1545,10 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
     } else if (strcmp(name, "hist_variant") == 0) {
         ARGCHK(value >= 0 && value <= 2, "hist_variant must be 0 (auto), 1 (generic) or 2 (conflict-free where it applies)");
         c->hist_variant = (int)value;
+    } else if (strcmp(name, "bit_planes") == 0) {
+        ARGCHK(value == 0 || value == 1, "bit_planes must be 0 or 1");
+        c->use_planes = (int)value;
+        if (value == 0) c->planes_ready = false;
     } else if (strcmp(name, "grads_ahead") == 0) {
         c->grads_ahead = value != 0;
         if (!c->grads_ahead) c->grads_ready = false;

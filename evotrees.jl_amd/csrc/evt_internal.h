@@ -82,6 +82,14 @@ struct evt_ctx {
     // data
     uint8_t *xcm;   // F x N bytes (column-major N x F)
     uint8_t *xrm;   // N records of RS bytes
+    // Threshold bit planes: plane (f, b), b = 1..B-1, holds one bit per row, x_bin[row, f] <= b, 32 rows per word.
+    // The partition's decision for a numeric split is one bit of one plane; a node's rows, ascending and 2^depth apart,
+    // find theirs 8 times closer together than their bin bytes (1024 rows per 128-byte line instead of 128).
+    // Built before the first tree when F * (B - 1) * N / 8 bytes fit the budget (HBM capacity traded for bandwidth).
+    uint32_t *planes;
+    int64_t plane_words; // words per plane: ceil(N / 32), rounded up to a multiple of 32
+    bool planes_ready;   // the planes hold the current x_bin
+    int use_planes;      // option "bit_planes": 0 never, 1 when they fit the budget (default)
     float *y;
     float *pred;    // K x N
     float *grad;    // NK x N
@@ -254,6 +262,7 @@ int launch_init_pred(evt_ctx *c, const float *mu_dev, const float *offset_dev);
 // data layout
 int launch_transpose_validate(evt_ctx *c);
 int launch_binarize(evt_ctx *c, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev);
+int launch_build_planes(evt_ctx *c);
 int launch_binarize_cols(hipStream_t s, const double *x_dev, const double *edges_dev, const int32_t *edge_off_dev, uint8_t *xcm, int64_t n,
                          int F, int64_t ldx, int64_t ldo);
 int launch_eval_metric(evt_ctx *c, int metric, double *partial);

@@ -34,6 +34,37 @@ int launch_transpose_validate(evt_ctx *c) {
     return EVT_OK;
 }
 
+// Threshold bit planes of x_bin: word w of plane (f, b) holds, for rows 32 w .. 32 w + 31, the bit x_bin[row, f] <= b.
+// One thread reads its 32 bins once and writes one word of each of the feature's B - 1 planes (consecutive threads,
+// consecutive words).  Rows past the end read as bin 255: their bits are 0 in every plane.
+__global__ __launch_bounds__(256) void k_build_planes(const uint8_t *__restrict__ xcm, uint32_t *__restrict__ planes, int64_t N, int B,
+                                                     int64_t W) {
+    const int64_t w = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int f = blockIdx.y;
+    if (w >= W) return;
+    const uint8_t *col = xcm + (size_t)f * N;
+    uint32_t v[32];
+#pragma unroll
+    for (int k = 0; k < 32; k++) {
+        const int64_t row = 32 * w + k;
+        v[k] = row < N ? (uint32_t)col[row] : 255u;
+    }
+    uint32_t *out = planes + ((size_t)f * (B - 1)) * W + w;
+    for (int b = 1; b < B; b++) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int k = 0; k < 32; k++) word |= (v[k] <= (uint32_t)b ? 1u : 0u) << k;
+        out[(size_t)(b - 1) * W] = word;
+    }
+}
+
+int launch_build_planes(evt_ctx *c) {
+    dim3 grid((unsigned)((c->plane_words + 255) / 256), (unsigned)c->F);
+    hipLaunchKernelGGL(k_build_planes, grid, dim3(256), 0, c->stream, c->xcm, c->planes, c->N, c->B, c->plane_words);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
+}
+
 // Julia's isless on Float64 (the default order of searchsortedfirst): IEEE `<`, except that NaN sorts after everything and
 // -0.0 before 0.0.
 __device__ __forceinline__ bool jl_isless(double a, double b) {

@@ -51,7 +51,27 @@ struct PartArgs {
     const float *t_pred;
     int K, loss, fuse_pred, write_nidx;
     int stream_hint; // the binned matrix does not fit the last-level cache
+    // threshold bit planes (nullptr: none): numeric splits read one bit of plane (feature, cond_bin) per row
+    const uint32_t *planes;
+    int64_t plane_words;
+    int B;
 };
+
+// The word of the decision source that holds row `rid`: its bin byte, or - for a numeric split with bit planes - the
+// plane word whose bit (rid & 31) says x_bin[rid, f] <= cond_bin.
+template <bool NT>
+__device__ __forceinline__ uint32_t load_decision(const uint8_t *__restrict__ col, const uint32_t *__restrict__ plane, uint32_t rid) {
+    if (plane) {
+        const uint32_t *p = plane + (rid >> 5);
+        return NT ? __builtin_nontemporal_load(p) : *p;
+    }
+    const uint8_t *p = col + rid;
+    return (uint32_t)(NT ? __builtin_nontemporal_load(p) : *p);
+}
+__device__ __forceinline__ bool decide_left(uint32_t v, bool use_plane, uint32_t rid, bool numeric, uint32_t cb) {
+    if (use_plane) return (v >> (rid & 31u)) & 1u;
+    return numeric ? (v <= cb) : (v == cb);
+}
 
 // NT: the streaming hint on the gathered bin bytes (a template parameter: a run-time branch between two otherwise
 // identical loads is merged by the compiler, which drops the hint)
@@ -77,6 +97,7 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
         const uint32_t cb = (nd >> 16) & 0xFFu;
         const bool numeric = (nd & EVT_NODE_NUMERIC) != 0;
         const uint8_t *col = A.xcm + (size_t)f * A.N;
+        const uint32_t *plane = (A.planes && numeric && cb >= 1u && cb < (uint32_t)A.B) ? A.planes + ((size_t)f * (A.B - 1) + (cb - 1)) * A.plane_words : nullptr;
         int cnt = 0;
         // all row ids, then all bin bytes, are requested before the first is used; positions past the end read the
         // segment's last row (unconditional loads keep every request of the chunk in flight at once)
@@ -90,12 +111,11 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
         // a binned matrix larger than the last-level cache is gathered with the streaming hint: each byte's line would
         // displace data that is read again (row lists, gradient words) and is rarely hit a second time itself
 #pragma unroll
-        for (int it = 0; it < NI; it++) xbv[it] = NT ? __builtin_nontemporal_load(col + rid[it]) : col[rid[it]];
+        for (int it = 0; it < NI; it++) xbv[it] = load_decision<NT>(col, plane, rid[it]);
 #pragma unroll
         for (int it = 0; it < NI; it++) {
             const int64_t p = p0 + it * 256 + tid;
-            const uint32_t xb = xbv[it];
-            const bool flag = (p < pend) && (numeric ? (xb <= cb) : (xb == cb));
+            const bool flag = (p < pend) && decide_left(xbv[it], plane != nullptr, rid[it], numeric, cb);
             const unsigned long long bal = __ballot(flag);
             if (lane == 0) A.flagw[c * EVT_CHUNK_WORDS + it * 4 + wave] = bal;
             cnt += __popcll(bal);
@@ -206,6 +226,7 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
             numeric = (nd & EVT_NODE_NUMERIC) != 0;
         }
         const uint8_t *col = A.xcm + (size_t)f * A.N;
+        const uint32_t *plane = (A.planes && is_split && numeric && cb >= 1u && cb < (uint32_t)A.B) ? A.planes + ((size_t)f * (A.B - 1) + (cb - 1)) * A.plane_words : nullptr;
         // every request of the chunk goes out before the first result is used: row ids, then bin bytes, then (one
         // output) the predictions; positions past the end read the segment's last row and are not written
         constexpr int NI = EVT_CHUNK / 256;
@@ -217,7 +238,7 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
             rid[it] = A.is_cur[p < pend ? p : pend - 1];
         }
 #pragma unroll
-        for (int it = 0; it < NI; it++) xbv[it] = is_split ? (uint32_t)(NT ? __builtin_nontemporal_load(col + rid[it]) : col[rid[it]]) : 0u;
+        for (int it = 0; it < NI; it++) xbv[it] = is_split ? load_decision<NT>(col, plane, rid[it]) : 0u;
         const bool fast1 = A.fuse_pred && K == 1;
         if (fast1) {
 #pragma unroll
@@ -230,8 +251,7 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
                 const uint32_t row = rid[it];
                 int leaf = n;
                 if (is_split) {
-                    const uint32_t xb = xbv[it];
-                    const bool left = numeric ? (xb <= cb) : (xb == cb);
+                    const bool left = decide_left(xbv[it], plane != nullptr, row, numeric, cb);
                     leaf = 2 * n + (left ? 0 : 1);
                 }
                 if (A.write_nidx) A.nidx[row] = (uint32_t)leaf;
@@ -608,6 +628,9 @@ static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32
     A.fuse_pred = fuse_pred ? 1 : 0;
     A.write_nidx = c->write_nidx ? 1 : 0;
     A.stream_hint = ((size_t)c->N * c->F > ((size_t)256 << 20)) ? 1 : 0;
+    A.planes = c->planes_ready ? c->planes : nullptr;
+    A.plane_words = c->plane_words;
+    A.B = c->B;
 }
 
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur) {

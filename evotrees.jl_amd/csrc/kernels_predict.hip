@@ -101,6 +101,12 @@ __device__ __forceinline__ void add_tree(float *acc, const float *lp, int K, int
         if (loss == EVT_LOSS_MLOGLOSS) {
 #pragma unroll
             for (int k = 0; k < KMAX; k++) acc[k] = fmaxf(-15.0f, acc[k] - m);
+        } else if (loss == EVT_LOSS_LOGLOSS) { // several targets: each clamped to [-15, 15]
+#pragma unroll
+            for (int k = 0; k < KMAX; k++) acc[k] = fminf(fmaxf(acc[k], -15.0f), 15.0f);
+        } else if (EVT_IS_MLE2P(loss)) { // (location, raw scale) pairs: the scale outputs are floored at -15
+#pragma unroll
+            for (int k = 1; k < KMAX; k += 2) acc[k] = fmaxf(-15.0f, acc[k]);
         }
     }
 }
@@ -253,9 +259,19 @@ __global__ __launch_bounds__(RB) void k_predict_model_lds(const uint32_t *__rest
 #pragma unroll
         for (int j = 0; j < NT; j++) {
             const float *lp = cleaf + (size_t)K * (m[j].leaf_off + pos[j]);
+            if (KMAX > 4 && (K & 3) == 0) { // rows of 4 values: 16-byte loads (the value array starts on an allocation boundary)
 #pragma unroll
-            for (int k = 0; k < KMAX; k++)
-                if (k < K) lpv[j][k] = lp[k];
+                for (int k = 0; k < KMAX; k += 4) {
+                    if (k < K) {
+                        const float4 v = *reinterpret_cast<const float4 *>(lp + k);
+                        lpv[j][k] = v.x; lpv[j][k + 1] = v.y; lpv[j][k + 2] = v.z; lpv[j][k + 3] = v.w;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < KMAX; k++)
+                    if (k < K) lpv[j][k] = lp[k];
+            }
         }
         if (g + 1 < ngroups) {
 #pragma unroll
@@ -284,19 +300,19 @@ __global__ __launch_bounds__(256) void k_leaf_idx_model(const uint32_t *__restri
     for (int t = 0; t < ntrees; t++) out[(size_t)t * N + i] = (uint32_t)walk_packed(nodes + off[t], xcm, N, i);
 }
 
-template <int RB, int NT, int PRE, bool ALLNUM>
+template <int KMAX, int RB, int NT, int PRE, bool ALLNUM>
 static int launch_model_lds(hipStream_t s, const uint32_t *cnodes, const float *cleaf, const void *meta, int ntrees, const uint8_t *xcm, int64_t N,
                             int F, int max_int, int K, int loss, int apply_link, float *out) {
     static EvtDevOnce once;
     const int dev = EvtDevOnce::current();
     if (once.pending(dev)) {
-        HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_predict_model_lds<4, RB, NT, PRE, ALLNUM>),
+        HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_predict_model_lds<KMAX, RB, NT, PRE, ALLNUM>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         once.mark(dev);
     }
     const int S4 = (F + 3) >> 2;
     const size_t lds = (size_t)RB * S4 * 4 + 8 * (size_t)NT * max_int;
-    hipLaunchKernelGGL((k_predict_model_lds<4, RB, NT, PRE, ALLNUM>), dim3((unsigned)((N + RB - 1) / RB)), dim3(RB), lds, s, cnodes, cleaf,
+    hipLaunchKernelGGL((k_predict_model_lds<KMAX, RB, NT, PRE, ALLNUM>), dim3((unsigned)((N + RB - 1) / RB)), dim3(RB), lds, s, cnodes, cleaf,
                        static_cast<const ModelTree *>(meta), ntrees, xcm, N, F, S4, max_int, K, loss, apply_link, out);
     HIPCHK(hipGetLastError());
     return EVT_OK;
@@ -304,13 +320,16 @@ static int launch_model_lds(hipStream_t s, const uint32_t *cnodes, const float *
 
 // Launch shape of the LDS kernel for this model: 1 = 1024 rows per block, 4 trees side by side (one block per CU);
 // 2 = 512 rows, 2 trees (two blocks per CU); 3 = 512 rows, 1 tree; 4 = 256 rows, 1 tree; 0 = does not apply.
+// A row's running prediction and the leaf values of the trees walked side by side live in registers: up to 4 outputs
+// take any shape, 5 - 8 outputs at most two trees side by side, 9 - 16 outputs one tree at a time.
 int predict_lds_shape(int F, int max_int, int K, int hint) {
-    if (K > 4 || F >= 1024 || max_int < 0) return 0;
+    if (K > EVT_MAX_K || F >= 1024 || max_int < 0) return 0;
     const size_t S = 4 * (size_t)((F + 3) >> 2), mi = (size_t)(max_int > 0 ? max_int : 1);
+    const int first = K <= 4 ? 1 : (K <= 8 ? 2 : 3);
     const bool fits[5] = {false, 4 * mi <= 8 * 1024 && 1024 * S + 32 * mi <= 150 * 1024, 2 * mi <= 8 * 512 && 512 * S + 16 * mi <= 80 * 1024,
                           mi <= 8 * 512 && 512 * S + 8 * mi <= 80 * 1024, mi <= 16 * 256 && 256 * S + 8 * mi <= 80 * 1024};
-    if (hint >= 1 && hint <= 4 && fits[hint]) return hint; // a sweep's choice, when the shape allows it
-    for (int sh = 1; sh <= 4; sh++)
+    if (hint >= first && hint <= 4 && fits[hint]) return hint; // a sweep's choice, when the shape allows it
+    for (int sh = first; sh <= 4; sh++)
         if (fits[sh]) return sh;
     return 0;
 }
@@ -320,13 +339,22 @@ int launch_predict_model_lds(hipStream_t s, const uint32_t *cnodes, const float 
                              int F, int max_int, int K, int loss, int apply_link, int all_numeric, int shape, float *out) {
     const int mi = max_int > 0 ? max_int : 1;
     shape = predict_lds_shape(F, max_int, K, shape);
-#define EVT_PM(RB_, NT_, PRE_)                                                                                                          \
-    return all_numeric ? launch_model_lds<RB_, NT_, PRE_, true>(s, cnodes, cleaf, meta, ntrees, xcm, N, F, mi, K, loss, apply_link, out) \
-                       : launch_model_lds<RB_, NT_, PRE_, false>(s, cnodes, cleaf, meta, ntrees, xcm, N, F, mi, K, loss, apply_link, out)
-    if (shape == 1) { EVT_PM(1024, 4, 8); }
-    if (shape == 2) { EVT_PM(512, 2, 8); }
-    if (shape == 3) { EVT_PM(512, 1, 8); }
-    if (shape == 4) { EVT_PM(256, 1, 16); }
+#define EVT_PM(KM_, RB_, NT_, PRE_)                                                                                                          \
+    return all_numeric ? launch_model_lds<KM_, RB_, NT_, PRE_, true>(s, cnodes, cleaf, meta, ntrees, xcm, N, F, mi, K, loss, apply_link, out) \
+                       : launch_model_lds<KM_, RB_, NT_, PRE_, false>(s, cnodes, cleaf, meta, ntrees, xcm, N, F, mi, K, loss, apply_link, out)
+    if (K <= 4) {
+        if (shape == 1) { EVT_PM(4, 1024, 4, 8); }
+        if (shape == 2) { EVT_PM(4, 512, 2, 8); }
+        if (shape == 3) { EVT_PM(4, 512, 1, 8); }
+        if (shape == 4) { EVT_PM(4, 256, 1, 16); }
+    } else if (K <= 8) {
+        if (shape == 2) { EVT_PM(8, 512, 2, 8); }
+        if (shape == 3) { EVT_PM(8, 512, 1, 8); }
+        if (shape == 4) { EVT_PM(8, 256, 1, 16); }
+    } else {
+        if (shape == 3) { EVT_PM(16, 512, 1, 8); }
+        if (shape == 4) { EVT_PM(16, 256, 1, 16); }
+    }
 #undef EVT_PM
     evt_set_error("internal: model shape does not fit the LDS predict kernel");
     return EVT_ERR_ARG;

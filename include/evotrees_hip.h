@@ -243,7 +243,7 @@ int evt_get_quant(evt_handle h, int32_t *qbits /* 2K+1 */, int32_t *qexp /* 2K+1
  * The transposition to nobs x K (src/predict.jl:134) is left to the host.
  * x_bin and out may be host or device pointers (device memory is used in place); feattypes and the tree arrays are host
  * arrays.  Models whose trees are full heaps (2^depth - 1 entries, as the reference stores them) of depth
- * <= 13 with K <= 4 and fewer than 1024 features are walked from LDS; others from global memory, with
+ * <= 13 and fewer than 1024 features are walked from LDS (any K up to 16); others from global memory, with
  * identical results. */
 int evt_predict(int64_t nobs, int32_t nfeats, const uint8_t *x_bin_colmajor, const uint8_t *feattypes,
                 int32_t loss, int32_t K, int32_t ntrees, const int64_t *tree_off, const int64_t *feat,
@@ -299,6 +299,9 @@ int evt_get_profile(evt_handle h, int64_t *launches, double *ms, int64_t *units)
 int evt_reset_profile(evt_handle h);
 /* Options: "hist_blocks", "hist_threads", "hist_min_rows", "hist_seg_cost", "hist_variant" (launch shape,
  * work split and kernel variant of the histogram builder, for sweeps; results do not depend on them);
+ * "bit_planes" (1, default: before the first tree the library derives one bit plane per
+ * (feature, bin threshold) from x_bin - F * (nbins - 1) * nobs / 8 bytes, taken only when that is at most 16 GiB and a third of the free
+ * memory - and the row partition reads its decisions there; 0: it gathers bin bytes; same trees, bit for bit);
  * "record_nidx" (1: the partition also records every sampled row's final node while the tree grows;
  * 0, default: evt_get_nidx derives it afterwards by walking the finished tree); "defer_pred" (1, default:
  * leaf values of a tree grown on every row are added in row order by the next pass over the rows;

@@ -194,6 +194,13 @@ def test_grow_tree_matches_oracle(evt, loss, weights, N, F, B, D, tt, n_js, rows
     t_again = h.grow_tree(js, gp, mask=mask, cond=cond)
     assert_tree_bits(t_again, t_fx)
     assert np.array_equal(h.get_nidx(), nidx_fx)
+    # the partition's two decision sources - threshold bit planes (default when they fit) and gathered bin bytes - agree
+    h.set_option("bit_planes", 0)
+    h.set_option("record_nidx", 1)
+    assert_tree_bits(h.grow_tree(js, gp, mask=mask, cond=cond), t_fx)
+    assert np.array_equal(h.get_nidx(), nidx_fx)
+    h.set_option("bit_planes", 1)
+    h.set_option("record_nidx", 0)
     # launch shape must not change a bit of the result (integer accumulation is order independent)
     h.set_option("hist_blocks", 37)
     h.set_option("hist_threads", 256)
@@ -428,6 +435,11 @@ def _random_tree(rng, depth, F, B, K):
     (5000, 33, 16, [6] * 9, 2, "gaussian_mle"),
     (4000, 20, 16, [5, 7, 1, 7], 2, "logistic_mle"),
     (3000, 9, 32, [4] * 5, 6, "logistic_mle"),
+    # more than four outputs walked from LDS: two trees side by side up to 8 outputs, one at a time up to 16
+    (9000, 100, 64, [11, 11, 3, 11, 11, 11], 8, "mlogloss"),
+    (5000, 28, 128, [8] * 7, 16, "mlogloss"),
+    (4097, 150, 32, [7, 3, 7, 1, 6, 7], 5, "mse"),
+    (3000, 250, 16, [5, 6, 6, 4, 6], 12, "poisson"),
 ])
 @pytest.mark.parametrize("categorical", [True, False])
 def test_model_predict_random_trees(evt, N, F, B, depths, K, loss, categorical):
@@ -501,6 +513,36 @@ def test_device_binarize(evt):
             got_left = (h.get_pred()[:, 0] - before) == 1.0
             assert np.array_equal(got_left, want <= cb), (j, cb)
     h.close()
+
+
+@pytest.mark.parametrize("loss,K", [("logloss", 6), ("gaussian_mle", 8), ("logistic_mle", 16), ("mlogloss", 8), ("mlogloss", 12), ("mlogloss", 16),
+                                    ("mse", 5), ("poisson", 16)])
+@pytest.mark.parametrize("ntrees", [3, 9])
+def test_model_predict_many_outputs_with_clamps(evt, loss, K, ntrees):
+    """More than four outputs (multi-class, several targets), with leaf values large enough that the per-tree clamps of
+    predict! (src/predict.jl:16-62: [-15, 15] for logloss, floor -15 on the scale outputs and on the shifted mlogloss
+    scores) act on most rows: 3 trees take the kernel that gathers from global memory, 9 trees the one that walks
+    from LDS; both must equal the oracle's tree-by-tree predict!, bit for bit."""
+    rng = np.random.default_rng(1234 + K)
+    N, F, B = 6001, 37, 32
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    ft = np.ones(F, np.uint8)
+    trees = []
+    for d in [7, 4, 9, 1, 7, 8, 9, 3, 9][:ntrees]:
+        t = _random_tree(rng, d, F, B, K)
+        t.pred[:] = (rng.standard_normal(t.pred.shape) * 9.0).astype(np.float32)
+        trees.append(t)
+    want = np.zeros((N, K), np.float32)
+    for t in trees:
+        orc.predict_tree(orc.LOSS_IDS[loss], K, x_bin, ft, t, want)
+    if loss in ("logloss", "gaussian_mle", "logistic_mle", "mlogloss"):
+        assert (np.abs(want) == 15).any()  # a clamp was hit
+    raw = evt._lib.predict_model(x_bin, ft, loss, K, trees, apply_link=False)
+    assert np.array_equal(raw.view(np.uint32), want.view(np.uint32))
+    if loss != "poisson":  # exp of sums of this size overflows Float32 on both sides
+        linked = evt._lib.predict_model(x_bin, ft, loss, K, trees, apply_link=True)
+        orc.apply_link(orc.LOSS_IDS[loss], K, want)
+        np.testing.assert_allclose(linked, want, rtol=RTOL, atol=1e-7)
 
 
 # --------------------------------------------------------------------------- error paths (forced from the host)
