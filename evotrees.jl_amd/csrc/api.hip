@@ -180,7 +180,7 @@ extern "C" int evt_destroy(evt_handle c) {
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
         LevelTab &L = c->lvl[l];
-        void *lp[] = {L.hdr, L.act_node, L.cprefix, L.bnode, L.bstart, L.bprefix};
+        void *lp[] = {L.hdr, L.act_node, L.cprefix, L.bnode, L.bstart, L.bprefix, L.cdesc};
         for (void *p : lp)
             if (p) (void)hipFree(p);
     }
@@ -345,6 +345,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
         ALLOC(c->lvl[l].bnode, c->maxlvl + 2);
         ALLOC(c->lvl[l].bstart, c->maxlvl + 2);
         ALLOC(c->lvl[l].bprefix, c->maxlvl + 2);
+        ALLOC(c->lvl[l].cdesc, c->max_chunks + 1);
     }
     ALLOC(c->js, c->F);
     ALLOC(c->jsmap, c->RS);

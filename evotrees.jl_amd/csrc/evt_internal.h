@@ -44,6 +44,7 @@ struct LevelTab {
     int32_t *bnode;    // build nodes
     int64_t *bstart;   // their segment starts
     int64_t *bprefix;  // exclusive prefix of their lengths, n_build+1 entries
+    uint4 *cdesc;      // per chunk of the level: {node, first position, end of the node's segment, first chunk of the node}
 };
 
 struct TreeDev {

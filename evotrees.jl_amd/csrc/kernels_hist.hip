@@ -42,6 +42,12 @@ struct HistArgs {
     int min_rows;
     int seg_cost;
     int a0; // first global channel of this launch (channels beyond EVT_HIST_GROUP take further launches)
+    // level bookkeeping that rides along with the first launch of a level: the partition kernels' chunk descriptors
+    const int32_t *act_node;
+    const int64_t *cprefix;
+    const int64_t *seg_start;
+    const int64_t *seg_len;
+    uint4 *cdesc;
 };
 
 // First node of a block's span: the largest i with bprefix[i] <= start.  bprefix ascends from 0, so that is the number
@@ -69,6 +75,31 @@ __device__ __forceinline__ unsigned long long load_gq(const unsigned long long *
     return gq[(size_t)a * N + id];
 }
 
+// Chunk descriptors of the level, for the partition kernels that run after the split search: chunk c of the level is
+// chunk c - c0 of node n, whose segment ends at `end`: {n, first position, end, c0}.  One wavefront per chunk finds the
+// owner (all its loads independent); the work hides behind the histogram kernel's own set-up.
+__device__ __forceinline__ void fill_chunk_descriptors(const HistArgs &A) {
+    if (blockIdx.y != 0 || A.a0 != 0) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int n_act = (int)A.hdr[LH_N_ACT];
+    const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
+    for (int64_t c = (int64_t)blockIdx.x * nwaves + wave; c < n_chunks; c += (int64_t)gridDim.x * nwaves) {
+        int cnt = 0;
+        for (int k0 = 0; k0 < n_act; k0 += 64) {
+            const int k = k0 + lane;
+            const bool hit = (k < n_act) && (A.cprefix[k < n_act ? k : 0] <= c);
+            cnt += __popcll(__ballot(hit));
+        }
+        if (lane == 0) {
+            const int i = cnt - 1;
+            const int n = A.act_node[i];
+            const int64_t c0 = A.cprefix[i];
+            const int64_t seg = A.seg_start[n], len = A.seg_len[n];
+            A.cdesc[c] = make_uint4((uint32_t)n, (uint32_t)(seg + (c - c0) * EVT_CHUNK), (uint32_t)(seg + len), (uint32_t)c0);
+        }
+    }
+}
+
 template <int NA, bool PACK>
 __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     extern __shared__ unsigned long long H[]; // [NA][tile slots][B]
@@ -76,6 +107,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     const int lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
     const int n_build = (int)A.hdr[LH_N_BUILD];
     const int64_t total = A.hdr[LH_TOTAL_BUILD];
+    fill_chunk_descriptors(A);
     if (n_build <= 0 || total <= 0) return;
     if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0 && A.a0 == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
 
@@ -306,6 +338,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     const int lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
     const int n_build = (int)A.hdr[LH_N_BUILD];
     const int64_t total = A.hdr[LH_TOTAL_BUILD];
+    fill_chunk_descriptors(A);
     if (n_build <= 0 || total <= 0) return;
     if (blockIdx.x == 0 && tid == 0 && A.a0 == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
 
@@ -596,6 +629,11 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
     A.bnode = L.bnode;
     A.bstart = L.bstart;
     A.bprefix = L.bprefix;
+    A.act_node = L.act_node;
+    A.cprefix = L.cprefix;
+    A.seg_start = c->seg_start;
+    A.seg_len = c->seg_len;
+    A.cdesc = L.cdesc;
     A.jsmap = c->jsmap;
     A.hist = c->hist;
     A.stats = c->stats;

@@ -32,6 +32,7 @@ __device__ __forceinline__ int find_owner(const int64_t *__restrict__ pre, int n
 
 struct PartArgs {
     const int64_t *hdr;
+    const uint4 *cdesc; // per chunk: {node, first position, end of the node's segment, first chunk of the node}
     const int32_t *act_node;
     const int64_t *cprefix;
     const int32_t *status;
@@ -78,29 +79,15 @@ __device__ __forceinline__ bool decide_left(uint32_t v, bool use_plane, uint32_t
 template <bool NT>
 __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n_act = (int)A.hdr[LH_N_ACT];
+    // the first descriptor is requested together with the level's chunk count (the grid never exceeds the table)
+    uint4 cd = A.cdesc[blockIdx.x];
     const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
     __shared__ int s_cnt[4];
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const int i = find_owner(A.cprefix, n_act, c);
-        const int n = A.act_node[i];
-        if (A.status[n] != ST_SPLIT) {
-            if (tid == 0) A.chunk_nleft[c] = 0;
-            continue;
-        }
-        const int64_t cl = c - A.cprefix[i];
-        const int64_t seg = A.seg_start[n], len = A.seg_len[n];
-        const int64_t p0 = seg + cl * EVT_CHUNK;
-        const int64_t pend = seg + len;
-        const uint32_t nd = A.t_packed[n - 1];
-        const int f = (int)(nd & 0xFFFFu) - 1;
-        const uint32_t cb = (nd >> 16) & 0xFFu;
-        const bool numeric = (nd & EVT_NODE_NUMERIC) != 0;
-        const uint8_t *col = A.xcm + (size_t)f * A.N;
-        const uint32_t *plane = (A.planes && numeric && cb >= 1u && cb < (uint32_t)A.B) ? A.planes + ((size_t)f * (A.B - 1) + (cb - 1)) * A.plane_words : nullptr;
-        int cnt = 0;
-        // all row ids, then all bin bytes, are requested before the first is used; positions past the end read the
-        // segment's last row (unconditional loads keep every request of the chunk in flight at once)
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x, cd = A.cdesc[c < n_chunks ? c : 0]) {
+        // the chunk's descriptor names its node and its positions: the row ids are requested together with the node's
+        // state, one trip to memory after the descriptor
+        const int n = (int)cd.x;
+        const int64_t p0 = cd.y, pend = cd.z;
         constexpr int NI = EVT_CHUNK / 256;
         uint32_t rid[NI], xbv[NI];
 #pragma unroll
@@ -108,6 +95,17 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
             const int64_t p = p0 + it * 256 + tid;
             rid[it] = A.is_cur[p < pend ? p : pend - 1];
         }
+        if (A.status[n] != ST_SPLIT) {
+            if (tid == 0) A.chunk_nleft[c] = 0;
+            continue;
+        }
+        const uint32_t nd = A.t_packed[n - 1];
+        const int f = (int)(nd & 0xFFFFu) - 1;
+        const uint32_t cb = (nd >> 16) & 0xFFu;
+        const bool numeric = (nd & EVT_NODE_NUMERIC) != 0;
+        const uint8_t *col = A.xcm + (size_t)f * A.N;
+        const uint32_t *plane = (A.planes && numeric && cb >= 1u && cb < (uint32_t)A.B) ? A.planes + ((size_t)f * (A.B - 1) + (cb - 1)) * A.plane_words : nullptr;
+        int cnt = 0;
         // a binned matrix larger than the last-level cache is gathered with the streaming hint: each byte's line would
         // displace data that is read again (row lists, gradient words) and is rarely hit a second time itself
 #pragma unroll
@@ -129,37 +127,39 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
 
 __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n_act = (int)A.hdr[LH_N_ACT];
+    uint4 cd = A.cdesc[blockIdx.x];
     const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
     __shared__ unsigned long long s_w[EVT_CHUNK_WORDS];
     __shared__ int s_pre[EVT_CHUNK_WORDS];
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const int i = find_owner(A.cprefix, n_act, c);
-        const int n = A.act_node[i];
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x, cd = A.cdesc[c < n_chunks ? c : 0]) {
+        const int n = (int)cd.x;
+        const int64_t p0 = cd.y, pend = cd.z, c0 = cd.w;
+        const int64_t cl = c - c0;
+        const int64_t seg = p0 - cl * EVT_CHUNK;
+        // everything the chunk needs is requested at once, behind the descriptor: node state, the count pass's ballots
+        // and prefixes, the left child's size and the row ids (positions past the end read the segment's last row)
         const int st = A.status[n];
-        const int64_t cl = c - A.cprefix[i];
-        const int64_t seg = A.seg_start[n], len = A.seg_len[n];
-        const int64_t p0 = seg + cl * EVT_CHUNK;
-        const int64_t pend = seg + len;
+        const unsigned long long fw = A.flagw[c * EVT_CHUNK_WORDS + (tid & (EVT_CHUNK_WORDS - 1))];
+        const int64_t lpre_c = A.chunk_lpre[c], lpre_0 = A.chunk_lpre[c0];
+        const int64_t nl_node = A.seg_len[2 * n];
+        constexpr int NI = EVT_CHUNK / 256;
+        uint32_t rid[NI];
+#pragma unroll
+        for (int it = 0; it < NI; it++) {
+            const int64_t p = p0 + it * 256 + tid;
+            rid[it] = A.is_cur[p < pend ? p : pend - 1];
+        }
         if (st == ST_SPLIT) {
-            if (tid < EVT_CHUNK_WORDS) s_w[tid] = A.flagw[c * EVT_CHUNK_WORDS + tid];
+            if (tid < EVT_CHUNK_WORDS) s_w[tid] = fw;
             __syncthreads();
             if (tid == 0) {
                 int run = 0;
                 for (int t = 0; t < EVT_CHUNK_WORDS; t++) { s_pre[t] = run; run += __popcll(s_w[t]); }
             }
             __syncthreads();
-            const int64_t lbase = A.chunk_lpre[c] - A.chunk_lpre[A.cprefix[i]]; // lefts of this node before this chunk
-            const int64_t nl_node = A.seg_len[2 * n];
+            const int64_t lbase = lpre_c - lpre_0; // lefts of this node before this chunk
             const int64_t dstL = seg + lbase;
             const int64_t dstR = seg + nl_node + (cl * EVT_CHUNK - lbase);
-            constexpr int NI = EVT_CHUNK / 256;
-            uint32_t rid[NI];
-#pragma unroll
-            for (int it = 0; it < NI; it++) {
-                const int64_t p = p0 + it * 256 + tid;
-                rid[it] = A.is_cur[p < pend ? p : pend - 1];
-            }
 #pragma unroll
             for (int it = 0; it < NI; it++) {
                 const int64_t p = p0 + it * 256 + tid;
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
             for (int it = 0; it < EVT_CHUNK / 256; it++) {
                 const int64_t p = p0 + it * 256 + tid;
                 if (p < pend) {
-                    const uint32_t row = A.is_cur[p];
+                    const uint32_t row = rid[it];
                     if (A.write_nidx) A.nidx[row] = (uint32_t)n;
                     if (A.fuse_pred) {
                         float *pr = A.pred + (size_t)K * row;
@@ -203,18 +203,22 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
 template <bool NT>
 __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
     const int tid = threadIdx.x;
-    const int n_act = (int)A.hdr[LH_N_ACT];
+    uint4 cd = A.cdesc[blockIdx.x];
     const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
     const int K = A.K;
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const int i = find_owner(A.cprefix, n_act, c);
-        const int n = A.act_node[i];
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x, cd = A.cdesc[c < n_chunks ? c : 0]) {
+        const int n = (int)cd.x;
+        const int64_t p0 = cd.y, pend = cd.z;
+        constexpr int NI = EVT_CHUNK / 256;
+        uint32_t rid[NI], xbv[NI];
+        float prv[NI];
+#pragma unroll
+        for (int it = 0; it < NI; it++) {
+            const int64_t p = p0 + it * 256 + tid;
+            rid[it] = A.is_cur[p < pend ? p : pend - 1];
+        }
         const int st = A.status[n];
         if (st != ST_SPLIT && st != ST_LEAF) continue;
-        const int64_t cl = c - A.cprefix[i];
-        const int64_t seg = A.seg_start[n], len = A.seg_len[n];
-        const int64_t p0 = seg + cl * EVT_CHUNK;
-        const int64_t pend = seg + len;
         const bool is_split = (st == ST_SPLIT);
         int f = 0;
         uint32_t cb = 0;
@@ -227,16 +231,8 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
         }
         const uint8_t *col = A.xcm + (size_t)f * A.N;
         const uint32_t *plane = (A.planes && is_split && numeric && cb >= 1u && cb < (uint32_t)A.B) ? A.planes + ((size_t)f * (A.B - 1) + (cb - 1)) * A.plane_words : nullptr;
-        // every request of the chunk goes out before the first result is used: row ids, then bin bytes, then (one
-        // output) the predictions; positions past the end read the segment's last row and are not written
-        constexpr int NI = EVT_CHUNK / 256;
-        uint32_t rid[NI], xbv[NI];
-        float prv[NI];
-#pragma unroll
-        for (int it = 0; it < NI; it++) {
-            const int64_t p = p0 + it * 256 + tid;
-            rid[it] = A.is_cur[p < pend ? p : pend - 1];
-        }
+        // every request of the chunk goes out before the first result is used: row ids (above), then bin bytes or plane
+        // words, then (one output) the predictions; positions past the end read the segment's last row and are not written
 #pragma unroll
         for (int it = 0; it < NI; it++) xbv[it] = is_split ? load_decision<NT>(col, plane, rid[it]) : 0u;
         const bool fast1 = A.fuse_pred && K == 1;
@@ -607,6 +603,7 @@ int launch_tree_begin(evt_ctx *c, bool all_rows) {
 static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred, PartArgs &A) {
     const LevelTab &L = c->lvl[level & 1];
     A.hdr = L.hdr;
+    A.cdesc = L.cdesc;
     A.act_node = L.act_node;
     A.cprefix = L.cprefix;
     A.status = c->status;
