@@ -832,7 +832,6 @@ static int tree_stage_partition(evt_ctx *c) {
     prof_begin(c, EVT_K_PARTITION, level);
     if (level < last_split) {
         r = launch_part_count(c, level, is_cur);
-        if (r == EVT_OK) r = launch_level_next(c, level);
         if (r == EVT_OK) r = launch_part_scatter(c, level, is_cur, is_next, c->step.fuse_pred);
     } else {
         r = launch_final_fused(c, level, is_cur, c->step.fuse_pred);

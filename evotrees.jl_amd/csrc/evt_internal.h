@@ -275,7 +275,6 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level);
 int launch_obliv_select(evt_ctx *c, int level, const evt_params *p);
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur);
-int launch_level_next(evt_ctx *c, int level);
 int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred);
 int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred);
 int launch_nidx_from_segments(evt_ctx *c, int level, const uint32_t *is_cur);

@@ -52,6 +52,7 @@ struct PartArgs {
     const float *t_pred;
     int K, loss, fuse_pred, write_nidx;
     int stream_hint; // the binned matrix does not fit the last-level cache
+    int fold;        // scatter: the level's bookkeeping block rides along and the blocks add up chunk counts themselves
     // threshold bit planes (nullptr: none): numeric splits read one bit of plane (feature, cond_bin) per row
     const uint32_t *planes;
     int64_t plane_words;
@@ -125,13 +126,199 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
     }
 }
 
-__global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
+// ---- single-block scans -----------------------------------------------------------------------
+// Exclusive prefix over the threads of the block (up to 1024); returns the prefix, *total gets the sum.
+__device__ long long block_excl_scan(long long v, long long *total, long long *s_tmp /* [17] */) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    long long x = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        int lo = __shfl_up((int)(x & 0xffffffffll), o), hi = __shfl_up((int)(x >> 32), o);
+        long long y = ((long long)hi << 32) | (unsigned int)lo;
+        if (lane >= o) x += y;
+    }
+    __syncthreads(); // s_tmp may still be read from a previous call
+    if (lane == 63) s_tmp[wave] = x;
+    __syncthreads();
+    if (tid == 0) {
+        long long run = 0;
+        const int nw = blockDim.x >> 6;
+        for (int w = 0; w < nw; w++) { long long t = s_tmp[w]; s_tmp[w] = run; run += t; }
+        s_tmp[16] = run;
+    }
+    __syncthreads();
+    *total = s_tmp[16];
+    return s_tmp[wave] + x - v;
+}
+
+struct NextArgs {
+    const int64_t *hdr;
+    const int32_t *act_node;
+    const int64_t *cprefix;
+    int32_t *status;
+    int64_t *seg_start;
+    int64_t *seg_len;
+    const int32_t *chunk_nleft;
+    int64_t *chunk_lpre;
+    // next level
+    int64_t *n_hdr;
+    int32_t *n_act_node;
+    int64_t *n_cprefix;
+    int32_t *n_bnode;
+    int64_t *n_bstart;
+    int64_t *n_bprefix;
+    int64_t seg_cost; // cost units added per build node in the histogram kernel's span space
+};
+
+// Two exclusive prefixes in one pass (same shape as block_excl_scan); s_tmp holds 34 values.
+__device__ void block_excl_scan2(long long va, long long vb, long long *pa, long long *pb, long long *ta, long long *tb, long long *s_tmp) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    long long xa = va, xb = vb;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int al = __shfl_up((int)(xa & 0xffffffffll), o), ah = __shfl_up((int)(xa >> 32), o);
+        const int bl = __shfl_up((int)(xb & 0xffffffffll), o), bh = __shfl_up((int)(xb >> 32), o);
+        if (lane >= o) {
+            xa += ((long long)ah << 32) | (unsigned int)al;
+            xb += ((long long)bh << 32) | (unsigned int)bl;
+        }
+    }
+    __syncthreads(); // s_tmp may still be read from a previous call
+    if (lane == 63) {
+        s_tmp[wave] = xa;
+        s_tmp[17 + wave] = xb;
+    }
+    __syncthreads();
+    if (tid < 2) {
+        long long *t = s_tmp + 17 * tid;
+        long long run = 0;
+        const int nw = blockDim.x >> 6;
+        for (int w = 0; w < nw; w++) { long long x = t[w]; t[w] = run; run += x; }
+        t[16] = run;
+    }
+    __syncthreads();
+    *ta = s_tmp[16];
+    *tb = s_tmp[33];
+    *pa = s_tmp[wave] + xa - va;
+    *pb = s_tmp[17 + wave] + xb - vb;
+}
+
+// One block turns the chunk counts of a level into the next level's tables (children's segments, which child is
+// built, active nodes, chunk prefix, build list).  It rides along as the last block of the scatter kernel, whose other
+// blocks need nothing from it: they add up the chunk counts of their own node themselves.  Loads that do not depend on
+// each other are issued together (fixed-trip loops over clamped indices instead of data-dependent ones).
+__device__ void level_next_block(const NextArgs &A, long long *s_tmp /* [34] */) {
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int n_act = (int)A.hdr[LH_N_ACT];
+    const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
+    long long total;
+    // A: exclusive scan of the chunks' left counts
+    {
+        constexpr int SP = 8;
+        const int64_t span = (n_chunks + nthr - 1) / nthr;
+        const int64_t c0 = (int64_t)tid * span, c1 = (c0 + span < n_chunks) ? c0 + span : n_chunks;
+        if (span <= SP) {
+            int v[SP];
+#pragma unroll
+            for (int k = 0; k < SP; k++) {
+                const int64_t c = c0 + k;
+                const int x = A.chunk_nleft[c < c1 ? c : 0];
+                v[k] = c < c1 ? x : 0;
+            }
+            long long s = 0;
+#pragma unroll
+            for (int k = 0; k < SP; k++) s += v[k];
+            long long pre = block_excl_scan(s, &total, s_tmp);
+#pragma unroll
+            for (int k = 0; k < SP; k++) {
+                if (c0 + k < c1) A.chunk_lpre[c0 + k] = pre;
+                pre += v[k];
+            }
+        } else {
+            long long s = 0;
+            for (int64_t c = c0; c < c1; c++) s += A.chunk_nleft[c];
+            long long pre = block_excl_scan(s, &total, s_tmp);
+            for (int64_t c = c0; c < c1; c++) { A.chunk_lpre[c] = pre; pre += A.chunk_nleft[c]; }
+        }
+        if (tid == 0) A.chunk_lpre[n_chunks] = total;
+    }
+    __syncthreads();
+    // B: children segments + three scans over the active nodes (children count, chunks, build rows)
+    const int span = (n_act + nthr - 1) / nthr;
+    const int i0 = tid * span, i1 = (i0 + span < n_act) ? i0 + span : n_act;
+    long long s_pos = 0, s_chunks = 0, s_brows = 0;
+    for (int i = i0; i < i1; i++) {
+        const int n = A.act_node[i];
+        const int64_t cp0 = A.cprefix[i], cp1 = A.cprefix[i + 1];
+        const int st = A.status[n];
+        const int64_t len = A.seg_len[n], start = A.seg_start[n];
+        const int64_t nl = A.chunk_lpre[cp1] - A.chunk_lpre[cp0];
+        if (st != ST_SPLIT) continue;
+        const int64_t nr = len - nl;
+        A.seg_start[2 * n] = start;
+        A.seg_len[2 * n] = nl;
+        A.seg_start[2 * n + 1] = start + nl;
+        A.seg_len[2 * n + 1] = nr;
+        const bool build_left = nr >= nl; // the smaller child is built, tie -> left (src/fit.jl:123-129)
+        A.status[2 * n] = build_left ? ST_BUILD : ST_SUBTRACT;
+        A.status[2 * n + 1] = build_left ? ST_SUBTRACT : ST_BUILD;
+        s_pos += 1;
+        s_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
+        s_brows += (build_left ? nl : nr) + A.seg_cost;
+    }
+    // children count (low 24 bits) and chunk count share one scan; the build rows take the other
+    long long t_pc, t_brows, p_pc, p_brows;
+    block_excl_scan2((s_chunks << 24) | s_pos, s_brows, &p_pc, &p_brows, &t_pc, &t_brows, s_tmp);
+    long long p_pos = p_pc & 0xFFFFFF, p_chunks = p_pc >> 24;
+    const long long t_pos = t_pc & 0xFFFFFF, t_chunks = t_pc >> 24;
+    for (int i = i0; i < i1; i++) {
+        const int n = A.act_node[i];
+        if (A.status[n] != ST_SPLIT) continue;
+        const int64_t nl = A.seg_len[2 * n], nr = A.seg_len[2 * n + 1];
+        const int64_t start = A.seg_start[2 * n];
+        const bool build_left = nr >= nl;
+        A.n_act_node[2 * p_pos] = 2 * n;
+        A.n_act_node[2 * p_pos + 1] = 2 * n + 1;
+        A.n_cprefix[2 * p_pos] = p_chunks;
+        A.n_cprefix[2 * p_pos + 1] = p_chunks + (nl + EVT_CHUNK - 1) / EVT_CHUNK;
+        A.n_bnode[p_pos] = build_left ? 2 * n : 2 * n + 1;
+        A.n_bstart[p_pos] = build_left ? start : start + nl;
+        A.n_bprefix[p_pos] = p_brows;
+        p_pos += 1;
+        p_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
+        p_brows += (build_left ? nl : nr) + A.seg_cost;
+    }
+    if (tid == 0) {
+        A.n_cprefix[2 * t_pos] = t_chunks;
+        A.n_bprefix[t_pos] = t_brows;
+        A.n_hdr[LH_N_ACT] = 2 * t_pos;
+        A.n_hdr[LH_N_CHUNKS] = t_chunks;
+        A.n_hdr[LH_N_BUILD] = t_pos;
+        A.n_hdr[LH_TOTAL_BUILD] = t_brows;
+    }
+}
+
+// The same bookkeeping as a kernel of its own (one block of 1024 threads), for inputs with thousands of chunks per level,
+// where every scatter block adding up its node's chunk counts would cost more than this launch.
+__global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
+    __shared__ long long s_tmp[34];
+    level_next_block(A, s_tmp);
+}
+
+__global__ __launch_bounds__(256) void k_part_scatter(PartArgs A, NextArgs NX) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __shared__ long long s_tmp[34];
+    const bool fold = A.fold != 0;
+    if (fold && blockIdx.x == gridDim.x - 1) { // the level's bookkeeping, beside the blocks that move the rows
+        level_next_block(NX, s_tmp);
+        return;
+    }
+    const int64_t G = fold ? gridDim.x - 1 : gridDim.x;
     uint4 cd = A.cdesc[blockIdx.x];
     const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
     __shared__ unsigned long long s_w[EVT_CHUNK_WORDS];
     __shared__ int s_pre[EVT_CHUNK_WORDS];
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x, cd = A.cdesc[c < n_chunks ? c : 0]) {
+    for (int64_t c = blockIdx.x; c < n_chunks; c += G, cd = A.cdesc[c < n_chunks ? c : 0]) {
         const int n = (int)cd.x;
         const int64_t p0 = cd.y, pend = cd.z, c0 = cd.w;
         const int64_t cl = c - c0;
@@ -140,8 +327,20 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
         // and prefixes, the left child's size and the row ids (positions past the end read the segment's last row)
         const int st = A.status[n];
         const unsigned long long fw = A.flagw[c * EVT_CHUNK_WORDS + (tid & (EVT_CHUNK_WORDS - 1))];
-        const int64_t lpre_c = A.chunk_lpre[c], lpre_0 = A.chunk_lpre[c0];
-        const int64_t nl_node = A.seg_len[2 * n];
+        // lefts of this node before this chunk, and in all of the node: the block adds up the node's chunk counts itself
+        // (a node's chunks are few, or the sums are spread over the 256 threads)
+        const int64_t c1 = c0 + (pend - seg + EVT_CHUNK - 1) / EVT_CHUNK;
+        long long sum_before = 0, sum_node = 0;
+        if (fold) {
+            for (int64_t k = c0 + tid; k < c1; k += 256) {
+                const int v = A.chunk_nleft[k];
+                sum_node += v;
+                sum_before += (k < c) ? v : 0;
+            }
+        } else { // the bookkeeping kernel ran before this one: prefix of the chunk counts, children's sizes
+            sum_before = A.chunk_lpre[c] - A.chunk_lpre[c0];
+            sum_node = A.seg_len[2 * n];
+        }
         constexpr int NI = EVT_CHUNK / 256;
         uint32_t rid[NI];
 #pragma unroll
@@ -150,6 +349,14 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
             rid[it] = A.is_cur[p < pend ? p : pend - 1];
         }
         if (st == ST_SPLIT) {
+            if (fold) {
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) {
+                    sum_before += __shfl_xor(sum_before, o);
+                    sum_node += __shfl_xor(sum_node, o);
+                }
+                if (lane == 0) { s_tmp[wave] = sum_before; s_tmp[4 + wave] = sum_node; }
+            }
             if (tid < EVT_CHUNK_WORDS) s_w[tid] = fw;
             __syncthreads();
             if (tid == 0) {
@@ -157,7 +364,8 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A) {
                 for (int t = 0; t < EVT_CHUNK_WORDS; t++) { s_pre[t] = run; run += __popcll(s_w[t]); }
             }
             __syncthreads();
-            const int64_t lbase = lpre_c - lpre_0; // lefts of this node before this chunk
+            const int64_t lbase = fold ? s_tmp[0] + s_tmp[1] + s_tmp[2] + s_tmp[3] : sum_before; // lefts of this node before this chunk
+            const int64_t nl_node = fold ? s_tmp[4] + s_tmp[5] + s_tmp[6] + s_tmp[7] : sum_node;
             const int64_t dstL = seg + lbase;
             const int64_t dstR = seg + nl_node + (cl * EVT_CHUNK - lbase);
 #pragma unroll
@@ -263,178 +471,6 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
                 }
             }
         }
-    }
-}
-
-// ---- single-block scans -----------------------------------------------------------------------
-// Exclusive prefix over the 1024 threads of the block; returns the prefix, *total gets the sum.
-__device__ long long block_excl_scan(long long v, long long *total, long long *s_tmp /* [17] */) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    long long x = v;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        int lo = __shfl_up((int)(x & 0xffffffffll), o), hi = __shfl_up((int)(x >> 32), o);
-        long long y = ((long long)hi << 32) | (unsigned int)lo;
-        if (lane >= o) x += y;
-    }
-    __syncthreads(); // s_tmp may still be read from a previous call
-    if (lane == 63) s_tmp[wave] = x;
-    __syncthreads();
-    if (tid == 0) {
-        long long run = 0;
-        const int nw = blockDim.x >> 6;
-        for (int w = 0; w < nw; w++) { long long t = s_tmp[w]; s_tmp[w] = run; run += t; }
-        s_tmp[16] = run;
-    }
-    __syncthreads();
-    *total = s_tmp[16];
-    return s_tmp[wave] + x - v;
-}
-
-struct NextArgs {
-    const int64_t *hdr;
-    const int32_t *act_node;
-    const int64_t *cprefix;
-    int32_t *status;
-    int64_t *seg_start;
-    int64_t *seg_len;
-    const int32_t *chunk_nleft;
-    int64_t *chunk_lpre;
-    // next level
-    int64_t *n_hdr;
-    int32_t *n_act_node;
-    int64_t *n_cprefix;
-    int32_t *n_bnode;
-    int64_t *n_bstart;
-    int64_t *n_bprefix;
-    int64_t seg_cost; // cost units added per build node in the histogram kernel's span space
-};
-
-// Two exclusive prefixes in one pass (same shape as block_excl_scan); s_tmp holds 34 values.
-__device__ void block_excl_scan2(long long va, long long vb, long long *pa, long long *pb, long long *ta, long long *tb, long long *s_tmp) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    long long xa = va, xb = vb;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const int al = __shfl_up((int)(xa & 0xffffffffll), o), ah = __shfl_up((int)(xa >> 32), o);
-        const int bl = __shfl_up((int)(xb & 0xffffffffll), o), bh = __shfl_up((int)(xb >> 32), o);
-        if (lane >= o) {
-            xa += ((long long)ah << 32) | (unsigned int)al;
-            xb += ((long long)bh << 32) | (unsigned int)bl;
-        }
-    }
-    __syncthreads(); // s_tmp may still be read from a previous call
-    if (lane == 63) {
-        s_tmp[wave] = xa;
-        s_tmp[17 + wave] = xb;
-    }
-    __syncthreads();
-    if (tid < 2) {
-        long long *t = s_tmp + 17 * tid;
-        long long run = 0;
-        const int nw = blockDim.x >> 6;
-        for (int w = 0; w < nw; w++) { long long x = t[w]; t[w] = run; run += x; }
-        t[16] = run;
-    }
-    __syncthreads();
-    *ta = s_tmp[16];
-    *tb = s_tmp[33];
-    *pa = s_tmp[wave] + xa - va;
-    *pb = s_tmp[17 + wave] + xb - vb;
-}
-
-// One block turns the chunk counts of a level into the next level's tables.  It runs between two grid-wide kernels,
-// so its latency is what counts: loads that do not depend on each other are issued together (fixed-trip loops over
-// clamped indices instead of data-dependent ones) and values are kept in registers between the passes.
-__global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
-    const int tid = threadIdx.x;
-    __shared__ long long s_tmp[34];
-    const int n_act = (int)A.hdr[LH_N_ACT];
-    const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
-    long long total;
-    // A: exclusive scan of the chunks' left counts
-    {
-        constexpr int SP = 8;
-        const int64_t span = (n_chunks + 1023) / 1024;
-        const int64_t c0 = (int64_t)tid * span, c1 = (c0 + span < n_chunks) ? c0 + span : n_chunks;
-        if (span <= SP) {
-            int v[SP];
-#pragma unroll
-            for (int k = 0; k < SP; k++) {
-                const int64_t c = c0 + k;
-                const int x = A.chunk_nleft[c < c1 ? c : 0];
-                v[k] = c < c1 ? x : 0;
-            }
-            long long s = 0;
-#pragma unroll
-            for (int k = 0; k < SP; k++) s += v[k];
-            long long pre = block_excl_scan(s, &total, s_tmp);
-#pragma unroll
-            for (int k = 0; k < SP; k++) {
-                if (c0 + k < c1) A.chunk_lpre[c0 + k] = pre;
-                pre += v[k];
-            }
-        } else {
-            long long s = 0;
-            for (int64_t c = c0; c < c1; c++) s += A.chunk_nleft[c];
-            long long pre = block_excl_scan(s, &total, s_tmp);
-            for (int64_t c = c0; c < c1; c++) { A.chunk_lpre[c] = pre; pre += A.chunk_nleft[c]; }
-        }
-        if (tid == 0) A.chunk_lpre[n_chunks] = total;
-    }
-    __syncthreads();
-    // B: children segments + three scans over the active nodes (children count, chunks, build rows)
-    const int span = (n_act + 1023) / 1024;
-    const int i0 = tid * span, i1 = (i0 + span < n_act) ? i0 + span : n_act;
-    long long s_pos = 0, s_chunks = 0, s_brows = 0;
-    for (int i = i0; i < i1; i++) {
-        const int n = A.act_node[i];
-        const int64_t cp0 = A.cprefix[i], cp1 = A.cprefix[i + 1];
-        const int st = A.status[n];
-        const int64_t len = A.seg_len[n], start = A.seg_start[n];
-        const int64_t nl = A.chunk_lpre[cp1] - A.chunk_lpre[cp0];
-        if (st != ST_SPLIT) continue;
-        const int64_t nr = len - nl;
-        A.seg_start[2 * n] = start;
-        A.seg_len[2 * n] = nl;
-        A.seg_start[2 * n + 1] = start + nl;
-        A.seg_len[2 * n + 1] = nr;
-        const bool build_left = nr >= nl; // the smaller child is built, tie -> left (src/fit.jl:123-129)
-        A.status[2 * n] = build_left ? ST_BUILD : ST_SUBTRACT;
-        A.status[2 * n + 1] = build_left ? ST_SUBTRACT : ST_BUILD;
-        s_pos += 1;
-        s_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
-        s_brows += (build_left ? nl : nr) + A.seg_cost;
-    }
-    // children count (low 24 bits) and chunk count share one scan; the build rows take the other
-    long long t_pc, t_brows, p_pc, p_brows;
-    block_excl_scan2((s_chunks << 24) | s_pos, s_brows, &p_pc, &p_brows, &t_pc, &t_brows, s_tmp);
-    long long p_pos = p_pc & 0xFFFFFF, p_chunks = p_pc >> 24;
-    const long long t_pos = t_pc & 0xFFFFFF, t_chunks = t_pc >> 24;
-    for (int i = i0; i < i1; i++) {
-        const int n = A.act_node[i];
-        if (A.status[n] != ST_SPLIT) continue;
-        const int64_t nl = A.seg_len[2 * n], nr = A.seg_len[2 * n + 1];
-        const int64_t start = A.seg_start[2 * n];
-        const bool build_left = nr >= nl;
-        A.n_act_node[2 * p_pos] = 2 * n;
-        A.n_act_node[2 * p_pos + 1] = 2 * n + 1;
-        A.n_cprefix[2 * p_pos] = p_chunks;
-        A.n_cprefix[2 * p_pos + 1] = p_chunks + (nl + EVT_CHUNK - 1) / EVT_CHUNK;
-        A.n_bnode[p_pos] = build_left ? 2 * n : 2 * n + 1;
-        A.n_bstart[p_pos] = build_left ? start : start + nl;
-        A.n_bprefix[p_pos] = p_brows;
-        p_pos += 1;
-        p_chunks += (nl + EVT_CHUNK - 1) / EVT_CHUNK + (nr + EVT_CHUNK - 1) / EVT_CHUNK;
-        p_brows += (build_left ? nl : nr) + A.seg_cost;
-    }
-    if (tid == 0) {
-        A.n_cprefix[2 * t_pos] = t_chunks;
-        A.n_bprefix[t_pos] = t_brows;
-        A.n_hdr[LH_N_ACT] = 2 * t_pos;
-        A.n_hdr[LH_N_CHUNKS] = t_chunks;
-        A.n_hdr[LH_N_BUILD] = t_pos;
-        A.n_hdr[LH_TOTAL_BUILD] = t_brows;
     }
 }
 
@@ -625,6 +661,7 @@ static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32
     A.fuse_pred = fuse_pred ? 1 : 0;
     A.write_nidx = c->write_nidx ? 1 : 0;
     A.stream_hint = ((size_t)c->N * c->F > ((size_t)256 << 20)) ? 1 : 0;
+    A.fold = 0;
     A.planes = c->planes_ready ? c->planes : nullptr;
     A.plane_words = c->plane_words;
     A.B = c->B;
@@ -639,10 +676,39 @@ int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur) {
     return EVT_OK;
 }
 
+static void fill_next_args(evt_ctx *c, int level, NextArgs &A) {
+    const LevelTab &L = c->lvl[level & 1];
+    const LevelTab &Nx = c->lvl[(level + 1) & 1];
+    A.hdr = L.hdr;
+    A.act_node = L.act_node;
+    A.cprefix = L.cprefix;
+    A.status = c->status;
+    A.seg_start = c->seg_start;
+    A.seg_len = c->seg_len;
+    A.chunk_nleft = c->chunk_nleft;
+    A.chunk_lpre = c->chunk_lpre;
+    A.n_hdr = Nx.hdr;
+    A.n_act_node = Nx.act_node;
+    A.n_cprefix = Nx.cprefix;
+    A.n_bnode = Nx.bnode;
+    A.n_bstart = Nx.bstart;
+    A.n_bprefix = Nx.bprefix;
+    A.seg_cost = c->hist_seg_cost;
+}
+
+// Moves the rows of the level's split nodes to their children and, in one extra block, writes the next level's tables.
 int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred) {
     PartArgs A;
     fill_part_args(c, level, is_cur, is_next, fuse_pred, A);
-    hipLaunchKernelGGL(k_part_scatter, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
+    NextArgs NX;
+    fill_next_args(c, level, NX);
+    // up to a thousand chunks per level the bookkeeping rides along in the scatter kernel (one launch less per level)
+    A.fold = c->max_chunks <= 1024 + c->maxlvl ? 1 : 0;
+    if (!A.fold) {
+        hipLaunchKernelGGL(k_level_next, dim3(1), dim3(1024), 0, c->stream, NX);
+        HIPCHK(hipGetLastError());
+    }
+    hipLaunchKernelGGL(k_part_scatter, dim3(grid_for_chunks(c->max_chunks) + (A.fold ? 1 : 0)), dim3(256), 0, c->stream, A, NX);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -677,26 +743,3 @@ int launch_nidx_from_segments(evt_ctx *c, int level, const uint32_t *is_cur) {
     return EVT_OK;
 }
 
-int launch_level_next(evt_ctx *c, int level) {
-    const LevelTab &L = c->lvl[level & 1];
-    const LevelTab &Nx = c->lvl[(level + 1) & 1];
-    NextArgs A;
-    A.hdr = L.hdr;
-    A.act_node = L.act_node;
-    A.cprefix = L.cprefix;
-    A.status = c->status;
-    A.seg_start = c->seg_start;
-    A.seg_len = c->seg_len;
-    A.chunk_nleft = c->chunk_nleft;
-    A.chunk_lpre = c->chunk_lpre;
-    A.n_hdr = Nx.hdr;
-    A.n_act_node = Nx.act_node;
-    A.n_cprefix = Nx.cprefix;
-    A.n_bnode = Nx.bnode;
-    A.n_bstart = Nx.bstart;
-    A.n_bprefix = Nx.bprefix;
-    A.seg_cost = c->hist_seg_cost;
-    hipLaunchKernelGGL(k_level_next, dim3(1), dim3(1024), 0, c->stream, A);
-    HIPCHK(hipGetLastError());
-    return EVT_OK;
-}
