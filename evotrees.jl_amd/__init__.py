@@ -18,7 +18,7 @@ from . import _lib
 from ._lib import EvtError, Handle, TreeArrays, make_params  # noqa: F401
 
 __all__ = ["EvoTreeRegressor", "EvoTreeCount", "EvoTreeClassifier", "EvoTreeMLE", "EvoTree", "Tree", "fit", "predict", "predict_leaf_idx", "init",
-           "grow_evotree", "update", "okay_to_continue", "get_edges", "check_args", "CallBack", "init_logger", "update_logger", "EvtError"]
+           "grow_evotree", "update", "okay_to_continue", "get_edges", "get_edges_table", "binarize_table", "check_args", "CallBack", "init_logger", "update_logger", "EvtError"]
 
 _GPU_DEVICES = ("gpu", "rocm", "amd", "hip")
 _EXP_LINK = ("poisson", "gamma", "tweedie")
@@ -233,6 +233,111 @@ def _link_offset(loss, offset, N, K):
     return offset.astype(np.float32)
 
 
+def _is_table(data):
+    """Tables.istable: a pandas DataFrame or a dict of equally long columns."""
+    if isinstance(data, dict):
+        return True
+    return hasattr(data, "columns") and hasattr(data, "dtypes")
+
+
+def _column(data, name):
+    """Tables.getcolumn as a numpy array or a pandas Categorical."""
+    col = data[name]
+    if hasattr(col, "dtype") and str(col.dtype) == "category":
+        return col.array if hasattr(col, "array") else col
+    return np.asarray(col)
+
+
+def _is_categorical(col):
+    return hasattr(col, "categories") and hasattr(col, "codes")
+
+
+def _table_names(data):
+    return [str(c) for c in (data.keys() if isinstance(data, dict) else data.columns)]
+
+
+def get_edges_table(data, feature_names, nbins, rng):
+    """get_edges for Tables input, src/fit-utils.jl:26-63: a Bool column is a two-level categorical feature, a
+    categorical column is split on its levels (`==`, or `<=` when its levels are ordered), a Real column on the unique
+    quantiles of the sampled rows."""
+    nrow = len(_column(data, feature_names[0]))
+    nobs = min(nrow, 1000 * nbins)
+    idx = np.sort(rng.choice(nrow, nobs, replace=False)) if nobs < nrow else np.arange(nrow)
+    q = np.arange(1, nbins) / nbins
+    edges, featbins, feattypes = [], [], []
+    for name in feature_names:
+        col = _column(data, name)
+        if _is_categorical(col):
+            e = list(col.categories)
+            nb, ft = len(e), bool(col.ordered)
+            if nb > nbins:
+                raise RuntimeError("Max categorical levels is limited to `nbins` (%d). Feature %s has %d levels. Consider using larger "
+                                   "`nbins`, up to 255." % (nbins, name, nb))
+        elif col.dtype == np.bool_:
+            e, nb, ft = [False, True], 2, False
+        elif col.dtype.kind in "iuf":
+            sub = np.asarray(col[idx], np.float64)
+            e = np.unique(np.quantile(sub, q))
+            if e.shape[0] == 1:
+                e = np.array([sub.min()])
+            e = np.ascontiguousarray(e)
+            nb, ft = len(e) + 1, True
+        else:
+            raise RuntimeError("Invalid feature eltype: %s is %s" % (name, col.dtype))
+        edges.append(e)
+        featbins.append(nb)
+        feattypes.append(1 if ft else 0)
+    return edges, np.array(featbins, np.uint8), np.array(feattypes, np.uint8)
+
+
+def binarize_table(data, feature_names, edges):
+    """binarize for Tables input, src/fit-utils.jl:74-92 -> (F, N) uint8 (the memory order of Julia's N x F matrix)."""
+    nrow = len(_column(data, feature_names[0]))
+    out = np.empty((len(feature_names), nrow), np.uint8)
+    for j, name in enumerate(feature_names):
+        col = _column(data, name)
+        if _is_categorical(col):
+            if list(col.categories) != list(edges[j]):  # levelcode refers to the training levels
+                col = col.set_categories(list(edges[j]))
+            codes = np.asarray(col.codes)
+            if (codes < 0).any():
+                raise RuntimeError("feature %s holds missing values or levels the model was not trained on" % name)
+            out[j] = codes + 1
+        elif col.dtype == np.bool_:
+            out[j] = col.astype(np.uint8) + 1
+        elif col.dtype.kind in "iuf":
+            out[j] = binarize(np.asarray(col, np.float64)[:, None], [edges[j]])[0]
+        else:
+            raise RuntimeError("Invalid feature eltype: %s is %s" % (name, col.dtype))
+    return out
+
+
+def _table_features(data, target_names, weight_name, offset_name, feature_names):
+    """Feature columns of a table: the names given, or every Real / categorical column that is not the target, the
+    weight or the offset (src/init.jl:253-282)."""
+    names = _table_names(data)
+    if feature_names is None:
+        skip = set(target_names) | {weight_name, offset_name}
+        out = []
+        for n in names:
+            col = _column(data, n)
+            if n not in skip and (_is_categorical(col) or col.dtype == np.bool_ or col.dtype.kind in "iuf"):
+                out.append(n)
+        return out
+    out = [feature_names] if isinstance(feature_names, str) else [str(f) for f in feature_names]
+    for n in out:
+        if n not in names:
+            raise AssertionError("feature %s is not a column of the table" % n)
+    return out
+
+
+def _table_target(data, target_name):
+    names = [str(t) for t in target_name] if isinstance(target_name, (list, tuple)) else [str(target_name)]
+    if len(names) == 1:
+        return names, np.asarray(data[names[0]])
+    return names, np.stack([np.asarray(data[t]) for t in names])  # targets x observations
+
+
 class Cache:
     """What CacheBaseGPU holds on the host side: the device handle plus RNG and sampling sizes."""
 
@@ -242,18 +347,32 @@ class Cache:
         self.next_mask = None  # ... or drawn only (few rows: the upload is not worth a second stream)
 
 
-def init(config, x_train, y_train, w_train=None, offset_train=None, feature_names=None, device=None):
-    """init / init_core for the GPU device (src/init.jl:316-339; ext/EvoTreesKernelAbstractionsExt/init.jl:1-151)."""
+def init(config, x_train, y_train=None, w_train=None, offset_train=None, feature_names=None, device=None, target_name=None, weight_name=None,
+         offset_name=None):
+    """init / init_core for the GPU device (src/init.jl:236-339; ext/EvoTreesKernelAbstractionsExt/init.jl:1-151).  x_train is a
+    matrix (with y_train, w_train, offset_train) or a table (with target_name, weight_name, offset_name)."""
     _device_check(config.device if device is None else device)
-    x = np.asarray(x_train)
-    if x.ndim != 2:
-        raise ValueError("x_train must be a matrix")
-    N, F = x.shape
-    feature_names = ["feat_%d" % (j + 1) for j in range(F)] if feature_names is None else [str(f) for f in feature_names]
-    if len(feature_names) != F:
-        raise AssertionError("length(feature_names) must equal size(x_train, 2)")
     rng = np.random.default_rng(config.seed)
-    edges, featbins, feattypes = get_edges(x, config.nbins, rng)
+    table = _is_table(x_train)
+    if table:
+        if target_name is None:
+            raise TypeError("target_name is required for a table")
+        target_names, y_train = _table_target(x_train, target_name)
+        feature_names = _table_features(x_train, target_names, weight_name, offset_name, feature_names)
+        w_train = None if weight_name is None else np.asarray(x_train[str(weight_name)])
+        offset_train = None if offset_name is None else np.asarray(x_train[str(offset_name)])
+        F = len(feature_names)
+        N = len(_column(x_train, feature_names[0]))
+        edges, featbins, feattypes = get_edges_table(x_train, feature_names, config.nbins, rng)
+    else:
+        x = np.asarray(x_train)
+        if x.ndim != 2:
+            raise ValueError("x_train must be a matrix")
+        N, F = x.shape
+        feature_names = ["feat_%d" % (j + 1) for j in range(F)] if feature_names is None else [str(f) for f in feature_names]
+        if len(feature_names) != F:
+            raise AssertionError("length(feature_names) must equal size(x_train, 2)")
+        edges, featbins, feattypes = get_edges(x, config.nbins, rng)
     K, y32, mu, target_levels = _init_target(config.loss, y_train)
     if y32.shape[0] != N:
         raise AssertionError("target length must equal the number of rows")
@@ -267,8 +386,10 @@ def init(config, x_train, y_train, w_train=None, offset_train=None, feature_name
         offset = _link_offset(config.loss, offset_train, N, K)
         mu = np.zeros_like(mu)  # neutral bias when an offset is given (src/init.jl:164)
     h = Handle(N, F, config.nbins, K, config.max_depth, config.loss, config.tree_type)
-    x_FN = np.ascontiguousarray(x.T, np.float64)
-    h.binarize(x_FN, edges)
+    if table:  # Bool and categorical columns have no edges to search: binned on the host as the reference does
+        h.set_xbin(binarize_table(x_train, feature_names, edges))
+    else:
+        h.binarize(np.ascontiguousarray(x.T, np.float64), edges)
     mono = np.zeros(F, np.int32)
     for k, v in config.monotone_constraints.items():
         mono[int(k) - 1] = int(v)
@@ -335,9 +456,17 @@ class CallBack:
     """CallBack (src/callback.jl:21-135) on the device: a second handle holds the binned eval rows, their
     running prediction, target and weights; each call adds one tree and evaluates the metric there."""
 
-    def __init__(self, config, m, x_eval, y_eval, w_eval=None, offset_eval=None):
-        x = np.asarray(x_eval)
-        N, F = x.shape
+    def __init__(self, config, m, x_eval, y_eval=None, w_eval=None, offset_eval=None, target_name=None, weight_name=None, offset_name=None):
+        table = _is_table(x_eval)
+        if table:  # the Tables form, src/callback.jl:31-80
+            _, y_eval = _table_target(x_eval, target_name)
+            w_eval = None if weight_name is None else np.asarray(x_eval[str(weight_name)])
+            offset_eval = None if offset_name is None else np.asarray(x_eval[str(offset_name)])
+            x_bin = binarize_table(x_eval, m.info["feature_names"], m.info["edges"])
+            F, N = x_bin.shape
+        else:
+            x = np.asarray(x_eval)
+            N, F = x.shape
         self.metric = config.metric
         self.maximise = _MAXIMISE[config.metric]
         if m.loss_type == "mlogloss":
@@ -351,7 +480,10 @@ class CallBack:
         offset = None if offset_eval is None else _link_offset(m.loss_type, offset_eval, N, m.K)
         h = Handle(N, F, config.nbins, m.K, 1, m.loss_type, "binary")
         try:
-            h.binarize(np.ascontiguousarray(x.T, np.float64), m.info["edges"])
+            if table:
+                h.set_xbin(x_bin)
+            else:
+                h.binarize(np.ascontiguousarray(x.T, np.float64), m.info["edges"])
             h.set_feature_meta(m.info["feattypes"], None)
             h.set_target(y32, w, np.zeros(m.K, np.float32), offset)  # p = zeros (+ offset'), src/callback.jl:104, :82
         except Exception:
@@ -392,15 +524,31 @@ def update_logger(logger, it, metric):
         logger["iter_since_best"] += logger["iter"][-1] - logger["iter"][-2]
 
 
-def fit(config, x_train=None, y_train=None, w_train=None, offset_train=None, x_eval=None, y_eval=None, w_eval=None, offset_eval=None,
-        feature_names=None, print_every_n=9999, device=None, verbosity=1, return_cache=False):
-    """fit(params; x_train, y_train, ..., x_eval, y_eval, ...), src/fit.jl:388-437."""
-    if x_train is None or y_train is None:
-        raise TypeError("x_train and y_train are required")
-    m, cache = init(config, x_train, y_train, w_train=w_train, offset_train=offset_train, feature_names=feature_names, device=device)
+def fit(config, dtrain=None, x_train=None, y_train=None, w_train=None, offset_train=None, x_eval=None, y_eval=None, w_eval=None, offset_eval=None,
+        feature_names=None, print_every_n=9999, device=None, verbosity=1, return_cache=False, target_name=None, weight_name=None,
+        offset_name=None, deval=None):
+    """fit(params; x_train, y_train, ..., x_eval, y_eval, ...), src/fit.jl:388-437, and the Tables form
+    fit(params, dtrain; target_name, feature_names, weight_name, offset_name, deval), src/fit.jl:302-345."""
+    if dtrain is not None:
+        if not _is_table(dtrain):
+            raise AssertionError("fit(params, dtrain) only accepts Tables compatible input for `dtrain` (a DataFrame or a dict of columns)")
+        m, cache = init(config, dtrain, feature_names=feature_names, device=device, target_name=target_name, weight_name=weight_name,
+                        offset_name=offset_name)
+        m.info["target_names"] = [str(t) for t in target_name] if isinstance(target_name, (list, tuple)) else [str(target_name)]
+        x_eval, y_eval = None, None
+    else:
+        if x_train is None or y_train is None:
+            raise TypeError("x_train and y_train are required")
+        m, cache = init(config, x_train, y_train, w_train=w_train, offset_train=offset_train, feature_names=feature_names, device=device)
     logger, cb = None, None
     try:
-        if x_eval is not None and y_eval is not None:
+        if dtrain is not None and deval is not None:
+            cb = CallBack(config, m, deval, target_name=target_name, weight_name=weight_name, offset_name=offset_name)
+            logger = init_logger(config.metric, cb.maximise, config.early_stopping_rounds, config.early_stopping_tolerance)
+            cb(logger, 0, m.trees[-1])
+            if verbosity > 0:
+                print("initialization: %s = %.6g" % (config.metric, logger["metrics"][-1]))
+        elif x_eval is not None and y_eval is not None:
             cb = CallBack(config, m, x_eval, y_eval, w_eval=w_eval, offset_eval=offset_eval)
             logger = init_logger(config.metric, cb.maximise, config.early_stopping_rounds, config.early_stopping_tolerance)
             cb(logger, 0, m.trees[-1])
@@ -470,6 +618,10 @@ def predict(m, data, ntree_limit=None, device="gpu"):
     ntree_limit = ntrees if ntree_limit is None else ntree_limit
     if ntree_limit > ntrees:
         raise RuntimeError("ntree_limit is larger than number of trees %d." % ntrees)
+    if _is_table(data):  # Bool / categorical columns: binned on the host (src/fit-utils.jl:74-92), walked on the device
+        x_bin = binarize_table(data, m.info["feature_names"], m.info["edges"])
+        p = _lib.predict_model(x_bin, m.info["feattypes"], m.loss_type, m.K, m.trees[:ntree_limit], apply_link=True)
+        return p[:, 0].copy() if m.K == 1 else p
     x_FN = np.ascontiguousarray(np.asarray(data).T, np.float64)
     p = _lib.predict_model_f64(x_FN, m.info["edges"], m.info["feattypes"], m.loss_type, m.K, m.trees[:ntree_limit], apply_link=True)
     return p[:, 0].copy() if m.K == 1 else p
@@ -482,5 +634,5 @@ def predict_leaf_idx(m, data, ntree_limit=None, device="gpu"):
     ntree_limit = ntrees if ntree_limit is None else ntree_limit
     if ntree_limit > ntrees:
         raise RuntimeError("ntree_limit is larger than number of trees %d." % ntrees)
-    x_bin = binarize(data, m.info["edges"])
+    x_bin = binarize_table(data, m.info["feature_names"], m.info["edges"]) if _is_table(data) else binarize(data, m.info["edges"])
     return _lib.predict_leaf_idx(x_bin, m.info["feattypes"], m.trees[:ntree_limit])
