@@ -134,12 +134,14 @@ def prepare(evt, cfg, opts=None):
 
 class Rounds:
     """Boosting rounds on a prepared handle, as the host mirror's grow_evotree drives them: gradients, the column sample,
-    the tree in two halves with the next round's mask drawn (and for many rows uploaded) in between."""
+    the row mask drawn on the device from one 64-bit draw of the host's generator, the tree.  host_mask=True draws one
+    byte per row on the host instead (the reference's rand!(rng, mask), src/subsample.jl:7) and uploads it while the
+    previous tree grows."""
 
-    # below a few million rows a round is bound by the host's launches and the second stream's copy costs more than it hides
+    # below a few million rows the second stream's copy of a host-drawn mask costs more than it hides
     STAGE_MASK_MIN_ROWS = 4_000_000
 
-    def __init__(self, evt, h, cfg, rng):
+    def __init__(self, evt, h, cfg, rng, host_mask=False):
         self.evt, self.h, self.cfg, self.rng = evt, h, cfg, rng
         self.N, self.F = cfg["N"], cfg["F"]
         self.K = 2 if cfg["loss"] == "gaussian_mle" else 1
@@ -149,27 +151,40 @@ class Rounds:
         self.L = evt._lib.load()
         self.tree = evt.Tree(self.K, h.nnodes)
         self.tree_out = self.tree.as_out()
-        # the host owns the row-sampling RNG (one uniform byte per row, drawn every round): raw 64-bit words viewed as bytes;
-        # numpy's fastest bulk generator: the draw is host work inside the timed region
+        self.host_mask = host_mask
+        # host-drawn masks: raw 64-bit words viewed as bytes, numpy's fastest bulk generator (4 ns per word)
         self.mask_rng = np.random.Generator(np.random.SFC64(124))
         self.staged = False
         self.nxt = None
+        self.nxt_draws = None
         h.set_option("grads_ahead", 1)  # one tree per round: the next round's gradients are queued behind the tree
 
     def draw_mask(self):
         return None if self.cond >= 255 else self.mask_rng.bit_generator.random_raw((self.N + 7) // 8).view(np.uint8)[:self.N]
 
-    def one_round(self):
-        evt, h, L, F = self.evt, self.h, self.L, self.F
-        h.update_grads()
+    def draws(self):
+        """The host generator's draws of one round: the mask's seed, then the column sample."""
+        seed = int(self.rng.integers(0, 1 << 64, dtype=np.uint64)) if self.cond < 255 and not self.host_mask else None
+        F = self.F
         js = np.arange(1, F + 1, dtype=np.uint32) if self.nfs >= F else (np.sort(self.rng.choice(F, self.nfs, replace=False)) + 1).astype(np.uint32)
-        if self.staged:
+        return seed, js
+
+    def one_round(self):
+        evt, h, L = self.evt, self.h, self.L
+        h.update_grads()
+        seed, js = self.nxt_draws if self.nxt_draws is not None else self.draws()
+        if seed is not None:
+            h.draw_mask(seed)
+            evt._lib.check(L.evt_grow_tree_begin_staged(h._h, self.cond, evt._lib.ptr(js), js.shape[0], self.params))
+        elif self.staged:
             evt._lib.check(L.evt_grow_tree_begin_staged(h._h, self.cond, evt._lib.ptr(js), js.shape[0], self.params))
         else:
             mask = self.nxt if self.nxt is not None else self.draw_mask()
             evt._lib.check(L.evt_grow_tree_begin(h._h, evt._lib.ptr(mask), self.cond, evt._lib.ptr(js), js.shape[0], self.params))
-        if self.cond < 255:
-            # the next round's mask is drawn (and, for many rows, uploaded) while the device grows this round's tree
+        # the host's work for the next round while the device grows this round's tree
+        self.nxt_draws = self.draws()
+        if self.cond < 255 and self.host_mask:
+            # one byte per row, drawn and (for many rows) uploaded
             self.nxt = self.draw_mask()
             if self.N >= self.STAGE_MASK_MIN_ROWS:
                 h.stage_mask(self.nxt)
@@ -212,7 +227,7 @@ def hist_roofline(cfg, prof_hist, nfs, NK):
     return achieved, bytes_per_row
 
 
-def side_workload(evt, name, steps, h=None, y=None, mu=None, rng=None):
+def side_workload(evt, name, steps, h=None, y=None, mu=None, rng=None, host_mask=False):
     """One of BASELINE.json's other configurations, a few dozen rounds: ms per round, seconds per 200 rounds and the
     histogram kernel's fraction of the HBM peak.  cfg3s runs on the headline workload's own handle (same matrix)."""
     cfg = dict(WORKLOADS[name])
@@ -220,7 +235,7 @@ def side_workload(evt, name, steps, h=None, y=None, mu=None, rng=None):
     t_init = None
     if own:
         h, y, mu, rng, t_init = prepare(evt, cfg)
-    r = Rounds(evt, h, cfg, rng)
+    r = Rounds(evt, h, cfg, rng, host_mask=host_mask)
     ms, ph, sampled = r.timed(steps, 3)
     K = r.K
     ach, _ = hist_roofline(cfg, ph, r.nfs, 2 * K + 1)
@@ -436,6 +451,10 @@ def main():
         side = {}
         try:
             side["cfg3s"] = side_workload(evt, "cfg3s", args.side_steps, h, y, mu, rng)
+            side["cfg3s"]["mask"] = "drawn on the device from one 64-bit seed per tree (evt_draw_mask)"
+            # the same rounds with one byte per row drawn by the host every round and uploaded while the last tree grows
+            side["cfg3s_hostmask"] = side_workload(evt, "cfg3s", max(1, args.side_steps // 2), h, y, mu, rng, host_mask=True)
+            side["cfg3s_hostmask"]["mask"] = "drawn on the host (numpy, 4 ns per 8 bytes), uploaded on a second stream"
         except Exception as e:  # measurement aid only
             side["cfg3s"] = {"error": str(e)}
         out["workloads"] = side

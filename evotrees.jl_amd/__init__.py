@@ -5,7 +5,8 @@ hot path: learner configs (src/learners.jl), `fit(config; x_train, y_train, ...)
 
 Everything data parallel runs in libevotrees_hip.so through the C ABI; this module only keeps
 what the reference keeps on the host: argument checks, quantile edges, the bias, the random
-row mask / column sample, and the list of trees.  There is no CPU compute path: `device` must be
+column sample, the seed of each tree's row mask (the mask bytes themselves are drawn on the
+device from it), and the list of trees.  There is no CPU compute path: `device` must be
 a GPU device name and the shared library must be present.
 
 Julia is not available where this package is developed, so the host side is Python; the random
@@ -15,7 +16,7 @@ Julia run with the same seed — the trees are identical for identical masks/col
 import numpy as np
 
 from . import _lib
-from ._lib import EvtError, Handle, TreeArrays, make_params  # noqa: F401
+from ._lib import EvtError, Handle, TreeArrays, make_params, splitmix_mask  # noqa: F401
 
 __all__ = ["EvoTreeRegressor", "EvoTreeCount", "EvoTreeClassifier", "EvoTreeMLE", "EvoTree", "Tree", "fit", "predict", "predict_leaf_idx", "init",
            "grow_evotree", "update", "okay_to_continue", "get_edges", "get_edges_table", "binarize_table", "check_args", "CallBack", "init_logger", "update_logger", "EvtError"]
@@ -343,8 +344,7 @@ class Cache:
 
     def __init__(self, handle, rng, nfs, params, N, F, config=None):
         self.handle, self.rng, self.nfs, self.params, self.N, self.F, self.config = handle, rng, nfs, params, N, F, config
-        self.mask_staged = False  # the row mask of the next tree has been drawn and uploaded while the device grew the last one
-        self.next_mask = None  # ... or drawn only (few rows: the upload is not worth a second stream)
+        self.next_draw = None  # (mask seed, column sample) of the next tree, drawn while the device grew the last one
 
 
 def init(config, x_train, y_train=None, w_train=None, offset_train=None, feature_names=None, device=None, target_name=None, weight_name=None,
@@ -405,44 +405,39 @@ def init(config, x_train, y_train=None, w_train=None, offset_train=None, feature
     return m, Cache(h, rng, nfs, params, N, F, config)
 
 
-# Rows from which the next tree's mask is drawn and uploaded while the current tree grows; below, a round is bound by the
-# host's launches and the second stream's copy costs more than it hides.
-STAGE_MASK_MIN_ROWS = 4_000_000
-
-
 def grow_evotree(m, cache, config):
-    """grow_evotree!, src/fit.jl:6-42 (device twin ext/.../fit.jl:1-21): gradients, then bagging_size trees."""
+    """grow_evotree!, src/fit.jl:6-42 (device twin ext/.../fit.jl:1-21): gradients, then bagging_size trees.
+
+    The row mask of a tree (rand!(rng, mask), src/subsample.jl:7) is drawn on the device from ONE 64-bit draw of the
+    fit's generator per tree (Handle.draw_mask: SplitMix64 keyed by that draw; splitmix_mask gives the same bytes on the
+    host): numpy needs 4 ns per 8 mask bytes, which at a million rows is already longer than the device takes to grow
+    the tree.  The bytes are compared with round(UInt8, 255 * rowsample) exactly as an uploaded mask is."""
     h = cache.handle
     h.update_grads()
     cond = int(np.rint(255 * config.rowsample))  # round(UInt8, 255*rowsample), src/subsample.jl:9
-    for _ in range(config.bagging_size):
-        # all rows pass `mask <= 255`, so the draw is skipped when nothing can be dropped
-        mask = None
-        staged = cache.mask_staged  # this tree's mask was drawn and uploaded while the device grew the last tree
-        if cond < 255 and not staged:
-            mask = cache.next_mask if cache.next_mask is not None else cache.rng.integers(0, 256, cache.N, dtype=np.uint8)
-            cache.next_mask = None
+
+    def draw():
+        # the generator's draws of one tree, in the reference's order (mask, then columns; src/fit.jl:13-20).  All rows
+        # pass `mask <= 255`, so nothing is drawn for the mask when nothing can be dropped
+        seed = int(cache.rng.integers(0, 1 << 64, dtype=np.uint64)) if cond < 255 else None
         if cache.nfs >= cache.F:
             js = np.arange(1, cache.F + 1, dtype=np.uint32)
         else:
             js = (np.sort(cache.rng.choice(cache.F, cache.nfs, replace=False)) + 1).astype(np.uint32)
+        return seed, js
+
+    for _ in range(config.bagging_size):
+        seed, js = cache.next_draw if cache.next_draw is not None else draw()
+        cache.next_draw = None
         t = Tree(m.K, h.nnodes)
         out = t.as_out()
         try:
-            if staged:
-                cache.mask_staged = False
+            if seed is not None:
+                h.draw_mask(seed)
                 _lib.check(_lib.load().evt_grow_tree_begin_staged(h._h, cond, _lib.ptr(js), js.shape[0], cache.params))
             else:
-                _lib.check(_lib.load().evt_grow_tree_begin(h._h, _lib.ptr(mask), cond, _lib.ptr(js), js.shape[0], cache.params))
-            if cond < 255:
-                # the next draw of the RNG stream is the next tree's mask: made (and, for many rows, uploaded) while the
-                # device grows this tree
-                nm = cache.rng.integers(0, 256, cache.N, dtype=np.uint8)
-                if cache.N >= STAGE_MASK_MIN_ROWS:
-                    h.stage_mask(nm)
-                    cache.mask_staged = True
-                else:
-                    cache.next_mask = nm
+                _lib.check(_lib.load().evt_grow_tree_begin(h._h, None, cond, _lib.ptr(js), js.shape[0], cache.params))
+            cache.next_draw = draw()  # the next tree's draws, made while the device grows this one
             _lib.check(_lib.load().evt_grow_tree_end(h._h, out))
         except EvtError as e:
             if e.code == _lib.EVT_ERR_EMPTY:

@@ -21,7 +21,7 @@ KERNEL_CLASSES = ["grad", "hist", "scan", "partition", "predict", "other"]
 EXPORTS = [
     "evt_last_error", "evt_device_count", "evt_create", "evt_destroy", "evt_set_xbin", "evt_binarize_f64",
     "evt_set_target", "evt_set_feature_meta", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
-    "evt_grow_tree_begin", "evt_grow_tree_end", "evt_stage_mask", "evt_grow_tree_begin_staged",
+    "evt_grow_tree_begin", "evt_grow_tree_end", "evt_stage_mask", "evt_grow_tree_begin_staged", "evt_draw_mask",
     "evt_tree_open", "evt_hist_build", "evt_split_scan", "evt_update_nodes_idx", "evt_tree_close", "evt_peek_tree",
     "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
     "evt_predict", "evt_predict_f64", "evt_predict_leaf_idx", "evt_eval_metric", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
@@ -74,6 +74,7 @@ def load():
         "evt_grow_tree_begin": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams)],
         "evt_grow_tree_end": [vp, C.POINTER(EvtTreeOut)],
         "evt_stage_mask": [vp, vp],
+        "evt_draw_mask": [vp, C.c_uint64],
         "evt_grow_tree_begin_staged": [vp, C.c_uint8, vp, i32, C.POINTER(EvtParams)],
         "evt_tree_open": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams)],
         "evt_hist_build": [vp, i32],
@@ -238,6 +239,11 @@ class Handle:
         assert mask.shape == (self.N,)
         check(load().evt_stage_mask(self._h, ptr(mask)))
 
+    def draw_mask(self, seed):
+        """The next tree's row mask drawn on the device: SplitMix64 started at `seed`, 8 mask bytes per output (see
+        splitmix_mask for the same bytes on the host).  Takes the place of stage_mask."""
+        check(load().evt_draw_mask(self._h, int(seed) & 0xFFFFFFFFFFFFFFFF))
+
     def grow_tree_begin_staged(self, js, params, cond):
         """grow_tree_begin with the mask last given to stage_mask."""
         js = np.ascontiguousarray(js, np.uint32)
@@ -344,6 +350,19 @@ class Handle:
 
     def synchronize(self):
         check(load().evt_synchronize(self._h))
+
+
+def splitmix_mask(seed, N):
+    """The bytes Handle.draw_mask(seed) writes on the device, computed on the host: output w (from 0) of SplitMix64
+    started at `seed` holds mask bytes 8w .. 8w+7, little end first."""
+    M = (1 << 64) - 1
+    with np.errstate(over="ignore"):
+        w = np.arange(1, (int(N) + 7) // 8 + 1, dtype=np.uint64)
+        z = np.uint64(int(seed) & M) + w * np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        z ^= z >> np.uint64(31)
+    return z.astype("<u8").view(np.uint8)[:int(N)]
 
 
 def make_params(eta=0.1, L2=1.0, lambda_=0.0, gamma=0.0, min_weight=1.0, bagging_size=1, update_pred=True):

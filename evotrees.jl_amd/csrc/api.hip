@@ -255,7 +255,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     // the flushes per node
     c->hist_blocks = 256;
     c->hist_threads = 1024;
-    c->hist_min_rows = 2048;
+    c->hist_min_rows = 1024;
     c->hist_variant = 0;
     c->hist_seg_cost = 2048;
     c->record_nidx = false;
@@ -351,7 +351,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->jsmap, c->RS);
     ALLOC(c->feattypes, c->F);
     ALLOC(c->mono, c->F);
-    ALLOC(c->absmax, EVT_MC_MAX_NK);
+    ALLOC(c->absmax, EVT_ABSMAX_STRIPES * EVT_MC_MAX_NK);
     for (int s = 0; s < 2; s++) {
         ALLOC(c->qexp_buf[s], EVT_MC_MAX_NK);
         ALLOC(c->qscale_buf[s], 2 * EVT_MC_MAX_NK);
@@ -385,7 +385,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
         c->h_feattypes = ft;
         hipError_t e2 = hipMemcpy(c->feattypes, ft.data(), c->F, hipMemcpyHostToDevice);
         if (e2 == hipSuccess) e2 = hipMemset(c->mono, 0, sizeof(int32_t) * c->F);
-        if (e2 == hipSuccess) e2 = hipMemset(c->absmax, 0, sizeof(uint32_t) * EVT_MC_MAX_NK);
+        if (e2 == hipSuccess) e2 = hipMemset(c->absmax, 0, sizeof(uint32_t) * EVT_ABSMAX_STRIPES * EVT_MC_MAX_NK);
         if (e2 == hipSuccess) e2 = hipMemset(c->nidx, 0, sizeof(uint32_t) * N);
         if (e2 == hipSuccess) e2 = hipMemset(c->errflag, 0, sizeof(int32_t));
         if (e2 != hipSuccess) {
@@ -740,8 +740,7 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
         // before the next tree, which starts after this one has been collected
         {
             const size_t o_js = c->blob_bytes, o_map = c->blob_bytes + (size_t)c->F * 4;
-            int rr = launch_copy_words(c, c->h_stage_dev + o_js, c->js, sizeof(uint32_t) * n_js);
-            if (rr == EVT_OK) rr = launch_copy_words(c, c->h_stage_dev + o_map, c->jsmap, sizeof(uint16_t) * c->RS);
+            int rr = launch_copy_words2(c, c->h_stage_dev + o_js, c->js, sizeof(uint32_t) * n_js, c->h_stage_dev + o_map, c->jsmap, sizeof(uint16_t) * c->RS);
             if (rr != EVT_OK) return rr;
         }
         c->n_js_last = n_js;
@@ -936,11 +935,33 @@ extern "C" int evt_stage_mask(evt_handle c, const uint8_t *mask) {
     });
 }
 
+// The next tree's mask drawn by the device from a 64-bit seed (no nobs-byte draw on the host, no upload): written on
+// the handle's own stream into the buffer the tree in flight does not read.
+extern "C" int evt_draw_mask(evt_handle c, uint64_t seed) {
+    return guarded([&]() -> int {
+    ARGCHK(c != nullptr, "handle is NULL");
+    HIPCHK(hipSetDevice(c->device));
+    if (c->step.phase != 0) {
+        evt_set_error("a tree opened with evt_tree_open has not been closed (evt_tree_close)");
+        return EVT_ERR_STATE;
+    }
+    if (!c->mask_next) {
+        int r = dev_alloc(&c->mask_next, (size_t)c->N);
+        if (r != EVT_OK) return r;
+    }
+    c->mask_next_valid = false;
+    int r = launch_draw_mask(c, c->mask_next, (unsigned long long)seed);
+    if (r != EVT_OK) return r;
+    c->mask_next_valid = true;
+    return EVT_OK;
+    });
+}
+
 extern "C" int evt_grow_tree_begin_staged(evt_handle c, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
     return guarded([&]() -> int {
     CTXCHK(c);
     if (!c->mask_next_valid) {
-        evt_set_error("evt_grow_tree_begin_staged: no mask has been staged since the last tree (evt_stage_mask)");
+        evt_set_error("evt_grow_tree_begin_staged: no mask has been staged since the last tree (evt_stage_mask / evt_draw_mask)");
         return EVT_ERR_STATE;
     }
     int r = tree_open(c, nullptr, true, cond, js, n_js, p, false);

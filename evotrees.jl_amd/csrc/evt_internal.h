@@ -20,6 +20,9 @@
 #define EVT_MAX_NK 5  // gradient rows of the one- and two-output losses (register arrays of the specialised kernels)
 #define EVT_MAX_NA 5
 #define EVT_MAX_K 16     // classes of the multi-class loss
+// the running maxima of the gradient rows are kept in EVT_ABSMAX_STRIPES copies, one 160-byte stripe each, and a block
+// raises the copy of stripe blockIdx % EVT_ABSMAX_STRIPES: same-address atomics queue up one behind the other
+#define EVT_ABSMAX_STRIPES 32
 #define EVT_MC_MAX_NK 40 // >= 2 * EVT_MAX_K + 1: sizes of the per-row quantisation tables and of the generic kernels' arrays
 #define EVT_HIST_GROUP 4 // accumulator channels one histogram launch handles; more channels take several launches
 #define EVT_METRIC_BLOCKS 1024 // partial sums of the evaluation metric
@@ -119,7 +122,7 @@ struct evt_ctx {
     uint16_t *jsmap;   // [RS] slot of feature f (0-based), 0xFFFF = not sampled / padding
     uint8_t *feattypes;
     int32_t *mono;
-    uint32_t *absmax;  // [EVT_MC_MAX_NK] float bits
+    uint32_t *absmax;  // [EVT_ABSMAX_STRIPES][EVT_MC_MAX_NK] float bits
     int32_t *qexp;     // [EVT_MC_MAX_NK]; points into qexp_buf: the tables of the gradients quantised last
     int32_t *qbits;    // [EVT_MC_MAX_NK]
     double *qscale;    // [2 * EVT_MC_MAX_NK]: decode scale per global channel, then encode multiplier per gradient row
@@ -271,6 +274,7 @@ int launch_eval_metric(evt_ctx *c, int metric, double *partial);
 int launch_tree_begin(evt_ctx *c, bool all_rows);
 int launch_iota(evt_ctx *c, uint32_t *dst, int64_t n);
 int launch_compact_mask(evt_ctx *c, uint8_t cond);
+int launch_draw_mask(evt_ctx *c, uint8_t *mask, unsigned long long seed);
 int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level);
 int launch_obliv_select(evt_ctx *c, int level, const evt_params *p);
@@ -280,6 +284,7 @@ int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_
 int launch_nidx_from_segments(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_copy_to_host(evt_ctx *c, const void *src_dev, void *dst_host_dev, size_t nbytes);
 int launch_copy_words(evt_ctx *c, const void *src, void *dst, size_t nbytes);
+int launch_copy_words2(evt_ctx *c, const void *src0, void *dst0, size_t nbytes0, const void *src1, void *dst1, size_t nbytes1);
 int launch_fill_u32(evt_ctx *c, uint32_t *dst, uint32_t v, int64_t n);
 int launch_fill_bytes(evt_ctx *c, void *dst, int64_t nbytes);
 // predict

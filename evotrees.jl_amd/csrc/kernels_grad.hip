@@ -41,6 +41,18 @@ __device__ __forceinline__ void mle2p_grad_hess(float loc, float raw, float y, f
     }
 }
 
+// Raises the running maximum of gradient row k.  Same-address atomics from thousands of blocks queue up one behind the
+// other (about 20 ns each - 40 us for the 2048 blocks of a gradient pass), so the maximum is kept in
+// EVT_ABSMAX_STRIPES copies on different cache lines, a block raises the copy its index selects, and the one reader
+// (k_quant_setup) takes the largest.  The value only grows while a pass runs: a block whose own maximum is already
+// covered by what a device-scope load shows skips the atomic.
+__device__ __forceinline__ void absmax_raise(uint32_t *absmax, int k, float m) {
+    if (!(m > 0.0f)) return;
+    uint32_t *p = absmax + (blockIdx.x % EVT_ABSMAX_STRIPES) * EVT_MC_MAX_NK + k;
+    const uint32_t u = __float_as_uint(m);
+    if (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < u) atomicMax(p, u);
+}
+
 // LOSS: 0 mse (src/loss.jl:52), 1 logloss (:54-57), 2 gaussian_mle (:194-203), 3 poisson (:59-62),
 // 4 gamma (:64-67), 5 tweedie with rho = 1.5 (:69-76).
 // grad rows: [g_1..g_K, h_1..h_K, w]; every written value is multiplied by w (src/loss.jl:104-108, :223-233).
@@ -105,7 +117,7 @@ __global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const f
     if (threadIdx.x < 2 * K) {
         const int k = threadIdx.x;
         const float m = fmaxf(fmaxf(s_m[0][k], s_m[1][k]), fmaxf(s_m[2][k], s_m[3][k]));
-        if (m > 0.0f) atomicMax(&absmax[k], __float_as_uint(m));
+        absmax_raise(absmax, k, m);
     }
 }
 
@@ -189,7 +201,7 @@ __global__ __launch_bounds__(256) void k_grads_mt(float *__restrict__ pred, cons
             if (threadIdx.x == 0) {
                 const float mm = fmaxf(fmaxf(s_m[0], s_m[1]), fmaxf(s_m[2], s_m[3]));
                 const int row = k < EVT_MAX_K ? k : K + kk;
-                if (mm > 0.0f) atomicMax(&absmax[row], __float_as_uint(mm));
+                absmax_raise(absmax, row, mm);
             }
         }
     }
@@ -243,7 +255,7 @@ __global__ __launch_bounds__(256) void k_grads_mlogloss(float *__restrict__ pred
             __syncthreads();
             if (threadIdx.x == 0) {
                 const float mm = fmaxf(fmaxf(s_m[0], s_m[1]), fmaxf(s_m[2], s_m[3]));
-                if (mm > 0.0f) atomicMax(&absmax[k < EVT_MAX_K ? kk : K + kk], __float_as_uint(mm));
+                absmax_raise(absmax, k < EVT_MAX_K ? kk : K + kk, mm);
             }
         }
     }
@@ -257,7 +269,7 @@ __global__ __launch_bounds__(256) void k_absmax(const float *__restrict__ grad, 
         for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256)
             m = fmaxf(m, fabsf(grad[(size_t)NK * i + k]));
         const float v = wave_max_f32(m);
-        if ((threadIdx.x & 63) == 0 && v > 0.0f) atomicMax(&absmax[k], __float_as_uint(v));
+        if ((threadIdx.x & 63) == 0) absmax_raise(absmax, k, v);
     }
 }
 
@@ -268,7 +280,12 @@ __global__ void k_quant_setup(uint32_t *absmax, const int32_t *qbits, int32_t *q
                               int NK, int NAg, int loss, int unit_w) {
     int k = threadIdx.x;
     if (k < NK) {
-        float m = __uint_as_float(absmax[k]);
+        uint32_t mu = 0u;
+        for (int st = 0; st < EVT_ABSMAX_STRIPES; st++) {
+            const uint32_t v = absmax[st * EVT_MC_MAX_NK + k]; // non-negative floats order as their bit patterns
+            mu = v > mu ? v : mu;
+        }
+        float m = __uint_as_float(mu);
         int e = 0;
         if (m > 0.0f) {
             e = ilogbf(m) + 1;
@@ -277,7 +294,8 @@ __global__ void k_quant_setup(uint32_t *absmax, const int32_t *qbits, int32_t *q
         }
         qexp[k] = e;
         qmul[k] = scalbn(1.0, qbits[k] - e);
-        if (k < NK - 1) absmax[k] = 0u;
+        if (k < NK - 1)
+            for (int st = 0; st < EVT_ABSMAX_STRIPES; st++) absmax[st * EVT_MC_MAX_NK + k] = 0u;
     }
     __syncthreads();
     if (k < NAg) {
@@ -383,12 +401,15 @@ int launch_check_unit_weight(evt_ctx *c) {
     return EVT_OK;
 }
 
+__global__ void k_absmax_clear(uint32_t *absmax, int k0, int k1) {
+    const int n = k1 - k0;
+    for (int i = threadIdx.x; i < n * EVT_ABSMAX_STRIPES; i += blockDim.x) absmax[(i / n) * EVT_MC_MAX_NK + k0 + i % n] = 0u;
+}
+
 // absmax over rows [k0, k1) of the current gradient matrix
 int launch_absmax_rows(evt_ctx *c, int k0, int k1) {
-    {
-        int r = launch_fill_u32(c, c->absmax + k0, 0u, k1 - k0);
-        if (r != EVT_OK) return r;
-    }
+    hipLaunchKernelGGL(k_absmax_clear, dim3(1), dim3(256), 0, c->stream, c->absmax, k0, k1);
+    HIPCHK(hipGetLastError());
     int64_t nb = (c->N + 255) / 256;
     if (nb > 2048) nb = 2048;
     hipLaunchKernelGGL(k_absmax, dim3((unsigned)nb), dim3(256), 0, c->stream, c->grad, c->N, c->NK, k0, k1, c->absmax);

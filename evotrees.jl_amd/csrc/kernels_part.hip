@@ -532,23 +532,43 @@ __global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) {
 }
 
 // ---- row subsampling: is = rows with mask <= cond, ascending (src/subsample.jl:6-38) -----------
+__device__ __forceinline__ int wave_sum_i32(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// A thread takes 8 consecutive mask bytes (one load); the 8 flags of 8 neighbouring threads make one 64-row flag word.
 __global__ __launch_bounds__(256) void k_mask_count(const uint8_t *mask, uint8_t cond, int64_t N, int64_t n_chunks,
                                                    unsigned long long *flagw, int32_t *chunk_nleft) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    __shared__ int s_cnt[4];
+    static_assert(EVT_CHUNK == 2048 && EVT_CHUNK_WORDS == 32, "a chunk is 256 threads x 8 bytes");
+    const int tid = threadIdx.x;
+    __shared__ unsigned long long s_w[EVT_CHUNK_WORDS];
+    uint8_t *s_b = reinterpret_cast<uint8_t *>(s_w);
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        int cnt = 0;
-#pragma unroll
-        for (int it = 0; it < EVT_CHUNK / 256; it++) {
-            const int64_t p = c * EVT_CHUNK + it * 256 + tid;
-            const bool flag = (p < N) && (mask[p] <= cond);
-            const unsigned long long bal = __ballot(flag);
-            if (lane == 0) flagw[c * EVT_CHUNK_WORDS + it * 4 + wave] = bal;
-            cnt += __popcll(bal);
+        const int64_t p0 = c * EVT_CHUNK + (int64_t)tid * 8;
+        unsigned long long v = ~0ull; // bytes past the end read as 255
+        if (p0 + 8 <= N) {
+            v = *reinterpret_cast<const unsigned long long *>(mask + p0);
+        } else {
+            for (int j = 0; j < 8; j++)
+                if (p0 + j < N) v = (v & ~(0xFFull << (8 * j))) | ((unsigned long long)mask[p0 + j] << (8 * j));
         }
-        if (lane == 0) s_cnt[wave] = cnt;
+        unsigned flags = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const bool keep = (p0 + j < N) && ((uint8_t)(v >> (8 * j)) <= cond);
+            flags |= keep ? (1u << j) : 0u;
+        }
+        s_b[tid] = (uint8_t)flags; // little end first: byte t of the chunk's flag words covers rows 8t .. 8t+7
         __syncthreads();
-        if (tid == 0) chunk_nleft[c] = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+        if (tid < 64) {
+            const unsigned long long w = tid < EVT_CHUNK_WORDS ? s_w[tid] : 0ull;
+            if (tid < EVT_CHUNK_WORDS) flagw[c * EVT_CHUNK_WORDS + tid] = w;
+            int cnt = __popcll(w);
+            cnt = wave_sum_i32(cnt);
+            if (tid == 0) chunk_nleft[c] = cnt;
+        }
         __syncthreads();
     }
 }
@@ -565,20 +585,36 @@ __global__ __launch_bounds__(1024) void k_mask_scan(const int32_t *chunk_nleft, 
     if (tid == 0) chunk_lpre[n_chunks] = total;
 }
 
+// SELF: no k_mask_scan has run - every block adds up the counts of the chunks before its own (a few hundred values:
+// cheaper than the launch), and the block of the last chunk leaves the total where k_tree_begin reads it.
+template <bool SELF>
 __global__ __launch_bounds__(256) void k_mask_scatter(int64_t N, int64_t n_chunks, const unsigned long long *flagw,
-                                                     const int64_t *chunk_lpre, uint32_t *is_out) {
+                                                     const int32_t *chunk_nleft, int64_t *chunk_lpre, uint32_t *is_out) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     __shared__ unsigned long long s_w[EVT_CHUNK_WORDS];
     __shared__ int s_pre[EVT_CHUNK_WORDS];
+    __shared__ int s_sum[4];
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
         if (tid < EVT_CHUNK_WORDS) s_w[tid] = flagw[c * EVT_CHUNK_WORDS + tid];
+        int64_t base;
+        if (SELF) {
+            int part = 0;
+            for (int64_t k = tid; k < c; k += 256) part += chunk_nleft[k];
+            part = wave_sum_i32(part);
+            if (lane == 0) s_sum[wave] = part;
+        }
         __syncthreads();
         if (tid == 0) {
             int run = 0;
             for (int t = 0; t < EVT_CHUNK_WORDS; t++) { s_pre[t] = run; run += __popcll(s_w[t]); }
         }
+        if (SELF) {
+            base = (int64_t)s_sum[0] + s_sum[1] + s_sum[2] + s_sum[3];
+            if (c == n_chunks - 1 && tid == 0) chunk_lpre[n_chunks] = base + chunk_nleft[c];
+        } else {
+            base = chunk_lpre[c];
+        }
         __syncthreads();
-        const int64_t base = chunk_lpre[c];
 #pragma unroll
         for (int it = 0; it < EVT_CHUNK / 256; it++) {
             const int64_t p = c * EVT_CHUNK + it * 256 + tid;
@@ -588,6 +624,35 @@ __global__ __launch_bounds__(256) void k_mask_scatter(int64_t N, int64_t n_chunk
         }
         __syncthreads();
     }
+}
+
+// The row mask drawn on the device instead of uploaded: the mask's 8-byte word w is output w of SplitMix64 (Steele,
+// Lea, Flood 2014: the state advances by the odd constant 0x9E3779B97F4A7C15 per output, each output is the state
+// passed through two multiply-xorshift rounds) started at state `seed`, stored little end first - byte i of the mask
+// is bits 8*(i%8).. of output i/8.  Stands in for rand!(rng, mask) of src/subsample.jl:7 when the caller accepts a
+// counter-based stream keyed by one 64-bit draw of its own generator per tree.
+__global__ __launch_bounds__(256) void k_draw_mask(uint8_t *mask, int64_t N, unsigned long long seed) {
+    const int64_t nwords = (N + 7) >> 3;
+    for (int64_t w = (int64_t)blockIdx.x * 256 + threadIdx.x; w < nwords; w += (int64_t)gridDim.x * 256) {
+        unsigned long long z = seed + (unsigned long long)(w + 1) * 0x9E3779B97F4A7C15ull;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        z ^= z >> 31;
+        if ((w + 1) * 8 <= N) {
+            reinterpret_cast<unsigned long long *>(mask)[w] = z;
+        } else {
+            for (int j = 0; w * 8 + j < N; j++) mask[w * 8 + j] = (uint8_t)(z >> (8 * j));
+        }
+    }
+}
+
+int launch_draw_mask(evt_ctx *c, uint8_t *mask, unsigned long long seed) {
+    const int64_t nwords = (c->N + 7) >> 3;
+    int64_t g = (nwords + 255) / 256;
+    if (g > 8192) g = 8192;
+    hipLaunchKernelGGL(k_draw_mask, dim3((unsigned)g), dim3(256), 0, c->stream, mask, c->N, seed);
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
 }
 
 static unsigned grid_for_chunks(int64_t max_chunks) {
@@ -602,9 +667,14 @@ int launch_compact_mask(evt_ctx *c, uint8_t cond) {
     unsigned g = grid_for_chunks(n_chunks);
     hipLaunchKernelGGL(k_mask_count, dim3(g), dim3(256), 0, c->stream, c->mask, cond, c->N, n_chunks, c->flagw, c->chunk_nleft);
     HIPCHK(hipGetLastError());
+    if (n_chunks <= 1024) { // the scatter's blocks add up the counts before their chunk themselves
+        hipLaunchKernelGGL(k_mask_scatter<true>, dim3(g), dim3(256), 0, c->stream, c->N, n_chunks, c->flagw, c->chunk_nleft, c->chunk_lpre, c->is_a);
+        HIPCHK(hipGetLastError());
+        return EVT_OK;
+    }
     hipLaunchKernelGGL(k_mask_scan, dim3(1), dim3(1024), 0, c->stream, c->chunk_nleft, c->chunk_lpre, n_chunks);
     HIPCHK(hipGetLastError());
-    hipLaunchKernelGGL(k_mask_scatter, dim3(g), dim3(256), 0, c->stream, c->N, n_chunks, c->flagw, c->chunk_lpre, c->is_a);
+    hipLaunchKernelGGL(k_mask_scatter<false>, dim3(g), dim3(256), 0, c->stream, c->N, n_chunks, c->flagw, c->chunk_nleft, c->chunk_lpre, c->is_a);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

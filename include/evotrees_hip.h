@@ -175,6 +175,15 @@ int evt_grow_tree_end(evt_handle h, evt_tree_out *tree);
 int evt_stage_mask(evt_handle h, const uint8_t *mask);
 int evt_grow_tree_begin_staged(evt_handle h, uint8_t cond, const uint32_t *js, int32_t n_js,
                                const evt_params *params);
+/* The staged mask drawn by the device instead of uploaded, for a caller that does not need the byte stream of its own
+ * generator (rand!(rng, mask), src/subsample.jl:7) but only a reproducible one: the caller draws ONE 64-bit seed per
+ * tree from its generator and the mask's 8-byte word w becomes output w of SplitMix64 started at that seed
+ * (z = seed + (w + 1) * 0x9E3779B97F4A7C15; z = (z ^ z >> 30) * 0xBF58476D1CE4E5B9; z = (z ^ z >> 27) *
+ * 0x94D049BB133111EB; z ^= z >> 31), little end first: byte i of the mask is bits 8 * (i % 8) and up of word i / 8.
+ * A row is kept when its byte <= cond, as with an uploaded mask, so P[keep] = (cond + 1) / 256 all the same.  Queued
+ * on the handle's stream (also behind a tree in flight), no host work per row; follow it with
+ * evt_grow_tree_begin_staged.  The trees equal, bit for bit, those grown from the same bytes uploaded. */
+int evt_draw_mask(evt_handle h, uint64_t seed);
 
 /*
  * The same tree, one kernel stage at a time: the stages are the reference's own per-level calls, so each can be

@@ -43,3 +43,17 @@ def test_host_config_checks(evt):
         evt.init(evt.EvoTreeRegressor(device="cpu"), [[1.0]], [1.0])
     assert evt.EvoTreeMLE().min_weight == 8.0 and evt.EvoTreeRegressor().min_weight == 1.0
     assert evt.EvoTreeRegressor(**{"lambda": 0.5}).lambda_ == 0.5
+
+
+def test_splitmix_mask_known_answers(evt):
+    # SplitMix64's published outputs: seed 0 (the reference C source's first three) and seed 1234567 (first five)
+    import numpy as np
+    got = evt.splitmix_mask(0, 24).view("<u8")
+    assert [int(v) for v in got] == [0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4, 0x06C45D188009454F]
+    got = evt.splitmix_mask(1234567, 40).view("<u8")
+    assert [int(v) for v in got] == [6457827717110365317, 3203168211198807973, 9817491932198370423, 4593380528125082431,
+                                     16408922859458223821]
+    # little end first, and a length that is not a multiple of eight cuts the last word short
+    m = evt.splitmix_mask(0, 13)
+    assert m.dtype == np.uint8 and m.shape == (13,)
+    assert list(m[:8]) == [0xAF, 0xCD, 0x1D, 0x7B, 0x39, 0xA8, 0x20, 0xE2] and list(m[8:]) == [0xF4, 0x65, 0xB9, 0xA1, 0x6A]

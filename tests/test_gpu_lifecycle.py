@@ -193,6 +193,57 @@ def test_mask_staged_while_the_last_tree_grows(evt):
     hb.close()
 
 
+def test_mask_drawn_on_the_device(evt):
+    """evt_draw_mask writes the bytes splitmix_mask computes on the host (pinned there by SplitMix64's published outputs):
+    the rows in the tree are exactly those with byte <= cond, for thresholds that cut the bytes in different places and a
+    row count that is not a multiple of eight, and the trees equal those grown from the same bytes uploaded.  A mask is
+    used once."""
+    N, F, B, D = 60003, 9, 32, 6
+    x_bin, y, w, mu = make_data(23, N, F, B, "mse", weights=False)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    gp = evt.make_params(eta=0.3)
+
+    def make():
+        h = evt.Handle(N, F, B, 1, D, "mse")
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        return h
+
+    ha, hb = make(), make()
+    seeds = [0, 1, 0xFFFFFFFFFFFFFFFF, 0x0123456789ABCDEF, 42, 7]
+    conds = [128, 0, 254, 1, 77, 200]
+    for r, (seed, cond) in enumerate(zip(seeds, conds)):
+        mask = evt.splitmix_mask(seed, N)
+        ha.update_grads()
+        ta = ha.grow_tree(js, gp, mask=mask, cond=cond)
+        hb.update_grads()
+        hb.draw_mask(seed)
+        hb.grow_tree_begin_staged(js, gp, cond)
+        if r == 2:
+            hb_next = seeds[r + 1]
+            hb.draw_mask(hb_next)  # queued behind the tree in flight, used by the next round
+        tb = hb.grow_tree_end()
+        assert_tree_bits(ta, tb)
+        nb = hb.get_nidx()
+        assert np.array_equal(nb != 0, mask <= cond), (r, seed, cond)
+        assert np.array_equal(ha.get_nidx(), nb)
+        if r == 2:  # the mask drawn while tree 2 was in flight serves tree 3
+            mask = evt.splitmix_mask(seeds[3], N)
+            ha.update_grads()
+            ta = ha.grow_tree(js, gp, mask=mask, cond=conds[3])
+            hb.update_grads()
+            hb.grow_tree_begin_staged(js, gp, conds[3])
+            tb = hb.grow_tree_end()
+            assert_tree_bits(ta, tb)
+            assert np.array_equal(hb.get_nidx() != 0, mask <= conds[3])
+    assert np.array_equal(ha.get_pred().view(np.uint32), hb.get_pred().view(np.uint32))
+    with pytest.raises(evt.EvtError) as ei:
+        hb.grow_tree_begin_staged(js, gp, 128)
+    assert ei.value.code == evt._lib.EVT_ERR_STATE
+    ha.close()
+    hb.close()
+
+
 def test_grow_tree_in_two_halves(evt):
     """evt_grow_tree_begin / evt_grow_tree_end give the trees and predictions of evt_grow_tree, bit for bit; between
     the two halves the handle refuses every other call (and still answers afterwards); an end without a begin and an
