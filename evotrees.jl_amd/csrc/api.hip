@@ -814,7 +814,7 @@ static int tree_stage_scan(evt_ctx *c) {
     } else {
         r = launch_scan(c, level, p, false);
         if (r == EVT_OK && obliv) r = launch_obliv_select(c, level, p);
-        if (r == EVT_OK && level == last_split) r = launch_scan(c, c->D, p, true); // leaf values of level D
+        if (r == EVT_OK && level == last_split && !scan_folds_leaves(c)) r = launch_scan(c, c->D, p, true); // leaf values of level D
     }
     prof_end(c);
     if (r != EVT_OK) return r;

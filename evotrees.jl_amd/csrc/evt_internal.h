@@ -277,6 +277,7 @@ int launch_compact_mask(evt_ctx *c, uint8_t cond);
 int launch_draw_mask(evt_ctx *c, uint8_t *mask, unsigned long long seed);
 int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level);
+bool scan_folds_leaves(const evt_ctx *c);
 int launch_obliv_select(evt_ctx *c, int level, const evt_params *p);
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred);

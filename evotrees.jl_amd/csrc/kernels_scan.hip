@@ -32,6 +32,7 @@ struct ScanArgs {
     double eta, lambda, L2, gamma, min_weight;
     int bagging;
     int nfs, B, F, K, NK, NAg, loss, level, leaf_level, oblivious, zero_children;
+    int fold_leaves; // the level's children are leaves: their weight and values are written along with the split (no pass of their own)
 };
 
 // ---- wavefront primitives -----------------------------------------------------------------
@@ -410,6 +411,7 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
     if (wave == 0) { // pass 1 already materialised h[n] for subtract nodes
         const int f = (int)A.js[bj] - 1;
         const bool numeric = A.feattypes[f] != 0;
+        long long qc[NAG]; // lane 0: the left child's sums, lane 1: the right child's
         for (int ag = 0; ag < NAG; ag++) {
             const int64_t o = ((int64_t)bj * NAG + ag) * B;
             long long s = 0;
@@ -422,6 +424,16 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
                 A.node_sum[(int64_t)(2 * n) * NAG + ag] = s;
                 A.node_sum[(int64_t)(2 * n + 1) * NAG + ag] = s_Sq[ag] - s;
             }
+            qc[ag] = (lane & 1) ? s_Sq[ag] - s : s;
+        }
+        if (A.fold_leaves && lane < 2) {
+            // what the leaf-level pass would compute from node_sum (same integers, same expressions)
+            const int cn = 2 * n + lane;
+            double v[EVT_MAX_NK];
+            decode_vals(qc, s_sc, A.loss, NK, v);
+            A.tree.w[cn - 1] = (float)v[NK - 1];
+            for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (cn - 1) + k] = (float)leaf_value(v, k, K, A.eta, A.bagging, A.lambda, A.L2);
+            A.status[cn] = ST_LEAF;
         }
     }
     // the children's histogram slices start from zero (the build child accumulates into it): with one block per node
@@ -787,6 +799,9 @@ __global__ __launch_bounds__(256) void k_scan_fin_mc(ScanArgs A, int ngroups) {
     }
 }
 
+// The pass over the last split level also writes its children's leaf values (binary trees with the fixed channel layouts).
+bool scan_folds_leaves(const evt_ctx *c) { return !c->mc && c->tree_type != EVT_TREE_OBLIVIOUS && c->D > 1; }
+
 int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     ScanArgs A;
     A.sbest = reinterpret_cast<ScanBest *>(c->sbest);
@@ -807,6 +822,7 @@ int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     A.leaf_level = leaf_level ? 1 : 0;
     A.oblivious = (c->tree_type == EVT_TREE_OBLIVIOUS) ? 1 : 0;
     A.zero_children = (level + 1 < c->D) ? 1 : 0; // children at the last level never get a histogram
+    A.fold_leaves = (!leaf_level && scan_folds_leaves(c) && level + 1 == c->D) ? 1 : 0;
     const unsigned nodes = 1u << (level - 1);
     const int ngroups = (A.nfs + 3) / 4; // 4 waves per block, one sampled feature each
     dim3 grid(nodes, (unsigned)ngroups);
