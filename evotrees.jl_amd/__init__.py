@@ -77,7 +77,10 @@ class _Learner:
         args["tree_type"] = str(args["tree_type"]).lstrip(":")
         if args["loss"] not in self._losses:
             raise ValueError("Invalid loss. Must be one of: %s" % (list(self._losses),))
-        args["metric"] = args["loss"] if args["metric"] is None else str(args["metric"]).lstrip(":")
+        if args["metric"] is None:  # the loss itself; mae for the credibility losses (src/learners.jl:76-81)
+            args["metric"] = "mae" if args["loss"] in ("cred_var", "cred_std") else args["loss"]
+        else:
+            args["metric"] = str(args["metric"]).lstrip(":")
         if args["metric"] not in self._metrics:
             raise ValueError("Invalid metric. Must be one of: %s" % (list(self._metrics),))
         args["monotone_constraints"] = dict(args["monotone_constraints"] or {})
@@ -86,8 +89,10 @@ class _Learner:
 
 
 class EvoTreeRegressor(_Learner):
-    """EvoTreeRegressor (src/learners.jl:1-119); losses mse, logloss, poisson, gamma, tweedie."""
-    _losses = ("mse", "logloss", "poisson", "gamma", "tweedie")
+    """EvoTreeRegressor (src/learners.jl:1-119); losses mse, logloss, poisson, gamma, tweedie, mae, cred_var, cred_std (of the
+    reference's list the quantile losses are not served: their leaf values are quantiles of the leaf's residuals, not
+    functions of the histogram)."""
+    _losses = ("mse", "logloss", "poisson", "gamma", "tweedie", "mae", "cred_var", "cred_std")
     _metrics = ("mse", "rmse", "mae", "logloss", "poisson", "gamma", "tweedie")
 
 

@@ -12,7 +12,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libevotrees_hip.so")
 
 EVT_OK, EVT_ERR_ARG, EVT_ERR_HIP, EVT_ERR_STATE, EVT_ERR_EMPTY, EVT_ERR_NOMEM = 0, -1, -2, -3, -4, -5
-LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5, "mlogloss": 6, "logistic_mle": 7}
+LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5, "mlogloss": 6, "logistic_mle": 7, "mae": 8,
+            "cred_var": 9, "cred_std": 10}
 METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8, "logistic_mle": 9}
 TREE_TYPES = {"binary": 0, "oblivious": 1}
 KERNEL_CLASSES = ["grad", "hist", "scan", "partition", "predict", "other"]

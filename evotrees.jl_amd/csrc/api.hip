@@ -211,8 +211,9 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ARGCHK(nfeats >= 1 && nfeats <= 1024, "nfeats must be in [1, 1024]");
     ARGCHK(nbins >= 2 && nbins <= 255, "nbins must be in [2, 255]");
     ARGCHK(max_depth >= 1 && max_depth <= EVT_MAX_DEPTH, "max_depth must be in [1, 16]");
-    ARGCHK(loss >= 0 && loss <= EVT_LOSS_LOGISTIC_MLE,
-           "loss must be one of mse (0), logloss (1), gaussian_mle (2), poisson (3), gamma (4), tweedie (5), mlogloss (6), logistic_mle (7)");
+    ARGCHK(loss >= 0 && loss <= EVT_LOSS_LAST,
+           "loss must be one of mse (0), logloss (1), gaussian_mle (2), poisson (3), gamma (4), tweedie (5), mlogloss (6), logistic_mle (7), mae (8), "
+           "cred_var (9), cred_std (10)");
     ARGCHK(tree_type == EVT_TREE_BINARY || tree_type == EVT_TREE_OBLIVIOUS, "tree_type must be binary (0) or oblivious (1)");
     if (loss == EVT_LOSS_MLOGLOSS) ARGCHK(K >= 2 && K <= EVT_MAX_K, "mlogloss needs 2 <= K <= 16 classes");
     else if (EVT_IS_MLE2P(loss)) ARGCHK(K >= 2 && K <= EVT_MAX_K && K % 2 == 0, "gaussian_mle / logistic_mle need K = 2 x targets, 2 <= K <= 16");
@@ -516,8 +517,8 @@ extern "C" int evt_binarize_f64(evt_handle c, const double *x_colmajor, const do
 static void set_channels(evt_ctx *c) {
     // LDS channels (rows of the gradient matrix that need their own accumulator)
     int na = 0;
-    if (c->loss == EVT_LOSS_MSE && c->K == 1) {
-        c->chan_k[na++] = 0;                   // g ; h == 2w is derived
+    if (EVT_TWO_CHAN(c->loss, c->K)) {
+        c->chan_k[na++] = 0;                   // g ; h is derived (mse: 2w, mae: 0)
         if (!c->unit_w) c->chan_k[na++] = 2;   // w
     } else {
         for (int k = 0; k < c->NK - 1; k++) c->chan_k[na++] = k;
@@ -525,7 +526,7 @@ static void set_channels(evt_ctx *c) {
     }
     c->NA = na;
     for (int a = na; a < EVT_MC_MAX_NK; a++) c->chan_k[a] = 0;
-    c->NAg = (c->loss == EVT_LOSS_MSE && c->K == 1) ? 2 : c->NK;
+    c->NAg = EVT_TWO_CHAN(c->loss, c->K) ? 2 : c->NK;
     int qbg = 62 - ceil_log2_i64(c->N);
     if (qbg > 40) qbg = 40;
     for (int k = 0; k < c->NK; k++) c->h_qbits[k] = qbg;
@@ -1367,7 +1368,7 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
                           const int32_t *edge_off = nullptr) {
     ARGCHK(nobs >= 1 && nfeats >= 1 && ntrees >= 1, "nobs, nfeats, ntrees must be >= 1");
     ARGCHK((x_bin || x_f64) && tree_off && feat && cond_bin && split, "NULL argument");
-    ARGCHK(leaf_out || (pred && out && K >= 1 && K <= EVT_MAX_K && loss >= 0 && loss <= EVT_LOSS_LOGISTIC_MLE), "invalid prediction arguments");
+    ARGCHK(leaf_out || (pred && out && K >= 1 && K <= EVT_MAX_K && loss >= 0 && loss <= EVT_LOSS_LAST), "invalid prediction arguments");
     std::vector<int32_t> eoff;
     if (x_f64) {
         ARGCHK(edges && edge_off, "NULL argument");

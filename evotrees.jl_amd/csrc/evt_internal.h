@@ -228,6 +228,11 @@ void evt_set_error(const char *fmt, ...);
 // A split node in one 32-bit word: feature id (1-based) | cond_bin << 16 | split << 24 | numeric << 25.  Leaves are 0.
 // the two-parameter MLE losses: outputs come in (location, raw scale) pairs
 #define EVT_IS_MLE2P(loss) ((loss) == EVT_LOSS_GAUSSIAN_MLE || (loss) == EVT_LOSS_LOGISTIC_MLE)
+#define EVT_IS_CRED(loss) ((loss) == EVT_LOSS_CRED_VAR || (loss) == EVT_LOSS_CRED_STD)
+#define EVT_LOSS_LAST EVT_LOSS_CRED_STD
+// One-target mse and mae need no accumulator for their second gradient row (mse: h = 2w; mae: h = 0, and neither its
+// gain nor its leaf value reads it): their histograms hold the channels {g, w} only.
+#define EVT_TWO_CHAN(loss, K) (((loss) == EVT_LOSS_MSE || (loss) == EVT_LOSS_MAE) && (K) == 1)
 #define EVT_NODE_SPLIT (1u << 24)
 #define EVT_NODE_NUMERIC (1u << 25)
 #ifdef __HIPCC__

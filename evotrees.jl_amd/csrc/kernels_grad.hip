@@ -54,7 +54,7 @@ __device__ __forceinline__ void absmax_raise(uint32_t *absmax, int k, float m) {
 }
 
 // LOSS: 0 mse (src/loss.jl:52), 1 logloss (:54-57), 2 gaussian_mle (:194-203), 3 poisson (:59-62),
-// 4 gamma (:64-67), 5 tweedie with rho = 1.5 (:69-76).
+// 4 gamma (:64-67), 5 tweedie with rho = 1.5 (:69-76), 8 mae (:78), 9 cred_var / cred_std (:80-83).
 // grad rows: [g_1..g_K, h_1..h_K, w]; every written value is multiplied by w (src/loss.jl:104-108, :223-233).
 template <int LOSS>
 __global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const float *__restrict__ y, float *__restrict__ grad, int64_t N,
@@ -91,6 +91,13 @@ __global__ __launch_bounds__(256) void k_grads(float *__restrict__ pred, const f
             const float a = powf(e, 0.5f), b = powf(e, -0.5f);
             out[0] = (2.0f * (a - y[i] * b)) * w;
             out[1] = (2.0f * (0.5f * a - (-0.5f) * y[i] * b)) * w;
+        } else if (LOSS == 8) { // mae (src/loss.jl:78): the residual, no second-order row
+            out[0] = (y[i] - pred[i]) * w;
+            out[1] = 0.0f * w;
+        } else if (LOSS == 9) { // credibility losses (src/loss.jl:80-83): residual and its square
+            const float d = y[i] - pred[i];
+            out[0] = d * w;
+            out[1] = (d * d) * w;
         } else {
             float g1, g2, h1, h2;
             mle2p_grad_hess<LOSS>(pred[2 * i], pred[2 * i + 1], y[i], g1, g2, h1, h2);
@@ -141,6 +148,13 @@ __device__ __forceinline__ void grad_hess_one(float pk, float yk, float &g, floa
         const float e = expf(pk);
         g = 2.0f * (1.0f - yk / e);
         h = 2.0f * yk / e;
+    } else if (LOSS == 8) {
+        g = yk - pk;
+        h = 0.0f;
+    } else if (LOSS == 9) {
+        const float d = yk - pk;
+        g = d;
+        h = d * d;
     } else {
         const float e = expf(pk);
         const float a = powf(e, 0.5f), b = powf(e, -0.5f);
@@ -300,7 +314,7 @@ __global__ void k_quant_setup(uint32_t *absmax, const int32_t *qbits, int32_t *q
     __syncthreads();
     if (k < NAg) {
         // global channel ag -> gradient row: mse {g, w}; otherwise identity; last channel is w (or the row count)
-        int kk = (loss == 0 && NK == 3) ? (k == 0 ? 0 : 2) : k; // one-target mse: channels {g, w}
+        int kk = EVT_TWO_CHAN(loss, (NK - 1) / 2) ? (k == 0 ? 0 : 2) : k; // one-target mse / mae: channels {g, w}
         if (k == NAg - 1 && unit_w) qscale_g[k] = 1.0;
         else qscale_g[k] = scalbn(1.0, qexp[kk] - qbits[kk]);
     }
@@ -343,6 +357,9 @@ int launch_grads(evt_ctx *c) {
         case EVT_LOSS_POISSON: MT(3); break;
         case EVT_LOSS_GAMMA: MT(4); break;
         case EVT_LOSS_LOGISTIC_MLE: MT(7); break;
+        case EVT_LOSS_MAE: MT(8); break;
+        case EVT_LOSS_CRED_VAR:
+        case EVT_LOSS_CRED_STD: MT(9); break;
         default: MT(5); break;
         }
 #undef MT
@@ -361,6 +378,10 @@ int launch_grads(evt_ctx *c) {
         hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_GAMMA)
         hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+    else if (c->loss == EVT_LOSS_MAE)
+        hipLaunchKernelGGL(k_grads<8>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+    else if (EVT_IS_CRED(c->loss))
+        hipLaunchKernelGGL(k_grads<9>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_MLOGLOSS)
         hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else
@@ -427,7 +448,7 @@ int launch_quantize(evt_ctx *c) {
                        c->loss, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
     hipLaunchKernelGGL(k_quantize, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, c->gq, c->N, c->NK, c->NA,
-                       (c->loss == EVT_LOSS_MSE && c->K == 1) ? 1 : 0, qmul, c->unit_w ? 1 : 0);
+                       EVT_TWO_CHAN(c->loss, c->K) ? 1 : 0, qmul, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

@@ -742,9 +742,9 @@ __global__ __launch_bounds__(256) void k_hist_export(const long long *__restrict
         double ch[EVT_MC_MAX_NK];
         for (int ag = 0; ag < NAg; ag++) ch[ag] = (double)hn[((int64_t)jp * NAg + ag) * B + b] * qscale[ag];
         double *o = out + (((int64_t)node * F + f) * B + b) * NK;
-        if (loss == 0 && NK == 3) {
+        if (EVT_TWO_CHAN(loss, (NK - 1) / 2)) { // channels {g, w}: h = 2w (mse) or 0 (mae)
             o[0] = ch[0];
-            o[1] = 2.0 * ch[1];
+            o[1] = (loss == EVT_LOSS_MSE) ? 2.0 * ch[1] : 0.0;
             o[2] = ch[1];
         } else {
             for (int k = 0; k < NK; k++) o[k] = ch[k];

@@ -80,17 +80,57 @@ __device__ __forceinline__ double term_gh(double g, double h, double w, double l
 
 // fixed-point channel sums -> the 2K+1 Float64 statistics [g.., h.., w]
 __device__ __forceinline__ void decode_vals(const long long *q, const double *sc, int loss, int NK, double *out) {
-    if (loss == EVT_LOSS_MSE && NK == 3) { // one-target mse: channels {g, w}, h = 2w
+    if (EVT_TWO_CHAN(loss, (NK - 1) / 2)) { // one-target mse / mae: channels {g, w}; h = 2w (mse), 0 (mae)
         double w = (double)q[1] * sc[1];
         out[0] = (double)q[0] * sc[0];
-        out[1] = 2.0 * w;
+        out[1] = (loss == EVT_LOSS_MSE) ? 2.0 * w : 0.0;
         out[2] = w;
     } else {
         for (int k = 0; k < NK; k++) out[k] = (double)q[k] * sc[k];
     }
 }
 
-__device__ __forceinline__ double leaf_value(const double *S, int k, int K, double eta, int bagging, double lambda, double L2) {
+// _term_cred with _cred_Z (src/split.jl:3-4, src/loss.jl:275-290): Z |m1| / (1 + L2 / w), Z = VHM / (VHM + EVPV) for
+// cred_var and the same ratio of square roots for cred_std, VHM = (m1 / w)^2, EVPV = max(eps, m2 / w - VHM)
+__device__ __forceinline__ double term_cred(int loss, double m1, double m2, double w, double L2) {
+    const double mean = m1 / w;
+    const double VHM = mean * mean;
+    double EVPV = m2 / w - VHM;
+    if (!(EVPV > DBL_EPSILON)) EVPV = DBL_EPSILON;
+    const double Z = (loss == EVT_LOSS_CRED_VAR) ? VHM / (VHM + EVPV) : sqrt(VHM) / (sqrt(VHM) + sqrt(EVPV));
+    return Z * fabs(m1) / (1.0 + L2 / w);
+}
+
+// One output's term of node_gain (src/split.jl:58-78): zero for mae.
+__device__ __forceinline__ double node_gain_k(int loss, double g, double h, double w, double lambda, double L2) {
+    if (loss == EVT_LOSS_MAE) return 0.0;
+    if (EVT_IS_CRED(loss)) return term_cred(loss, g, h, w, L2);
+    return term_gh(g, h, w, lambda, L2);
+}
+
+// One output's term of split_gain (src/split.jl:108-141): left + right.  (Sg, Sh, w_p) are the node's totals.  mae:
+// _term_shift (src/split.jl:2), |g / w - mu_p| w / d on either side with d = max(eps, 1 + lambda + L2 / w).
+__device__ __forceinline__ double split_gain_k(int loss, double Sg, double Sh, double w_p, double g_l, double h_l, double w_l, double w_r,
+                                               double lambda, double L2) {
+    if (loss == EVT_LOSS_MAE) {
+        double d_l = 1.0 + lambda + L2 / w_l, d_r = 1.0 + lambda + L2 / w_r;
+        if (!(d_l > DBL_EPSILON)) d_l = DBL_EPSILON;
+        if (!(d_r > DBL_EPSILON)) d_r = DBL_EPSILON;
+        const double mu_p = Sg / w_p;
+        return fabs(g_l / w_l - mu_p) * w_l / d_l + fabs((Sg - g_l) / w_r - mu_p) * w_r / d_r;
+    }
+    if (EVT_IS_CRED(loss)) return term_cred(loss, g_l, h_l, w_l, L2) + term_cred(loss, Sg - g_l, Sh - h_l, w_r, L2);
+    return term_gh(g_l, h_l, w_l, lambda, L2) + term_gh(Sg - g_l, Sh - h_l, w_r, lambda, L2);
+}
+
+// pred_leaf_cpu! / pred_scalar (src/predict.jl:198-262) for output k
+__device__ __forceinline__ double leaf_value(int loss, const double *S, int k, int K, double eta, int bagging, double lambda, double L2) {
+    if (EVT_IS_CRED(loss)) return eta / (double)bagging * S[k] / (S[2 * K] + L2);
+    if (loss == EVT_LOSS_MAE) {
+        double d = S[2 * K] + lambda * S[2 * K] + L2;
+        if (!(d > DBL_EPSILON)) d = DBL_EPSILON;
+        return eta / (double)bagging * S[k] / d;
+    }
     double d = S[K + k] + lambda * S[2 * K] + L2;
     if (!(d > DBL_EPSILON)) d = DBL_EPSILON;
     return -eta / (double)bagging * S[k] / d;
@@ -225,7 +265,7 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     for (int k = 0; k < NK; k++) S[k] = s_S[k];
 
     double gain_p = 0.0;
-    for (int k = 0; k < K; k++) gain_p += term_gh(S[k], S[K + k], S[2 * K], A.lambda, A.L2);
+    for (int k = 0; k < K; k++) gain_p += node_gain_k(A.loss, S[k], S[K + k], S[2 * K], A.lambda, A.L2);
     const double w_p = S[NK - 1];
 
     double wbest = -INFINITY;
@@ -272,15 +312,14 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
                         if (constraint != 0) {
                             double SR[EVT_MAX_NK];
                             for (int k = 0; k < NK; k++) SR[k] = S[k] - SL[k];
-                            const double predL = leaf_value(SL, 0, K, A.eta, A.bagging, A.lambda, A.L2);
-                            const double predR = leaf_value(SR, 0, K, A.eta, A.bagging, A.lambda, A.L2);
+                            const double predL = leaf_value(A.loss, SL, 0, K, A.eta, A.bagging, A.lambda, A.L2);
+                            const double predR = leaf_value(A.loss, SR, 0, K, A.eta, A.bagging, A.lambda, A.L2);
                             ok = (constraint == -1 && predL > predR) || (constraint == 1 && predL < predR);
                         }
                         if (ok) {
                             double sg = 0.0;
                             for (int k = 0; k < K; k++) {
-                                const double g_l = SL[k], h_l = SL[K + k];
-                                sg += term_gh(g_l, h_l, w_l, A.lambda, A.L2) + term_gh(S[k] - g_l, S[K + k] - h_l, w_r, A.lambda, A.L2);
+                                sg += split_gain_k(A.loss, S[k], S[K + k], w_p, SL[k], SL[K + k], w_l, w_r, A.lambda, A.L2);
                             }
                             gain = sg - gain_p;
                         }
@@ -368,7 +407,7 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
     if (tid == 0) A.tree.w[n - 1] = (float)S[NK - 1];
 
     if (A.leaf_level) {
-        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
+        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(A.loss, S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
         if (tid == 0) A.status[n] = ST_LEAF;
         return;
     }
@@ -401,7 +440,7 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
             A.tree.packed[n - 1] = evt_pack_node(feat, bb, A.feattypes[feat - 1] != 0);
             A.status[n] = ST_SPLIT;
         } else {
-            for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (n - 1) + k] = (float)leaf_value(S, k, K, A.eta, A.bagging, A.lambda, A.L2);
+            for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (n - 1) + k] = (float)leaf_value(A.loss, S, k, K, A.eta, A.bagging, A.lambda, A.L2);
             A.status[n] = ST_LEAF;
         }
     }
@@ -432,7 +471,7 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
             double v[EVT_MAX_NK];
             decode_vals(qc, s_sc, A.loss, NK, v);
             A.tree.w[cn - 1] = (float)v[NK - 1];
-            for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (cn - 1) + k] = (float)leaf_value(v, k, K, A.eta, A.bagging, A.lambda, A.L2);
+            for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (cn - 1) + k] = (float)leaf_value(A.loss, v, k, K, A.eta, A.bagging, A.lambda, A.L2);
             A.status[cn] = ST_LEAF;
         }
     }
@@ -524,7 +563,7 @@ __global__ __launch_bounds__(1024) void k_obliv_select(OblivArgs A) {
         decode_vals(Sq, s_sc, A.loss, NK, S);
         if (lane == 0) A.tree.w[n - 1] = (float)S[NK - 1];
         if (!found) {
-            if (lane < K) A.tree.pred[(int64_t)K * (n - 1) + lane] = (float)leaf_value(S, lane, K, A.eta, A.bagging, A.lambda, A.L2);
+            if (lane < K) A.tree.pred[(int64_t)K * (n - 1) + lane] = (float)leaf_value(A.loss, S, lane, K, A.eta, A.bagging, A.lambda, A.L2);
             if (lane == 0) A.status[n] = ST_LEAF;
             continue;
         }
@@ -637,7 +676,7 @@ __global__ __launch_bounds__(256) void k_scan_mc(ScanArgs A) {
 
     node_totals_mc(A, n, hn, blockIdx.y == 0, s_Sq, s_S, s_sc);
     double gain_p = 0.0;
-    for (int k = 0; k < K; k++) gain_p += term_gh(s_S[k], s_S[K + k], s_S[2 * K], A.lambda, A.L2);
+    for (int k = 0; k < K; k++) gain_p += node_gain_k(A.loss, s_S[k], s_S[K + k], s_S[2 * K], A.lambda, A.L2);
     const double w_p = s_S[NK - 1];
 
     double wbest = -INFINITY;
@@ -668,7 +707,7 @@ __global__ __launch_bounds__(256) void k_scan_mc(ScanArgs A) {
 #pragma unroll
             for (int t = 0; t < BPL; t++) {
                 const double g_l = (double)gq[t] * s_sc[k], h_l = (double)hq[t] * s_sc[K + k];
-                sg[t] += term_gh(g_l, h_l, w_l[t], A.lambda, A.L2) + term_gh(Sg - g_l, Sh - h_l, w_r[t], A.lambda, A.L2);
+                sg[t] += split_gain_k(A.loss, Sg, Sh, w_p, g_l, h_l, w_l[t], w_r[t], A.lambda, A.L2);
             }
         }
         double lg = -INFINITY;
@@ -731,7 +770,7 @@ __global__ __launch_bounds__(256) void k_scan_fin_mc(ScanArgs A, int ngroups) {
     node_totals_mc(A, n, hn, true, s_Sq, s_S, s_sc);
     if (tid == 0) A.tree.w[n - 1] = (float)s_S[NK - 1];
     if (A.leaf_level) {
-        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(s_S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
+        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(A.loss, s_S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
         if (tid == 0) A.status[n] = ST_LEAF;
         return;
     }
@@ -769,7 +808,7 @@ __global__ __launch_bounds__(256) void k_scan_fin_mc(ScanArgs A, int ngroups) {
     }
     __syncthreads();
     if (!s_dec[0]) {
-        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(s_S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
+        if (tid < K) A.tree.pred[(int64_t)K * (n - 1) + tid] = (float)leaf_value(A.loss, s_S, tid, K, A.eta, A.bagging, A.lambda, A.L2);
         return;
     }
     bj = s_dec[1]; bb = s_dec[2];

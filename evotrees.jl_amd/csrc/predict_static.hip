@@ -92,7 +92,7 @@ extern "C" int evt_predict_static(void *stream, int64_t nobs, int32_t nfeats, co
                                   const uint8_t *cond_bin_dev, const float *pred_dev, const uint8_t *split_dev, int32_t apply_link,
                                   float *out_dev, int32_t *status_dev) {
     ARGCHK(nobs >= 1 && nfeats >= 1 && nfeats <= 65535 && ntrees >= 1, "nobs, nfeats (<= 65535), ntrees must be >= 1");
-    ARGCHK(K >= 1 && K <= EVT_MAX_K && loss >= 0 && loss <= EVT_LOSS_LOGISTIC_MLE, "invalid loss or K");
+    ARGCHK(K >= 1 && K <= EVT_MAX_K && loss >= 0 && loss <= EVT_LOSS_LAST, "invalid loss or K");
     ARGCHK(total_nodes >= ntrees, "total_nodes is smaller than the number of trees");
     if (total_nodes > (int64_t)EVT_STATIC_MAX_NODES) {
         evt_set_error("evt_predict_static: the model has %lld nodes, the static work area holds %lld (use evt_predict)", (long long)total_nodes,

@@ -50,7 +50,12 @@ enum {
     EVT_LOSS_GAMMA = 4,
     EVT_LOSS_TWEEDIE = 5,
     EVT_LOSS_MLOGLOSS = 6, /* K classes, y holds the 1-based class (level code) as a Float32 */
-    EVT_LOSS_LOGISTIC_MLE = 7 /* the other two-parameter MLE loss (src/loss.jl:205-217): outputs and clamps as gaussian_mle */
+    EVT_LOSS_LOGISTIC_MLE = 7, /* the other two-parameter MLE loss (src/loss.jl:205-217): outputs and clamps as gaussian_mle */
+    EVT_LOSS_MAE = 8,      /* rows [(y - p) w, 0, w] (src/loss.jl:78, :130-142); gain = shift of the children's mean residual
+                              (src/split.jl:2, :68, :119-130); leaf = eta * sum(g) / (w + lambda w + L2) (src/predict.jl:250-258) */
+    EVT_LOSS_CRED_VAR = 9, /* credibility losses: rows [d w, d^2 w, w], d = y - p (src/loss.jl:80-83, :173-185); gain terms */
+    EVT_LOSS_CRED_STD = 10 /* Z |m1| / (1 + L2 / w), Z the ratio of variances / of standard deviations (src/loss.jl:275-290,
+                              src/split.jl:3-4, :70-78, :132-141); leaf = eta * sum(g) / (w + L2) (src/predict.jl:211-217) */
 };
 /* evaluation metrics, metric_dict of src/metrics.jl:209-224 (in-scope subset) */
 enum {

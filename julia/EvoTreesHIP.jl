@@ -57,11 +57,12 @@ check(rc::Integer) = rc == 0 ? nothing : error(lasterr())
 
 const LOSS_ID = Dict{Any,Cint}(
     EvoTrees.MSE => 0, EvoTrees.LogLoss => 1, EvoTrees.GaussianMLE => 2, EvoTrees.Poisson => 3,
-    EvoTrees.Gamma => 4, EvoTrees.Tweedie => 5, EvoTrees.MLogLoss => 6, EvoTrees.LogisticMLE => 7)
+    EvoTrees.Gamma => 4, EvoTrees.Tweedie => 5, EvoTrees.MLogLoss => 6, EvoTrees.LogisticMLE => 7,
+    EvoTrees.MAE => 8, EvoTrees.CredVar => 9, EvoTrees.CredStd => 10)
 const METRIC_ID = Dict{Symbol,Cint}(
     :mse => 0, :rmse => 1, :mae => 2, :logloss => 3, :gaussian_mle => 4, :poisson => 5, :gamma => 6,
     :tweedie => 7, :mlogloss => 8, :logistic_mle => 9)
-loss_id(::Type{L}) where {L} = haskey(LOSS_ID, L) ? LOSS_ID[L] : error("loss $L is not supported by libevotrees_hip (mse, logloss, poisson, gamma, tweedie, mlogloss, gaussian_mle, logistic_mle)")
+loss_id(::Type{L}) where {L} = haskey(LOSS_ID, L) ? LOSS_ID[L] : error("loss $L is not supported by libevotrees_hip (mse, logloss, poisson, gamma, tweedie, mlogloss, gaussian_mle, logistic_mle, mae, cred_var, cred_std)")
 
 # ---------------------------------------------------------------------------------------------------------------
 # device_array_type / device_ones: `init` calls both before `init_core` (src/init.jl:331-333, :283-285).  Host arrays

@@ -51,6 +51,10 @@
 #define ORC_GAMMA 4
 #define ORC_TWEEDIE 5
 #define ORC_MLOGLOSS 6
+#define ORC_MAE 8
+#define ORC_CRED_VAR 9
+#define ORC_CRED_STD 10
+#define ORC_IS_CRED(l) ((l) == ORC_CRED_VAR || (l) == ORC_CRED_STD)
 #define ORC_MAX_NK 40 /* 2K+1 with up to 16 classes, rounded up */
 
 typedef struct {
@@ -167,6 +171,13 @@ void orc_update_grads(const orc_params *p, int64_t N, const float *pred, const f
                 float e = expf(pk);
                 gg = 2.0f * (1.0f - yk / e);
                 hh = 2.0f * yk / e;
+            } else if (p->loss == ORC_MAE) { /* mae_grad_hess, src/loss.jl:78 (update_grads! :130-142) */
+                gg = yk - pk;
+                hh = 0.0f;
+            } else if (ORC_IS_CRED(p->loss)) { /* cred_grad_hess, src/loss.jl:80-83 (update_grads! :173-185) */
+                float d = yk - pk;
+                gg = d;
+                hh = d * d;
             } else { /* tweedie, src/loss.jl:69-76, rho = 1.5 */
                 float e = expf(pk);
                 float a = powf(e, 0.5f), b = powf(e, -0.5f);
@@ -367,16 +378,53 @@ static inline double term_gh(double g, double h, double w, double lambda, double
     return g * g / d / 2.0;
 }
 
-/* node_gain — src/split.jl:58-66 */
-static double node_gain(const double *S, int K, double lambda, double L2, double eps) {
+/* _term_shift — src/split.jl:2 */
+static inline double term_shift(double g, double w, double mu_p, double d) { return fabs(g / w - mu_p) * w / d; }
+
+/* _cred_Z — src/loss.jl:275-290: VHM = (m1 / w)^2, EVPV = max(eps, m2 / w - VHM); the ratio of variances (cred_var) or of
+ * standard deviations (cred_std).  _term_cred — src/split.jl:3-4. */
+static inline double term_cred(int loss, double m1, double m2, double w, double L2, double eps) {
+    double mean = m1 / w;
+    double VHM = mean * mean;
+    double EVPV = m2 / w - VHM;
+    if (!(EVPV > eps)) EVPV = eps;
+    double Z = (loss == ORC_CRED_VAR) ? VHM / (VHM + EVPV) : sqrt(VHM) / (sqrt(VHM) + sqrt(EVPV));
+    return Z * fabs(m1) / (1.0 + L2 / w);
+}
+
+/* node_gain — src/split.jl:58-66 (gradient losses), :68 (mae: zero), :70-78 (credibility losses) */
+static double node_gain(int loss, const double *S, int K, double lambda, double L2, double eps) {
     double w = S[2 * K], gain = 0.0;
+    if (loss == ORC_MAE) return 0.0;
+    if (ORC_IS_CRED(loss)) {
+        for (int k = 0; k < K; k++) gain += term_cred(loss, S[k], S[K + k], w, L2, eps);
+        return gain;
+    }
     for (int k = 0; k < K; k++) gain += term_gh(S[k], S[K + k], w, lambda, L2, eps);
     return gain;
 }
 
-/* split_gain — src/split.jl:108-117 */
-static double split_gain(const double *S, const double *SL, int K, double w_l, double w_r, double lambda, double L2, double eps) {
+/* split_gain — src/split.jl:108-117 (gradient losses), :119-130 (mae), :132-141 (credibility losses) */
+static double split_gain(int loss, const double *S, const double *SL, int K, double w_l, double w_r, double lambda, double L2, double eps) {
     double gain = 0.0;
+    if (loss == ORC_MAE) {
+        double w_p = S[2 * K];
+        double d_l = 1.0 + lambda + L2 / w_l, d_r = 1.0 + lambda + L2 / w_r;
+        if (!(d_l > eps)) d_l = eps;
+        if (!(d_r > eps)) d_r = eps;
+        for (int k = 0; k < K; k++) {
+            double mu_p = S[k] / w_p;
+            gain += term_shift(SL[k], w_l, mu_p, d_l) + term_shift(S[k] - SL[k], w_r, mu_p, d_r);
+        }
+        return gain;
+    }
+    if (ORC_IS_CRED(loss)) {
+        for (int k = 0; k < K; k++) {
+            double m1l = SL[k], m2l = SL[K + k];
+            gain += term_cred(loss, m1l, m2l, w_l, L2, eps) + term_cred(loss, S[k] - m1l, S[K + k] - m2l, w_r, L2, eps);
+        }
+        return gain;
+    }
     for (int k = 0; k < K; k++) {
         double g_l = SL[k], h_l = SL[K + k];
         gain += term_gh(g_l, h_l, w_l, lambda, L2, eps) + term_gh(S[k] - g_l, S[K + k] - h_l, w_r, lambda, L2, eps);
@@ -384,22 +432,39 @@ static double split_gain(const double *S, const double *SL, int K, double w_l, d
     return gain;
 }
 
-/* pred_scalar — src/predict.jl:205-208 (GradientRegression), :235-238 (MLE2P) */
+/* pred_scalar — src/predict.jl:205-208 (GradientRegression), :235-238 (MLE2P), :219-221 (credibility), :259-262 (mae) */
 static double pred_scalar(const double *S, const orc_params *p) {
     int K = p->K;
+    if (ORC_IS_CRED(p->loss)) return p->eta / (double)p->bagging_size * S[0] / (S[2 * K] + p->L2);
+    if (p->loss == ORC_MAE) {
+        double d = S[2 * K] + p->lambda * S[2 * K] + p->L2;
+        if (!(d > DBL_EPSILON)) d = DBL_EPSILON;
+        return p->eta / (double)p->bagging_size * S[0] / d;
+    }
     double d = S[K] + p->lambda * S[2 * K] + p->L2;
     if (!(d > DBL_EPSILON)) d = DBL_EPSILON;
     return -p->eta / (double)p->bagging_size * S[0] / d;
 }
 
 /* pred_leaf_cpu! — src/predict.jl:198-204 (GradientRegression), :224-234 (MLE2P; for one
- * target the index pairs are (1,3),(2,4), i.e. (k, K+k) as well).  Stored as Float32. */
+ * target the index pairs are (1,3),(2,4), i.e. (k, K+k) as well), :211-217 (credibility), :250-258 (mae).
+ * Stored as Float32. */
 static void pred_leaf(float *tree_pred, int n, const double *S, const orc_params *p) {
     int K = p->K;
     for (int k = 0; k < K; k++) {
-        double d = S[K + k] + p->lambda * S[2 * K] + p->L2;
-        if (!(d > DBL_EPSILON)) d = DBL_EPSILON;
-        tree_pred[(size_t)K * (n - 1) + k] = (float)(-p->eta / (double)p->bagging_size * S[k] / d);
+        double v;
+        if (ORC_IS_CRED(p->loss)) {
+            v = p->eta / (double)p->bagging_size * S[k] / (S[2 * K] + p->L2);
+        } else if (p->loss == ORC_MAE) {
+            double d = S[2 * K] + p->lambda * S[2 * K] + p->L2;
+            if (!(d > DBL_EPSILON)) d = DBL_EPSILON;
+            v = p->eta / (double)p->bagging_size * S[k] / d;
+        } else {
+            double d = S[K + k] + p->lambda * S[2 * K] + p->L2;
+            if (!(d > DBL_EPSILON)) d = DBL_EPSILON;
+            v = -p->eta / (double)p->bagging_size * S[k] / d;
+        }
+        tree_pred[(size_t)K * (n - 1) + k] = (float)v;
     }
 }
 
@@ -418,7 +483,7 @@ static void scan_node(orc_cache *c, int n, const uint32_t *js, int nj, int mode,
     const double *S = c->sum + (size_t)n * NK;
     double SL[ORC_MAX_NK], SR[ORC_MAX_NK];
     int64_t SLq[ORC_MAX_NK];
-    double gain_p = node_gain(S, K, p->lambda, p->L2, eps);
+    double gain_p = node_gain(p->loss, S, K, p->lambda, p->L2, eps);
     double w_p = S[NK - 1];
     for (int jj = 0; jj < nj; jj++) {
         int j = (int)js[jj] - 1;
@@ -447,7 +512,7 @@ static void scan_node(orc_cache *c, int n, const uint32_t *js, int nj, int mode,
                     double predL = pred_scalar(SL, p), predR = pred_scalar(SR, p);
                     ok = (constraint == -1 && predL > predR) || (constraint == 1 && predL < predR);
                 }
-                if (ok) sink(ctx, split_gain(S, SL, K, w_l, w_r, p->lambda, p->L2, eps) - gain_p, j + 1, bin + 1);
+                if (ok) sink(ctx, split_gain(p->loss, S, SL, K, w_l, w_r, p->lambda, p->L2, eps) - gain_p, j + 1, bin + 1);
             }
         }
     }
@@ -720,7 +785,7 @@ void orc_predict_tree(int32_t loss, int32_t K, int64_t N, const uint8_t *x_bin, 
             float m = -INFINITY;
             for (int k = 0; k < K; k++) { pr[k] += lp[k]; if (pr[k] > m) m = pr[k]; }
             for (int k = 0; k < K; k++) { float v = pr[k] - m; pr[k] = v > -15.0f ? v : -15.0f; }
-        } else if (loss == ORC_MSE || (loss >= ORC_POISSON && loss != ORC_LOGISTIC_MLE)) {
+        } else if (loss == ORC_MSE || (loss >= ORC_POISSON && loss != ORC_LOGISTIC_MLE)) { /* generic method, src/predict.jl:68-81, for mae and the credibility losses */
             for (int k = 0; k < K; k++) pr[k] += lp[k];
         } else if (loss == ORC_LOGLOSS) {
             for (int k = 0; k < K; k++) {
@@ -756,7 +821,7 @@ void orc_apply_link(int32_t loss, int32_t K, int64_t N, float *pred) {
             float isum = 0.0f;
             for (int k = 0; k < K; k++) { pred[(size_t)K * i + k] = expf(pred[(size_t)K * i + k]); isum += pred[(size_t)K * i + k]; }
             for (int k = 0; k < K; k++) pred[(size_t)K * i + k] /= isum;
-        } else if (loss >= ORC_POISSON && loss != ORC_LOGISTIC_MLE) {
+        } else if (loss >= ORC_POISSON && loss <= ORC_TWEEDIE) {
             for (int k = 0; k < K; k++) pred[(size_t)K * i + k] = expf(pred[(size_t)K * i + k]);
         }
     }

@@ -27,15 +27,62 @@ def term(g, h, w, lam, L2):
     return g * g / np.maximum(EPS, h + lam * w + L2) / 2.0
 
 
-def leaf_value(S, K, eta, lam, L2, bagging=1):
+def cred_term(kind, m1, m2, w, L2):
+    """Credibility-weighted absolute sum: Z |m1| / (1 + L2 / w) with Z = between / (between + within), on variances
+    (cred_var) or on standard deviations (cred_std); the within-variance is floored at eps."""
+    between = (m1 / w) ** 2
+    within = np.maximum(EPS, m2 / w - between)
+    if kind == "cred_std":
+        between, within = np.sqrt(between), np.sqrt(within)
+    return between / (between + within) * np.abs(m1) / (1.0 + L2 / w)
+
+
+def side_terms(kind, S, L, K, wl, wr, lam, L2):
+    """Gain of the two sides summed over the K outputs; L holds the left sums of every candidate (rows)."""
+    g = np.zeros(L.shape[0])
+    for k in range(K):
+        if kind == "mae":  # absolute shift of each side's mean residual from the parent's, weighted
+            mu_p = S[k] / S[2 * K]
+            dl = np.maximum(EPS, 1.0 + lam + L2 / wl)
+            dr = np.maximum(EPS, 1.0 + lam + L2 / wr)
+            g = g + (np.abs(L[:, k] / wl - mu_p) * wl / dl + np.abs((S[k] - L[:, k]) / wr - mu_p) * wr / dr)
+        elif kind in ("cred_var", "cred_std"):
+            g = g + (cred_term(kind, L[:, k], L[:, K + k], wl, L2) + cred_term(kind, S[k] - L[:, k], S[K + k] - L[:, K + k], wr, L2))
+        else:
+            g = g + (term(L[:, k], L[:, K + k], wl, lam, L2) + term(S[k] - L[:, k], S[K + k] - L[:, K + k], wr, lam, L2))
+    return g
+
+
+def parent_gain(kind, S, K, lam, L2):
+    if kind == "mae":
+        return 0.0
+    if kind in ("cred_var", "cred_std"):
+        return sum(cred_term(kind, S[k], S[K + k], S[2 * K], L2) for k in range(K))
+    return sum(term(S[k], S[K + k], S[2 * K], lam, L2) for k in range(K))
+
+
+def leaf_value(S, K, eta, lam, L2, bagging=1, kind="gh"):
+    if kind == "mae":
+        return np.array([eta / bagging * S[k] / max(EPS, S[2 * K] + lam * S[2 * K] + L2) for k in range(K)])
+    if kind in ("cred_var", "cred_std"):
+        return np.array([eta / bagging * S[k] / (S[2 * K] + L2) for k in range(K)])
     return np.array([-eta / bagging * S[k] / max(EPS, S[K + k] + lam * S[2 * K] + L2) for k in range(K)])
 
 
-def gains_matrix(h, S, js, feattypes, mono, K, lam, L2, min_weight, eta):
+def first_output_value(kind, L, K, w, eta, lam, L2):
+    """Leaf value of output 1 for every candidate side (monotone constraints compare the two sides' values)."""
+    if kind == "mae":
+        return eta * L[:, 0] / np.maximum(EPS, w + lam * w + L2)
+    if kind in ("cred_var", "cred_std"):
+        return eta * L[:, 0] / (w + L2)
+    return -eta * L[:, 0] / np.maximum(EPS, L[:, K] + lam * w + L2)
+
+
+def gains_matrix(h, S, js, feattypes, mono, K, lam, L2, min_weight, eta, kind="gh"):
     """Returns gains[jpos, bin] (-inf where not a candidate), for features js (1-based)."""
     nbins = h.shape[1]
     out = np.full((len(js), nbins), -np.inf)
-    gp = sum(term(S[k], S[K + k], S[2 * K], lam, L2) for k in range(K))
+    gp = parent_gain(kind, S, K, lam, L2)
     for jp, j in enumerate(js):
         hj = h[j - 1]
         if feattypes[j - 1]:
@@ -45,21 +92,18 @@ def gains_matrix(h, S, js, feattypes, mono, K, lam, L2, min_weight, eta):
         wl = L[:, 2 * K]
         wr = S[2 * K] - wl
         ok = (wl > min_weight) & (wr > min_weight)
-        g = np.zeros(L.shape[0])
-        for k in range(K):
-            g = g + (term(L[:, k], L[:, K + k], wl, lam, L2) + term(S[k] - L[:, k], S[K + k] - L[:, K + k], wr, lam, L2))
-        g = g - gp
-        if mono[j - 1] != 0:
-            pl = -eta * L[:, 0] / np.maximum(EPS, L[:, K] + lam * wl + L2)
-            R = S[None, :] - L
-            pr = -eta * R[:, 0] / np.maximum(EPS, R[:, K] + lam * wr + L2)
-            ok &= (pl > pr) if mono[j - 1] == -1 else (pl < pr)
+        with np.errstate(divide="ignore", invalid="ignore"):
+            g = side_terms(kind, S, L, K, wl, wr, lam, L2) - gp
+            if mono[j - 1] != 0:
+                pl = first_output_value(kind, L, K, wl, eta, lam, L2)
+                pr = first_output_value(kind, S[None, :] - L, K, wr, eta, lam, L2)
+                ok &= (pl > pr) if mono[j - 1] == -1 else (pl < pr)
         out[jp, : L.shape[0]] = np.where(ok, g, -np.inf)
     return out
 
 
 def grow(x_bin_FN, grad, rows, js, K, nbins, max_depth, eta=0.1, lam=0.0, L2=1.0, gamma=0.0, min_weight=1.0,
-         feattypes=None, mono=None, oblivious=False):
+         feattypes=None, mono=None, oblivious=False, kind="gh"):
     F, N = x_bin_FN.shape
     feattypes = np.ones(F, bool) if feattypes is None else np.asarray(feattypes, bool)
     mono = np.zeros(F, int) if mono is None else np.asarray(mono, int)
@@ -77,14 +121,14 @@ def grow(x_bin_FN, grad, rows, js, K, nbins, max_depth, eta=0.1, lam=0.0, L2=1.0
         if depth == max_depth:
             for n in active:
                 T["w"][n - 1] = sums[n][2 * K]
-                T["pred"][n - 1] = leaf_value(sums[n], K, eta, lam, L2)
+                T["pred"][n - 1] = leaf_value(sums[n], K, eta, lam, L2, kind=kind)
             break
         G = {}
         for n in active:
             r = np.flatnonzero(label == n)
             hists[n] = dense_hist(x_bin_FN, grad, r, nbins)
             T["w"][n - 1] = sums[n][2 * K]
-            G[n] = gains_matrix(hists[n], sums[n], js, feattypes, mono, K, lam, L2, min_weight, eta)
+            G[n] = gains_matrix(hists[n], sums[n], js, feattypes, mono, K, lam, L2, min_weight, eta, kind=kind)
         decisions = {}
         if not oblivious:
             for n in active:
@@ -125,7 +169,7 @@ def grow(x_bin_FN, grad, rows, js, K, nbins, max_depth, eta=0.1, lam=0.0, L2=1.0
                 sums[2 * n + 1] = sums[n] - SL
                 nxt += [2 * n, 2 * n + 1]
             else:
-                T["pred"][n - 1] = leaf_value(sums[n], K, eta, lam, L2)
+                T["pred"][n - 1] = leaf_value(sums[n], K, eta, lam, L2, kind=kind)
         active = nxt
     return T, label, hists, sums
 

@@ -88,7 +88,8 @@ def _sinus(rng, n):
 
 @pytest.mark.parametrize("cfg_kw", [dict(loss="mse", metric="mae"), dict(loss="logloss"), dict(loss="gamma"), dict(loss="tweedie"),
                                     dict(loss="poisson", learner="count"), dict(loss="gaussian_mle", learner="mle"),
-                                    dict(loss="logistic_mle", learner="mle")])
+                                    dict(loss="logistic_mle", learner="mle"), dict(loss="mae"), dict(loss="cred_var"),
+                                    dict(loss="cred_std", metric="rmse")])
 def test_fit_with_eval_logger_matches_oracle_replay(evt, cfg_kw):
     # every logged value equals the oracle's metric of the oracle's own replay of the model on the eval rows
     rng = np.random.default_rng(7)
@@ -103,6 +104,8 @@ def test_fit_with_eval_logger_matches_oracle_replay(evt, cfg_kw):
     m = evt.fit(cfg, x_train=X[tr], y_train=Y[tr], x_eval=X[ev], y_eval=Y[ev], w_eval=w_ev, verbosity=0)
     lg = m.info["logger"]
     assert lg["name"] == cfg.metric and lg["iter"] == list(range(13)) and lg["nrounds"] == 12
+    if cfg.loss in ("mae", "cred_var"):
+        assert cfg.metric == "mae"  # the credibility losses are tracked by mae unless told otherwise (src/learners.jl:76-81)
     assert lg["maximise"] == (cfg.loss in ("gaussian_mle", "logistic_mle"))
     xb = evt.binarize(X[ev], m.info["edges"])
     ft = np.ones(1, np.uint8)

@@ -44,6 +44,10 @@ CASES = [
     ("gaussian_mle", 8, True, 3000, 6, 255, 3, "binary", 6, 1.0, False),
     ("logistic_mle", 2, True, 12000, 14, 32, 5, "binary", 14, 1.0, False),
     ("logistic_mle", 3, False, 9000, 40, 64, 4, "oblivious", 25, 0.5, True),
+    ("mae", 3, True, 12000, 14, 32, 5, "binary", 14, 1.0, False),
+    ("mae", 2, False, 9000, 40, 64, 4, "oblivious", 25, 0.5, True),
+    ("cred_var", 2, True, 12000, 14, 32, 5, "binary", 10, 1.0, True),
+    ("cred_std", 4, False, 9000, 20, 16, 4, "binary", 20, 0.5, False),
 ]
 
 
@@ -60,7 +64,7 @@ def test_multi_target_tree_against_the_oracle(evt, loss, T, weights, N, F, B, D,
     orc.update_grads(op, pred0, y, grad)
     h.update_grads()
     g_dev = h.get_grads()
-    if loss == "mse":
+    if loss in ("mse", "mae", "cred_var", "cred_std"):
         assert np.array_equal(g_dev.view(np.uint32), grad.view(np.uint32))
     else:
         # (1 - r^2 / s^2) and (1 - z tanh(z / 2)) cancel, which magnifies the last-bit differences between two libm's exp / tanh:
@@ -106,7 +110,7 @@ def test_multi_target_tree_against_the_oracle(evt, loss, T, weights, N, F, B, D,
         assert abs(float(t_gpu.gain[n0]) - float(t_ref.gain[n0])) <= 1e-6 * abs(float(t_ref.gain[n0])) + 1e-12
     # the evaluation metric on the updated prediction
     metric = {"mse": "mse", "logloss": "logloss", "poisson": "poisson", "gamma": "gamma", "tweedie": "tweedie",
-              "gaussian_mle": "gaussian_mle", "logistic_mle": "logistic_mle"}[loss]
+              "gaussian_mle": "gaussian_mle", "logistic_mle": "logistic_mle", "mae": "mae", "cred_var": "mae", "cred_std": "mae"}[loss]
     got = h.eval_metric(metric)
     want = orc.eval_metric(metric, K, p_orc, y, w)
     assert abs(got - want) <= 1e-5 * abs(want) + 1e-9

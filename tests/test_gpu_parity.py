@@ -83,7 +83,8 @@ def assert_tree_close(t_gpu, t_ref, pred_atol=1e-9):
 # --------------------------------------------------------------------------- gradients
 @pytest.mark.parametrize("loss,weights", [("mse", False), ("mse", True), ("logloss", True), ("gaussian_mle", False),
                                           ("gaussian_mle", True), ("poisson", True), ("gamma", False), ("tweedie", True),
-                                          ("mlogloss", False), ("mlogloss", True), ("logistic_mle", False), ("logistic_mle", True)])
+                                          ("mlogloss", False), ("mlogloss", True), ("logistic_mle", False), ("logistic_mle", True),
+                                          ("mae", False), ("mae", True), ("cred_var", True), ("cred_std", False)])
 def test_gradient_kernel(evt, loss, weights):
     N, F, B = 70001, 5, 16
     x_bin, y, w, mu = make_data(1, N, F, B, loss, weights)
@@ -94,7 +95,7 @@ def test_gradient_kernel(evt, loss, weights):
     orc.update_grads(op, pred0, y, grad)
     K = op.K
     assert np.array_equal(g_gpu[:, 2 * K], grad[:, 2 * K])  # weight row untouched
-    if loss == "mse":
+    if loss in ("mse", "mae", "cred_var", "cred_std"):
         assert np.array_equal(g_gpu.view(np.uint32), grad.view(np.uint32))  # exact Float32 arithmetic
     else:
         # terms like (1 - z tanh(z / 2)) cancel: the absolute bound is a few ulp of the largest gradient
@@ -134,6 +135,13 @@ CASES = [
     ("mlogloss", False, 20000, 100, 16, 4, "binary", 100, 1.0, dict(K=2)),
     ("mlogloss", False, 20000, 10, 32, 4, "oblivious", 10, 1.0, dict(K=5)),
     ("mlogloss", True, 12000, 9, 128, 4, "binary", 9, 1.0, dict(K=16, min_weight=2.0)),
+    ("mae", False, 30000, 12, 32, 6, "binary", 12, 1.0, {}),
+    ("mae", True, 40000, 100, 64, 6, "binary", 60, 0.6, dict(lambda_=0.3, L2=0.5, gamma=0.01)),
+    ("mae", False, 20000, 10, 16, 5, "oblivious", 10, 1.0, {}),
+    ("cred_var", False, 30000, 12, 32, 6, "binary", 12, 1.0, {}),
+    ("cred_var", True, 40000, 100, 64, 6, "binary", 100, 0.7, dict(L2=2.0, min_weight=4.0)),
+    ("cred_std", False, 30000, 20, 64, 6, "binary", 14, 1.0, dict(L2=0.0)),
+    ("cred_std", True, 20000, 10, 16, 5, "oblivious", 10, 0.8, {}),
     ("mse", False, 60000, 5, 8, 14, "binary", 5, 1.0, dict(min_weight=0.0)),   # deep: most leaves hold a handful of rows
     ("logloss", True, 3000, 4, 4, 16, "binary", 4, 0.9, dict(min_weight=0.0)),  # deepest supported tree, far more nodes than rows
 ]

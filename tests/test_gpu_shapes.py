@@ -12,7 +12,7 @@ from test_gpu_parity import assert_tree_bits, make_data, setup_pair
 pytestmark = pytest.mark.gpu
 
 TIES = []  # (case, text) of every case whose structure differs from the Float64 oracle by an exact tie
-LOSSES = ["mse", "logloss", "gaussian_mle", "poisson", "gamma", "tweedie", "mlogloss", "logistic_mle"]
+LOSSES = ["mse", "logloss", "gaussian_mle", "poisson", "gamma", "tweedie", "mlogloss", "logistic_mle", "mae", "cred_var", "cred_std"]
 
 
 def _cases():

@@ -730,3 +730,166 @@ def test_logistic_mle_metric_link_and_predict():
     p = np.zeros((2, 2), np.float32)
     orc.predict_tree(orc.LOSS_IDS["logistic_mle"], 2, x_bin, np.ones(1, np.uint8), t, p)
     assert p.tolist() == [[2.0, -15.0], [-3.0, 1.0]]
+
+
+# ---------------------------------------------------------------- mae and the credibility losses
+KIND = {"mae": "mae", "cred_var": "cred_var", "cred_std": "cred_std"}
+
+
+@pytest.mark.parametrize("loss", ["mae", "cred_var", "cred_std"])
+def test_residual_loss_grads_closed_form(loss):
+    """mae: [(y - p) w, 0, w]; credibility: [d w, d^2 w, w] with d = y - p (src/loss.jl:78-83), in Float32."""
+    N = 500
+    x_bin, y, pred, grad = make_data(61, N, 3, 8, "mse", weights=True)
+    w = grad[:, 2].copy()
+    p = orc.make_params(loss, nbins=8, max_depth=3)
+    orc.update_grads(p, pred, y, grad)
+    d = y - pred[:, 0]
+    assert np.array_equal(grad[:, 0], d * w)
+    assert np.array_equal(grad[:, 1], (np.zeros_like(d) if loss == "mae" else (d * d) * w))
+    assert np.array_equal(grad[:, 2], w)
+
+
+def _stump(loss, x_bin, y, pred, grad, B, lam=0.0, L2=0.0, eta=1.0, min_weight=1.0):
+    p = orc.make_params(loss, nbins=B, max_depth=2, lambda_=lam, L2=L2, eta=eta, min_weight=min_weight)
+    orc.update_grads(p, pred, y, grad)
+    o = orc.Oracle(p, x_bin)
+    rows = np.arange(x_bin.shape[1], dtype=np.uint32)
+    js = np.arange(1, x_bin.shape[0] + 1, dtype=np.uint32)
+    t, nidx = o.grow_tree(grad, rows, js, mode=0)
+    o.close()
+    return t, nidx
+
+
+def test_mae_stump_is_the_largest_weighted_shift_of_the_mean_residual():
+    """With lambda = L2 = 0 and unit weights the mae gain of a split is nL |mean_L - mean| + nR |mean_R - mean|
+    (= 2 nL |mean_L - mean|, the two shifts balance), the parent's gain is zero, and a leaf predicts eta times its mean
+    residual: checked from the raw residuals, no histogram."""
+    N, F, B = 400, 4, 8
+    x_bin, y, pred, grad = make_data(62, N, F, B, "mse", weights=False)
+    t, nidx = _stump("mae", x_bin, y, pred, grad, B, eta=0.7)
+    d = (y - pred[:, 0]).astype(np.float64)
+    best = (-1.0, 0, 0)
+    for j in range(F):
+        for b in range(1, B):  # numeric: bins 1 .. B-1
+            L = x_bin[j] <= b
+            nL, nR = L.sum(), (~L).sum()
+            if nL > 1 and nR > 1:
+                g = nL * abs(d[L].mean() - d.mean()) + nR * abs(d[~L].mean() - d.mean())
+                assert abs(g - 2 * nL * abs(d[L].mean() - d.mean())) < 1e-9 * max(1.0, g)
+                if g > best[0] * (1 + 1e-12) + 1e-12:
+                    best = (g, j + 1, b)
+    assert t.split[0] == 1 and (int(t.feat[0]), int(t.cond_bin[0])) == best[1:]
+    np.testing.assert_allclose(t.gain[0], best[0], rtol=1e-5)
+    L = x_bin[best[1] - 1] <= best[2]
+    np.testing.assert_allclose(t.pred[1, 0], 0.7 * d[L].mean(), rtol=1e-5)
+    np.testing.assert_allclose(t.pred[2, 0], 0.7 * d[~L].mean(), rtol=1e-5)
+    assert np.array_equal(nidx, np.where(L, 2, 3))
+
+
+@pytest.mark.parametrize("loss", ["cred_var", "cred_std"])
+def test_cred_stump_from_raw_residual_moments(loss):
+    """Unit weights, L2 = 0: a side's term is Z |sum d| with Z = mean^2 / (mean^2 + var) = mean^2 / mean(d^2) for
+    cred_var and |mean| / (|mean| + std) for cred_std (population variance); the recorded gain is left + right - parent;
+    a leaf predicts eta * mean residual.  All from numpy's mean / var / std of the raw residuals."""
+    N, F, B = 400, 4, 8
+    x_bin, y, pred, grad = make_data(63, N, F, B, "mse", weights=False)
+    y = (y + 0.8).astype(np.float32)  # residuals with a clear mean
+    t, nidx = _stump(loss, x_bin, y, pred, grad, B, eta=0.5)
+    d = (y - pred[:, 0]).astype(np.float64)
+
+    def term(v):
+        m, var = v.mean(), v.var()
+        Z = m * m / (m * m + var) if loss == "cred_var" else abs(m) / (abs(m) + np.sqrt(var))
+        return Z * abs(v.sum())
+
+    if loss == "cred_var":  # the same credibility written with the second moment only
+        assert abs(term(d) - abs(d.sum()) ** 3 / (len(d) * (d * d).sum())) < 1e-9 * term(d)
+    best = (-np.inf, 0, 0)
+    for j in range(F):
+        for b in range(1, B):
+            L = x_bin[j] <= b
+            if L.sum() > 1 and (~L).sum() > 1:
+                g = term(d[L]) + term(d[~L]) - term(d)
+                if g > best[0] + 1e-12 * abs(g):
+                    best = (g, j + 1, b)
+    assert t.split[0] == 1 and (int(t.feat[0]), int(t.cond_bin[0])) == best[1:]
+    np.testing.assert_allclose(t.gain[0], best[0], rtol=1e-5)
+    L = x_bin[best[1] - 1] <= best[2]
+    np.testing.assert_allclose(t.pred[1, 0], 0.5 * d[L].mean(), rtol=1e-5)
+    np.testing.assert_allclose(t.pred[2, 0], 0.5 * d[~L].mean(), rtol=1e-5)
+
+
+@pytest.mark.parametrize("loss,weights,lam,L2,gamma,minw", [
+    ("mae", False, 0.0, 1.0, 0.0, 1.0),
+    ("mae", True, 0.5, 0.3, 0.05, 2.0),
+    ("cred_var", False, 0.0, 1.0, 0.0, 1.0),
+    ("cred_var", True, 0.0, 0.4, 0.01, 2.0),
+    ("cred_std", False, 0.0, 0.0, 0.0, 1.0),
+    ("cred_std", True, 0.0, 2.0, 0.02, 3.0),
+])
+def test_residual_loss_tree_against_bruteforce(loss, weights, lam, L2, gamma, minw):
+    N, F, B, D = 900, 6, 16, 5
+    x_bin, y, pred, grad = make_data(64, N, F, B, "mse", weights)
+    p = orc.make_params(loss, nbins=B, max_depth=D, lambda_=lam, L2=L2, gamma=gamma, min_weight=minw, eta=0.3)
+    orc.update_grads(p, pred, y, grad)
+    rng = np.random.default_rng(65)
+    rows = np.sort(rng.choice(N, 640, replace=False)).astype(np.uint32)
+    js = np.array([1, 2, 4, 6], np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t, nidx = o.grow_tree(grad, rows, js, mode=0)
+    T, label, hists, sums = brute.grow(x_bin, grad, rows, js, 1, B, D, eta=0.3, lam=lam, L2=L2, gamma=gamma, min_weight=minw, kind=KIND[loss])
+    assert trees_equal_struct(t, T)
+    assert t.split.sum() >= 3
+    np.testing.assert_allclose(t.gain, T["gain"], rtol=1e-5)
+    np.testing.assert_allclose(t.pred, T["pred"], rtol=1e-5, atol=1e-9)
+    np.testing.assert_allclose(t.w, T["w"], rtol=1e-6)
+    assert np.array_equal(nidx.astype(np.int64), label)
+    # fixed-point mode: same structure on this data, values to 1e-5
+    qbits = np.full(3, 38, np.int32)
+    qbits[0] = 30
+    o.set_quant(grad, qbits)
+    t1, nidx1 = o.grow_tree(grad, rows, js, mode=1)
+    assert trees_equal_struct(t1, T) and np.array_equal(nidx1, nidx)
+    np.testing.assert_allclose(t1.pred, t.pred, rtol=1e-5, atol=1e-9)
+    o.close()
+
+
+@pytest.mark.parametrize("loss", ["mae", "cred_std"])
+def test_residual_loss_monotone_and_oblivious_against_bruteforce(loss):
+    N, F, B, D = 700, 5, 12, 4
+    x_bin, y, pred, grad = make_data(66, N, F, B, "mse", weights=True)
+    y = (y + 0.02 * x_bin[0] - 0.03 * x_bin[2]).astype(np.float32)
+    mono = np.array([1, 0, -1, 0, 0], np.int32)
+    rows = np.arange(N, dtype=np.uint32)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    for tt in ("binary", "oblivious"):
+        p = orc.make_params(loss, nbins=B, max_depth=D, tree_type=tt, eta=0.2, L2=0.5, min_weight=3.0)
+        orc.update_grads(p, pred, y, grad)
+        o = orc.Oracle(p, x_bin, monotone=mono)
+        t, nidx = o.grow_tree(grad, rows, js, mode=0)
+        T, label, _, _ = brute.grow(x_bin, grad, rows, js, 1, B, D, eta=0.2, L2=0.5, min_weight=3.0, mono=mono, oblivious=(tt == "oblivious"),
+                                    kind=KIND[loss])
+        assert trees_equal_struct(t, T), tt
+        assert t.split.sum() >= 1
+        np.testing.assert_allclose(t.pred, T["pred"], rtol=1e-5, atol=1e-9)
+        assert np.array_equal(nidx.astype(np.int64), label)
+        o.close()
+
+
+def test_residual_loss_predict_adds_and_link_is_identity():
+    """The generic predict! (src/predict.jl:68-81) adds the leaf value, no clamp; apply_prediction_link! leaves these
+    losses alone (src/predict.jl:105-116)."""
+    N, F, B = 50, 3, 4
+    rng = np.random.default_rng(67)
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    t = orc.Tree(1, 3)
+    t.split[0] = 1; t.feat[0] = 2; t.cond_bin[0] = 2
+    t.pred[1, 0] = 40.0; t.pred[2, 0] = -40.0
+    for loss in ("mae", "cred_var", "cred_std"):
+        pred = np.full((N, 1), 3.0, np.float32)
+        orc.predict_tree(orc.LOSS_IDS[loss], 1, x_bin, np.ones(F, np.uint8), t, pred)
+        assert np.array_equal(pred[:, 0], np.where(x_bin[1] <= 2, 43.0, -37.0).astype(np.float32))
+        q = pred.copy()
+        orc.apply_link(orc.LOSS_IDS[loss], 1, q)
+        assert np.array_equal(q, pred)
