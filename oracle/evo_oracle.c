@@ -55,6 +55,10 @@
 #define ORC_CRED_VAR 9
 #define ORC_CRED_STD 10
 #define ORC_IS_CRED(l) ((l) == ORC_CRED_VAR || (l) == ORC_CRED_STD)
+#define ORC_QUANTILE 11
+#define ORC_MULTIQUANTILE 12
+#define ORC_IS_QUANTILE(l) ((l) == ORC_QUANTILE || (l) == ORC_MULTIQUANTILE)
+#define ORC_IS_SHIFT(l) ((l) == ORC_MAE || ORC_IS_QUANTILE(l)) /* gains of Union{MAE,Quantile}, src/split.jl:68, :119 */
 #define ORC_MAX_NK 40 /* 2K+1 with up to 16 classes, rounded up */
 
 typedef struct {
@@ -65,6 +69,8 @@ typedef struct {
     int32_t tree_type;    /* 0 binary (grow_tree!), 1 oblivious (grow_otree!)              */
     int32_t bagging_size; /* divides the leaf value (src/predict.jl:202)                   */
     double eta, L2, lambda, gamma, min_weight;
+    int32_t n_alphas;     /* 1: params.alpha (quantile); K: params.alphas (multiquantile)  */
+    double alphas[16];
 } orc_params;
 
 typedef struct {
@@ -171,6 +177,17 @@ void orc_update_grads(const orc_params *p, int64_t N, const float *pred, const f
                 float e = expf(pk);
                 gg = 2.0f * (1.0f - yk / e);
                 hh = 2.0f * yk / e;
+            } else if (ORC_IS_QUANTILE(p->loss)) {
+                /* quantile_grad_diff, src/loss.jl:85-91; update_grads! :144-156 (quantile: one alpha, a target column per
+                 * output) and :158-171 (multiquantile: one target, an alpha per output).  The first row is alpha or
+                 * alpha - 1 (Float64) times the weight, the second the raw residual, NOT weighted. */
+                const int mq = (p->loss == ORC_MULTIQUANTILE);
+                const double alpha = mq ? p->alphas[k] : p->alphas[0];
+                if (mq) yk = y[i];
+                const float diff = yk - pk;
+                g[k] = (float)((diff > 0.0f ? alpha : alpha - 1.0) * (double)w);
+                g[K + k] = diff;
+                continue;
             } else if (p->loss == ORC_MAE) { /* mae_grad_hess, src/loss.jl:78 (update_grads! :130-142) */
                 gg = yk - pk;
                 hh = 0.0f;
@@ -395,7 +412,7 @@ static inline double term_cred(int loss, double m1, double m2, double w, double 
 /* node_gain — src/split.jl:58-66 (gradient losses), :68 (mae: zero), :70-78 (credibility losses) */
 static double node_gain(int loss, const double *S, int K, double lambda, double L2, double eps) {
     double w = S[2 * K], gain = 0.0;
-    if (loss == ORC_MAE) return 0.0;
+    if (ORC_IS_SHIFT(loss)) return 0.0;
     if (ORC_IS_CRED(loss)) {
         for (int k = 0; k < K; k++) gain += term_cred(loss, S[k], S[K + k], w, L2, eps);
         return gain;
@@ -407,7 +424,7 @@ static double node_gain(int loss, const double *S, int K, double lambda, double 
 /* split_gain — src/split.jl:108-117 (gradient losses), :119-130 (mae), :132-141 (credibility losses) */
 static double split_gain(int loss, const double *S, const double *SL, int K, double w_l, double w_r, double lambda, double L2, double eps) {
     double gain = 0.0;
-    if (loss == ORC_MAE) {
+    if (ORC_IS_SHIFT(loss)) {
         double w_p = S[2 * K];
         double d_l = 1.0 + lambda + L2 / w_l, d_r = 1.0 + lambda + L2 / w_r;
         if (!(d_l > eps)) d_l = eps;
@@ -466,6 +483,47 @@ static void pred_leaf(float *tree_pred, int n, const double *S, const orc_params
         }
         tree_pred[(size_t)K * (n - 1) + k] = (float)v;
     }
+}
+
+/* Statistics.quantile(v, p) with its defaults alpha = beta = 1 (the stdlib the reference calls; Hyndman & Fan's
+ * definition 7, numpy's "linear"): on the sorted values, aleph = fma(n, p, 1 - p), j = clamp(trunc(aleph), 1, n - 1),
+ * gamma = clamp(aleph - j, 0, 1), result v[j] + gamma * (v[j+1] - v[j]) with the difference taken in the values' own
+ * Float32 and the rest in Float64.  v is sorted here (ascending). */
+static int cmp_f32(const void *a, const void *b) {
+    float x = *(const float *)a, y = *(const float *)b;
+    return (x > y) - (x < y);
+}
+static double jl_quantile(float *v, int64_t n, double p) {
+    qsort(v, (size_t)n, sizeof(float), cmp_f32);
+    double aleph = fma((double)n, p, 1.0 - p);
+    int64_t j = (int64_t)aleph;
+    if (j > n - 1) j = n - 1; /* clamp(x, lo, hi) = ifelse(x > hi, hi, ifelse(x < lo, lo, x)) */
+    else if (j < 1) j = 1;
+    double gamma = aleph - (double)j;
+    if (gamma > 1.0) gamma = 1.0;
+    else if (gamma < 0.0) gamma = 0.0;
+    float a, b;
+    if (n == 1) { a = v[0]; b = v[0]; }
+    else { a = v[j - 1]; b = v[j]; }
+    if (isfinite(a) && isfinite(b)) return (double)a + gamma * (double)(b - a);
+    return (1.0 - gamma) * (double)a + gamma * (double)b;
+}
+
+/* pred_leaf_cpu! of the quantile losses — src/predict.jl:265-272 (quantile: max(eps, denom)) and :275-281
+ * (multiquantile): eta / bagging * quantile(residuals of the leaf's rows, alpha) / (1 + lambda + L2 / w).  rows: the
+ * node's row ids; the residual of output k is row K + k of the gradient matrix. */
+static void pred_leaf_quantile(float *tree_pred, int n, const double *S, const orc_params *p, const float *grad, const uint32_t *rows, int64_t nrows) {
+    const int K = p->K, NK = 2 * K + 1;
+    float *v = (float *)malloc(sizeof(float) * (size_t)(nrows > 0 ? nrows : 1));
+    double denom = 1.0 + p->lambda + p->L2 / S[2 * K];
+    if (p->loss == ORC_QUANTILE && !(denom > DBL_EPSILON)) denom = DBL_EPSILON;
+    for (int k = 0; k < K; k++) {
+        for (int64_t t = 0; t < nrows; t++) v[t] = grad[(int64_t)NK * rows[t] + K + k];
+        const double alpha = (p->loss == ORC_MULTIQUANTILE) ? p->alphas[k] : p->alphas[0];
+        const double q = nrows > 0 ? jl_quantile(v, nrows, alpha) : 0.0;
+        tree_pred[(size_t)K * (n - 1) + k] = (float)(p->eta / (double)p->bagging_size * q / denom);
+    }
+    free(v);
 }
 
 typedef void (*scan_sink)(void *ctx, double gain, int j, int bin);
@@ -645,7 +703,8 @@ int orc_grow_tree(orc_cache *c, const float *grad, const uint32_t *is_in, int64_
                 int n = n_current[t];
                 const double *S = c->sum + (size_t)n * NK;
                 t_w[n - 1] = (float)S[NK - 1];
-                pred_leaf(t_pred, n, S, p);
+                if (ORC_IS_QUANTILE(p->loss)) pred_leaf_quantile(t_pred, n, S, p, grad, c->is + c->seg_off[n], c->seg_len[n]);
+                else pred_leaf(t_pred, n, S, p);
                 if (nidx_out) for (int64_t q = 0; q < c->seg_len[n]; q++) nidx_out[c->is[c->seg_off[n] + q]] = (uint32_t)n;
             }
         } else {
@@ -743,7 +802,8 @@ int orc_grow_tree(orc_cache *c, const float *grad, const uint32_t *is_in, int64_
                     if (len - nl >= nl) { n_next[nnext++] = 2 * n; n_next[nnext++] = 2 * n + 1; }
                     else { n_next[nnext++] = 2 * n + 1; n_next[nnext++] = 2 * n; }
                 } else {
-                    pred_leaf(t_pred, n, c->sum + (size_t)n * NK, p);
+                    if (ORC_IS_QUANTILE(p->loss)) pred_leaf_quantile(t_pred, n, c->sum + (size_t)n * NK, p, grad, c->is + c->seg_off[n], c->seg_len[n]);
+                    else pred_leaf(t_pred, n, c->sum + (size_t)n * NK, p);
                     /* rows of a finished node: record before later splits overwrite the buffer */
                     if (nidx_out) for (int64_t q = 0; q < c->seg_len[n]; q++) nidx_out[c->is[c->seg_off[n] + q]] = (uint32_t)n;
                 }
@@ -833,6 +893,26 @@ void orc_apply_link(int32_t loss, int32_t K, int64_t N, float *pred) {
  * metric: 0 mse, 1 rmse, 2 mae, 3 logloss, 4 gaussian_mle, 5 poisson, 6 gamma, 7 tweedie, 9 logistic_mle, 8 mlogloss (:59-77,
  * eval[i] = w[i] * (log(sum_k exp(p[k,i])) - p[y[i], i]), not divided by K).
  */
+/* quantile / multiquantile metrics — src/metrics.jl:4-6 (the pinball loss of one output in Float32, alpha given as
+ * T(params.alpha), src/callback.jl:62-66), :83-84 (quantile: averaged over the K outputs like every other metric, one
+ * target column each) and :117-134 (multiquantile: one target, alphas[k] for output k).  metric: 10 quantile, 11 multiquantile. */
+double orc_eval_metric_quantile(int32_t metric, int32_t K, int64_t N, const float *pred, const float *y, const float *w, const float *alphas) {
+    double num = 0.0, den = 0.0;
+    for (int64_t i = 0; i < N; i++) {
+        float wi = w ? w[i] : 1.0f, acc = 0.0f;
+        for (int k = 0; k < K; k++) {
+            float pk = pred[(size_t)K * i + k], yk = (metric == 11) ? y[i] : y[(size_t)K * i + k];
+            float alpha = (metric == 11) ? alphas[k] : alphas[0];
+            float up = yk - pk, dn = pk - yk;
+            acc += alpha * (up > 0.0f ? up : 0.0f) + (1.0f - alpha) * (dn > 0.0f ? dn : 0.0f);
+        }
+        float ev = wi * acc / (float)K;
+        num += (double)ev;
+        den += (double)wi;
+    }
+    return num / den;
+}
+
 double orc_eval_metric(int32_t metric, int32_t K, int64_t N, const float *pred, const float *y, const float *w) {
     double num = 0.0, den = 0.0;
     for (int64_t i = 0; i < N; i++) {

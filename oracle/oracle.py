@@ -13,8 +13,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libevo_oracle.so")
 
 LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5, "mlogloss": 6, "logistic_mle": 7, "mae": 8,
-            "cred_var": 9, "cred_std": 10}
-METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8, "logistic_mle": 9}
+            "cred_var": 9, "cred_std": 10, "quantile": 11, "multiquantile": 12}
+METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8, "logistic_mle": 9, "quantile": 10, "multiquantile": 11}
 TREE_TYPES = {"binary": 0, "oblivious": 1}
 
 
@@ -31,6 +31,8 @@ class OrcParams(C.Structure):
         ("lambda_", C.c_double),
         ("gamma", C.c_double),
         ("min_weight", C.c_double),
+        ("n_alphas", C.c_int32),
+        ("alphas", C.c_double * 16),
     ]
 
 
@@ -84,6 +86,8 @@ def lib():
         L.orc_apply_link.restype = None
         L.orc_eval_metric.argtypes = [i32, i32, i64, vp, vp, vp]
         L.orc_eval_metric.restype = C.c_double
+        L.orc_eval_metric_quantile.argtypes = [i32, i32, i64, vp, vp, vp, vp]
+        L.orc_eval_metric_quantile.restype = C.c_double
         _lib = L
     return _lib
 
@@ -93,11 +97,18 @@ def _p(a):
 
 
 def make_params(loss="mse", nbins=64, max_depth=6, tree_type="binary", bagging_size=1, eta=0.1, L2=1.0,
-                lambda_=0.0, gamma=0.0, min_weight=1.0, K=None):
+                lambda_=0.0, gamma=0.0, min_weight=1.0, K=None, alpha=0.5, alphas=None):
+    """alpha: the quantile loss's level (every output); alphas: the multiquantile loss's levels, one output each."""
+    if loss == "multiquantile":
+        al = [float(a) for a in alphas]
+        K = len(al)
+    else:
+        al = [float(alpha)]
     if K is None:
         K = 2 if loss in ("gaussian_mle", "logistic_mle") else 1
+    arr = (C.c_double * 16)(*(al + [0.0] * (16 - len(al))))
     return OrcParams(LOSS_IDS[loss], K, nbins, max_depth, TREE_TYPES[tree_type], bagging_size, eta, L2, lambda_,
-                     gamma, min_weight)
+                     gamma, min_weight, len(al), arr)
 
 
 class Tree:
@@ -223,7 +234,10 @@ def apply_link(loss_id, K, pred):
     lib().orc_apply_link(loss_id, K, pred.shape[0], _p(pred))
 
 
-def eval_metric(metric, K, pred, y, w=None):
+def eval_metric(metric, K, pred, y, w=None, alphas=None):
     """pred (N, K) f32 raw (link not applied), y (N,) f32, w (N,) f32 or None."""
     w = None if w is None else np.ascontiguousarray(w, np.float32)
+    if metric in ("quantile", "multiquantile"):
+        al = np.ascontiguousarray(alphas, np.float32).reshape(-1)
+        return lib().orc_eval_metric_quantile(METRIC_IDS[metric], K, pred.shape[0], _p(pred), _p(y), _p(w), _p(al))
     return lib().orc_eval_metric(METRIC_IDS[metric], K, pred.shape[0], _p(pred), _p(y), _p(w))

@@ -41,7 +41,7 @@ def side_terms(kind, S, L, K, wl, wr, lam, L2):
     """Gain of the two sides summed over the K outputs; L holds the left sums of every candidate (rows)."""
     g = np.zeros(L.shape[0])
     for k in range(K):
-        if kind == "mae":  # absolute shift of each side's mean residual from the parent's, weighted
+        if kind in ("mae", "quantile"):  # absolute shift of each side's mean first-row value from the parent's, weighted
             mu_p = S[k] / S[2 * K]
             dl = np.maximum(EPS, 1.0 + lam + L2 / wl)
             dr = np.maximum(EPS, 1.0 + lam + L2 / wr)
@@ -54,7 +54,7 @@ def side_terms(kind, S, L, K, wl, wr, lam, L2):
 
 
 def parent_gain(kind, S, K, lam, L2):
-    if kind == "mae":
+    if kind in ("mae", "quantile"):
         return 0.0
     if kind in ("cred_var", "cred_std"):
         return sum(cred_term(kind, S[k], S[K + k], S[2 * K], L2) for k in range(K))
@@ -103,7 +103,10 @@ def gains_matrix(h, S, js, feattypes, mono, K, lam, L2, min_weight, eta, kind="g
 
 
 def grow(x_bin_FN, grad, rows, js, K, nbins, max_depth, eta=0.1, lam=0.0, L2=1.0, gamma=0.0, min_weight=1.0,
-         feattypes=None, mono=None, oblivious=False, kind="gh"):
+         feattypes=None, mono=None, oblivious=False, kind="gh", alphas=None, clamp_denom=True):
+    """kind "quantile": gains as mae on the first gradient rows; a leaf's value of output k is eta times numpy's
+    linear-interpolation quantile (level alphas[k]) of the leaf's rows' residuals, row K + k of grad, over
+    1 + lam + L2 / w (floored at eps when clamp_denom)."""
     F, N = x_bin_FN.shape
     feattypes = np.ones(F, bool) if feattypes is None else np.asarray(feattypes, bool)
     mono = np.zeros(F, int) if mono is None else np.asarray(mono, int)
@@ -112,6 +115,16 @@ def grow(x_bin_FN, grad, rows, js, K, nbins, max_depth, eta=0.1, lam=0.0, L2=1.0
              gain=np.zeros(nn, np.float32), pred=np.zeros((nn, K), np.float32), split=np.zeros(nn, np.uint8))
     label = np.zeros(N, np.int64)
     label[rows] = 1
+
+    def leaf_of(n):
+        if kind != "quantile":
+            return leaf_value(sums[n], K, eta, lam, L2, kind=kind)
+        r = np.flatnonzero(label == n)
+        d = 1.0 + lam + L2 / sums[n][2 * K]
+        if clamp_denom:
+            d = max(EPS, d)
+        return np.array([eta * np.quantile(grad[r, K + k].astype(np.float64), alphas[k], method="linear") / d for k in range(K)])
+
     sums = {1: grad[rows].astype(np.float64).sum(axis=0)}
     hists = {}
     active = [1]
@@ -121,7 +134,7 @@ def grow(x_bin_FN, grad, rows, js, K, nbins, max_depth, eta=0.1, lam=0.0, L2=1.0
         if depth == max_depth:
             for n in active:
                 T["w"][n - 1] = sums[n][2 * K]
-                T["pred"][n - 1] = leaf_value(sums[n], K, eta, lam, L2, kind=kind)
+                T["pred"][n - 1] = leaf_of(n)
             break
         G = {}
         for n in active:
@@ -169,7 +182,7 @@ def grow(x_bin_FN, grad, rows, js, K, nbins, max_depth, eta=0.1, lam=0.0, L2=1.0
                 sums[2 * n + 1] = sums[n] - SL
                 nxt += [2 * n, 2 * n + 1]
             else:
-                T["pred"][n - 1] = leaf_value(sums[n], K, eta, lam, L2, kind=kind)
+                T["pred"][n - 1] = leaf_of(n)
         active = nxt
     return T, label, hists, sums
 

@@ -893,3 +893,108 @@ def test_residual_loss_predict_adds_and_link_is_identity():
         q = pred.copy()
         orc.apply_link(orc.LOSS_IDS[loss], 1, q)
         assert np.array_equal(q, pred)
+
+
+# ---------------------------------------------------------------- quantile losses
+def test_quantile_grads_closed_form():
+    """Row k: alpha (residual > 0) or alpha - 1, a Float64, times the weight, rounded to Float32; row K + k: the raw
+    residual, not weighted (src/loss.jl:85-91, :144-171)."""
+    N = 400
+    x_bin, y, pred, grad = make_data(71, N, 3, 8, "mse", weights=True)
+    w = grad[:, 2].copy()
+    p = orc.make_params("quantile", nbins=8, max_depth=3, alpha=0.3)
+    orc.update_grads(p, pred, y, grad)
+    d = y - pred[:, 0]
+    want = (np.where(d > 0, 0.3, 0.3 - 1.0) * w.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(grad[:, 0], want) and np.array_equal(grad[:, 1], d) and np.array_equal(grad[:, 2], w)
+    # multiquantile: one target, an alpha per output
+    al = [0.1, 0.5, 0.9]
+    pm = orc.make_params("multiquantile", nbins=8, max_depth=3, alphas=al)
+    assert pm.K == 3
+    predm = (np.random.default_rng(72).standard_normal((N, 3)) * 0.3).astype(np.float32)
+    gm = np.zeros((N, 7), np.float32)
+    gm[:, 6] = w
+    orc.update_grads(pm, predm, y, gm)
+    for k in range(3):
+        dk = y - predm[:, k]
+        assert np.array_equal(gm[:, k], (np.where(dk > 0, al[k], al[k] - 1.0) * w.astype(np.float64)).astype(np.float32))
+        assert np.array_equal(gm[:, 3 + k], dk)
+
+
+@pytest.mark.parametrize("alpha,n", [(0.5, 1), (0.5, 2), (0.1, 11), (0.9, 11), (0.25, 400), (0.999, 57), (0.0, 9), (1.0, 9)])
+def test_leaf_quantile_is_numpys_linear_quantile(alpha, n):
+    """A depth-1 tree is one leaf over all rows: its value is eta * quantile(residuals, alpha) (lambda = L2 = 0), with the
+    quantile of Hyndman & Fan's definition 7 - numpy's "linear" method on the same Float32 residuals."""
+    rng = np.random.default_rng(73)
+    x_bin = rng.integers(1, 5, size=(2, n), dtype=np.uint8)
+    y = rng.standard_normal(n).astype(np.float32)
+    pred = np.zeros((n, 1), np.float32)
+    grad = np.zeros((n, 3), np.float32)
+    grad[:, 2] = 1.0
+    p = orc.make_params("quantile", nbins=4, max_depth=1, eta=0.7, L2=0.0, alpha=alpha)
+    orc.update_grads(p, pred, y, grad)
+    o = orc.Oracle(p, x_bin)
+    t, nidx = o.grow_tree(grad, np.arange(n, dtype=np.uint32), np.array([1, 2], np.uint32), mode=0)
+    want = 0.7 * np.quantile(y.astype(np.float64), alpha, method="linear")
+    np.testing.assert_allclose(t.pred[0, 0], want, rtol=1e-6, atol=1e-7)
+    o.close()
+
+
+def test_pinball_metric_against_sklearn():
+    from sklearn.metrics import mean_pinball_loss
+    rng = np.random.default_rng(74)
+    N = 3000
+    y = rng.standard_normal(N).astype(np.float32)
+    p1 = (y + rng.standard_normal(N) * 0.5).astype(np.float32).reshape(N, 1)
+    w = (rng.random(N) + 0.5).astype(np.float32)
+    for alpha in (0.1, 0.5, 0.8):
+        got = orc.eval_metric("quantile", 1, p1, y, w, alphas=[alpha])
+        np.testing.assert_allclose(got, mean_pinball_loss(y, p1[:, 0], sample_weight=w, alpha=alpha), rtol=1e-5)
+    al = [0.2, 0.5, 0.9]
+    p3 = (y[:, None] + rng.standard_normal((N, 3)) * 0.5).astype(np.float32)
+    got = orc.eval_metric("multiquantile", 3, p3, y, None, alphas=al)
+    want = np.mean([mean_pinball_loss(y, p3[:, k], alpha=al[k]) for k in range(3)])
+    np.testing.assert_allclose(got, want, rtol=1e-5)
+    # quantile loss with several targets: one alpha, averaged over the outputs
+    Y2 = np.stack([y, -y], axis=1).astype(np.float32)
+    got = orc.eval_metric("quantile", 2, p3[:, :2].copy(), Y2, w, alphas=[0.3])
+    want = np.mean([mean_pinball_loss(Y2[:, k], p3[:, k], sample_weight=w, alpha=0.3) for k in range(2)])
+    np.testing.assert_allclose(got, want, rtol=1e-5)
+
+
+@pytest.mark.parametrize("loss,weights,lam,L2,tt", [
+    ("quantile", False, 0.0, 0.0, "binary"),
+    ("quantile", True, 0.4, 0.7, "binary"),
+    ("quantile", True, 0.0, 1.0, "oblivious"),
+    ("multiquantile", False, 0.0, 1.0, "binary"),
+    ("multiquantile", True, 0.2, 0.5, "binary"),
+])
+def test_quantile_tree_against_bruteforce(loss, weights, lam, L2, tt):
+    N, F, B, D = 900, 6, 16, 5
+    x_bin, y, pred, grad0 = make_data(75, N, F, B, "mse", weights)
+    y = (y + 0.03 * x_bin[1]).astype(np.float32)
+    if loss == "multiquantile":
+        al = [0.15, 0.5, 0.85]
+        p = orc.make_params(loss, nbins=B, max_depth=D, tree_type=tt, lambda_=lam, L2=L2, eta=0.3, min_weight=2.0, alphas=al)
+        K = 3
+        pred = (np.random.default_rng(76).standard_normal((N, K)) * 0.2).astype(np.float32)
+    else:
+        al = [0.7]
+        p = orc.make_params(loss, nbins=B, max_depth=D, tree_type=tt, lambda_=lam, L2=L2, eta=0.3, min_weight=2.0, alpha=0.7)
+        K = 1
+    grad = np.zeros((N, 2 * K + 1), np.float32)
+    grad[:, 2 * K] = grad0[:, 2]
+    orc.update_grads(p, pred, y, grad)
+    rng = np.random.default_rng(77)
+    rows = np.sort(rng.choice(N, 700, replace=False)).astype(np.uint32)
+    js = np.array([1, 2, 3, 5], np.uint32)
+    o = orc.Oracle(p, x_bin)
+    t, nidx = o.grow_tree(grad, rows, js, mode=0)
+    T, label, hists, sums = brute.grow(x_bin, grad, rows, js, K, B, D, eta=0.3, lam=lam, L2=L2, min_weight=2.0, oblivious=(tt == "oblivious"),
+                                       kind="quantile", alphas=al * (K if len(al) == 1 else 1), clamp_denom=(loss == "quantile"))
+    assert trees_equal_struct(t, T)
+    assert t.split.sum() >= 3
+    np.testing.assert_allclose(t.gain, T["gain"], rtol=1e-5)
+    np.testing.assert_allclose(t.pred, T["pred"], rtol=1e-5, atol=1e-7)
+    assert np.array_equal(nidx.astype(np.int64), label)
+    o.close()
