@@ -25,7 +25,7 @@ _GPU_DEVICES = ("gpu", "rocm", "amd", "hip")
 _EXP_LINK = ("poisson", "gamma", "tweedie")
 # is_maximise, src/metrics.jl:195-207
 _MAXIMISE = {"mse": False, "rmse": False, "mae": False, "logloss": False, "poisson": False, "gamma": False, "tweedie": False,
-             "gaussian_mle": True, "logistic_mle": True, "mlogloss": False}
+             "gaussian_mle": True, "logistic_mle": True, "mlogloss": False, "quantile": False, "multiquantile": False}
 
 
 def _device_check(device):
@@ -57,6 +57,13 @@ def check_args(args):
         raise ValueError("bagging_size must be >= 1")
     rng("early_stopping_rounds", 1, float("inf"))
     rng("early_stopping_tolerance", 0.0, float("inf"))
+    if "alpha" in args:
+        rng("alpha", 0.0, 1.0)
+    if args.get("loss") == "multiquantile":  # check_alphas, src/learners.jl:504-515
+        al = [float(a) for a in (args.get("alphas") or [])]
+        if not al or any(not (0.0 < a < 1.0) for a in al) or any(b <= a for a, b in zip(al, al[1:])):
+            raise ValueError("Invalid value for parameter `alphas`: %s. `alphas` must be a non-empty, strictly increasing vector with "
+                             "values in (0, 1)." % (args.get("alphas"),))
 
 
 class _Learner:
@@ -89,11 +96,11 @@ class _Learner:
 
 
 class EvoTreeRegressor(_Learner):
-    """EvoTreeRegressor (src/learners.jl:1-119); losses mse, logloss, poisson, gamma, tweedie, mae, cred_var, cred_std (of the
-    reference's list the quantile losses are not served: their leaf values are quantiles of the leaf's residuals, not
-    functions of the histogram)."""
-    _losses = ("mse", "logloss", "poisson", "gamma", "tweedie", "mae", "cred_var", "cred_std")
-    _metrics = ("mse", "rmse", "mae", "logloss", "poisson", "gamma", "tweedie")
+    """EvoTreeRegressor (src/learners.jl:1-119); losses mse, logloss, poisson, gamma, tweedie, mae, quantile (level `alpha`),
+    multiquantile (levels `alphas`, one output each), cred_var, cred_std."""
+    _losses = ("mse", "logloss", "poisson", "gamma", "tweedie", "mae", "quantile", "multiquantile", "cred_var", "cred_std")
+    _metrics = ("mse", "rmse", "mae", "logloss", "poisson", "gamma", "tweedie", "quantile", "multiquantile")
+    _defaults = dict(_Learner._defaults, alpha=0.5, alphas=(0.1, 0.5, 0.9))
 
 
 class EvoTreeCount(_Learner):
@@ -186,7 +193,7 @@ def _target_rows(y):
     return y
 
 
-def _init_target(loss, y):
+def _init_target(loss, y, alphas=None):
     """_init_target, src/init.jl:10-146 (in-scope branches).  Returns K, y (Float32; (N,) for one target, (N, T) for a
     T x N matrix target), mu, target levels."""
     y = np.asarray(y)
@@ -206,6 +213,12 @@ def _init_target(loss, y):
         mu = np.log(prop).astype(np.float32)
         mu = mu - mu.max()
         return K, codes, mu.astype(np.float32), levels
+    if loss == "multiquantile":  # src/init.jl:101-105: one target, an output per level, each starting at its quantile of y
+        if y.ndim != 1:
+            raise RuntimeError("Multi-target (matrix target) is not supported for loss multiquantile: its outputs are the levels.")
+        y32 = y.astype(np.float32)
+        mu = np.quantile(y32.astype(np.float64), [float(a) for a in alphas], method="linear").astype(np.float32)
+        return mu.shape[0], y32, mu, None
     rows = _target_rows(y).astype(np.float32)  # T x N
     if loss == "logloss" and (rows.min() < 0 or rows.max() > 1):
         raise AssertionError("logloss targets must be in [0, 1]")
@@ -378,7 +391,7 @@ def init(config, x_train, y_train=None, w_train=None, offset_train=None, feature
         if len(feature_names) != F:
             raise AssertionError("length(feature_names) must equal size(x_train, 2)")
         edges, featbins, feattypes = get_edges(x, config.nbins, rng)
-    K, y32, mu, target_levels = _init_target(config.loss, y_train)
+    K, y32, mu, target_levels = _init_target(config.loss, y_train, getattr(config, "alphas", None))
     if y32.shape[0] != N:
         raise AssertionError("target length must equal the number of rows")
     w = None
@@ -399,6 +412,7 @@ def init(config, x_train, y_train=None, w_train=None, offset_train=None, feature
     for k, v in config.monotone_constraints.items():
         mono[int(k) - 1] = int(v)
     h.set_feature_meta(feattypes, mono)
+    _set_levels(h, config)
     h.set_target(y32, w, mu, offset)
     info = dict(nrounds=0, feature_names=feature_names, target_levels=target_levels, target_isordered=False, edges=edges, featbins=featbins,
                 feattypes=feattypes)
@@ -452,6 +466,14 @@ def grow_evotree(m, cache, config):
     m.info["nrounds"] += 1
 
 
+def _set_levels(h, config):
+    """params.alpha / params.alphas of the quantile losses and metrics (src/callback.jl:62-66)."""
+    if config.loss == "multiquantile":
+        h.set_alphas([float(a) for a in config.alphas])
+    elif hasattr(config, "alpha"):
+        h.set_alphas([float(config.alpha)])
+
+
 class CallBack:
     """CallBack (src/callback.jl:21-135) on the device: a second handle holds the binned eval rows, their
     running prediction, target and weights; each call adds one tree and evaluates the metric there."""
@@ -485,6 +507,7 @@ class CallBack:
             else:
                 h.binarize(np.ascontiguousarray(x.T, np.float64), m.info["edges"])
             h.set_feature_meta(m.info["feattypes"], None)
+            _set_levels(h, config)
             h.set_target(y32, w, np.zeros(m.K, np.float32), offset)  # p = zeros (+ offset'), src/callback.jl:104, :82
         except Exception:
             h.close()

@@ -13,15 +13,15 @@ LIB_PATH = os.path.join(_HERE, "libevotrees_hip.so")
 
 EVT_OK, EVT_ERR_ARG, EVT_ERR_HIP, EVT_ERR_STATE, EVT_ERR_EMPTY, EVT_ERR_NOMEM = 0, -1, -2, -3, -4, -5
 LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5, "mlogloss": 6, "logistic_mle": 7, "mae": 8,
-            "cred_var": 9, "cred_std": 10}
-METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8, "logistic_mle": 9}
+            "cred_var": 9, "cred_std": 10, "quantile": 11, "multiquantile": 12}
+METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8, "logistic_mle": 9, "quantile": 10, "multiquantile": 11}
 TREE_TYPES = {"binary": 0, "oblivious": 1}
 KERNEL_CLASSES = ["grad", "hist", "scan", "partition", "predict", "other"]
 
 # every symbol include/evotrees_hip.h declares
 EXPORTS = [
     "evt_last_error", "evt_device_count", "evt_create", "evt_destroy", "evt_set_xbin", "evt_binarize_f64",
-    "evt_set_target", "evt_set_feature_meta", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
+    "evt_set_target", "evt_set_feature_meta", "evt_set_alphas", "evt_update_grads", "evt_set_grads", "evt_grow_tree",
     "evt_grow_tree_begin", "evt_grow_tree_end", "evt_stage_mask", "evt_grow_tree_begin_staged", "evt_draw_mask",
     "evt_tree_open", "evt_hist_build", "evt_split_scan", "evt_update_nodes_idx", "evt_tree_close", "evt_peek_tree",
     "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
@@ -69,6 +69,7 @@ def load():
         "evt_binarize_f64": [vp, vp, vp, vp],
         "evt_set_target": [vp, vp, vp, vp, vp],
         "evt_set_feature_meta": [vp, vp, vp],
+        "evt_set_alphas": [vp, vp, i32],
         "evt_update_grads": [vp],
         "evt_set_grads": [vp, vp],
         "evt_grow_tree": [vp, vp, C.c_uint8, vp, i32, C.POINTER(EvtParams), C.POINTER(EvtTreeOut)],
@@ -196,7 +197,7 @@ class Handle:
         mu = np.ascontiguousarray(mu, np.float32)
         offset = None if offset is None else np.ascontiguousarray(offset, np.float32)
         # one value per row and target: (N,) for one target, (N, T) C-order (Julia's T x N) for several
-        T = 1 if self.loss == "mlogloss" else (self.K // 2 if self.loss in ("gaussian_mle", "logistic_mle") else self.K)
+        T = 1 if self.loss in ("mlogloss", "multiquantile") else (self.K // 2 if self.loss in ("gaussian_mle", "logistic_mle") else self.K)
         assert (y.shape == (self.N,) and T == 1) or y.shape == (self.N, T)
         assert mu.shape == (self.K,)
         check(load().evt_set_target(self._h, ptr(y), ptr(w), ptr(mu), ptr(offset)))
@@ -284,6 +285,11 @@ class Handle:
 
     def predict_tree(self, tree):
         check(load().evt_predict_tree(self._h, tree.feat.shape[0], ptr(tree.feat), ptr(tree.cond_bin), ptr(tree.pred), ptr(tree.split)))
+
+    def set_alphas(self, alphas):
+        """Levels of the quantile losses and metrics: one value (quantile) or one per output (multiquantile)."""
+        a = np.ascontiguousarray(np.atleast_1d(alphas), np.float64)
+        check(load().evt_set_alphas(self._h, ptr(a), a.shape[0]))
 
     def eval_metric(self, metric):
         """Metric of the handle's prediction against its target and weights (the eval CallBack's feval)."""

@@ -175,7 +175,8 @@ extern "C" int evt_destroy(evt_handle c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     void *ptrs[] = {c->xcm, c->xrm, c->y, c->pred, c->grad, c->gq, c->is_a, c->is_b, c->nidx, c->mask, c->flagw, c->chunk_nleft, c->chunk_lpre,
                     c->hist, c->seg_start, c->seg_len, c->status, c->node_sum, c->tree_blob, c->tree.packed, c->js, c->jsmap, c->feattypes, c->mono, c->absmax, c->qexp_buf[0], c->qexp_buf[1], c->qbits,
-                    c->qscale_buf[0], c->qscale_buf[1], c->planes, c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id, c->pt_nodes, c->pt_pred, c->mask_next};
+                    c->qscale_buf[0], c->qscale_buf[1], c->planes, c->metric_partial, c->errflag, c->ogains, c->sbest, c->is_id, c->pt_nodes, c->pt_pred, c->mask_next,
+                    c->alphas, c->alphas_f, c->qkeys_a, c->qkeys_b, c->qtemp};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     for (int l = 0; l < 2; l++) {
@@ -202,6 +203,14 @@ extern "C" int evt_destroy(evt_handle c) {
     });
 }
 
+static hipError_t upload_alphas(evt_ctx *c) {
+    float af[EVT_MAX_K];
+    for (int k = 0; k < EVT_MAX_K; k++) af[k] = (float)c->h_alphas[k];
+    hipError_t e = hipMemcpy(c->alphas, c->h_alphas, sizeof(double) * EVT_MAX_K, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(c->alphas_f, af, sizeof(float) * EVT_MAX_K, hipMemcpyHostToDevice);
+    return e;
+}
+
 extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K, int32_t max_depth, int32_t loss, int32_t tree_type,
                           evt_handle *out) {
     return guarded([&]() -> int {
@@ -213,7 +222,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ARGCHK(max_depth >= 1 && max_depth <= EVT_MAX_DEPTH, "max_depth must be in [1, 16]");
     ARGCHK(loss >= 0 && loss <= EVT_LOSS_LAST,
            "loss must be one of mse (0), logloss (1), gaussian_mle (2), poisson (3), gamma (4), tweedie (5), mlogloss (6), logistic_mle (7), mae (8), "
-           "cred_var (9), cred_std (10)");
+           "cred_var (9), cred_std (10), quantile (11), multiquantile (12)");
     ARGCHK(tree_type == EVT_TREE_BINARY || tree_type == EVT_TREE_OBLIVIOUS, "tree_type must be binary (0) or oblivious (1)");
     if (loss == EVT_LOSS_MLOGLOSS) ARGCHK(K >= 2 && K <= EVT_MAX_K, "mlogloss needs 2 <= K <= 16 classes");
     else if (EVT_IS_MLE2P(loss)) ARGCHK(K >= 2 && K <= EVT_MAX_K && K % 2 == 0, "gaussian_mle / logistic_mle need K = 2 x targets, 2 <= K <= 16");
@@ -231,7 +240,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     memset((void *)&c->device, 0, sizeof(int));
     c->stream = nullptr;
     c->N = nobs; c->F = nfeats; c->B = nbins; c->K = K; c->NK = 2 * K + 1; c->D = max_depth; c->loss = loss; c->tree_type = tree_type;
-    c->T = (loss == EVT_LOSS_MLOGLOSS) ? 1 : (EVT_IS_MLE2P(loss) ? K / 2 : K);
+    c->T = (loss == EVT_LOSS_MLOGLOSS || loss == EVT_LOSS_MULTIQUANTILE) ? 1 : (EVT_IS_MLE2P(loss) ? K / 2 : K);
     c->mc = (loss == EVT_LOSS_MLOGLOSS) || K > (EVT_IS_MLE2P(loss) ? 2 : 1);
     c->nnodes = (1 << max_depth) - 1;
     c->maxlvl = 1 << (max_depth - 1);
@@ -247,6 +256,9 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->tree_blob = nullptr;
     memset(c->lvl, 0, sizeof(c->lvl));
     c->js = nullptr; c->jsmap = nullptr; c->feattypes = nullptr; c->mono = nullptr; c->absmax = nullptr; c->qexp = nullptr; c->qbits = nullptr;
+    c->alphas = nullptr; c->alphas_f = nullptr; c->qkeys_a = c->qkeys_b = nullptr; c->qtemp = nullptr; c->qtemp_bytes = 0;
+    c->n_alphas = 1;
+    for (int k = 0; k < EVT_MAX_K; k++) c->h_alphas[k] = 0.5;
     c->qscale = nullptr; c->qexp_buf[0] = c->qexp_buf[1] = nullptr; c->qscale_buf[0] = c->qscale_buf[1] = nullptr; c->q_cur = c->q_tree = 0;
     c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->sbest = nullptr;
     c->h_stage = nullptr; c->h_stage_dev = nullptr; c->h_stage_bytes = 0;
@@ -353,6 +365,8 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->feattypes, c->F);
     ALLOC(c->mono, c->F);
     ALLOC(c->absmax, EVT_ABSMAX_STRIPES * EVT_MC_MAX_NK);
+    ALLOC(c->alphas, EVT_MAX_K);
+    ALLOC(c->alphas_f, EVT_MAX_K);
     for (int s = 0; s < 2; s++) {
         ALLOC(c->qexp_buf[s], EVT_MC_MAX_NK);
         ALLOC(c->qscale_buf[s], 2 * EVT_MC_MAX_NK);
@@ -389,6 +403,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
         if (e2 == hipSuccess) e2 = hipMemset(c->absmax, 0, sizeof(uint32_t) * EVT_ABSMAX_STRIPES * EVT_MC_MAX_NK);
         if (e2 == hipSuccess) e2 = hipMemset(c->nidx, 0, sizeof(uint32_t) * N);
         if (e2 == hipSuccess) e2 = hipMemset(c->errflag, 0, sizeof(int32_t));
+        if (e2 == hipSuccess) e2 = upload_alphas(c);
         if (e2 != hipSuccess) {
             evt_set_error("initial fills failed: %s", hipGetErrorString(e2));
             evt_destroy(c);
@@ -583,6 +598,28 @@ extern "C" int evt_set_target(evt_handle c, const float *y, const float *w, cons
     });
 }
 
+extern "C" int evt_set_alphas(evt_handle c, const double *alphas, int32_t n) {
+    return guarded([&]() -> int {
+    CTXCHK(c);
+    ARGCHK(alphas != nullptr, "alphas is NULL");
+    if (c->loss == EVT_LOSS_MULTIQUANTILE) ARGCHK(n == c->K, "the multiquantile loss takes one level per output (n == K)");
+    else ARGCHK(n == 1, "one level (n == 1) unless the loss is multiquantile");
+    double a[EVT_MAX_K];
+    HIPCHK(hipMemcpy(a, alphas, sizeof(double) * n, hipMemcpyDefault));
+    for (int k = 0; k < n; k++) {
+        ARGCHK(a[k] >= 0.0 && a[k] <= 1.0, "a quantile level must be in [0, 1]");
+        ARGCHK(k == 0 || a[k] > a[k - 1], "quantile levels must be strictly increasing");
+    }
+    HIPCHK(hipStreamSynchronize(c->stream)); // kernels queued earlier read the old levels
+    for (int k = 0; k < EVT_MAX_K; k++) c->h_alphas[k] = (k < n) ? a[k] : a[n - 1];
+    c->n_alphas = n;
+    HIPCHK(upload_alphas(c));
+    c->have_grads = false; // the gradients of the quantile losses depend on the levels
+    c->grads_ready = false;
+    return EVT_OK;
+    });
+}
+
 extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, const int32_t *monotone) {
     return guarded([&]() -> int {
     CTXCHK(c);
@@ -595,6 +632,7 @@ extern "C" int evt_set_feature_meta(evt_handle c, const uint8_t *feattypes, cons
         ARGCHK(mo[j] >= -1 && mo[j] <= 1, "monotone constraints must be -1, 0 or 1");
         // the reference has no pred_scalar method for the multi-class loss (src/predict.jl:205-238): a constraint cannot be evaluated there
         ARGCHK(mo[j] == 0 || c->loss != EVT_LOSS_MLOGLOSS, "monotone constraints are not defined for mlogloss");
+        ARGCHK(mo[j] == 0 || !EVT_IS_QUANTILE(c->loss), "monotone constraints are not defined for the quantile losses"); // no pred_scalar either
         // with several targets the reference's pred_scalar (src/predict.jl:205-208, :235-238) still reads the statistics at the
         // one-target positions, i.e. another target's gradient as the hessian: refused rather than reproduced
         ARGCHK(mo[j] == 0 || !c->mc, "monotone constraints are not defined for more than one target");
@@ -725,7 +763,8 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
     c->last_cond = cond;
     c->q_tree = c->q_cur; // this tree is grown on (and decoded with) the tables of the gradients quantised last
     // a tree grown in stages records the node of every row on the way, so that evt_get_nidx can show it after each stage
-    const bool rec_nidx = c->record_nidx || staged;
+    // ... and so does a quantile loss: its leaves are valued from the rows they hold once the tree is complete
+    const bool rec_nidx = c->record_nidx || staged || EVT_IS_QUANTILE(c->loss);
     c->nidx_valid = rec_nidx;
 
     // per-tree small uploads through pinned memory
@@ -750,12 +789,17 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
 
     // With every row in the tree the leaf of each row is recorded while growing and its value is added later, in row
     // order (fused into the next gradient pass): a scattered 4-byte write per row instead of a scattered read-modify-write.
-    const bool defer = p->update_pred && all_rows && c->defer_pred;
+    // (a quantile loss's leaf values do not exist before the tree is complete: always deferred)
+    const bool defer = p->update_pred && all_rows && (c->defer_pred || EVT_IS_QUANTILE(c->loss));
     const bool fuse_pred = p->update_pred && all_rows && !defer;
     c->write_nidx = rec_nidx || defer;
 
     int r = ensure_planes(c);
     if (r != EVT_OK) return r;
+    if (EVT_IS_QUANTILE(c->loss)) {
+        r = quantile_leaf_buffers(c);
+        if (r != EVT_OK) return r;
+    }
     prof_begin(c, EVT_K_OTHER, 0);
     r = launch_apply_pending(c); // an earlier tree's values go in before its node ids are overwritten
     if (r != EVT_OK) return r;
@@ -858,6 +902,12 @@ static int tree_close(evt_ctx *c) {
     const bool all_rows = c->step.all_rows, defer = c->step.defer;
     int r;
     c->step.phase = 0;
+    if (EVT_IS_QUANTILE(c->loss)) { // pred_leaf_cpu! of the quantile losses: every leaf's value from the residuals of its rows
+        prof_begin(c, EVT_K_OTHER, 0);
+        r = launch_quantile_leaves(c, p);
+        prof_end(c);
+        if (r != EVT_OK) return r;
+    }
     if (p->update_pred && !all_rows) {
         // rows outside the sample are predicted too (src/fit.jl:37): walk the new tree for all rows
         prof_begin(c, EVT_K_PREDICT, 0);
@@ -1270,7 +1320,9 @@ extern "C" int evt_eval_metric(evt_handle c, int32_t metric, double *value_out) 
     return guarded([&]() -> int {
     CTXCHK(c);
     ARGCHK(value_out, "value_out is NULL");
-    ARGCHK(metric >= 0 && metric <= EVT_METRIC_LOGISTIC_MLE, "unknown metric");
+    ARGCHK(metric >= 0 && metric <= EVT_METRIC_MULTIQUANTILE, "unknown metric");
+    ARGCHK(metric != EVT_METRIC_MULTIQUANTILE || c->loss == EVT_LOSS_MULTIQUANTILE,
+           "multiquantile is the metric of the multiquantile loss (one target, a level per output) and of no other");
     ARGCHK((metric == EVT_METRIC_GAUSSIAN_MLE) == (c->loss == EVT_LOSS_GAUSSIAN_MLE),
            "gaussian_mle is the metric of the gaussian_mle loss and of no other");
     ARGCHK((metric == EVT_METRIC_LOGISTIC_MLE) == (c->loss == EVT_LOSS_LOGISTIC_MLE),

@@ -71,7 +71,7 @@ struct evt_ctx {
     hipStream_t stream;
     int64_t N;
     int32_t F, B, K, NK, D, loss, tree_type;
-    int32_t T;         // target columns of y: K for the gradient-regression losses, K / 2 for gaussian_mle, 1 (the class) for mlogloss
+    int32_t T;         // target columns of y: K for the gradient-regression losses, K / 2 for gaussian_mle, 1 for mlogloss (the class) and multiquantile
     bool mc;           // more outputs than the specialised kernels take: run-time channel count (multi-class, several targets)
     int32_t nnodes;    // 2^D - 1
     int32_t maxlvl;    // 2^(D-1)
@@ -123,6 +123,14 @@ struct evt_ctx {
     uint8_t *feattypes;
     int32_t *mono;
     uint32_t *absmax;  // [EVT_ABSMAX_STRIPES][EVT_MC_MAX_NK] float bits
+    // quantile losses: levels (Float64 for the gradients, Float32 for the metrics) and the sort buffers of the leaf pass
+    double h_alphas[EVT_MAX_K];
+    int32_t n_alphas;
+    double *alphas;        // [EVT_MAX_K]
+    float *alphas_f;       // [EVT_MAX_K]
+    unsigned long long *qkeys_a, *qkeys_b; // [N] (node, residual) keys, unsorted / sorted
+    void *qtemp;
+    size_t qtemp_bytes;
     int32_t *qexp;     // [EVT_MC_MAX_NK]; points into qexp_buf: the tables of the gradients quantised last
     int32_t *qbits;    // [EVT_MC_MAX_NK]
     double *qscale;    // [2 * EVT_MC_MAX_NK]: decode scale per global channel, then encode multiplier per gradient row
@@ -229,10 +237,13 @@ void evt_set_error(const char *fmt, ...);
 // the two-parameter MLE losses: outputs come in (location, raw scale) pairs
 #define EVT_IS_MLE2P(loss) ((loss) == EVT_LOSS_GAUSSIAN_MLE || (loss) == EVT_LOSS_LOGISTIC_MLE)
 #define EVT_IS_CRED(loss) ((loss) == EVT_LOSS_CRED_VAR || (loss) == EVT_LOSS_CRED_STD)
-#define EVT_LOSS_LAST EVT_LOSS_CRED_STD
-// One-target mse and mae need no accumulator for their second gradient row (mse: h = 2w; mae: h = 0, and neither its
-// gain nor its leaf value reads it): their histograms hold the channels {g, w} only.
-#define EVT_TWO_CHAN(loss, K) (((loss) == EVT_LOSS_MSE || (loss) == EVT_LOSS_MAE) && (K) == 1)
+#define EVT_IS_QUANTILE(loss) ((loss) == EVT_LOSS_QUANTILE || (loss) == EVT_LOSS_MULTIQUANTILE)
+// losses whose gain is the weighted shift of the children's mean first-row value (Union{MAE,Quantile}, src/split.jl:68, :119)
+#define EVT_IS_SHIFT(loss) ((loss) == EVT_LOSS_MAE || EVT_IS_QUANTILE(loss))
+#define EVT_LOSS_LAST EVT_LOSS_MULTIQUANTILE
+// One-target mse, mae and quantile need no accumulator for their second gradient row (mse: h = 2w; mae: h = 0; quantile:
+// the raw residual, read per row when the leaves are valued; no gain reads it): their histograms hold the channels {g, w} only.
+#define EVT_TWO_CHAN(loss, K) (((loss) == EVT_LOSS_MSE || EVT_IS_SHIFT(loss)) && (K) == 1)
 #define EVT_NODE_SPLIT (1u << 24)
 #define EVT_NODE_NUMERIC (1u << 25)
 #ifdef __HIPCC__
@@ -280,6 +291,8 @@ int launch_tree_begin(evt_ctx *c, bool all_rows);
 int launch_iota(evt_ctx *c, uint32_t *dst, int64_t n);
 int launch_compact_mask(evt_ctx *c, uint8_t cond);
 int launch_draw_mask(evt_ctx *c, uint8_t *mask, unsigned long long seed);
+int quantile_leaf_buffers(evt_ctx *c);
+int launch_quantile_leaves(evt_ctx *c, const evt_params *p);
 int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level);
 bool scan_folds_leaves(const evt_ctx *c);

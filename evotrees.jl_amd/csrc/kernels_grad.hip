@@ -275,6 +275,53 @@ __global__ __launch_bounds__(256) void k_grads_mlogloss(float *__restrict__ pred
     }
 }
 
+// The quantile losses (src/loss.jl:85-91, :144-171): row k = (alpha or alpha - 1, a Float64) * w, row K + k = the raw
+// residual (not weighted: the leaf pass takes its quantile).  multi: one target column and a level per output
+// (multiquantile); otherwise one level and a target column per output (quantile).
+__global__ __launch_bounds__(256) void k_grads_quantile(float *__restrict__ pred, const float *__restrict__ y, float *__restrict__ grad, int64_t N,
+                                                       int K, int multi, const double *__restrict__ alphas, uint32_t *absmax,
+                                                       const uint32_t *__restrict__ pend_nidx, const float *__restrict__ pend_leaf, int unit_w) {
+    const int NK = 2 * K + 1;
+    const int T = multi ? 1 : K;
+    __shared__ float s_m[4];
+    float mx[2 * EVT_MAX_K];
+#pragma unroll
+    for (int k = 0; k < 2 * EVT_MAX_K; k++) mx[k] = 0.0f;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
+        float *pr = pred + (size_t)K * i;
+        float *g = grad + (size_t)NK * i;
+        const float *yi = y + (size_t)T * i;
+        const float w = unit_w ? 1.0f : g[NK - 1];
+        if (pend_nidx) evt_add_leaf(pr, pend_leaf + (size_t)K * (pend_nidx[i] - 1), K, EVT_LOSS_QUANTILE);
+#pragma unroll
+        for (int k = 0; k < EVT_MAX_K; k++) {
+            if (k < K) {
+                const double alpha = multi ? alphas[k] : alphas[0];
+                const float diff = (multi ? yi[0] : yi[k]) - pr[k];
+                const float gg = (float)((diff > 0.0f ? alpha : alpha - 1.0) * (double)w);
+                g[k] = gg;
+                g[K + k] = diff;
+                mx[k] = fmaxf(mx[k], fabsf(gg));
+                mx[EVT_MAX_K + k] = fmaxf(mx[EVT_MAX_K + k], fabsf(diff));
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 2 * EVT_MAX_K; k++) {
+        const int kk = k < EVT_MAX_K ? k : k - EVT_MAX_K;
+        if (kk < K) { // uniform
+            const float m = wave_max_f32(mx[k]);
+            __syncthreads();
+            if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                const float mm = fmaxf(fmaxf(s_m[0], s_m[1]), fmaxf(s_m[2], s_m[3]));
+                absmax_raise(absmax, k < EVT_MAX_K ? kk : K + kk, mm);
+            }
+        }
+    }
+}
+
 // max |v| of every gradient row of an existing gradient matrix (injected gradients, weight row)
 __global__ __launch_bounds__(256) void k_absmax(const float *__restrict__ grad, int64_t N, int NK, int k0, int k1, uint32_t *absmax) {
     // one gradient row at a time: any number of rows without per-thread arrays
@@ -347,6 +394,12 @@ int launch_grads(evt_ctx *c) {
     dim3 grid((unsigned)nb);
     const uint32_t *pn = c->pend_pred ? c->nidx : nullptr; // the last tree's leaf values are added on the way
     c->pend_pred = false;
+    if (EVT_IS_QUANTILE(c->loss)) {
+        hipLaunchKernelGGL(k_grads_quantile, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->loss == EVT_LOSS_MULTIQUANTILE ? 1 : 0,
+                           c->alphas, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        HIPCHK(hipGetLastError());
+        return EVT_OK;
+    }
     const bool multi_target = c->loss != EVT_LOSS_MLOGLOSS && c->K > (EVT_IS_MLE2P(c->loss) ? 2 : 1);
     if (multi_target) {
 #define MT(L_) hipLaunchKernelGGL(k_grads_mt<L_>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0)
@@ -458,7 +511,19 @@ int launch_quantize(evt_ctx *c) {
 // (:43, :111), accumulated in Float64.  Two stages with a fixed shape (EVT_METRIC_BLOCKS partial sums, then one
 // block) keep the summation order, hence the result, independent of scheduling.
 __device__ __forceinline__ float metric_value_one(int metric, float pk, float yk);
-__device__ __forceinline__ float metric_value(int metric, int K, const float *__restrict__ pred, const float *__restrict__ y, int64_t i) {
+// T: target columns of y (K, or 1 when every output is measured against the one target: _target(y::AbstractVector, k, i) = y[i],
+// src/loss.jl:49).  alphas: the levels of the quantile metrics as Float32 (src/callback.jl:62-66).
+__device__ __forceinline__ float metric_value(int metric, int K, int T, const float *__restrict__ pred, const float *__restrict__ y, int64_t i,
+                                              const float *__restrict__ alphas) {
+    if (metric == EVT_METRIC_QUANTILE || metric == EVT_METRIC_MULTIQUANTILE) { // src/metrics.jl:4-6, :83-84, :117-134
+        float acc = 0.0f;
+        for (int k = 0; k < K; k++) {
+            const float pk = pred[(size_t)K * i + k], yk = y[(size_t)T * i + (T == 1 ? 0 : k)];
+            const float alpha = (metric == EVT_METRIC_MULTIQUANTILE) ? alphas[k] : alphas[0];
+            acc += alpha * fmaxf(yk - pk, 0.0f) + (1.0f - alpha) * fmaxf(pk - yk, 0.0f);
+        }
+        return acc;
+    }
     if (metric == EVT_METRIC_MLOGLOSS) { // src/metrics.jl:59-77
         float isum = 0.0f;
         for (int k = 0; k < K; k++) isum += expf(pred[(size_t)K * i + k]);
@@ -480,7 +545,7 @@ __device__ __forceinline__ float metric_value(int metric, int K, const float *__
         return acc;
     }
     float acc = 0.0f; // src/metrics.jl:39-43: the per-target values are added in Float32, starting from zero
-    for (int k = 0; k < K; k++) acc += metric_value_one(metric, pred[(size_t)K * i + k], y[(size_t)K * i + k]);
+    for (int k = 0; k < K; k++) acc += metric_value_one(metric, pred[(size_t)K * i + k], y[(size_t)T * i + (T == 1 ? 0 : k)]);
     return acc;
 }
 
@@ -518,13 +583,13 @@ __device__ __forceinline__ double block_sum_f64(double v, double *s_red) {
 }
 
 __global__ __launch_bounds__(256) void k_metric_partial(const float *__restrict__ pred, const float *__restrict__ y,
-                                                       const float *__restrict__ grad, int64_t N, int NK, int K, int metric, float kdiv,
-                                                       double *__restrict__ partial) {
+                                                       const float *__restrict__ grad, int64_t N, int NK, int K, int T, int metric, float kdiv,
+                                                       const float *__restrict__ alphas, double *__restrict__ partial) {
     __shared__ double s_red[4];
     double num = 0.0, den = 0.0;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < N; i += (int64_t)gridDim.x * 256) {
         const float w = grad[(size_t)NK * i + NK - 1];
-        const float ev = w * metric_value(metric, K, pred, y, i) / kdiv;
+        const float ev = w * metric_value(metric, K, T, pred, y, i, alphas) / kdiv;
         num += (double)ev;
         den += (double)w;
     }
@@ -556,8 +621,11 @@ int launch_eval_metric(evt_ctx *c, int metric, double *partial) {
     int64_t nb = (c->N + 255) / 256;
     if (nb > EVT_METRIC_BLOCKS) nb = EVT_METRIC_BLOCKS;
     const float kdiv = (metric == EVT_METRIC_MLOGLOSS) ? 1.0f : (float)((metric == EVT_METRIC_GAUSSIAN_MLE || metric == EVT_METRIC_LOGISTIC_MLE) ? c->K / 2 : c->K);
-    hipLaunchKernelGGL(k_metric_partial, dim3((unsigned)nb), dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->NK, c->K, metric, kdiv,
-                       partial);
+    // y has K columns for the losses whose outputs each have a target; the multi-class, two-parameter and multiquantile
+    // metrics index their own layouts
+    const int T = (c->loss == EVT_LOSS_MULTIQUANTILE) ? 1 : c->K;
+    hipLaunchKernelGGL(k_metric_partial, dim3((unsigned)nb), dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->NK, c->K, T, metric, kdiv,
+                       c->alphas_f, partial);
     HIPCHK(hipGetLastError());
     hipLaunchKernelGGL(k_metric_final, dim3(1), dim3(256), 0, c->stream, partial, (int)nb, metric, partial + 2 * EVT_METRIC_BLOCKS);
     HIPCHK(hipGetLastError());

@@ -103,7 +103,7 @@ __device__ __forceinline__ double term_cred(int loss, double m1, double m2, doub
 
 // One output's term of node_gain (src/split.jl:58-78): zero for mae.
 __device__ __forceinline__ double node_gain_k(int loss, double g, double h, double w, double lambda, double L2) {
-    if (loss == EVT_LOSS_MAE) return 0.0;
+    if (EVT_IS_SHIFT(loss)) return 0.0;
     if (EVT_IS_CRED(loss)) return term_cred(loss, g, h, w, L2);
     return term_gh(g, h, w, lambda, L2);
 }
@@ -112,7 +112,7 @@ __device__ __forceinline__ double node_gain_k(int loss, double g, double h, doub
 // _term_shift (src/split.jl:2), |g / w - mu_p| w / d on either side with d = max(eps, 1 + lambda + L2 / w).
 __device__ __forceinline__ double split_gain_k(int loss, double Sg, double Sh, double w_p, double g_l, double h_l, double w_l, double w_r,
                                                double lambda, double L2) {
-    if (loss == EVT_LOSS_MAE) {
+    if (EVT_IS_SHIFT(loss)) {
         double d_l = 1.0 + lambda + L2 / w_l, d_r = 1.0 + lambda + L2 / w_r;
         if (!(d_l > DBL_EPSILON)) d_l = DBL_EPSILON;
         if (!(d_r > DBL_EPSILON)) d_r = DBL_EPSILON;
@@ -125,6 +125,7 @@ __device__ __forceinline__ double split_gain_k(int loss, double Sg, double Sh, d
 
 // pred_leaf_cpu! / pred_scalar (src/predict.jl:198-262) for output k
 __device__ __forceinline__ double leaf_value(int loss, const double *S, int k, int K, double eta, int bagging, double lambda, double L2) {
+    if (EVT_IS_QUANTILE(loss)) return 0.0; // valued from the leaf's rows once the tree is complete (launch_quantile_leaves)
     if (EVT_IS_CRED(loss)) return eta / (double)bagging * S[k] / (S[2 * K] + L2);
     if (loss == EVT_LOSS_MAE) {
         double d = S[2 * K] + lambda * S[2 * K] + L2;

@@ -54,8 +54,14 @@ enum {
     EVT_LOSS_MAE = 8,      /* rows [(y - p) w, 0, w] (src/loss.jl:78, :130-142); gain = shift of the children's mean residual
                               (src/split.jl:2, :68, :119-130); leaf = eta * sum(g) / (w + lambda w + L2) (src/predict.jl:250-258) */
     EVT_LOSS_CRED_VAR = 9, /* credibility losses: rows [d w, d^2 w, w], d = y - p (src/loss.jl:80-83, :173-185); gain terms */
-    EVT_LOSS_CRED_STD = 10 /* Z |m1| / (1 + L2 / w), Z the ratio of variances / of standard deviations (src/loss.jl:275-290,
+    EVT_LOSS_CRED_STD = 10, /* Z |m1| / (1 + L2 / w), Z the ratio of variances / of standard deviations (src/loss.jl:275-290,
                               src/split.jl:3-4, :70-78, :132-141); leaf = eta * sum(g) / (w + L2) (src/predict.jl:211-217) */
+    EVT_LOSS_QUANTILE = 11, /* one level alpha for every output; rows [(alpha or alpha - 1) w, y - p, w] (src/loss.jl:85-91,
+                              :144-156); gains as mae; a leaf's value is eta * quantile(residuals of its rows, alpha) /
+                              max(eps, 1 + lambda + L2 / w) (src/predict.jl:265-272) - computed on the device by sorting
+                              (node, residual) pairs once the tree is complete.  Levels: evt_set_alphas */
+    EVT_LOSS_MULTIQUANTILE = 12 /* K levels on ONE target (y has one column): output k follows alphas[k] (src/loss.jl:158-171,
+                              src/predict.jl:275-281) */
 };
 /* evaluation metrics, metric_dict of src/metrics.jl:209-224 (in-scope subset) */
 enum {
@@ -68,7 +74,9 @@ enum {
     EVT_METRIC_GAMMA = 6,
     EVT_METRIC_TWEEDIE = 7,
     EVT_METRIC_MLOGLOSS = 8,
-    EVT_METRIC_LOGISTIC_MLE = 9
+    EVT_METRIC_LOGISTIC_MLE = 9,
+    EVT_METRIC_QUANTILE = 10,     /* pinball loss at the handle's alpha, averaged over the outputs (src/metrics.jl:4-6, :83-84) */
+    EVT_METRIC_MULTIQUANTILE = 11 /* pinball loss of output k at alphas[k] against the one target (src/metrics.jl:117-134) */
 };
 /* params.tree_type, src/learners.jl:45 */
 enum { EVT_TREE_BINARY = 0, EVT_TREE_OBLIVIOUS = 1 };
@@ -134,10 +142,16 @@ int evt_set_target(evt_handle h, const float *y, const float *w, const float *mu
 
 /* feattypes[j] != 0: numeric (<=), 0: categorical (==); monotone[j] in {-1,0,1}
  * (cache.feattypes / cache.monotone_constraints, src/init.jl:183-187).  NULL = all numeric / none.
- * A constraint is refused (EVT_ERR_ARG) for mlogloss and for more than one target: the reference has no
- * pred_scalar for the former, and for the latter its pred_scalar (src/predict.jl:205-208, :235-238) reads the
+ * A constraint is refused (EVT_ERR_ARG) for mlogloss, the quantile losses and for more than one target: the reference
+ * has no pred_scalar for the former two, and for the latter its pred_scalar (src/predict.jl:205-208, :235-238) reads the
  * statistics at the one-target positions. */
 int evt_set_feature_meta(evt_handle h, const uint8_t *feattypes, const int32_t *monotone);
+
+/* Levels of the quantile losses and metrics: params.alpha (n = 1: the quantile loss, every output) or params.alphas
+ * (n = K: the multiquantile loss, one output each; strictly increasing, src/learners.jl:504-515), each in [0, 1]
+ * (src/learners.jl:539).  A handle starts with alpha = 0.5, the reference's default (src/learners.jl:44).  The gradients
+ * use the Float64 values (src/loss.jl:85-91), the metrics T(alpha) (src/callback.jl:62-66). */
+int evt_set_alphas(evt_handle h, const double *alphas, int32_t n);
 
 /* update_grads!(cache.∇, cache.pred, cache.y, L, params): src/loss.jl:100-111, :219-236;
  * device twin ext/.../loss.jl:183-191. */
@@ -244,7 +258,9 @@ int evt_get_nidx(evt_handle h, uint32_t *nidx_out /* nobs */);
 /* Histogram of the last tree in the reference layout h∇[k, bin, feat, node] Float64
  * ((2K+1) x nbins x nfeats x (2^max_depth-1), src/init.jl:204); only slices of nodes that were
  * scanned (or, inside a tree grown in stages, built from rows at the current level) and features in js are
- * defined, the rest is zero. */
+ * defined, the rest is zero.  The second gradient row has no accumulator for one-output mse, mae and quantile: it is
+ * exported as derived (mse: twice the weight), as zero (mae, where the row is zero) or as zero in place of the sum of
+ * residuals (quantile: the reference accumulates it and reads it nowhere). */
 int evt_get_hist(evt_handle h, double *hist_out);
 /* Fixed-point parameters of the last update: gradient row k is accumulated as
  * rint(v * 2^(qbits[k]-qexp[k])) in int64. */

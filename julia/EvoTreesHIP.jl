@@ -58,11 +58,11 @@ check(rc::Integer) = rc == 0 ? nothing : error(lasterr())
 const LOSS_ID = Dict{Any,Cint}(
     EvoTrees.MSE => 0, EvoTrees.LogLoss => 1, EvoTrees.GaussianMLE => 2, EvoTrees.Poisson => 3,
     EvoTrees.Gamma => 4, EvoTrees.Tweedie => 5, EvoTrees.MLogLoss => 6, EvoTrees.LogisticMLE => 7,
-    EvoTrees.MAE => 8, EvoTrees.CredVar => 9, EvoTrees.CredStd => 10)
+    EvoTrees.MAE => 8, EvoTrees.CredVar => 9, EvoTrees.CredStd => 10, EvoTrees.Quantile => 11, EvoTrees.MultiQuantile => 12)
 const METRIC_ID = Dict{Symbol,Cint}(
     :mse => 0, :rmse => 1, :mae => 2, :logloss => 3, :gaussian_mle => 4, :poisson => 5, :gamma => 6,
-    :tweedie => 7, :mlogloss => 8, :logistic_mle => 9)
-loss_id(::Type{L}) where {L} = haskey(LOSS_ID, L) ? LOSS_ID[L] : error("loss $L is not supported by libevotrees_hip (mse, logloss, poisson, gamma, tweedie, mlogloss, gaussian_mle, logistic_mle, mae, cred_var, cred_std)")
+    :tweedie => 7, :mlogloss => 8, :logistic_mle => 9, :quantile => 10, :multiquantile => 11)
+loss_id(::Type{L}) where {L} = haskey(LOSS_ID, L) ? LOSS_ID[L] : error("loss $L is not supported by libevotrees_hip (mse, logloss, poisson, gamma, tweedie, mlogloss, gaussian_mle, logistic_mle, mae, cred_var, cred_std, quantile, multiquantile)")
 
 # ---------------------------------------------------------------------------------------------------------------
 # device_array_type / device_ones: `init` calls both before `init_core` (src/init.jl:331-333, :283-285).  Host arrays
@@ -121,6 +121,16 @@ end
 # y as the ABI takes it: Float32, one value per row (the UInt32 level codes of mlogloss included) or the reference's
 # targets x nobs matrix (src/init.jl:11-16); w == ones -> NULL (the row count then stands for the weight); offset is
 # nobs x K on the host (src/init.jl:168-174 adds offset'), K x nobs across the ABI.
+# params.alpha (every output of the quantile loss; also the level of the :quantile metric) or params.alphas (one output
+# each, multiquantile): src/loss.jl:144-171, src/callback.jl:62-66
+function upload_levels!(h::Ptr{Cvoid}, params, ::Type{L}) where {L}
+    a = L == EvoTrees.MultiQuantile ? Vector{Float64}(params.alphas) :
+        (hasproperty(params, :alpha) ? Float64[params.alpha] : Float64[])
+    isempty(a) && return nothing
+    GC.@preserve a check(ccall((:evt_set_alphas, LIB), Cint, (Ptr{Cvoid}, Ptr{Float64}, Cint), h, a, length(a)))
+    return nothing
+end
+
 function upload_target!(h::Ptr{Cvoid}, y, w::AbstractVector, μ::AbstractVector, offset)
     yf = y isa Array{Float32} ? y : Array{Float32}(y)
     wf = w isa Vector{Float32} ? w : Vector{Float32}(w)
@@ -165,6 +175,7 @@ function EvoTrees.init_core(params::EvoTypes, ::Type{<:HIPDevice}, data, feature
     end
     ft = Vector{UInt8}(feattypes)
     GC.@preserve ft monotone check(ccall((:evt_set_feature_meta, LIB), Cint, (Ptr{Cvoid}, Ptr{UInt8}, Ptr{Int32}), h, ft, monotone))
+    upload_levels!(h, params, L)
     upload_target!(h, y, w, μ, offset)
     # one tree per round: the next round's gradients are computed while the host stores the tree
     params.bagging_size == 1 && check(ccall((:evt_set_option, LIB), Cint, (Ptr{Cvoid}, Cstring, Int64), h, "grads_ahead", 1))
@@ -302,6 +313,7 @@ function callback_core(params, m::EvoTree{L,K}, data, y_eval, w_eval, offset_eva
     GC.@preserve ft check(ccall((:evt_set_feature_meta, LIB), Cint, (Ptr{Cvoid}, Ptr{UInt8}, Ptr{Int32}), h, ft, Ptr{Int32}(C_NULL)))
     y = L == EvoTrees.MLogLoss ? Float32.(EvoTrees.eval_levelcode(y_eval, m.info[:target_levels])) : Float32.(y_eval)
     w = isnothing(w_eval) ? ones(Float32, nobs) : Vector{Float32}(w_eval)
+    upload_levels!(h, params, L)
     upload_target!(h, y, w, zeros(Float32, K), eval_offset(L, offset_eval))      # p = 0 (+ offset'), src/callback.jl:38,75
     return CallBackHIP(EvoTrees.metric_dict[params.metric], cache, METRIC_ID[params.metric])
 end

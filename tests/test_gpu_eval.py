@@ -18,11 +18,14 @@ METRICS_OF = {
     "gamma": ["gamma"],
     "tweedie": ["tweedie", "rmse"],
     "mlogloss": ["mlogloss"],
+    "quantile": ["quantile", "mae", "mse"],
+    "multiquantile": ["multiquantile"],
 }
 
 
 @pytest.mark.parametrize("loss,weights", [("mse", True), ("logloss", False), ("gaussian_mle", True), ("poisson", True),
-                                          ("gamma", False), ("tweedie", True), ("mlogloss", True), ("logistic_mle", True)])
+                                          ("gamma", False), ("tweedie", True), ("mlogloss", True), ("logistic_mle", True),
+                                          ("quantile", True), ("multiquantile", False)])
 def test_eval_metric_matches_oracle(evt, loss, weights):
     N, F, B, D = 70001, 6, 32, 4
     x_bin, y, w, mu = make_data(41, N, F, B, loss, weights)
@@ -37,10 +40,13 @@ def test_eval_metric_matches_oracle(evt, loss, weights):
         pred = h.get_pred()
         for metric in METRICS_OF[loss]:
             got = h.eval_metric(metric)
-            want = orc.eval_metric(metric, op.K, pred, y, w)
+            want = orc.eval_metric(metric, op.K, pred, y, w, alphas=list(op.alphas[:op.n_alphas]))
             exact_rows = metric in ("mse", "rmse", "mae")  # per-row Float32 values identical, only the Float64 sum order differs
             np.testing.assert_allclose(got, want, rtol=1e-12 if exact_rows else RTOL)
             assert got == h.eval_metric(metric)  # fixed summation order: reproducible to the bit
+    if loss != "multiquantile":
+        with pytest.raises(evt.EvtError):
+            h.eval_metric("multiquantile")
     if loss not in ("gaussian_mle", "mlogloss", "logistic_mle"):
         with pytest.raises(evt.EvtError):
             h.eval_metric("gaussian_mle")
@@ -89,7 +95,8 @@ def _sinus(rng, n):
 @pytest.mark.parametrize("cfg_kw", [dict(loss="mse", metric="mae"), dict(loss="logloss"), dict(loss="gamma"), dict(loss="tweedie"),
                                     dict(loss="poisson", learner="count"), dict(loss="gaussian_mle", learner="mle"),
                                     dict(loss="logistic_mle", learner="mle"), dict(loss="mae"), dict(loss="cred_var"),
-                                    dict(loss="cred_std", metric="rmse")])
+                                    dict(loss="cred_std", metric="rmse"), dict(loss="quantile", alpha=0.8),
+                                    dict(loss="multiquantile", alphas=[0.2, 0.5, 0.8])])
 def test_fit_with_eval_logger_matches_oracle_replay(evt, cfg_kw):
     # every logged value equals the oracle's metric of the oracle's own replay of the model on the eval rows
     rng = np.random.default_rng(7)
@@ -114,7 +121,8 @@ def test_fit_with_eval_logger_matches_oracle_replay(evt, cfg_kw):
     for i, t in enumerate(m.trees):
         orc.predict_tree(orc.LOSS_IDS[cfg.loss], m.K, xb, ft, t, p)
         # a mean log-likelihood can pass through zero: the absolute bound is 1e-6 of the per-row values' scale (~1)
-        np.testing.assert_allclose(lg["metrics"][i], orc.eval_metric(cfg.metric, m.K, p, y32, w_ev), rtol=RTOL, atol=1e-6)
+        al = list(cfg.alphas) if cfg.loss == "multiquantile" else [getattr(cfg, "alpha", 0.5)]
+        np.testing.assert_allclose(lg["metrics"][i], orc.eval_metric(cfg.metric, m.K, p, y32, w_ev, alphas=al), rtol=RTOL, atol=1e-6)
     best = int(np.argmax(lg["metrics"]) if lg["maximise"] else np.argmin(lg["metrics"]))
     assert lg["best_iter"] == best and lg["best_metric"] == lg["metrics"][best]
     better = lg["metrics"][-1] > lg["metrics"][0] if lg["maximise"] else lg["metrics"][-1] < lg["metrics"][0]

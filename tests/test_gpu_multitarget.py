@@ -24,6 +24,8 @@ def make_targets(seed, N, F, B, loss, T, weights):
         y = np.floor(y * 3).astype(np.float32)
     elif loss in ("gamma", "tweedie"):
         y = (y + 0.1).astype(np.float32)
+    elif loss == "quantile":
+        y = (y - 0.95).astype(np.float32)  # residuals of both signs against the starting prediction near zero
     K = 2 * T if loss in ("gaussian_mle", "logistic_mle") else T
     w = (rng.random(N).astype(np.float32) + 0.5) if weights else None
     mu = (rng.standard_normal(K) * 0.1).astype(np.float32)
@@ -48,6 +50,8 @@ CASES = [
     ("mae", 2, False, 9000, 40, 64, 4, "oblivious", 25, 0.5, True),
     ("cred_var", 2, True, 12000, 14, 32, 5, "binary", 10, 1.0, True),
     ("cred_std", 4, False, 9000, 20, 16, 4, "binary", 20, 0.5, False),
+    ("quantile", 3, True, 12000, 14, 32, 5, "binary", 14, 1.0, False),
+    ("quantile", 2, False, 9000, 20, 16, 4, "oblivious", 20, 0.5, True),
 ]
 
 
@@ -64,7 +68,7 @@ def test_multi_target_tree_against_the_oracle(evt, loss, T, weights, N, F, B, D,
     orc.update_grads(op, pred0, y, grad)
     h.update_grads()
     g_dev = h.get_grads()
-    if loss in ("mse", "mae", "cred_var", "cred_std"):
+    if loss in ("mse", "mae", "cred_var", "cred_std", "quantile"):
         assert np.array_equal(g_dev.view(np.uint32), grad.view(np.uint32))
     else:
         # (1 - r^2 / s^2) and (1 - z tanh(z / 2)) cancel, which magnifies the last-bit differences between two libm's exp / tanh:
@@ -110,9 +114,9 @@ def test_multi_target_tree_against_the_oracle(evt, loss, T, weights, N, F, B, D,
         assert abs(float(t_gpu.gain[n0]) - float(t_ref.gain[n0])) <= 1e-6 * abs(float(t_ref.gain[n0])) + 1e-12
     # the evaluation metric on the updated prediction
     metric = {"mse": "mse", "logloss": "logloss", "poisson": "poisson", "gamma": "gamma", "tweedie": "tweedie",
-              "gaussian_mle": "gaussian_mle", "logistic_mle": "logistic_mle", "mae": "mae", "cred_var": "mae", "cred_std": "mae"}[loss]
+              "gaussian_mle": "gaussian_mle", "logistic_mle": "logistic_mle", "mae": "mae", "cred_var": "mae", "cred_std": "mae", "quantile": "quantile"}[loss]
     got = h.eval_metric(metric)
-    want = orc.eval_metric(metric, K, p_orc, y, w)
+    want = orc.eval_metric(metric, K, p_orc, y, w, alphas=[0.5])
     assert abs(got - want) <= 1e-5 * abs(want) + 1e-9
     if loss == "mse":
         assert abs(h.eval_metric("rmse") - np.sqrt(want)) <= 1e-5 * np.sqrt(want)

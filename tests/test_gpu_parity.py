@@ -20,7 +20,7 @@ RTOL = 1e-5
 
 
 def n_outputs(loss, K=None):
-    return 2 if loss in ("gaussian_mle", "logistic_mle") else ((K or 3) if loss == "mlogloss" else 1)
+    return 2 if loss in ("gaussian_mle", "logistic_mle") else ((K or 3) if loss in ("mlogloss", "multiquantile") else 1)
 
 
 def make_data(seed, N, F, nbins, loss="mse", weights=False, signal=True, K=None):
@@ -36,6 +36,8 @@ def make_data(seed, N, F, nbins, loss="mse", weights=False, signal=True, K=None)
         y = np.floor(y * 3).astype(np.float32)  # counts, zeros included
     elif loss in ("gamma", "tweedie"):
         y = (y + 0.1).astype(np.float32)  # strictly positive
+    elif loss in ("quantile", "multiquantile"):
+        y = (y - 0.85).astype(np.float32)  # residuals of both signs against the starting prediction near zero
     elif loss == "mlogloss":
         y = (np.minimum(np.floor(y / y.max() * K), K - 1) + 1).astype(np.float32)  # 1-based class, tied to the features
     w = (rng.random(N).astype(np.float32) + 0.5) if weights else None
@@ -51,6 +53,13 @@ def setup_pair(evt, loss, x_bin, y, w, mu, nbins, depth, tree_type="binary", fea
     h = evt.Handle(N, F, nbins, K, depth, loss, tree_type)
     h.set_xbin(x_bin)
     h.set_feature_meta(feattypes, mono)
+    if loss == "multiquantile":  # one level per output
+        pk = dict(pk, alphas=pk.get("alphas", [0.1, 0.5, 0.9]))
+        assert len(pk["alphas"]) == K
+        h.set_alphas(pk["alphas"])
+    elif loss == "quantile":
+        pk = dict(pk, alpha=pk.get("alpha", 0.5))
+        h.set_alphas([pk["alpha"]])
     h.set_target(y, w, mu)
     op = orc.make_params(loss, nbins=nbins, max_depth=depth, tree_type=tree_type, K=K, **pk)
     o = orc.Oracle(op, x_bin, feattypes, mono)
@@ -84,7 +93,8 @@ def assert_tree_close(t_gpu, t_ref, pred_atol=1e-9):
 @pytest.mark.parametrize("loss,weights", [("mse", False), ("mse", True), ("logloss", True), ("gaussian_mle", False),
                                           ("gaussian_mle", True), ("poisson", True), ("gamma", False), ("tweedie", True),
                                           ("mlogloss", False), ("mlogloss", True), ("logistic_mle", False), ("logistic_mle", True),
-                                          ("mae", False), ("mae", True), ("cred_var", True), ("cred_std", False)])
+                                          ("mae", False), ("mae", True), ("cred_var", True), ("cred_std", False),
+                                          ("quantile", True), ("quantile", False), ("multiquantile", True)])
 def test_gradient_kernel(evt, loss, weights):
     N, F, B = 70001, 5, 16
     x_bin, y, w, mu = make_data(1, N, F, B, loss, weights)
@@ -95,7 +105,7 @@ def test_gradient_kernel(evt, loss, weights):
     orc.update_grads(op, pred0, y, grad)
     K = op.K
     assert np.array_equal(g_gpu[:, 2 * K], grad[:, 2 * K])  # weight row untouched
-    if loss in ("mse", "mae", "cred_var", "cred_std"):
+    if loss in ("mse", "mae", "cred_var", "cred_std", "quantile", "multiquantile"):
         assert np.array_equal(g_gpu.view(np.uint32), grad.view(np.uint32))  # exact Float32 arithmetic
     else:
         # terms like (1 - z tanh(z / 2)) cancel: the absolute bound is a few ulp of the largest gradient
@@ -142,6 +152,12 @@ CASES = [
     ("cred_var", True, 40000, 100, 64, 6, "binary", 100, 0.7, dict(L2=2.0, min_weight=4.0)),
     ("cred_std", False, 30000, 20, 64, 6, "binary", 14, 1.0, dict(L2=0.0)),
     ("cred_std", True, 20000, 10, 16, 5, "oblivious", 10, 0.8, {}),
+    ("quantile", False, 30000, 12, 32, 6, "binary", 12, 1.0, dict(alpha=0.3)),
+    ("quantile", True, 40000, 100, 64, 6, "binary", 60, 0.6, dict(alpha=0.9, lambda_=0.2, L2=0.5, gamma=0.01)),
+    ("quantile", False, 20000, 10, 16, 5, "oblivious", 10, 1.0, {}),
+    ("quantile", True, 3000, 4, 4, 12, "binary", 4, 0.9, dict(alpha=0.05, min_weight=0.0)),  # leaves of one or two rows
+    ("multiquantile", True, 30000, 12, 32, 5, "binary", 12, 0.8, dict(alphas=[0.1, 0.5, 0.9])),
+    ("multiquantile", False, 20000, 20, 64, 4, "oblivious", 20, 1.0, dict(alphas=[0.25, 0.75], L2=0.0)),
     ("mse", False, 60000, 5, 8, 14, "binary", 5, 1.0, dict(min_weight=0.0)),   # deep: most leaves hold a handful of rows
     ("logloss", True, 3000, 4, 4, 16, "binary", 4, 0.9, dict(min_weight=0.0)),  # deepest supported tree, far more nodes than rows
 ]
@@ -151,7 +167,7 @@ CASES = [
 def test_grow_tree_matches_oracle(evt, loss, weights, N, F, B, D, tt, n_js, rowsample, pk):
     print("case", loss, weights, N, F, B, D, tt, n_js, rowsample, pk, flush=True)
     pk = dict(pk)
-    x_bin, y, w, mu = make_data(7, N, F, B, loss, weights, K=pk.pop("K", None))
+    x_bin, y, w, mu = make_data(7, N, F, B, loss, weights, K=pk.pop("K", None) or (len(pk["alphas"]) if "alphas" in pk else None))
     h, o, op, gp, pred0, grad0 = setup_pair(evt, loss, x_bin, y, w, mu, B, D, tt, **pk)
     rng = np.random.default_rng(99)
     grad = grad0.copy()
@@ -179,9 +195,14 @@ def test_grow_tree_matches_oracle(evt, loss, weights, N, F, B, D, tt, n_js, rows
     Hq = o.hist(fixed=True)
     scale = np.ldexp(1.0, (qe - qb).astype(np.int64))
     split_nodes = np.flatnonzero(t_gpu.split)
+    # one-output quantile: the second gradient row (the raw residual, read per row when the leaves are valued) has no
+    # accumulator on the device and is exported as zero; no gain reads its sum
+    chan = [0, 2] if loss in ("quantile", "multiquantile") and op.K == 1 else list(range(2 * op.K + 1))
     for n0 in split_nodes:
         want = Hq[n0][js - 1].astype(np.float64) * scale
-        assert np.array_equal(H_gpu[n0][js - 1], want), n0
+        assert np.array_equal(H_gpu[n0][js - 1][..., chan], want[..., chan]), n0
+        if len(chan) == 2:
+            assert not H_gpu[n0][js - 1][..., 1].any()
     # reference arithmetic (Float64 accumulation in row order): same structure, values within 1e-5
     t_ref, nidx_ref = o.grow_tree(grad, rows, js, mode=0)
     assert_tree_close(t_gpu, t_ref)
@@ -189,7 +210,7 @@ def test_grow_tree_matches_oracle(evt, loss, weights, N, F, B, D, tt, n_js, rows
     H_ref = o.hist()
     gmax = np.abs(grad).max(axis=0)
     for n0 in split_nodes:
-        np.testing.assert_allclose(H_gpu[n0][js - 1], H_ref[n0][js - 1], rtol=RTOL, atol=1e-6 * float(gmax.max()))
+        np.testing.assert_allclose(H_gpu[n0][js - 1][..., chan], H_ref[n0][js - 1][..., chan], rtol=RTOL, atol=1e-6 * float(gmax.max()))
     if D > 1 and N >= 5000:
         assert len(split_nodes) >= 1
     # predict! on the cache: all rows (also those outside the sample)
