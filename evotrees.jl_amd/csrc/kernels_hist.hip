@@ -76,27 +76,19 @@ __device__ __forceinline__ unsigned long long load_gq(const unsigned long long *
 }
 
 // Chunk descriptors of the level, for the partition kernels that run after the split search: chunk c of the level is
-// chunk c - c0 of node n, whose segment ends at `end`: {n, first position, end, c0}.  One wavefront per chunk finds the
-// owner (all its loads independent); the work hides behind the histogram kernel's own set-up.
+// chunk c - c0 of node n, whose segment ends at `end`: {n, first position, end, c0}.  One wavefront per active node
+// writes the descriptors of that node's chunks, cprefix[i] .. cprefix[i + 1] (two dependent trips to memory, then
+// stores); the work hides behind the histogram kernel's own set-up.
 __device__ __forceinline__ void fill_chunk_descriptors(const HistArgs &A) {
     if (blockIdx.y != 0 || A.a0 != 0) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int n_act = (int)A.hdr[LH_N_ACT];
-    const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
-    for (int64_t c = (int64_t)blockIdx.x * nwaves + wave; c < n_chunks; c += (int64_t)gridDim.x * nwaves) {
-        int cnt = 0;
-        for (int k0 = 0; k0 < n_act; k0 += 64) {
-            const int k = k0 + lane;
-            const bool hit = (k < n_act) && (A.cprefix[k < n_act ? k : 0] <= c);
-            cnt += __popcll(__ballot(hit));
-        }
-        if (lane == 0) {
-            const int i = cnt - 1;
-            const int n = A.act_node[i];
-            const int64_t c0 = A.cprefix[i];
-            const int64_t seg = A.seg_start[n], len = A.seg_len[n];
+    for (int i = (int)blockIdx.x * nwaves + wave; i < n_act; i += (int)gridDim.x * nwaves) {
+        const int n = A.act_node[i];
+        const int64_t c0 = A.cprefix[i], c1 = A.cprefix[i + 1];
+        const int64_t seg = A.seg_start[n], len = A.seg_len[n];
+        for (int64_t c = c0 + lane; c < c1; c += 64)
             A.cdesc[c] = make_uint4((uint32_t)n, (uint32_t)(seg + (c - c0) * EVT_CHUNK), (uint32_t)(seg + len), (uint32_t)c0);
-        }
     }
 }
 
