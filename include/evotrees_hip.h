@@ -41,7 +41,7 @@ typedef enum {
     EVT_ERR_NOMEM = -5
 } evt_status;
 
-/* loss ids: the in-scope subset of src/loss.jl:20-34 */
+/* loss ids: the losses of src/loss.jl:20-34 */
 enum {
     EVT_LOSS_MSE = 0,
     EVT_LOSS_LOGLOSS = 1,
@@ -115,9 +115,9 @@ int evt_device_count(int32_t *count);
  * Replaces init_core(params, ::Type{<:GPU}, ...) device allocation
  * (ext/EvoTreesKernelAbstractionsExt/init.jl:1-151): sizes every device buffer.
  * nbins in [2,255] (src/learners.jl:527).  K is the number of outputs (size(pred, 1) in the reference, at most 16):
- * the number of targets for mse / logloss / poisson / gamma / tweedie (1, or more with a matrix target,
- * src/init.jl:11-16, :142-150), twice the number of targets for gaussian_mle and logistic_mle (src/init.jl:68-100), the number of
- * classes (2..16) for mlogloss. */
+ * the number of targets for mse / logloss / poisson / gamma / tweedie / mae / quantile / cred_var / cred_std (1, or more with
+ * a matrix target, src/init.jl:11-16, :104-150), twice the number of targets for gaussian_mle and logistic_mle
+ * (src/init.jl:68-100), the number of classes (2..16) for mlogloss, the number of levels for multiquantile (src/init.jl:101-103). */
 int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K, int32_t max_depth, int32_t loss,
                int32_t tree_type, evt_handle *out);
 /* Frees all device memory; the slot post_fit_gc has in the reference (src/fit.jl:340). */
