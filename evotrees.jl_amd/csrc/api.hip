@@ -270,6 +270,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->hist_threads = 1024;
     c->hist_min_rows = 1024;
     c->hist_variant = 0;
+    c->scan_fused = 1;
     c->hist_seg_cost = 2048;
     c->record_nidx = false;
     c->nidx_valid = false;
@@ -1628,6 +1629,8 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
         if (!c->grads_ahead) c->grads_ready = false;
     } else if (strcmp(name, "record_nidx") == 0) {
         c->record_nidx = value != 0;
+    } else if (strcmp(name, "scan_fused") == 0) {
+        c->scan_fused = value != 0;
     } else if (strcmp(name, "defer_pred") == 0) {
         c->defer_pred = value != 0;
     } else if (strcmp(name, "hist_threads") == 0) {

@@ -165,7 +165,8 @@ struct evt_ctx {
 
     // tunables
     int hist_blocks, hist_threads, hist_min_rows, hist_seg_cost;
-    int hist_variant;  // 0 auto, 1 generic 16-byte-piece kernel, 2 conflict-free 8-byte-piece kernel where it applies
+    int hist_variant;
+    int scan_fused;    // option: the split search of a node with at most 16 sampled features runs in one kernel  // 0 auto, 1 generic 16-byte-piece kernel, 2 conflict-free 8-byte-piece kernel where it applies
     bool record_nidx;  // leaf finalisation also writes the node id of every sampled row
     bool nidx_valid;   // nidx holds the last tree's node ids
     bool defer_pred;   // a tree grown on every row records leaf ids and leaves the addition to the next row-order pass

@@ -171,11 +171,69 @@ __device__ __forceinline__ void node_totals(const ScanArgs &A, int n, const long
     __syncthreads();
 }
 
+// The decision for one node (get_best_split's threshold, src/fit-utils.jl:444-450; the Tree arrays, src/fit.jl:96-103;
+// a node without a split becomes a leaf, src/predict.jl:198-262): thread 0 holds the node's best candidate (bg, bj, bb)
+// and its feature (1-based id, type); S: the node's statistics (in shared memory).  Leaves {found, bj, bb} in s_dec.
+__device__ __forceinline__ void scan_decide(const ScanArgs &A, int n, const double *S, int *s_dec, double bg, int bj, int bb, int feat, bool numeric) {
+    const int K = A.K;
+    const int found = (bb != NO_BIN && bg > A.gamma) ? 1 : 0;
+    s_dec[0] = found; s_dec[1] = bj; s_dec[2] = bb;
+    if (found) {
+        A.tree.feat[n - 1] = feat;
+        A.tree.cond_bin[n - 1] = (uint8_t)bb;
+        A.tree.gain[n - 1] = (float)bg;
+        A.tree.split[n - 1] = 1;
+        A.tree.packed[n - 1] = evt_pack_node(feat, bb, numeric);
+        A.status[n] = ST_SPLIT;
+    } else {
+        for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (n - 1) + k] = (float)leaf_value(A.loss, S, k, K, A.eta, A.bagging, A.lambda, A.L2);
+        A.status[n] = ST_LEAF;
+    }
+}
+
+// Totals of the two children from the left child's (qL; right = parent - left, exact in integers; _child_sums!,
+// src/fit-utils.jl:472-486), by one lane.  With fold_leaves the children are leaves of the last level: their weight, values
+// and state are written here too - what the leaf-level pass would compute from node_sum (same integers, same expressions).
+template <int NAG>
+__device__ __forceinline__ void write_children(const ScanArgs &A, int n, const long long *qL, const long long *s_Sq, const double *s_sc) {
+    const int NK = A.NK, K = A.K;
+#pragma unroll
+    for (int child = 0; child < 2; child++) {
+        const int cn = 2 * n + child;
+        long long qc[NAG];
+#pragma unroll
+        for (int ag = 0; ag < NAG; ag++) {
+            qc[ag] = child ? s_Sq[ag] - qL[ag] : qL[ag];
+            A.node_sum[(int64_t)cn * NAG + ag] = qc[ag];
+        }
+        if (A.fold_leaves) {
+            double v[EVT_MAX_NK];
+            decode_vals(qc, s_sc, A.loss, NK, v);
+            A.tree.w[cn - 1] = (float)v[NK - 1];
+            for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (cn - 1) + k] = (float)leaf_value(A.loss, v, k, K, A.eta, A.bagging, A.lambda, A.L2);
+            A.status[cn] = ST_LEAF;
+        }
+    }
+}
+
+// the children's histogram slices start from zero (the build child accumulates into its own)
+template <int NAG>
+__device__ __forceinline__ void zero_children_slices(const ScanArgs &A, int n) {
+    long long *hc = A.hist + (int64_t)(2 * n - 1) * A.node_stride;
+    const int64_t used = (int64_t)A.nfs * NAG * A.B;
+    for (int64_t i = threadIdx.x; i < used; i += blockDim.x) {
+        hc[i] = 0;
+        hc[A.node_stride + i] = 0;
+    }
+}
+
 // Pass 1: grid (nodes of the level, feature groups); one wave per (node, sampled feature).
 // Writes the group's best candidate to sbest[node][group] (or the gain matrix for oblivious trees)
 // and, for subtract nodes, materialises h[n] = h[parent] - h[sibling].
-template <int NAG, int BPL>
-__global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
+// FUSED: one block of 16 waves per node covers every sampled feature (at most 16) and finishes the node itself
+// (scan_finish): one launch per level instead of two where a level is a chain of small kernels.
+template <int NAG, int BPL, bool FUSED>
+__global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const int n = (1 << (A.level - 1)) + blockIdx.x; // 1-based node id
     // The block's time is a chain of round trips to memory, so requests go out in as few dependent steps as the data
@@ -189,7 +247,9 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     asm volatile("" : "+v"(f)); // the feature id is requested ahead of the branch on the node state, not behind it
     if (st != ST_BUILD && st != ST_SUBTRACT) return;
     const bool is_sub = (st == ST_SUBTRACT);
-    const int B = A.B, NK = A.NK, K = A.K;
+    // the channel layout fixes the outputs: two-output MLE losses have five channels, every other shape here one output
+    constexpr int K = (NAG == 5) ? 2 : 1, NK = 2 * K + 1;
+    const int B = A.B;
     // BPL = bins per lane = ceil(nbins / 64), a template parameter so that nbins <= 64 keeps one bin per lane in registers
     long long *hn = A.hist + (int64_t)(n - 1) * A.node_stride;
     const long long *hp = A.hist + (int64_t)((n >> 1) - 1) * A.node_stride;
@@ -198,8 +258,10 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     __shared__ long long s_Sq[EVT_MAX_NA];
     __shared__ double s_S[EVT_MAX_NK];
     __shared__ double s_sc[EVT_MAX_NA];
-    __shared__ double s_wg[4];
-    __shared__ int s_wjp[4], s_wbin[4];
+    __shared__ double s_wg[16];
+    __shared__ int s_wjp[16], s_wbin[16];
+    __shared__ int s_wfeat[16]; // FUSED: feature of each wave (1-based id, negative when categorical)
+    __shared__ int s_dec[3];
 
     long long pre[NAG][BPL];
     long long vb[NAG][BPL];
@@ -254,15 +316,15 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
         }
         __syncthreads();
         if (tid == 0) {
-            double v[EVT_MAX_NK];
+            double v[NK];
             long long q[NAG];
             for (int ag = 0; ag < NAG; ag++) q[ag] = s_Sq[ag];
-            decode_vals(q, s_sc, A.loss, A.NK, v);
-            for (int k = 0; k < A.NK; k++) s_S[k] = v[k];
+            decode_vals(q, s_sc, A.loss, NK, v);
+            for (int k = 0; k < NK; k++) s_S[k] = v[k];
         }
         __syncthreads();
     }
-    double S[EVT_MAX_NK];
+    double S[NK];
     for (int k = 0; k < NK; k++) S[k] = s_S[k];
 
     double gain_p = 0.0;
@@ -304,14 +366,14 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
                         const long long prev = (t == 0) ? excl[ag] : pre[ag][t > 0 ? t - 1 : 0];
                         q[ag] = numeric ? pre[ag][t] : (pre[ag][t] - prev); // _acc_left!: accumulate vs single bin
                     }
-                    double SL[EVT_MAX_NK];
+                    double SL[NK];
                     decode_vals(q, s_sc, A.loss, NK, SL);
                     const double w_l = SL[NK - 1];
                     const double w_r = w_p - w_l;
                     if (w_l > A.min_weight && w_r > A.min_weight) {
                         ok = true;
                         if (constraint != 0) {
-                            double SR[EVT_MAX_NK];
+                            double SR[NK];
                             for (int k = 0; k < NK; k++) SR[k] = S[k] - SL[k];
                             const double predL = leaf_value(A.loss, SL, 0, K, A.eta, A.bagging, A.lambda, A.L2);
                             const double predR = leaf_value(A.loss, SR, 0, K, A.eta, A.bagging, A.lambda, A.L2);
@@ -346,14 +408,46 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
     }
     if (A.oblivious) return; // decision is taken for the whole level by k_obliv_select
 
-    if (lane == 0) { s_wg[wave] = wbest; s_wjp[wave] = wjp; s_wbin[wave] = wbin; }
+    if (lane == 0) {
+        s_wg[wave] = wbest; s_wjp[wave] = wjp; s_wbin[wave] = wbin;
+        if (FUSED) s_wfeat[wave] = numeric ? f + 1 : -(f + 1);
+    }
     __syncthreads();
+    double bg = -INFINITY;
+    int bj = NO_BIN, bb = NO_BIN;
     if (tid == 0) {
-        double bg = -INFINITY;
-        int bj = NO_BIN, bb = NO_BIN;
         for (int w = 0; w < nwaves; w++) {
             if (s_wg[w] > bg || (s_wg[w] == bg && s_wjp[w] < bj)) { bg = s_wg[w]; bj = s_wjp[w]; bb = s_wbin[w]; }
         }
+    }
+    if constexpr (FUSED) {
+        // the node is finished here: wave jp scanned sampled feature jp, so the winner's left totals are still in the
+        // registers of the lane that holds the winning bin - no second read of the histogram
+        if (tid == 0) {
+            A.tree.w[n - 1] = (float)S[NK - 1];
+            const int wf = (bb != NO_BIN) ? s_wfeat[bj] : 1;
+            scan_decide(A, n, s_S, s_dec, bg, bj, bb, wf < 0 ? -wf : wf, wf > 0);
+        }
+        __syncthreads();
+        if (!s_dec[0]) return;
+        if (have && jp == s_dec[1]) {
+            const int b0 = s_dec[2] - 1; // 0-based winning bin: lane b0 / BPL, position b0 % BPL
+            long long qL[NAG];
+#pragma unroll
+            for (int ag = 0; ag < NAG; ag++) {
+                long long v = 0;
+#pragma unroll
+                for (int t = 0; t < BPL; t++) {
+                    const long long prev = (t == 0) ? excl[ag] : pre[ag][t > 0 ? t - 1 : 0];
+                    const long long q = numeric ? pre[ag][t] : (pre[ag][t] - prev);
+                    if (t == b0 % BPL) v = q;
+                }
+                qL[ag] = v;
+            }
+            if (lane == b0 / BPL) write_children<NAG>(A, n, qL, s_Sq, s_sc);
+        }
+        if (A.zero_children) zero_children_slices<NAG>(A, n);
+    } else if (tid == 0) {
         ScanBest r;
         r.gain = bg; r.jp = bj; r.bin = bb;
         A.sbest[(int64_t)nodeidx * gridDim.y + blockIdx.y] = r;
@@ -367,7 +461,7 @@ __global__ __launch_bounds__(256) void k_scan(ScanArgs A) {
 // exact in integers) and zeroes the children's histogram slices.
 template <int NAG>
 __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x;
     const int n = (1 << (A.level - 1)) + blockIdx.x;
     if (blockIdx.y > 0) {
         // Blocks beyond the first of a node only clear the children's histogram slices (the build child accumulates
@@ -392,7 +486,7 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
         const int st = A.status[n];
         if (st != ST_BUILD && st != ST_SUBTRACT) return;
     }
-    const int B = A.B, NK = A.NK, K = A.K;
+    const int NK = A.NK, K = A.K;
     long long *hn = A.hist + (int64_t)(n - 1) * A.node_stride;
 
     __shared__ long long s_Sq[EVT_MAX_NA];
@@ -429,62 +523,37 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
         __syncthreads();
     }
     if (tid == 0) {
-        bg = s_g[0]; bj = s_j[0]; bb = s_b[0];
-        const int found = (bb != NO_BIN && bg > A.gamma) ? 1 : 0;
-        s_dec[0] = found; s_dec[1] = bj; s_dec[2] = bb;
-        if (found) {
-            const int feat = (int)A.js[bj];
-            A.tree.feat[n - 1] = feat;
-            A.tree.cond_bin[n - 1] = (uint8_t)bb;
-            A.tree.gain[n - 1] = (float)bg;
-            A.tree.split[n - 1] = 1;
-            A.tree.packed[n - 1] = evt_pack_node(feat, bb, A.feattypes[feat - 1] != 0);
-            A.status[n] = ST_SPLIT;
-        } else {
-            for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (n - 1) + k] = (float)leaf_value(A.loss, S, k, K, A.eta, A.bagging, A.lambda, A.L2);
-            A.status[n] = ST_LEAF;
+        const int bj0 = s_j[0], bb0 = s_b[0];
+        int feat = 0;
+        bool numeric = true;
+        if (bb0 != NO_BIN) {
+            feat = (int)A.js[bj0];
+            numeric = A.feattypes[feat - 1] != 0;
         }
+        scan_decide(A, n, s_S, s_dec, s_g[0], bj0, bb0, feat, numeric);
     }
     __syncthreads();
     if (!s_dec[0]) return;
     bj = s_dec[1]; bb = s_dec[2];
-    if (wave == 0) { // pass 1 already materialised h[n] for subtract nodes
+    if (tid < 64) { // wave 0; pass 1 already materialised h[n] for subtract nodes
+        const int lane = tid;
+        const int B = A.B;
         const int f = (int)A.js[bj] - 1;
         const bool numeric = A.feattypes[f] != 0;
-        long long qc[NAG]; // lane 0: the left child's sums, lane 1: the right child's
+        long long qL[NAG];
         for (int ag = 0; ag < NAG; ag++) {
             const int64_t o = ((int64_t)bj * NAG + ag) * B;
-            long long s = 0;
+            long long sL = 0;
             for (int b = lane; b < B; b += 64) {
                 const bool in = numeric ? (b + 1 <= bb) : (b + 1 == bb);
-                if (in) s += hn[o + b];
+                if (in) sL += hn[o + b];
             }
-            s = wave_sum_i64(s);
-            if (lane == 0) {
-                A.node_sum[(int64_t)(2 * n) * NAG + ag] = s;
-                A.node_sum[(int64_t)(2 * n + 1) * NAG + ag] = s_Sq[ag] - s;
-            }
-            qc[ag] = (lane & 1) ? s_Sq[ag] - s : s;
+            qL[ag] = wave_sum_i64(sL);
         }
-        if (A.fold_leaves && lane < 2) {
-            // what the leaf-level pass would compute from node_sum (same integers, same expressions)
-            const int cn = 2 * n + lane;
-            double v[EVT_MAX_NK];
-            decode_vals(qc, s_sc, A.loss, NK, v);
-            A.tree.w[cn - 1] = (float)v[NK - 1];
-            for (int k = 0; k < K; k++) A.tree.pred[(int64_t)K * (cn - 1) + k] = (float)leaf_value(A.loss, v, k, K, A.eta, A.bagging, A.lambda, A.L2);
-            A.status[cn] = ST_LEAF;
-        }
+        if (lane == 0) write_children<NAG>(A, n, qL, s_Sq, s_sc);
     }
-    // the children's histogram slices start from zero (the build child accumulates into it): with one block per node
-    // this block clears them, otherwise the node's other blocks have
-    if (!A.zero_children || gridDim.y > 1) return;
-    long long *hc = A.hist + (int64_t)(2 * n - 1) * A.node_stride;
-    const int64_t used = (int64_t)A.nfs * NAG * B;
-    for (int64_t i = tid; i < used; i += blockDim.x) {
-        hc[i] = 0;
-        hc[A.node_stride + i] = 0;
-    }
+    // with one block per node this block clears the children's slices, otherwise the node's other blocks have
+    if (A.zero_children && gridDim.y == 1) zero_children_slices<NAG>(A, n);
 }
 
 // Oblivious trees (grow_otree!, src/fit.jl:190-257): per-level decision from the sum of the
@@ -880,12 +949,20 @@ int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
         HIPCHK(hipGetLastError());
         return EVT_OK;
     }
+    // few sampled features: one block of 16 waves scans a node's features and finishes the node, no second launch
+    const bool fused = !leaf_level && !A.oblivious && A.nfs <= 16 && c->scan_fused;
 #define SCASE(NAG_)                                                                                     \
     case NAG_:                                                                                          \
+        if (fused) {                                                                                    \
+            if (bpl == 1) hipLaunchKernelGGL((k_scan<NAG_, 1, true>), dim3(nodes), dim3(1024), 0, c->stream, A);      \
+            else if (bpl == 2) hipLaunchKernelGGL((k_scan<NAG_, 2, true>), dim3(nodes), dim3(1024), 0, c->stream, A); \
+            else hipLaunchKernelGGL((k_scan<NAG_, 4, true>), dim3(nodes), dim3(1024), 0, c->stream, A);               \
+            break;                                                                                      \
+        }                                                                                               \
         if (!leaf_level) {                                                                              \
-            if (bpl == 1) hipLaunchKernelGGL((k_scan<NAG_, 1>), grid, dim3(256), 0, c->stream, A);      \
-            else if (bpl == 2) hipLaunchKernelGGL((k_scan<NAG_, 2>), grid, dim3(256), 0, c->stream, A); \
-            else hipLaunchKernelGGL((k_scan<NAG_, 4>), grid, dim3(256), 0, c->stream, A);               \
+            if (bpl == 1) hipLaunchKernelGGL((k_scan<NAG_, 1, false>), grid, dim3(256), 0, c->stream, A);      \
+            else if (bpl == 2) hipLaunchKernelGGL((k_scan<NAG_, 2, false>), grid, dim3(256), 0, c->stream, A); \
+            else hipLaunchKernelGGL((k_scan<NAG_, 4, false>), grid, dim3(256), 0, c->stream, A);               \
         }                                                                                               \
         if (!A.oblivious || leaf_level) hipLaunchKernelGGL(k_scan_fin<NAG_>, dim3(nodes, 1 + zero_blocks), dim3(256), 0, c->stream, A, ngroups); \
         break;
