@@ -77,13 +77,14 @@ def synth(cfg, seed=123):
     return x, y.astype(np.float32), rng
 
 
-def edges_from_sample(x_FN, nbins, rng):
-    """Quantile edges on <= 1000*nbins sampled rows (src/fit-utils.jl:9-16)."""
+def edges_from_sample(evt, x_FN, nbins, rng):
+    """Quantile edges on <= 1000*nbins sampled rows (src/fit-utils.jl:9-16), the features spread over threads as in the
+    reference's `@threads for j` and in the host mirror's get_edges."""
     F, N = x_FN.shape
     nobs = min(N, 1000 * nbins)
     idx = np.sort(rng.choice(N, nobs, replace=False)) if nobs < N else np.arange(N)
     q = np.arange(1, nbins) / nbins
-    return [np.ascontiguousarray(np.quantile(x_FN[j, idx], q)) for j in range(F)]
+    return evt._per_feature(lambda j: np.ascontiguousarray(np.quantile(x_FN[j, idx], q)), F)
 
 
 def bias(loss, y):
@@ -119,7 +120,7 @@ def prepare(evt, cfg, opts=None):
     t0 = time.time()
     x, y, rng = synth(cfg)
     t1 = time.time()
-    edges = edges_from_sample(x, B, rng)
+    edges = edges_from_sample(evt, x, B, rng)
     t2 = time.time()
     h = evt.Handle(N, F, B, K, D, loss, cfg["tree_type"])
     h.binarize(x, edges)

@@ -13,6 +13,9 @@ Julia is not available where this package is developed, so the host side is Pyth
 streams are numpy's (PCG64), not Julia's Xoshiro, hence models are not stream-identical to a
 Julia run with the same seed — the trees are identical for identical masks/column samples.
 """
+import os
+from concurrent.futures import ThreadPoolExecutor
+
 import numpy as np
 
 from . import _lib
@@ -144,19 +147,30 @@ class EvoTree:
         return predict(self, data, ntree_limit=ntree_limit, device=device)
 
 
+def _per_feature(fn, F):
+    """[fn(0), ..., fn(F - 1)], on a few threads when there are enough features (numpy's sorts release the GIL)."""
+    workers = min(16, os.cpu_count() or 1, F)
+    if workers < 2 or F < 8:
+        return [fn(j) for j in range(F)]
+    with ThreadPoolExecutor(workers) as ex:
+        return list(ex.map(fn, range(F)))
+
+
 def get_edges(x, nbins, rng):
     """get_edges, src/fit-utils.jl:7-24: type-7 quantiles at (1..nbins-1)/nbins of <= 1000*nbins sampled rows."""
     N, F = x.shape
     nobs = min(N, 1000 * nbins)
     idx = np.sort(rng.choice(N, nobs, replace=False)) if nobs < N else np.arange(N)
     q = np.arange(1, nbins) / nbins
-    edges = []
-    for j in range(F):
+
+    def one(j):
         col = np.asarray(x[idx, j], np.float64)
         e = np.quantile(col, q)  # numpy's default is the linear (type 7) rule Statistics.quantile uses
         if e.shape[0] == 1:
             e = np.array([col.min()])
-        edges.append(np.ascontiguousarray(e))
+        return np.ascontiguousarray(e)
+
+    edges = _per_feature(one, F)  # `@threads for j`, src/fit-utils.jl:15: the features are independent
     featbins = np.array([len(e) + 1 for e in edges], np.uint8)
     feattypes = np.ones(F, np.uint8)
     return edges, featbins, feattypes
