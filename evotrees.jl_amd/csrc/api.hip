@@ -271,6 +271,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->hist_min_rows = 1024;
     c->hist_variant = 0;
     c->scan_fused = 1;
+    c->hist_in_scatter = 1;
     c->hist_seg_cost = 2048;
     c->record_nidx = false;
     c->nidx_valid = false;
@@ -823,6 +824,7 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
     c->step.all_rows = all_rows;
     c->step.defer = defer;
     c->step.fuse_pred = fuse_pred;
+    c->step.hist_fused = !staged && scatter_can_build_hist(c, c->n_js_last);
     c->step.p = *p;
     // the root's list is the identity (kept, never written) or what the mask compaction left in is_a; the levels below
     // alternate between is_a and is_b
@@ -839,6 +841,10 @@ static inline int tree_last_split(const evt_ctx *c) { return (c->D > 1) ? c->D -
 // update_hist! for the build nodes of the level (src/fit-utils.jl:345-360)
 static int tree_stage_hist(evt_ctx *c) {
     const int level = c->step.level;
+    if (level > 1 && c->step.hist_fused) { // built by the scatter pass of the level above
+        c->step.phase = 2;
+        return EVT_OK;
+    }
     prof_begin_launch(c, EVT_K_HIST, level);
     int r = launch_hist_build(c, level, c->step.is_cur);
     c->launch_e0 = c->launch_e1 = nullptr;
@@ -1631,6 +1637,8 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
         c->record_nidx = value != 0;
     } else if (strcmp(name, "scan_fused") == 0) {
         c->scan_fused = value != 0;
+    } else if (strcmp(name, "hist_in_scatter") == 0) {
+        c->hist_in_scatter = value != 0;
     } else if (strcmp(name, "defer_pred") == 0) {
         c->defer_pred = value != 0;
     } else if (strcmp(name, "hist_threads") == 0) {

@@ -165,8 +165,9 @@ struct evt_ctx {
 
     // tunables
     int hist_blocks, hist_threads, hist_min_rows, hist_seg_cost;
-    int hist_variant;
-    int scan_fused;    // option: the split search of a node with at most 16 sampled features runs in one kernel  // 0 auto, 1 generic 16-byte-piece kernel, 2 conflict-free 8-byte-piece kernel where it applies
+    int hist_variant;  // 0 auto, 1 generic 16-byte-piece kernel, 2 conflict-free 8-byte-piece kernel where it applies
+    int scan_fused;    // option: the split search of a node with at most 16 sampled features runs in one kernel
+    int hist_in_scatter; // option: with 16-byte records and few chunks the partition's scatter pass builds the next level's histograms
     bool record_nidx;  // leaf finalisation also writes the node id of every sampled row
     bool nidx_valid;   // nidx holds the last tree's node ids
     bool defer_pred;   // a tree grown on every row records leaf ids and leaves the addition to the next row-order pass
@@ -180,6 +181,7 @@ struct evt_ctx {
         int phase; // 0 no tree open, 1 histogram next, 2 split search next, 3 partition next, 4 levels done
         int level;
         bool all_rows, defer, fuse_pred;
+        bool hist_fused; // levels below the root get their histograms from the scatter pass of the level above
         uint32_t *is_cur, *is_next; // row-id lists of the current level and of the one below
         evt_params p;
     } step;
@@ -251,6 +253,35 @@ void evt_set_error(const char *fmt, ...);
 __host__ __device__ __forceinline__ uint32_t evt_pack_node(int feat, int cond_bin, bool numeric) {
     return (uint32_t)feat | ((uint32_t)cond_bin << 16) | EVT_NODE_SPLIT | (numeric ? EVT_NODE_NUMERIC : 0u);
 }
+// The fixed-point word of channel a for one row.  The channel that shares its word with the row count holds 30 bits:
+// it is staged as a 32-bit word (half the plane to gather from) and widened here to (q << 16) + 1.
+template <bool PACK>
+__device__ __forceinline__ unsigned long long evt_load_gq(const unsigned long long *__restrict__ gq, int64_t N, int a, uint32_t id) {
+    if (PACK && a == 0) {
+        const long long q = (long long)reinterpret_cast<const int32_t *>(gq)[id];
+        return ((unsigned long long)q << EVT_PACK_CNT_BITS) + 1ull;
+    }
+    return gq[(size_t)a * N + id];
+}
+
+// Chunk descriptors of a level, for the partition kernels that run after the split search: chunk c of the level is
+// chunk c - c0 of node n, whose segment ends at `end`: {n, first position, end, c0}.  One wavefront per active node
+// writes the descriptors of that node's chunks, cprefix[i] .. cprefix[i + 1] (two dependent trips to memory, then
+// stores); `w` of `nw` wavefronts share the level's nodes.
+__device__ __forceinline__ void evt_fill_chunk_descriptors(const int64_t *__restrict__ hdr, const int32_t *__restrict__ act_node,
+                                                           const int64_t *__restrict__ cprefix, const int64_t *__restrict__ seg_start,
+                                                           const int64_t *__restrict__ seg_len, uint4 *cdesc, int w, int nw) {
+    const int lane = threadIdx.x & 63;
+    const int n_act = (int)hdr[LH_N_ACT];
+    for (int i = w; i < n_act; i += nw) {
+        const int n = act_node[i];
+        const int64_t c0 = cprefix[i], c1 = cprefix[i + 1];
+        const int64_t seg = seg_start[n], len = seg_len[n];
+        for (int64_t c = c0 + lane; c < c1; c += 64)
+            cdesc[c] = make_uint4((uint32_t)n, (uint32_t)(seg + (c - c0) * EVT_CHUNK), (uint32_t)(seg + len), (uint32_t)c0);
+    }
+}
+
 __device__ __forceinline__ void evt_add_leaf(float *pr, const float *lp, int K, int loss) {
     if (loss == EVT_LOSS_LOGLOSS) {
         for (int k = 0; k < K; k++) pr[k] = fminf(fmaxf(pr[k] + lp[k], -15.0f), 15.0f);
@@ -300,6 +331,7 @@ bool scan_folds_leaves(const evt_ctx *c);
 int launch_obliv_select(evt_ctx *c, int level, const evt_params *p);
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred);
+bool scatter_can_build_hist(const evt_ctx *c, int nfs);
 int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred);
 int launch_nidx_from_segments(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_copy_to_host(evt_ctx *c, const void *src_dev, void *dst_host_dev, size_t nbytes);

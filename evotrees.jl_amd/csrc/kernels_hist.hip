@@ -64,32 +64,13 @@ __device__ __forceinline__ int first_node_of_span(const int64_t *__restrict__ bp
     return cnt - 1;
 }
 
-// The fixed-point word of channel a for one row.  The channel that shares its word with the row count holds 30 bits:
-// it is staged as a 32-bit word (half the plane to gather from) and widened here to (q << 16) + 1.
-template <bool PACK>
-__device__ __forceinline__ unsigned long long load_gq(const unsigned long long *__restrict__ gq, int64_t N, int a, uint32_t id) {
-    if (PACK && a == 0) {
-        const long long q = (long long)reinterpret_cast<const int32_t *>(gq)[id];
-        return ((unsigned long long)q << EVT_PACK_CNT_BITS) + 1ull;
-    }
-    return gq[(size_t)a * N + id];
-}
-
-// Chunk descriptors of the level, for the partition kernels that run after the split search: chunk c of the level is
-// chunk c - c0 of node n, whose segment ends at `end`: {n, first position, end, c0}.  One wavefront per active node
-// writes the descriptors of that node's chunks, cprefix[i] .. cprefix[i + 1] (two dependent trips to memory, then
-// stores); the work hides behind the histogram kernel's own set-up.
+// Chunk descriptors of the level (evt_fill_chunk_descriptors): they ride along with the first launch of a level, spread
+// over the wavefronts of its first block column; the work hides behind the histogram kernel's own set-up.
 __device__ __forceinline__ void fill_chunk_descriptors(const HistArgs &A) {
     if (blockIdx.y != 0 || A.a0 != 0) return;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-    const int n_act = (int)A.hdr[LH_N_ACT];
-    for (int i = (int)blockIdx.x * nwaves + wave; i < n_act; i += (int)gridDim.x * nwaves) {
-        const int n = A.act_node[i];
-        const int64_t c0 = A.cprefix[i], c1 = A.cprefix[i + 1];
-        const int64_t seg = A.seg_start[n], len = A.seg_len[n];
-        for (int64_t c = c0 + lane; c < c1; c += 64)
-            A.cdesc[c] = make_uint4((uint32_t)n, (uint32_t)(seg + (c - c0) * EVT_CHUNK), (uint32_t)(seg + len), (uint32_t)c0);
-    }
+    const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    evt_fill_chunk_descriptors(A.hdr, A.act_node, A.cprefix, A.seg_start, A.seg_len, A.cdesc, (int)blockIdx.x * nwaves + wave,
+                               (int)gridDim.x * nwaves);
 }
 
 template <int NA, bool PACK>
@@ -177,7 +158,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
                 if (rc[u] != INV) {
                     vc[u] = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)rc[u] * A.RS + sub * 16);
 #pragma unroll
-                    for (int a = 0; a < NA; a++) gc[u][a] = load_gq<PACK>(A.gq, A.N, a, rc[u]);
+                    for (int a = 0; a < NA; a++) gc[u][a] = evt_load_gq<PACK>(A.gq, A.N, a, rc[u]);
                 }
             }
 #pragma unroll
@@ -192,7 +173,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
                     if (rn[u] != INV) {
                         vn[u] = *reinterpret_cast<const uint4 *>(A.xrm + (size_t)rn[u] * A.RS + sub * 16);
 #pragma unroll
-                        for (int a = 0; a < NA; a++) gn[u][a] = load_gq<PACK>(A.gq, A.N, a, rn[u]);
+                        for (int a = 0; a < NA; a++) gn[u][a] = evt_load_gq<PACK>(A.gq, A.N, a, rn[u]);
                     }
                 }
                 uint32_t rnn[U];
@@ -419,7 +400,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                 idc = load_id<NT>(isp + ((fetcher && p < nend) ? p : lastp));
             }
 #pragma unroll
-            for (int a = 0; a < NA; a++) gc[a] = load_gq<PACK>(A.gq, A.N, a, idc);
+            for (int a = 0; a < NA; a++) gc[a] = evt_load_gq<PACK>(A.gq, A.N, a, idc);
             {
                 const int64_t p = pw + itstride + mypos;
                 idn = load_id<NT>(isp + ((fetcher && p < nend) ? p : lastp));
@@ -437,7 +418,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             for (; pw < nend; pw += itstride) {
                 // next iteration's gradient words and the row ids of the one after: ahead of the records in issue order
 #pragma unroll
-                for (int a = 0; a < NA; a++) gn[a] = load_gq<PACK>(A.gq, A.N, a, idn);
+                for (int a = 0; a < NA; a++) gn[a] = evt_load_gq<PACK>(A.gq, A.N, a, idn);
                 uint32_t idnn;
                 {
                     const int64_t p = pw + 2 * itstride + mypos;

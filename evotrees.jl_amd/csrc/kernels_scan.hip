@@ -33,6 +33,13 @@ struct ScanArgs {
     int bagging;
     int nfs, B, F, K, NK, NAg, loss, level, leaf_level, oblivious, zero_children;
     int fold_leaves; // the level's children are leaves: their weight and values are written along with the split (no pass of their own)
+    // the level's chunk descriptors, written here when no histogram kernel runs at this level (cdesc == nullptr: not here)
+    const int64_t *hdr;
+    const int32_t *act_node;
+    const int64_t *cprefix;
+    const int64_t *seg_start;
+    const int64_t *seg_len;
+    uint4 *cdesc;
 };
 
 // ---- wavefront primitives -----------------------------------------------------------------
@@ -236,6 +243,13 @@ template <int NAG, int BPL, bool FUSED>
 __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const int n = (1 << (A.level - 1)) + blockIdx.x; // 1-based node id
+    if constexpr (FUSED) {
+        // the partition's chunk descriptors of this level, when the level's histograms came from the scatter pass above
+        // and no histogram kernel wrote them: the highest wavefronts take them (idle unless 16 features are sampled)
+        if (A.cdesc)
+            evt_fill_chunk_descriptors(A.hdr, A.act_node, A.cprefix, A.seg_start, A.seg_len, A.cdesc,
+                                       (int)blockIdx.x * nwaves + (nwaves - 1 - wave), (int)gridDim.x * nwaves);
+    }
     // The block's time is a chain of round trips to memory, so requests go out in as few dependent steps as the data
     // allows: node state and feature id first; then, in one batch of unconditional loads, the histogram slices, the
     // feature's type and constraint, the node totals and the decode scales.
@@ -932,6 +946,16 @@ int launch_scan(evt_ctx *c, int level, const evt_params *p, bool leaf_level) {
     A.oblivious = (c->tree_type == EVT_TREE_OBLIVIOUS) ? 1 : 0;
     A.zero_children = (level + 1 < c->D) ? 1 : 0; // children at the last level never get a histogram
     A.fold_leaves = (!leaf_level && scan_folds_leaves(c) && level + 1 == c->D) ? 1 : 0;
+    A.cdesc = nullptr;
+    if (c->step.hist_fused && level > 1 && !leaf_level) {
+        const LevelTab &L = c->lvl[level & 1];
+        A.hdr = L.hdr;
+        A.act_node = L.act_node;
+        A.cprefix = L.cprefix;
+        A.seg_start = c->seg_start;
+        A.seg_len = c->seg_len;
+        A.cdesc = L.cdesc;
+    }
     const unsigned nodes = 1u << (level - 1);
     const int ngroups = (A.nfs + 3) / 4; // 4 waves per block, one sampled feature each
     dim3 grid(nodes, (unsigned)ngroups);

@@ -338,7 +338,11 @@ int evt_reset_profile(evt_handle h);
  * 0: they are added while the tree's last level is partitioned; results do not depend on it); "grads_ahead"
  * (1: a tree grown with update_pred queues the next evt_update_grads behind itself, so the device computes it
  * while the host collects the tree, and that next call returns at once; meant for bagging_size 1 - with more
- * trees per round only the last one's work is used; 0, default; results do not depend on it). */
+ * trees per round only the last one's work is used; 0, default; results do not depend on it); "scan_fused"
+ * (1, default: with at most 16 sampled features one kernel searches and finishes a node's split, 0: two kernels)
+ * and "hist_in_scatter" (1, default: with at most 16 features and a quarter of a million rows the levels below
+ * the root get their histograms from the partition's scatter pass, one kernel less per level; 0: a histogram
+ * kernel per level) - same trees and histograms, bit for bit, either way. */
 int evt_set_option(evt_handle h, const char *name, int64_t value);
 /* Blocks until all work queued on the handle's stream is done. */
 int evt_synchronize(evt_handle h);

@@ -334,6 +334,39 @@ def test_gradients_queued_ahead_change_nothing(evt, loss, tt):
             assert_tree_bits(a, b)
 
 
+@pytest.mark.parametrize("loss,weights,rowsample", [("mse", False, 1.0), ("mse", True, 0.6), ("gaussian_mle", False, 1.0)])
+def test_histograms_built_by_the_scatter_pass_change_nothing(evt, loss, weights, rowsample):
+    """With 16-byte records and few chunks the levels below the root get their histograms from the partition's scatter
+    pass ("hist_in_scatter", on by default) instead of a histogram kernel per level: trees, histograms, node ids and
+    predictions are bit-identical either way over free-running rounds."""
+    N, F, B, D, R = 100000, 10, 64, 6, 5
+    x_bin, y, w, mu = make_data(91, N, F, B, loss, weights)
+    js = np.array([1, 2, 4, 5, 6, 8, 9, 10], np.uint32)
+    gp = evt.make_params(eta=0.4, min_weight=8.0 if loss == "gaussian_mle" else 1.0)
+    rng = np.random.default_rng(17)
+    masks = [None if rowsample >= 1 else rng.integers(0, 256, N, dtype=np.uint8) for _ in range(R)]
+    out = []
+    for on in (1, 0):
+        h = evt.Handle(N, F, B, mu.shape[0], D, loss)
+        h.set_option("hist_in_scatter", on)
+        h.set_option("record_nidx", 1)
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        rec = []
+        for r in range(R):
+            h.update_grads()
+            rec.append(h.grow_tree(js if r % 2 else np.arange(1, F + 1, dtype=np.uint32), gp, mask=masks[r], cond=int(np.rint(255 * rowsample))))
+            rec += [h.get_hist(), h.get_nidx()]
+        rec.append(h.get_pred())
+        h.close()
+        out.append(rec)
+    for a, b in zip(*out):
+        if isinstance(a, np.ndarray):
+            assert a.tobytes() == b.tobytes()
+        else:
+            assert_tree_bits(a, b)
+
+
 @pytest.mark.parametrize("bagging", [1, 2])
 def test_gradients_queued_ahead_with_bagging_and_read_back(evt, bagging):
     """A round of bagging_size trees is grown on ONE set of gradients (src/fit.jl:9-11): "grads_ahead" must not refresh

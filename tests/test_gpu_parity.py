@@ -160,6 +160,10 @@ CASES = [
     ("multiquantile", False, 20000, 20, 64, 4, "oblivious", 20, 1.0, dict(alphas=[0.25, 0.75], L2=0.0)),
     ("mse", False, 60000, 5, 8, 14, "binary", 5, 1.0, dict(min_weight=0.0)),   # deep: most leaves hold a handful of rows
     ("logloss", True, 3000, 4, 4, 16, "binary", 4, 0.9, dict(min_weight=0.0)),  # deepest supported tree, far more nodes than rows
+    # 16-byte records and few chunks: the levels below the root get their histograms from the partition's scatter pass
+    ("logloss", True, 50000, 13, 64, 7, "binary", 13, 1.0, {}),                          # three channels, weights
+    ("gaussian_mle", False, 30000, 16, 64, 5, "binary", 16, 1.0, dict(min_weight=8.0)),  # four channels, all 16 features sampled
+    ("gaussian_mle", True, 30000, 9, 32, 6, "binary", 7, 0.8, dict(min_weight=8.0)),     # five channels, row and column samples
 ]
 
 
