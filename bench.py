@@ -157,7 +157,9 @@ class Rounds:
         self.mask_rng = np.random.Generator(np.random.SFC64(124))
         self.staged = False
         self.nxt = None
-        self.nxt_draws = None
+        self.in_flight = 0
+        self.sampled = 0
+        self.prof_on = False
         h.set_option("grads_ahead", 1)  # one tree per round: the next round's gradients are queued behind the tree
 
     def draw_mask(self):
@@ -170,27 +172,42 @@ class Rounds:
         js = np.arange(1, F + 1, dtype=np.uint32) if self.nfs >= F else (np.sort(self.rng.choice(F, self.nfs, replace=False)) + 1).astype(np.uint32)
         return seed, js
 
-    def one_round(self):
+    def begin(self):
+        """Queues one round on the device: the gradient update, the round's draws, the tree."""
         evt, h, L = self.evt, self.h, self.L
         h.update_grads()
-        seed, js = self.nxt_draws if self.nxt_draws is not None else self.draws()
+        seed, js = self.draws()
         if seed is not None:
             h.draw_mask(seed)
             evt._lib.check(L.evt_grow_tree_begin_staged(h._h, self.cond, evt._lib.ptr(js), js.shape[0], self.params))
         elif self.staged:
+            self.staged = False
             evt._lib.check(L.evt_grow_tree_begin_staged(h._h, self.cond, evt._lib.ptr(js), js.shape[0], self.params))
         else:
             mask = self.nxt if self.nxt is not None else self.draw_mask()
+            self.nxt = None
             evt._lib.check(L.evt_grow_tree_begin(h._h, evt._lib.ptr(mask), self.cond, evt._lib.ptr(js), js.shape[0], self.params))
-        # the host's work for the next round while the device grows this round's tree
-        self.nxt_draws = self.draws()
+        self.in_flight += 1
+        self.sampled += 1 if self.prof_on else 0
+
+    def one_round(self, more=False):
+        """One round as grow_evotree drives it.  more=True: another round follows, and its tree is queued before this
+        round's is collected (the library takes two trees in flight), so the device does not idle while the host copies
+        the tree out and prepares the next call.  A host-drawn mask is drawn (and, for many rows, uploaded) while the
+        device grows this round's tree, so the next round is queued after this one has been collected."""
+        h = self.h
+        if self.in_flight == 0:
+            self.begin()
         if self.cond < 255 and self.host_mask:
-            # one byte per row, drawn and (for many rows) uploaded
-            self.nxt = self.draw_mask()
-            if self.N >= self.STAGE_MASK_MIN_ROWS:
-                h.stage_mask(self.nxt)
-                self.staged = True
-        evt._lib.check(L.evt_grow_tree_end(h._h, self.tree_out))
+            if more:
+                self.nxt = self.draw_mask()  # one byte per row
+                if self.N >= self.STAGE_MASK_MIN_ROWS:
+                    h.stage_mask(self.nxt)
+                    self.staged = True
+        elif more:
+            self.begin()
+        self.evt._lib.check(self.L.evt_grow_tree_end(h._h, self.tree_out))
+        self.in_flight -= 1
 
     def timed(self, steps, warmup, profile_every=4, no_profile=False):
         """`warmup` untimed rounds, then `steps` timed ones.  HIP events around the histogram launches only (the kernel
@@ -198,25 +215,28 @@ class Rounds:
         either side of the kernel it times (measured with rocprofv3 --kernel-trace), 90 us per round if every launch
         carried a pair.  Returns (ms per round, histogram profile, rounds sampled)."""
         h = self.h
-        for _ in range(warmup):
-            self.one_round()
+        for i in range(warmup):
+            self.one_round(more=i + 1 < warmup)
         h.synchronize()
         pe = max(1, profile_every)
         h.set_profiling(False)
         h.reset_profile()
-        sampled = 0
+        self.sampled = 0  # trees queued with the events switched on
         t1 = time.perf_counter()
+        # the switch applies to the trees queued after it: with the device one tree ahead that is the NEXT round's tree
+        # (and, in the first round, this round's as well)
         for step in range(steps):
             on = (not no_profile) and step % pe == 0
             if on:
                 h.set_profiling(["hist"])
-                sampled += 1
-            self.one_round()
+            self.prof_on = on
+            self.one_round(more=step + 1 < steps)
             if on:
                 h.set_profiling(False)
+            self.prof_on = False
         h.synchronize()
         t2 = time.perf_counter()
-        return (t2 - t1) * 1e3 / steps, h.get_profile()["hist"], sampled
+        return (t2 - t1) * 1e3 / steps, h.get_profile()["hist"], self.sampled
 
 
 def hist_roofline(cfg, prof_hist, nfs, NK):

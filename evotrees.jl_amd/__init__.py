@@ -376,7 +376,7 @@ class Cache:
 
     def __init__(self, handle, rng, nfs, params, N, F, config=None):
         self.handle, self.rng, self.nfs, self.params, self.N, self.F, self.config = handle, rng, nfs, params, N, F, config
-        self.next_draw = None  # (mask seed, column sample) of the next tree, drawn while the device grew the last one
+        self.pending = []  # trees queued on the device and not yet collected, oldest first (at most two)
 
 
 def init(config, x_train, y_train=None, w_train=None, offset_train=None, feature_names=None, device=None, target_name=None, weight_name=None,
@@ -438,40 +438,52 @@ def init(config, x_train, y_train=None, w_train=None, offset_train=None, feature
     return m, Cache(h, rng, nfs, params, N, F, config)
 
 
-def grow_evotree(m, cache, config):
+def _begin_tree(cache, config, first_of_round):
+    """Queues one tree on the device (the round's gradient update first): the generator's draws of the tree in the
+    reference's order (mask, then columns; src/fit.jl:13-20), then evt_grow_tree_begin.  All rows pass `mask <= 255`, so
+    nothing is drawn for the mask when nothing can be dropped."""
+    h = cache.handle
+    if first_of_round:
+        h.update_grads()
+    cond = int(np.rint(255 * config.rowsample))  # round(UInt8, 255*rowsample), src/subsample.jl:9
+    seed = int(cache.rng.integers(0, 1 << 64, dtype=np.uint64)) if cond < 255 else None
+    if cache.nfs >= cache.F:
+        js = np.arange(1, cache.F + 1, dtype=np.uint32)
+    else:
+        js = (np.sort(cache.rng.choice(cache.F, cache.nfs, replace=False)) + 1).astype(np.uint32)
+    if seed is not None:
+        h.draw_mask(seed)
+        _lib.check(_lib.load().evt_grow_tree_begin_staged(h._h, cond, _lib.ptr(js), js.shape[0], cache.params))
+    else:
+        _lib.check(_lib.load().evt_grow_tree_begin(h._h, None, cond, _lib.ptr(js), js.shape[0], cache.params))
+    cache.pending.append(Tree(h.K, h.nnodes))
+
+
+def grow_evotree(m, cache, config, more=False):
     """grow_evotree!, src/fit.jl:6-42 (device twin ext/.../fit.jl:1-21): gradients, then bagging_size trees.
 
     The row mask of a tree (rand!(rng, mask), src/subsample.jl:7) is drawn on the device from ONE 64-bit draw of the
     fit's generator per tree (Handle.draw_mask: SplitMix64 keyed by that draw; splitmix_mask gives the same bytes on the
     host): numpy needs 4 ns per 8 mask bytes, which at a million rows is already longer than the device takes to grow
-    the tree.  The bytes are compared with round(UInt8, 255 * rowsample) exactly as an uploaded mask is."""
+    the tree.  The bytes are compared with round(UInt8, 255 * rowsample) exactly as an uploaded mask is.
+
+    The device runs one tree ahead of the host: a tree is queued before the one before it is collected (the library
+    takes two trees in flight), so the device does not wait while the host copies a tree out and prepares the next
+    call.  Within a round that is always possible; `more=True` says that another round follows and that nothing is read
+    from the handle before it, so the next round's first tree is queued as well before this round's last is collected
+    (the next call finds it in cache.pending).  Draws, trees and predictions are those of strictly alternating calls."""
     h = cache.handle
-    h.update_grads()
-    cond = int(np.rint(255 * config.rowsample))  # round(UInt8, 255*rowsample), src/subsample.jl:9
-
-    def draw():
-        # the generator's draws of one tree, in the reference's order (mask, then columns; src/fit.jl:13-20).  All rows
-        # pass `mask <= 255`, so nothing is drawn for the mask when nothing can be dropped
-        seed = int(cache.rng.integers(0, 1 << 64, dtype=np.uint64)) if cond < 255 else None
-        if cache.nfs >= cache.F:
-            js = np.arange(1, cache.F + 1, dtype=np.uint32)
-        else:
-            js = (np.sort(cache.rng.choice(cache.F, cache.nfs, replace=False)) + 1).astype(np.uint32)
-        return seed, js
-
-    for _ in range(config.bagging_size):
-        seed, js = cache.next_draw if cache.next_draw is not None else draw()
-        cache.next_draw = None
-        t = Tree(m.K, h.nnodes)
-        out = t.as_out()
+    n = config.bagging_size
+    for b in range(n):
+        if not cache.pending:
+            _begin_tree(cache, config, b == 0)
+        if b + 1 < n:
+            _begin_tree(cache, config, False)
+        elif more:
+            _begin_tree(cache, config, True)
+        t = cache.pending.pop(0)
         try:
-            if seed is not None:
-                h.draw_mask(seed)
-                _lib.check(_lib.load().evt_grow_tree_begin_staged(h._h, cond, _lib.ptr(js), js.shape[0], cache.params))
-            else:
-                _lib.check(_lib.load().evt_grow_tree_begin(h._h, None, cond, _lib.ptr(js), js.shape[0], cache.params))
-            cache.next_draw = draw()  # the next tree's draws, made while the device grows this one
-            _lib.check(_lib.load().evt_grow_tree_end(h._h, out))
+            _lib.check(_lib.load().evt_grow_tree_end(h._h, t.as_out()))
         except EvtError as e:
             if e.code == _lib.EVT_ERR_EMPTY:
                 raise RuntimeError("no subsample observation - choose larger rowsample") from e
@@ -595,7 +607,8 @@ def fit(config, dtrain=None, x_train=None, y_train=None, w_train=None, offset_tr
             import warnings
             warnings.warn("To track eval metric in logger, both `x_eval` and `y_eval` must be provided.")
         for i in range(1, config.nrounds + 1):
-            grow_evotree(m, cache, config)
+            # without an eval set nothing is read between two rounds: the device may start the next one early
+            grow_evotree(m, cache, config, more=(logger is None and i < config.nrounds))
             if logger is not None:
                 cb(logger, i, m.trees[-1])  # as the reference: only the round's last tree reaches the eval prediction
                 if i % print_every_n == 0 and verbosity > 0:
@@ -624,7 +637,7 @@ def update(config, m, cache, x_train=None, y_train=None, w_train=None):
     any change other than a larger nrounds refits from scratch."""
     if okay_to_continue(config, m, cache):
         while m.info["nrounds"] < config.nrounds:
-            grow_evotree(m, cache, config)
+            grow_evotree(m, cache, config, more=m.info["nrounds"] + 1 < config.nrounds)
         cache.config = config
         return m, cache
     cache.handle.close()

@@ -227,8 +227,9 @@ class Handle:
         return t
 
     def grow_tree_begin(self, js, params, mask=None, cond=255):
-        """Queues one tree and returns while the device grows it; grow_tree_end collects it.  Nothing else may be
-        called on the handle in between (the host is free to prepare the next round, e.g. draw the next row mask)."""
+        """Queues one tree and returns while the device grows it; grow_tree_end collects it (the older one when two
+        are in flight).  While ONE tree is in flight the next round may be queued behind it (update_grads, draw_mask /
+        stage_mask, grow_tree_begin[_staged]); calls that read or rewrite the handle's state wait for grow_tree_end."""
         js = np.ascontiguousarray(js, np.uint32)
         if mask is not None:
             mask = np.ascontiguousarray(mask, np.uint8)

@@ -69,6 +69,7 @@ void prof_begin(evt_ctx *c, int cls, int level) {
     ProfRec r;
     r.cls = cls;
     r.level = level;
+    r.seq = c->tree_seq;
     auto get = [&]() {
         hipEvent_t e;
         if (!c->free_events.empty()) {
@@ -94,6 +95,7 @@ void prof_begin_launch(evt_ctx *c, int cls, int level) {
     ProfRec r;
     r.cls = cls;
     r.level = level;
+    r.seq = c->tree_seq;
     for (hipEvent_t *e : {&r.e0, &r.e1}) {
         if (!c->free_events.empty()) {
             *e = c->free_events.back();
@@ -111,10 +113,16 @@ void prof_end(evt_ctx *c) {
     c->prof_open = false;
     (void)hipEventRecord(c->recs.back().e1, c->stream);
 }
-// after a stream sync: fold finished event pairs into the per-class totals
-static void prof_collect(evt_ctx *c, const int64_t *stats_host) {
+// after a stream sync or the arrival of tree `upto_seq`: fold finished event pairs into the per-class totals.  stats_host:
+// the rows built per level of that tree, the units of its histogram launches; pairs of a tree queued behind it wait for
+// their own tree's counts.
+static void prof_collect(evt_ctx *c, const int64_t *stats_host, int64_t upto_seq = INT64_MAX) {
     std::vector<ProfRec> later; // pairs whose kernels are still queued (work placed behind the point the host waited for)
     for (auto &r : c->recs) {
+        if (r.seq > upto_seq) {
+            later.push_back(r);
+            continue;
+        }
         float ms = 0.0f;
         const hipError_t e = hipEventElapsedTime(&ms, r.e0, r.e1);
         if (e == hipErrorNotReady) {
@@ -185,13 +193,14 @@ extern "C" int evt_destroy(evt_handle c) {
         for (void *p : lp)
             if (p) (void)hipFree(p);
     }
-    if (c->h_stage) (void)hipHostFree(c->h_stage);
+    if (c->h_stage_base) (void)hipHostFree(c->h_stage_base);
     for (auto &r : c->recs) {
         (void)hipEventDestroy(r.e0);
         (void)hipEventDestroy(r.e1);
     }
     for (auto e : c->free_events) (void)hipEventDestroy(e);
-    if (c->tree_ev) (void)hipEventDestroy(c->tree_ev);
+    for (hipEvent_t e : c->tree_evs)
+        if (e) (void)hipEventDestroy(e);
     if (c->pt_stage) (void)hipHostFree(c->pt_stage);
     if (c->copy_stream) {
         (void)hipStreamSynchronize(c->copy_stream);
@@ -261,7 +270,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     for (int k = 0; k < EVT_MAX_K; k++) c->h_alphas[k] = 0.5;
     c->qscale = nullptr; c->qexp_buf[0] = c->qexp_buf[1] = nullptr; c->qscale_buf[0] = c->qscale_buf[1] = nullptr; c->q_cur = c->q_tree = 0;
     c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->sbest = nullptr;
-    c->h_stage = nullptr; c->h_stage_dev = nullptr; c->h_stage_bytes = 0;
+    c->h_stage = nullptr; c->h_stage_dev = nullptr; c->h_stage_bytes = 0; c->h_stage_base = nullptr; c->h_stage_dev_base = nullptr;
     c->n_js_last = 0;
     c->last_all_rows = true;
     // one block of 16 waves per CU: as many waves as two blocks of 8 (the LDS histogram caps a CU at 128 KB), half
@@ -279,10 +288,13 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->write_nidx = false;
     c->pend_pred = false;
     c->is_id = nullptr;
-    c->tree_in_flight = false;
+    c->tree_in_flight = 0;
+    c->slot_w = c->slot_r = 0;
+    c->tree_seq = 0;
+    c->slot_seq[0] = c->slot_seq[1] = 0;
     c->step.phase = 0;
     c->pt_nodes = nullptr; c->pt_pred = nullptr; c->pt_stage = nullptr; c->pt_stage_dev = nullptr; c->pt_cap = 0; c->pt_busy = false;
-    c->tree_ev = nullptr;
+    c->tree_evs[0] = c->tree_evs[1] = nullptr;
     c->mask_next = nullptr;
     c->copy_stream = nullptr;
     c->mask_next_valid = false;
@@ -302,7 +314,8 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     }
     hipError_t e = hipGetDevice(&c->device);
     if (e == hipSuccess) e = hipStreamCreate(&c->stream);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->tree_ev, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->tree_evs[0], hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->tree_evs[1], hipEventDisableTiming);
     if (e != hipSuccess) {
         evt_set_error("stream creation failed: %s", hipGetErrorString(e));
         if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -386,16 +399,19 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     }
     // pinned staging: tree read-back + small per-tree uploads
     c->h_stage_bytes = c->blob_bytes + (size_t)c->F * 4 + (size_t)c->RS * 2 + 1024;
-    if (hipHostMalloc((void **)&c->h_stage, c->h_stage_bytes, hipHostMallocDefault) != hipSuccess) {
+    c->h_stage_bytes = (c->h_stage_bytes + 255) / 256 * 256;
+    if (hipHostMalloc((void **)&c->h_stage_base, 2 * c->h_stage_bytes, hipHostMallocDefault) != hipSuccess) {
         evt_set_error("hipHostMalloc failed");
         evt_destroy(c);
         return EVT_ERR_NOMEM;
     }
-    if (hipHostGetDevicePointer((void **)&c->h_stage_dev, c->h_stage, 0) != hipSuccess) {
+    if (hipHostGetDevicePointer((void **)&c->h_stage_dev_base, c->h_stage_base, 0) != hipSuccess) {
         evt_set_error("pinned staging buffer is not addressable from the device");
         evt_destroy(c);
         return EVT_ERR_HIP;
     }
+    c->h_stage = c->h_stage_base;
+    c->h_stage_dev = c->h_stage_dev_base;
     // defaults: all numeric, no monotone constraint
     {
         std::vector<uint8_t> ft(c->F, 1);
@@ -434,6 +450,21 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
         HIPCHK(hipSetDevice((c)->device));                                                             \
         if ((c)->tree_in_flight) {                                                                     \
             evt_set_error("a tree begun with evt_grow_tree_begin has not been collected (evt_grow_tree_end)"); \
+            return EVT_ERR_STATE;                                                                      \
+        }                                                                                              \
+        if ((c)->step.phase != 0) {                                                                    \
+            evt_set_error("a tree opened with evt_tree_open has not been closed (evt_tree_close)");    \
+            return EVT_ERR_STATE;                                                                      \
+        }                                                                                              \
+    } while (0)
+// calls that only queue work behind what is already queued (the next tree, the next gradient update, the next mask) are
+// also allowed while ONE tree waits to be collected: two trees may be in flight, evt_grow_tree_end collects the older
+#define CTXCHK_QUEUE(c)                                                                                \
+    do {                                                                                               \
+        ARGCHK((c) != nullptr, "handle is NULL");                                                      \
+        HIPCHK(hipSetDevice((c)->device));                                                             \
+        if ((c)->tree_in_flight > 1) {                                                                 \
+            evt_set_error("two trees begun with evt_grow_tree_begin have not been collected (evt_grow_tree_end)"); \
             return EVT_ERR_STATE;                                                                      \
         }                                                                                              \
         if ((c)->step.phase != 0) {                                                                    \
@@ -686,7 +717,7 @@ static int queue_grads(evt_ctx *c) {
 
 extern "C" int evt_update_grads(evt_handle c) {
     return guarded([&]() -> int {
-    CTXCHK(c);
+    CTXCHK_QUEUE(c);
     if (!c->have_target) {
         evt_set_error("evt_set_target must be called before evt_update_grads");
         return EVT_ERR_STATE;
@@ -740,6 +771,10 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
         evt_set_error("x_bin, target and gradients must be set before evt_grow_tree");
         return EVT_ERR_STATE;
     }
+    // the tree's staging slot: the one the tree collected last (or never used) held
+    c->h_stage = c->h_stage_base + (size_t)c->slot_w * c->h_stage_bytes;
+    c->h_stage_dev = c->h_stage_dev_base + (size_t)c->slot_w * c->h_stage_bytes;
+    c->tree_seq += 1;
     // js: 1-based, strictly ascending
     std::vector<uint32_t> jsv(n_js);
     {
@@ -931,7 +966,8 @@ static int tree_close(evt_ctx *c) {
     // the tree (and the per-level row counts) comes back in one pinned transfer, queued behind the kernels
     r = launch_copy_to_host(c, c->tree_blob, c->h_stage_dev, c->blob_bytes);
     if (r != EVT_OK) return r;
-    HIPCHK(hipEventRecord(c->tree_ev, c->stream));
+    HIPCHK(hipEventRecord(c->tree_evs[c->slot_w], c->stream));
+    c->slot_seq[c->slot_w] = c->tree_seq;
     if (c->grads_ahead && p->update_pred && p->bagging_size == 1) {
         // the next round's gradient update runs while the host collects this tree and prepares the next call.  Not with
         // bagging: the trees of one round are all grown on the same gradients (src/fit.jl:9-11), and the library cannot
@@ -940,7 +976,8 @@ static int tree_close(evt_ctx *c) {
         if (r != EVT_OK) return r;
         c->grads_ready = true;
     }
-    c->tree_in_flight = true;
+    c->tree_in_flight += 1;
+    c->slot_w ^= 1;
     return EVT_OK;
 }
 
@@ -963,7 +1000,7 @@ static int tree_run_stages(evt_ctx *c, int r) {
 
 extern "C" int evt_grow_tree_begin(evt_handle c, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
     return guarded([&]() -> int {
-    CTXCHK(c);
+    CTXCHK_QUEUE(c);
     int r = tree_open(c, mask, false, cond, js, n_js, p, false);
     return tree_run_stages(c, r);
     });
@@ -978,6 +1015,10 @@ extern "C" int evt_stage_mask(evt_handle c, const uint8_t *mask) {
     HIPCHK(hipSetDevice(c->device));
     if (c->step.phase != 0) {
         evt_set_error("a tree opened with evt_tree_open has not been closed (evt_tree_close)");
+        return EVT_ERR_STATE;
+    }
+    if (c->tree_in_flight > 1) { // the older tree may still be reading the buffer this copy would overwrite
+        evt_set_error("evt_stage_mask with two trees in flight: collect the older one first (evt_grow_tree_end)");
         return EVT_ERR_STATE;
     }
     if (!c->copy_stream) HIPCHK(hipStreamCreateWithFlags(&c->copy_stream, hipStreamNonBlocking));
@@ -997,12 +1038,7 @@ extern "C" int evt_stage_mask(evt_handle c, const uint8_t *mask) {
 // the handle's own stream into the buffer the tree in flight does not read.
 extern "C" int evt_draw_mask(evt_handle c, uint64_t seed) {
     return guarded([&]() -> int {
-    ARGCHK(c != nullptr, "handle is NULL");
-    HIPCHK(hipSetDevice(c->device));
-    if (c->step.phase != 0) {
-        evt_set_error("a tree opened with evt_tree_open has not been closed (evt_tree_close)");
-        return EVT_ERR_STATE;
-    }
+    CTXCHK_QUEUE(c);
     if (!c->mask_next) {
         int r = dev_alloc(&c->mask_next, (size_t)c->N);
         if (r != EVT_OK) return r;
@@ -1017,7 +1053,7 @@ extern "C" int evt_draw_mask(evt_handle c, uint64_t seed) {
 
 extern "C" int evt_grow_tree_begin_staged(evt_handle c, uint8_t cond, const uint32_t *js, int32_t n_js, const evt_params *p) {
     return guarded([&]() -> int {
-    CTXCHK(c);
+    CTXCHK_QUEUE(c);
     if (!c->mask_next_valid) {
         evt_set_error("evt_grow_tree_begin_staged: no mask has been staged since the last tree (evt_stage_mask / evt_draw_mask)");
         return EVT_ERR_STATE;
@@ -1092,10 +1128,9 @@ extern "C" int evt_tree_close(evt_handle c) {
 }
 
 // host copy of the device's tree arrays (in the pinned staging buffer) -> the caller's arrays
-static int fill_tree_out(evt_ctx *c, evt_tree_out *tree) {
+static int fill_tree_out(evt_ctx *c, const uint8_t *hs, evt_tree_out *tree) {
     ARGCHK(tree->feat && tree->cond_bin && tree->w && tree->gain && tree->pred && tree->split, "tree output arrays must not be NULL");
     const int nn = c->nnodes, K = c->K;
-    const uint8_t *hs = c->h_stage;
     const int32_t *f32 = reinterpret_cast<const int32_t *>(hs + c->blob_feat);
     for (int n = 0; n < nn; n++) tree->feat[n] = (int64_t)f32[n];
     memcpy(tree->w, hs + c->blob_w, (size_t)nn * 4);
@@ -1114,21 +1149,23 @@ extern "C" int evt_grow_tree_end(evt_handle c, evt_tree_out *tree) {
         evt_set_error("evt_grow_tree_end without evt_grow_tree_begin");
         return EVT_ERR_STATE;
     }
-    c->tree_in_flight = false;
-    uint8_t *hs = c->h_stage;
+    // the older of the trees in flight
+    const int slot = c->slot_r;
+    c->tree_in_flight -= 1;
+    c->slot_r ^= 1;
+    const uint8_t *hs = c->h_stage_base + (size_t)slot * c->h_stage_bytes;
     const size_t o_stats = c->blob_stats;
-    HIPCHK(hipEventSynchronize(c->tree_ev)); // the tree has arrived; work queued behind it may still be running
+    HIPCHK(hipEventSynchronize(c->tree_evs[slot])); // the tree has arrived; work queued behind it may still be running
     const int64_t n_is = reinterpret_cast<const int64_t *>(hs + o_stats)[0];
-    if (c->profiling) {
-        c->prof_units[EVT_K_PARTITION] += n_is;
-        prof_collect(c, reinterpret_cast<const int64_t *>(hs + o_stats));
-        c->prof_units[EVT_K_SCAN] += 0;
+    if (c->profiling || !c->recs.empty()) {
+        if (c->profiling) c->prof_units[EVT_K_PARTITION] += n_is;
+        prof_collect(c, reinterpret_cast<const int64_t *>(hs + o_stats), c->slot_seq[slot]);
     }
     if (n_is == 0) { // the tree grown on no rows is a single zero leaf; report it as the reference does
         evt_set_error("no subsample observation - choose larger rowsample");
         return EVT_ERR_EMPTY;
     }
-    if (tree) return fill_tree_out(c, tree);
+    if (tree) return fill_tree_out(c, hs, tree);
     return EVT_OK;
     });
 }
@@ -1141,7 +1178,7 @@ extern "C" int evt_peek_tree(evt_handle c, evt_tree_out *tree) {
     int r = launch_copy_to_host(c, c->tree_blob, c->h_stage_dev, c->blob_bytes);
     if (r != EVT_OK) return r;
     HIPCHK(hipStreamSynchronize(c->stream));
-    return fill_tree_out(c, tree);
+    return fill_tree_out(c, c->h_stage, tree);
     });
 }
 
@@ -1578,9 +1615,7 @@ extern "C" int evt_predict_leaf_idx(int64_t nobs, int32_t nfeats, const uint8_t 
 // ---- measurement ----------------------------------------------------------------------------
 extern "C" int evt_set_profiling(evt_handle c, int32_t on) {
     return guarded([&]() -> int {
-    CTXCHK(c);
-    HIPCHK(hipStreamSynchronize(c->stream));
-    prof_collect(c, nullptr);
+    CTXCHK_QUEUE(c); // applies to what is queued from here on; pairs already recorded are folded in when their work is done
     c->profiling = (on == 1) ? 0x7fffffff : on; // 1: every class; otherwise a bit mask of EVT_K_* classes
     return EVT_OK;
     });

@@ -63,6 +63,7 @@ struct TreeDev {
 struct ProfRec {
     int cls;
     int level;
+    int64_t seq; // tree the launch belongs to (evt_ctx::tree_seq when it was queued)
     hipEvent_t e0, e1;
 };
 
@@ -146,8 +147,10 @@ struct evt_ctx {
     double *ogains;    // oblivious: [maxlvl][F][B]
     void *sbest;       // split search: best candidate per (node of the level, feature group), 16 B each
 
-    // host staging (pinned)
+    // host staging (pinned): two slots of h_stage_bytes each, so that a second tree can be queued before the first one
+    // has been collected.  h_stage / h_stage_dev point at the slot of the tree queued last.
     uint8_t *h_stage;
+    uint8_t *h_stage_base, *h_stage_dev_base;
     // evt_predict_tree: device copies of the tree handed in (packed nodes, leaf values) and the pinned buffer they are
     // uploaded through; kept between calls and grown on demand
     uint32_t *pt_nodes;
@@ -174,8 +177,11 @@ struct evt_ctx {
     bool write_nidx;   // the tree being grown records the node id of every row it places
     bool grads_ahead;    // option: a tree with update_pred queues the next gradient update behind itself
     bool grads_ready;    // the gradients of the predictions as they stand were computed ahead: evt_update_grads has nothing to do
-    hipEvent_t tree_ev;  // recorded behind the tree's transfer to the host: evt_grow_tree_end waits for this, not for the stream
-    bool tree_in_flight; // evt_grow_tree_begin has queued a tree that evt_grow_tree_end has not collected
+    hipEvent_t tree_evs[2]; // per slot, recorded behind the tree's transfer to the host: evt_grow_tree_end waits for this, not for the stream
+    int tree_in_flight;     // trees queued by evt_grow_tree_begin that evt_grow_tree_end has not collected (0..2)
+    int slot_w, slot_r;     // staging slot of the next tree queued / of the oldest tree not yet collected
+    int64_t tree_seq;       // trees opened so far; slot_seq: the tree each slot holds
+    int64_t slot_seq[2];
     // a tree grown one kernel stage at a time (evt_tree_open ... evt_tree_close); evt_grow_tree_begin drives the same stages
     struct {
         int phase; // 0 no tree open, 1 histogram next, 2 split search next, 3 partition next, 4 levels done

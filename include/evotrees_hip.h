@@ -181,15 +181,22 @@ int evt_grow_tree(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_
  * mask, src/subsample.jl:7; the reference's host does this between kernels of the device path,
  * ext/.../subsample.jl:2-8) with the device growing this round's tree.  begin reads mask and js before it
  * returns and queues all device work; end waits for it and fills the tree arrays (EVT_ERR_EMPTY when no row was
- * kept).  Between the two, every other call on the handle except evt_synchronize and evt_destroy returns
- * EVT_ERR_STATE.  evt_grow_tree is begin followed by end. */
+ * kept).  evt_grow_tree is begin followed by end.
+ * TWO trees may be in flight: the next tree's begin (either form), the evt_update_grads and evt_draw_mask that go with
+ * it and evt_set_profiling only queue work behind what is already queued, so they may be called while ONE tree waits
+ * to be collected; end then collects the older tree.  A host whose next round does not depend on this round's tree
+ * arrays (src/fit.jl:6-42 reads nothing back) thereby keeps the device busy while it collects a tree and prepares
+ * the next call.  With two trees in flight only evt_grow_tree_end, evt_synchronize and evt_destroy are accepted; every
+ * call not named here returns EVT_ERR_STATE while any tree is in flight.  The results are, bit for bit, those of
+ * begin / end strictly in turn. */
 int evt_grow_tree_begin(evt_handle h, const uint8_t *mask, uint8_t cond, const uint32_t *js, int32_t n_js,
                         const evt_params *params);
 int evt_grow_tree_end(evt_handle h, evt_tree_out *tree);
 /* The upload of the next tree's mask (nobs bytes over PCIe, src/subsample.jl:7-9 / ext/.../subsample.jl:2-8) taken off
  * the critical path: evt_stage_mask may be called while a tree begun with evt_grow_tree_begin is in flight; it copies
  * the mask on a stream of its own into a second device buffer and returns when the copy is done (the caller's buffer
- * is free again; the tree in flight keeps running).  evt_grow_tree_begin_staged is evt_grow_tree_begin with the mask
+ * is free again; the tree in flight keeps running; with TWO trees in flight it returns EVT_ERR_STATE, since the older
+ * tree may still read the buffer the copy goes to).  evt_grow_tree_begin_staged is evt_grow_tree_begin with the mask
  * staged last; EVT_ERR_STATE when none has been staged since the last tree.  Same trees, bit for bit. */
 int evt_stage_mask(evt_handle h, const uint8_t *mask);
 int evt_grow_tree_begin_staged(evt_handle h, uint8_t cond, const uint32_t *js, int32_t n_js,

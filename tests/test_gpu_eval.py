@@ -234,6 +234,22 @@ def test_classifier_fit_levels_logger_and_errors(evt):
         evt.Handle(10, 2, 8, 17, 2, "mlogloss")
 
 
+@pytest.mark.parametrize("kw", [dict(rowsample=0.6, colsample=0.5), dict(bagging_size=3, rowsample=0.8), dict()])
+def test_fit_running_one_tree_ahead_equals_fit_in_turn(evt, kw):
+    # without an eval set the device is given the next tree before the last one is collected (two trees in flight, also
+    # across rounds); with one, every tree is collected before the next call.  Same generator draws, same trees.
+    rng = np.random.default_rng(3)
+    X = rng.random((4000, 6))
+    Y = X[:, 0] * 2 + np.sin(6 * X[:, 1]) + 0.1 * rng.standard_normal(4000)
+    cfg = evt.EvoTreeRegressor(nrounds=9, nbins=32, eta=0.3, max_depth=5, seed=42, **kw)
+    m_ahead = evt.fit(cfg, x_train=X, y_train=Y)
+    m_turn = evt.fit(cfg, x_train=X, y_train=Y, x_eval=X[:500], y_eval=Y[:500], verbosity=0)
+    assert len(m_ahead.trees) == len(m_turn.trees) == 1 + 9 * cfg.bagging_size
+    for a, b in zip(m_ahead.trees, m_turn.trees):
+        for name in ("feat", "cond_bin", "split", "w", "gain", "pred"):
+            assert getattr(a, name).tobytes() == getattr(b, name).tobytes(), name
+
+
 def test_update_continues_on_the_kept_handle(evt):
     # MMI.update (src/MLJ.jl:38-57): only a larger nrounds continues; the result equals a single longer fit
     rng = np.random.default_rng(11)

@@ -246,8 +246,8 @@ def test_mask_drawn_on_the_device(evt):
 
 def test_grow_tree_in_two_halves(evt):
     """evt_grow_tree_begin / evt_grow_tree_end give the trees and predictions of evt_grow_tree, bit for bit; between
-    the two halves the handle refuses every other call (and still answers afterwards); an end without a begin and an
-    empty subsample are reported by the half that knows."""
+    the two halves the handle refuses every call that reads or rewrites its state (and still answers afterwards); an end
+    without a begin and an empty subsample are reported by the half that knows."""
     N, F, B, D = 40000, 11, 32, 6
     x_bin, y, w, mu = make_data(91, N, F, B, "logloss", weights=True)
     js = np.arange(1, F + 1, dtype=np.uint32)
@@ -271,7 +271,7 @@ def test_grow_tree_in_two_halves(evt):
         hb.grow_tree_begin(js, gp, mask=mb, cond=140)
         if sub:
             mb[:] = 0  # the mask has been read when begin returns
-        for call in (hb.update_grads, hb.get_pred, lambda: hb.eval_metric("logloss"), lambda: hb.grow_tree_begin(js, gp)):
+        for call in (hb.get_pred, hb.get_grads, lambda: hb.eval_metric("logloss"), lambda: hb.predict_tree(ta), lambda: hb.set_target(y, w, mu)):
             with pytest.raises(evt.EvtError) as ei:
                 call()
             assert ei.value.code == evt._lib.EVT_ERR_STATE
@@ -290,6 +290,83 @@ def test_grow_tree_in_two_halves(evt):
     hb.grow_tree(js, gp)  # the handle goes on working
     ha.close()
     hb.close()
+
+
+@pytest.mark.parametrize("loss,tt,bagging,sub", [("mse", "binary", 1, False), ("mse", "binary", 1, True), ("logloss", "oblivious", 1, True),
+                                                 ("gaussian_mle", "binary", 2, False), ("quantile", "binary", 1, True)])
+def test_two_trees_in_flight(evt, loss, tt, bagging, sub):
+    """The next tree (with its gradient update and its device-drawn mask) may be queued before the last one has been
+    collected: evt_grow_tree_end then hands out the older tree.  Trees, gradients and predictions are those of calls
+    strictly in turn, bit for bit, with and without the gradients queued ahead; with two trees in flight the handle
+    takes nothing but the collection of the older one; per-level row counts in the profile stay those of each tree."""
+    N, F, B, D, R = 50000, 10, 32, 6, 7
+    x_bin, y, w, mu = make_data(33, N, F, B, loss, weights=(loss == "logloss"))
+    rng = np.random.default_rng(5)
+    jss = [np.sort(rng.choice(F, 7, replace=False)).astype(np.uint32) + 1 if r % 3 == 1 else np.arange(1, F + 1, dtype=np.uint32) for r in range(R)]
+    seeds = [int(s) for s in rng.integers(0, 1 << 62, R)]
+    gp = evt.make_params(eta=0.3, bagging_size=bagging, min_weight=8.0 if loss == "gaussian_mle" else 1.0)
+    cond = 150
+
+    def make(ahead):
+        h = evt.Handle(N, F, B, mu.shape[0], D, loss, tt)
+        h.set_option("grads_ahead", ahead)
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        if loss == "quantile":
+            h.set_alphas([0.3])
+        return h
+
+    def begin(h, r):
+        if r % bagging == 0:
+            h.update_grads()
+        if sub:
+            h.draw_mask(seeds[r])
+            h.grow_tree_begin_staged(jss[r], gp, cond)
+        else:
+            h.grow_tree_begin(jss[r], gp)
+
+    ha = make(0)
+    ref = []
+    for r in range(R):
+        begin(ha, r)
+        ref.append(ha.grow_tree_end())
+    ha.update_grads()
+    ref_state = [ha.get_grads(), ha.get_pred()]
+    ha.close()
+    for ahead in (0, 1) if bagging == 1 else (0,):
+        hb = make(ahead)
+        hb.set_profiling(["hist"])
+        got = []
+        begin(hb, 0)
+        for r in range(1, R):
+            begin(hb, r)  # tree r - 1 has not been collected
+            if r == 2:
+                for call in (hb.update_grads, lambda: hb.grow_tree_begin(jss[r], gp), lambda: hb.draw_mask(1), hb.get_pred,
+                             lambda: hb.stage_mask(np.zeros(N, np.uint8)), lambda: hb.set_profiling(False)):
+                    with pytest.raises(evt.EvtError) as ei:
+                        call()
+                    assert ei.value.code == evt._lib.EVT_ERR_STATE
+            got.append(hb.grow_tree_end())
+            if r == 4:
+                with pytest.raises(evt.EvtError) as ei:
+                    hb.get_pred()  # one tree is still in flight
+                assert ei.value.code == evt._lib.EVT_ERR_STATE
+        got.append(hb.grow_tree_end())
+        with pytest.raises(evt.EvtError) as ei:
+            hb.grow_tree_end()
+        assert ei.value.code == evt._lib.EVT_ERR_STATE
+        for a, b in zip(ref, got):
+            assert_tree_bits(a, b)
+        prof = hb.get_profile()["hist"]
+        # rows built, as the histogram launches' events were matched with each tree's own per-level counts: the root
+        # level of every tree holds the tree's sampled rows (= the root's weight for unit weights)
+        if loss == "mse":
+            assert prof["launches"] == R  # 16-byte records, few chunks: only the root's histogram is a launch of its own
+            assert prof["units"] == sum(int(t.w[0]) for t in got)
+        hb.update_grads()
+        assert hb.get_grads().tobytes() == ref_state[0].tobytes()
+        assert hb.get_pred().tobytes() == ref_state[1].tobytes()
+        hb.close()
 
 
 @pytest.mark.parametrize("loss,tt", [("mse", "binary"), ("logloss", "oblivious"), ("gaussian_mle", "binary")])
