@@ -272,6 +272,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->stats = nullptr; c->errflag = nullptr; c->ogains = nullptr; c->sbest = nullptr;
     c->h_stage = nullptr; c->h_stage_dev = nullptr; c->h_stage_bytes = 0; c->h_stage_base = nullptr; c->h_stage_dev_base = nullptr;
     c->n_js_last = 0;
+    c->js_staged = false;
     c->last_all_rows = true;
     // one block of 16 waves per CU: as many waves as two blocks of 8 (the LDS histogram caps a CU at 128 KB), half
     // the flushes per node
@@ -805,7 +806,7 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
     c->nidx_valid = rec_nidx;
 
     // per-tree small uploads through pinned memory
-    if (c->n_js_last != n_js || c->js_last != jsv) { // the column sample changed: refresh the device copies
+    if (c->n_js_last != n_js || c->js_last != jsv || c->js_staged) { // the column sample changed: refresh the device copies
         uint32_t *h_js = reinterpret_cast<uint32_t *>(c->h_stage + c->blob_bytes);
         uint16_t *h_map = reinterpret_cast<uint16_t *>(c->h_stage + c->blob_bytes + (size_t)c->F * 4);
         for (int f = 0; f < c->RS; f++) h_map[f] = 0xFFFF;
@@ -813,13 +814,9 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
             h_js[i] = jsv[i];
             h_map[jsv[i] - 1] = (uint16_t)i;
         }
-        // read from the pinned buffer by a kernel (no trip through the copy engine); the buffer is not written again
-        // before the next tree, which starts after this one has been collected
-        {
-            const size_t o_js = c->blob_bytes, o_map = c->blob_bytes + (size_t)c->F * 4;
-            int rr = launch_copy_words2(c, c->h_stage_dev + o_js, c->js, sizeof(uint32_t) * n_js, c->h_stage_dev + o_map, c->jsmap, sizeof(uint16_t) * c->RS);
-            if (rr != EVT_OK) return rr;
-        }
+        // k_tree_begin reads them from the pinned buffer (this tree's staging slot, not written again before the tree has
+        // been collected)
+        c->js_staged = true;
         c->n_js_last = n_js;
         c->js_last = jsv;
     }
@@ -860,6 +857,7 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
     c->step.defer = defer;
     c->step.fuse_pred = fuse_pred;
     c->step.hist_fused = !staged && scatter_can_build_hist(c, c->n_js_last);
+    c->step.blob_sent = false;
     c->step.p = *p;
     // the root's list is the identity (kept, never written) or what the mask compaction left in is_a; the levels below
     // alternate between is_a and is_b
@@ -920,7 +918,10 @@ static int tree_stage_partition(evt_ctx *c) {
         r = launch_part_count(c, level, is_cur);
         if (r == EVT_OK) r = launch_part_scatter(c, level, is_cur, is_next, c->step.fuse_pred);
     } else {
-        r = launch_final_fused(c, level, is_cur, c->step.fuse_pred);
+        // the tree's last kernel unless its leaves are still to be valued (quantile losses) or the rows outside the sample
+        // are still to be predicted: the finished tree's transfer to the host rides along
+        const bool last_kernel = !EVT_IS_QUANTILE(c->loss) && !(c->step.p.update_pred && !c->step.all_rows);
+        r = launch_final_fused(c, level, is_cur, c->step.fuse_pred, last_kernel);
     }
     prof_end(c);
     if (r != EVT_OK) return r;
@@ -953,7 +954,7 @@ static int tree_close(evt_ctx *c) {
     if (p->update_pred && !all_rows) {
         // rows outside the sample are predicted too (src/fit.jl:37): walk the new tree for all rows
         prof_begin(c, EVT_K_PREDICT, 0);
-        r = launch_predict_tree_cache(c);
+        r = launch_predict_tree_cache(c, true); // with the tree's transfer to the host in its last blocks
         prof_end(c);
         if (r != EVT_OK) return r;
         if (c->profiling) c->prof_units[EVT_K_PREDICT] += c->N;
@@ -964,8 +965,10 @@ static int tree_close(evt_ctx *c) {
     }
 
     // the tree (and the per-level row counts) comes back in one pinned transfer, queued behind the kernels
-    r = launch_copy_to_host(c, c->tree_blob, c->h_stage_dev, c->blob_bytes);
-    if (r != EVT_OK) return r;
+    if (!c->step.blob_sent) {
+        r = launch_copy_to_host(c, c->tree_blob, c->h_stage_dev, c->blob_bytes);
+        if (r != EVT_OK) return r;
+    }
     HIPCHK(hipEventRecord(c->tree_evs[c->slot_w], c->stream));
     c->slot_seq[c->slot_w] = c->tree_seq;
     if (c->grads_ahead && p->update_pred && p->bagging_size == 1) {

@@ -162,6 +162,7 @@ struct evt_ctx {
     size_t h_stage_bytes;
     int32_t h_qbits[EVT_MC_MAX_NK];
     int32_t n_js_last;
+    bool js_staged; // the column sample sits in the pinned staging slot and has not reached the device copies yet (k_tree_begin takes it along)
     std::vector<uint32_t> js_last;
     std::vector<uint8_t> h_feattypes; // host copy: trees handed in from outside are packed with it
     bool last_all_rows;
@@ -188,6 +189,7 @@ struct evt_ctx {
         int level;
         bool all_rows, defer, fuse_pred;
         bool hist_fused; // levels below the root get their histograms from the scatter pass of the level above
+        bool blob_sent;  // the finished tree's transfer to the host rode along with the tree's last kernel
         uint32_t *is_cur, *is_next; // row-id lists of the current level and of the one below
         evt_params p;
     } step;
@@ -338,7 +340,7 @@ int launch_obliv_select(evt_ctx *c, int level, const evt_params *p);
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t *is_next, bool fuse_pred);
 bool scatter_can_build_hist(const evt_ctx *c, int nfs);
-int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred);
+int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred, bool send_blob);
 int launch_nidx_from_segments(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_copy_to_host(evt_ctx *c, const void *src_dev, void *dst_host_dev, size_t nbytes);
 int launch_copy_words(evt_ctx *c, const void *src, void *dst, size_t nbytes);
@@ -346,7 +348,7 @@ int launch_copy_words2(evt_ctx *c, const void *src0, void *dst0, size_t nbytes0,
 int launch_fill_u32(evt_ctx *c, uint32_t *dst, uint32_t v, int64_t n);
 int launch_fill_bytes(evt_ctx *c, void *dst, int64_t nbytes);
 // predict
-int launch_predict_tree_cache(evt_ctx *c);
+int launch_predict_tree_cache(evt_ctx *c, bool send_blob);
 int launch_hist_export(evt_ctx *c, double *out_dev);
 int launch_nidx_from_tree(evt_ctx *c, bool use_mask, uint8_t cond);
 

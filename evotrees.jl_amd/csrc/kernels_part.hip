@@ -15,6 +15,7 @@
 //             became leaves record the node id per row (and add the leaf value to the prediction).
 // No host round trip is needed between levels.
 #include "evt_internal.h"
+#include <algorithm>
 
 // largest i in [0, n) with pre[i] <= v   (pre ascending, pre[0] <= v): the number of such entries, less one.  Every
 // wavefront counts them for itself, 64 entries per step, all loads independent: one trip to memory where a binary
@@ -64,6 +65,11 @@ struct PartArgs {
     long long *hist;
     int64_t node_stride;
     int F, nfs, NAg;
+    // last pass of a tree: the finished tree's arrays go to the host's pinned buffer in copy_blocks extra blocks
+    const uint4 *copy_src;
+    uint4 *copy_dst;
+    int64_t copy_n;
+    int copy_blocks;
 };
 
 // The word of the decision source that holds row `rid`: its bin byte, or - for a numeric split with bit planes - the
@@ -506,10 +512,17 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A, NextArgs NX) {
 template <bool NT>
 __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
     const int tid = threadIdx.x;
+    const int64_t G = (int64_t)gridDim.x - A.copy_blocks;
+    if ((int64_t)blockIdx.x >= G) {
+        // the tree's arrays are complete (this is the tree's last kernel and writes none of them): their way back to the
+        // host rides along instead of taking a launch of its own
+        for (int64_t i = ((int64_t)blockIdx.x - G) * 256 + tid; i < A.copy_n; i += (int64_t)A.copy_blocks * 256) A.copy_dst[i] = A.copy_src[i];
+        return;
+    }
     uint4 cd = A.cdesc[blockIdx.x];
     const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
     const int K = A.K;
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x, cd = A.cdesc[c < n_chunks ? c : 0]) {
+    for (int64_t c = blockIdx.x; c < n_chunks; c += G, cd = A.cdesc[c < n_chunks ? c : 0]) {
         const int n = (int)cd.x;
         const int64_t p0 = cd.y, pend = cd.z;
         constexpr int NI = EVT_CHUNK / 256;
@@ -589,6 +602,10 @@ struct BeginArgs {
     int64_t seg_cost;
     int64_t root_words;
     int nnodes, K, D;
+    // the tree's column sample and its inverse map, from the pinned staging buffer to the device copies (0 words: unchanged)
+    const uint32_t *js_src, *map_src;
+    uint32_t *js_dst, *map_dst;
+    int js_words, map_words;
 };
 
 __global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) {
@@ -605,6 +622,8 @@ __global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) {
     for (int n = tid; n < A.nnodes + 2; n += 1024) A.status[n] = ST_INACTIVE;
     for (int64_t i = tid; i < A.root_words; i += 1024) A.hist[i] = 0;
     for (int d = tid; d <= A.D; d += 1024) A.stats[d] = 0;
+    for (int i = tid; i < A.js_words; i += 1024) A.js_dst[i] = A.js_src[i];
+    for (int i = tid; i < A.map_words; i += 1024) A.map_dst[i] = A.map_src[i];
     __syncthreads();
     if (tid == 0) {
         if (A.n_is_dev) A.n_is = *A.n_is_dev;
@@ -796,8 +815,21 @@ int launch_tree_begin(evt_ctx *c, bool all_rows) {
     A.nnodes = c->nnodes;
     A.K = c->K;
     A.D = c->D;
+    A.js_words = A.map_words = 0;
+    A.js_src = A.map_src = nullptr;
+    A.js_dst = A.map_dst = nullptr;
+    if (c->js_staged) { // read from the pinned buffer by the kernel (no trip through the copy engine, no launch of its own)
+        const size_t o_js = c->blob_bytes, o_map = c->blob_bytes + (size_t)c->F * 4;
+        A.js_src = reinterpret_cast<const uint32_t *>(c->h_stage_dev + o_js);
+        A.js_dst = c->js;
+        A.js_words = c->n_js_last;
+        A.map_src = reinterpret_cast<const uint32_t *>(c->h_stage_dev + o_map);
+        A.map_dst = reinterpret_cast<uint32_t *>(c->jsmap);
+        A.map_words = c->RS / 2;
+    }
     hipLaunchKernelGGL(k_tree_begin, dim3(1), dim3(1024), 0, c->stream, A);
     HIPCHK(hipGetLastError());
+    c->js_staged = false;
     return EVT_OK;
 }
 
@@ -836,6 +868,10 @@ static void fill_part_args(evt_ctx *c, int level, const uint32_t *is_cur, uint32
     A.hist = nullptr;
     A.node_stride = 0;
     A.F = A.nfs = A.NAg = 0;
+    A.copy_src = nullptr;
+    A.copy_dst = nullptr;
+    A.copy_n = 0;
+    A.copy_blocks = 0;
 }
 
 int launch_part_count(evt_ctx *c, int level, const uint32_t *is_cur) {
@@ -926,12 +962,20 @@ bool scatter_can_build_hist(const evt_ctx *c, int nfs) {
            c->NA <= EVT_MAX_NA && c->max_chunks <= 128 + c->maxlvl && (size_t)c->NA * nfs * c->B * 8 <= 32 * 1024;
 }
 
-int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred) {
+int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_pred, bool send_blob) {
     if (!fuse_pred && !c->write_nidx) return EVT_OK;
     PartArgs A;
     fill_part_args(c, level, is_cur, nullptr, fuse_pred, A);
-    if (A.stream_hint) hipLaunchKernelGGL(k_final_fused<true>, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
-    else hipLaunchKernelGGL(k_final_fused<false>, dim3(grid_for_chunks(c->max_chunks)), dim3(256), 0, c->stream, A);
+    if (send_blob) {
+        A.copy_src = reinterpret_cast<const uint4 *>(c->tree_blob);
+        A.copy_dst = reinterpret_cast<uint4 *>(c->h_stage_dev);
+        A.copy_n = (int64_t)(c->blob_bytes / 16);
+        A.copy_blocks = (int)std::min<int64_t>(64, (A.copy_n + 255) / 256);
+        c->step.blob_sent = true;
+    }
+    const dim3 grid(grid_for_chunks(c->max_chunks) + (unsigned)A.copy_blocks);
+    if (A.stream_hint) hipLaunchKernelGGL(k_final_fused<true>, grid, dim3(256), 0, c->stream, A);
+    else hipLaunchKernelGGL(k_final_fused<false>, grid, dim3(256), 0, c->stream, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

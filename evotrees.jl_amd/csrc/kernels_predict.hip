@@ -5,6 +5,7 @@
 // walk reads one bin byte per level, from the column-major x_bin (neighbouring rows share 64-byte sectors of
 // a column) or, in the whole-model kernel, from a copy of the block's rows in LDS.
 #include "evt_internal.h"
+#include <algorithm>
 
 __device__ __forceinline__ int walk_packed(const uint32_t *__restrict__ nodes, const uint8_t *__restrict__ xcm, int64_t N, int64_t i) {
     int nid = 1;
@@ -20,9 +21,17 @@ __device__ __forceinline__ int walk_packed(const uint32_t *__restrict__ nodes, c
     return nid;
 }
 
-// one tree added to pred (K x N), all rows
+// one tree added to pred (K x N), all rows.  copy_blocks extra blocks at the end of the grid carry copy_n 16-byte words
+// from copy_src to copy_dst: the finished tree's way back to the host's pinned buffer, when this is the tree's last kernel.
 __global__ __launch_bounds__(256) void k_predict_tree(const uint32_t *__restrict__ nodes, const float *__restrict__ leaf_pred,
-                                                     const uint8_t *__restrict__ xcm, int64_t N, int K, int loss, float *pred) {
+                                                     const uint8_t *__restrict__ xcm, int64_t N, int K, int loss, float *pred,
+                                                     const uint4 *__restrict__ copy_src, uint4 *__restrict__ copy_dst, int64_t copy_n,
+                                                     int copy_blocks) {
+    const int64_t G = (int64_t)gridDim.x - copy_blocks;
+    if ((int64_t)blockIdx.x >= G) {
+        for (int64_t k = ((int64_t)blockIdx.x - G) * 256 + threadIdx.x; k < copy_n; k += (int64_t)copy_blocks * 256) copy_dst[k] = copy_src[k];
+        return;
+    }
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= N) return;
     const int nid = walk_packed(nodes, xcm, N, i);
@@ -47,16 +56,20 @@ int launch_nidx_from_tree(evt_ctx *c, bool use_mask, uint8_t cond) {
     return EVT_OK;
 }
 
-int launch_predict_tree_cache(evt_ctx *c) {
-    hipLaunchKernelGGL(k_predict_tree, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->tree.packed, c->tree.pred, c->xcm,
-                       c->N, c->K, c->loss, c->pred);
+int launch_predict_tree_cache(evt_ctx *c, bool send_blob) {
+    const int64_t copy_n = send_blob ? (int64_t)(c->blob_bytes / 16) : 0;
+    const int copy_blocks = (int)std::min<int64_t>(64, (copy_n + 255) / 256);
+    hipLaunchKernelGGL(k_predict_tree, dim3((unsigned)((c->N + 255) / 256) + (unsigned)copy_blocks), dim3(256), 0, c->stream, c->tree.packed,
+                       c->tree.pred, c->xcm, c->N, c->K, c->loss, c->pred, reinterpret_cast<const uint4 *>(c->tree_blob),
+                       reinterpret_cast<uint4 *>(c->h_stage_dev), copy_n, copy_blocks);
     HIPCHK(hipGetLastError());
+    if (send_blob) c->step.blob_sent = true;
     return EVT_OK;
 }
 
 int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, const float *leaf_pred_dev) {
     hipLaunchKernelGGL(k_predict_tree, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, nodes_dev, leaf_pred_dev, c->xcm, c->N,
-                       c->K, c->loss, c->pred);
+                       c->K, c->loss, c->pred, static_cast<const uint4 *>(nullptr), static_cast<uint4 *>(nullptr), (int64_t)0, 0);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
