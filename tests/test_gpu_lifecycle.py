@@ -369,6 +369,41 @@ def test_two_trees_in_flight(evt, loss, tt, bagging, sub):
         hb.close()
 
 
+def test_empty_subsample_with_a_second_tree_in_flight(evt):
+    """A tree whose mask keeps no row is reported when it is collected (EVT_ERR_EMPTY), also when the next tree has been
+    queued behind it meanwhile; that next tree is collected as usual and equals the tree a handle grows that never saw
+    the empty one (a tree on no rows is a single zero leaf: it changes no prediction)."""
+    N, F, B, D = 30000, 8, 32, 5
+    x_bin, y, w, mu = make_data(12, N, F, B, "mse", weights=False)
+    js = np.arange(1, F + 1, dtype=np.uint32)
+    gp = evt.make_params(eta=0.3)
+
+    def make():
+        h = evt.Handle(N, F, B, 1, D, "mse")
+        h.set_xbin(x_bin)
+        h.set_target(y, w, mu)
+        return h
+
+    ha, hb = make(), make()
+    ha.update_grads()
+    t0 = ha.grow_tree(js, gp)
+    ha.update_grads()
+    t1 = ha.grow_tree(js, gp)
+    hb.update_grads()
+    assert_tree_bits(t0, hb.grow_tree(js, gp))
+    hb.update_grads()
+    hb.grow_tree_begin(js, gp, mask=np.full(N, 255, np.uint8), cond=10)  # keeps no row
+    hb.update_grads()
+    hb.grow_tree_begin(js, gp)                                            # queued behind it
+    with pytest.raises(evt.EvtError) as ei:
+        hb.grow_tree_end()
+    assert ei.value.code == evt._lib.EVT_ERR_EMPTY
+    assert_tree_bits(t1, hb.grow_tree_end())
+    assert ha.get_pred().tobytes() == hb.get_pred().tobytes()
+    ha.close()
+    hb.close()
+
+
 @pytest.mark.parametrize("loss,tt", [("mse", "binary"), ("logloss", "oblivious"), ("gaussian_mle", "binary")])
 def test_gradients_queued_ahead_change_nothing(evt, loss, tt):
     """With "grads_ahead" the gradient update of the next round is queued behind every tree and the next
