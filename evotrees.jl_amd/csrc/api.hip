@@ -6,7 +6,11 @@
 #include <string.h>
 
 #include <algorithm>
+#include <condition_variable>
+#include <memory>
+#include <mutex>
 #include <new>
+#include <thread>
 
 int launch_absmax_rows(evt_ctx *c, int k0, int k1);
 int launch_check_unit_weight(evt_ctx *c);
@@ -513,6 +517,125 @@ extern "C" int evt_set_xbin(evt_handle c, const uint8_t *x_bin_colmajor) {
     });
 }
 
+// A Float64 matrix in host memory (column-major, nobs x nfeats) -> bins, written in place at xcm (column j at xcm + j * nobs).
+// The matrix goes up in pieces (whole columns while they are short, row ranges of one column otherwise) through three pinned
+// buffers: a few worker threads copy piece k + 1 into its buffer while the DMA engine moves piece k, and the kernel that bins
+// a piece runs behind its copy on the same stream.  A copy straight from the caller's pageable memory is staged by the runtime
+// at about half the rate the bus gives pinned memory (31 against 57 GB/s on the box this was measured on), and one thread's
+// memcpy is no faster than that either.  The workers only copy memory, never call back into the caller's runtime, and are
+// joined before the call returns.
+struct CopyJob {
+    const char *src;
+    char *dst;
+    size_t n;
+};
+class CopyPool {
+    std::vector<std::thread> th;
+    std::mutex m;
+    std::condition_variable cv_go, cv_done;
+    const std::vector<CopyJob> *jobs = nullptr;
+    size_t gen = 0;
+    int pending = 0;
+    bool stop = false;
+    const int nt;
+    void run(int w) {
+        size_t seen = 0;
+        for (;;) {
+            std::unique_lock<std::mutex> lk(m);
+            cv_go.wait(lk, [&] { return stop || gen != seen; });
+            if (stop) return;
+            seen = gen;
+            const std::vector<CopyJob> *j = jobs;
+            lk.unlock();
+            for (const CopyJob &job : *j) { // worker w takes the w-th of nt slices of every job (cut at 64-byte multiples)
+                const size_t lo = (job.n * (size_t)w / nt) & ~(size_t)63;
+                const size_t hi = (w + 1 == nt) ? job.n : ((job.n * (size_t)(w + 1) / nt) & ~(size_t)63);
+                if (hi > lo) memcpy(job.dst + lo, job.src + lo, hi - lo);
+            }
+            lk.lock();
+            if (--pending == 0) cv_done.notify_one();
+        }
+    }
+
+  public:
+    explicit CopyPool(int n) : nt(n) {
+        for (int w = 0; w < n; w++) th.emplace_back([this, w] { run(w); });
+    }
+    ~CopyPool() {
+        {
+            std::lock_guard<std::mutex> lk(m);
+            stop = true;
+        }
+        cv_go.notify_all();
+        for (auto &t : th) t.join();
+    }
+    void copy(const std::vector<CopyJob> &j) { // returns when every job has been copied
+        std::unique_lock<std::mutex> lk(m);
+        jobs = &j;
+        pending = nt;
+        gen++;
+        cv_go.notify_all();
+        cv_done.wait(lk, [&] { return pending == 0; });
+    }
+};
+struct UploadSlots {
+    static const int NS = 3;
+    void *host[NS] = {nullptr, nullptr, nullptr};
+    double *dev[NS] = {nullptr, nullptr, nullptr};
+    hipEvent_t ev[NS] = {nullptr, nullptr, nullptr};
+    ~UploadSlots() {
+        for (int k = 0; k < NS; k++) {
+            if (ev[k]) (void)hipEventDestroy(ev[k]);
+            if (dev[k]) (void)hipFree(dev[k]);
+            if (host[k]) (void)hipHostFree(host[k]);
+        }
+    }
+};
+static int upload_binarize_f64(hipStream_t s, const double *x, int64_t nobs, int nfeats, const double *d_edges, const int32_t *d_eoff,
+                               uint8_t *xcm) {
+    const int64_t PIECE = (int64_t)32 << 20; // bytes
+    const int64_t rows_max = PIECE / 8;
+    const int64_t rows_piece = std::min(nobs, rows_max);
+    const int cols_piece = (nobs <= rows_max) ? (int)std::max<int64_t>(1, std::min<int64_t>(nfeats, rows_max / nobs)) : 1;
+    const size_t bytes = sizeof(double) * (size_t)rows_piece * cols_piece;
+    UploadSlots U;
+    for (int k = 0; k < UploadSlots::NS; k++) {
+        HIPCHK(hipHostMalloc(&U.host[k], bytes, hipHostMallocDefault));
+        HIPCHK(hipMalloc((void **)&U.dev[k], bytes));
+        HIPCHK(hipEventCreateWithFlags(&U.ev[k], hipEventDisableTiming));
+    }
+    // small inputs are copied by the calling thread; from a few pieces on, by up to six workers
+    const int64_t total_bytes = (int64_t)sizeof(double) * nobs * nfeats;
+    const int nworkers = total_bytes < ((int64_t)64 << 20) ? 0 : (int)std::min<unsigned>(6, std::max(1u, std::thread::hardware_concurrency() / 2));
+    std::unique_ptr<CopyPool> pool;
+    if (nworkers > 1) pool.reset(new CopyPool(nworkers));
+    std::vector<CopyJob> jobs;
+    int64_t piece = 0;
+    for (int j0 = 0; j0 < nfeats; j0 += cols_piece) {
+        const int nc = std::min(cols_piece, nfeats - j0);
+        for (int64_t r0 = 0; r0 < nobs; r0 += rows_piece, piece++) {
+            const int64_t n = std::min(rows_piece, nobs - r0);
+            const int k = (int)(piece % UploadSlots::NS);
+            if (piece >= UploadSlots::NS) HIPCHK(hipEventSynchronize(U.ev[k])); // the piece that used this buffer has been binned
+            double *h = static_cast<double *>(U.host[k]);
+            jobs.clear();
+            for (int j = 0; j < nc; j++)
+                jobs.push_back({reinterpret_cast<const char *>(x + (size_t)(j0 + j) * nobs + r0), reinterpret_cast<char *>(h + (size_t)j * n), sizeof(double) * (size_t)n});
+            if (pool) {
+                pool->copy(jobs);
+            } else {
+                for (const CopyJob &job : jobs) memcpy(job.dst, job.src, job.n);
+            }
+            HIPCHK(hipMemcpyAsync(U.dev[k], h, sizeof(double) * (size_t)n * nc, hipMemcpyHostToDevice, s));
+            const int r = launch_binarize_cols(s, U.dev[k], d_edges, d_eoff + j0, xcm + (size_t)j0 * nobs + r0, n, nc, n, nobs);
+            if (r != EVT_OK) return r;
+            HIPCHK(hipEventRecord(U.ev[k], s));
+        }
+    }
+    HIPCHK(hipStreamSynchronize(s));
+    return EVT_OK;
+}
+
 extern "C" int evt_binarize_f64(evt_handle c, const double *x_colmajor, const double *edges, const int32_t *edge_off) {
     return guarded([&]() -> int {
     CTXCHK(c);
@@ -531,31 +654,24 @@ extern "C" int evt_binarize_f64(evt_handle c, const double *x_colmajor, const do
     }
     double *d_edges = nullptr;
     int32_t *d_off = nullptr;
-    double *d_x = nullptr;
     HIPCHK(hipMalloc((void **)&d_edges, sizeof(double) * std::max(1, off[c->F])));
     hipError_t e = hipMalloc((void **)&d_off, sizeof(int32_t) * (c->F + 1));
     if (e == hipSuccess) e = hipMemcpyAsync(d_edges, edges, sizeof(double) * off[c->F], hipMemcpyDefault, c->stream);
     if (e == hipSuccess) e = hipMemcpyAsync(d_off, off.data(), sizeof(int32_t) * (c->F + 1), hipMemcpyHostToDevice, c->stream);
-    const double *xsrc = x_colmajor;
-    if (e == hipSuccess && !on_dev) {
-        e = hipMalloc((void **)&d_x, sizeof(double) * (size_t)c->N * c->F);
-        if (e == hipSuccess) e = hipMemcpyAsync(d_x, x_colmajor, sizeof(double) * (size_t)c->N * c->F, hipMemcpyHostToDevice, c->stream);
-        xsrc = d_x;
-    }
     int r = EVT_OK;
     if (e == hipSuccess) {
-        r = launch_binarize(c, xsrc, d_edges, d_off);
+        if (on_dev) r = launch_binarize(c, x_colmajor, d_edges, d_off);
+        else r = upload_binarize_f64(c->stream, x_colmajor, c->N, c->F, d_edges, d_off, c->xcm);
         if (r == EVT_OK) r = launch_transpose_validate(c);
         e = hipStreamSynchronize(c->stream);
     }
-    if (d_x) (void)hipFree(d_x);
     if (d_off) (void)hipFree(d_off);
     if (d_edges) (void)hipFree(d_edges);
+    if (r != EVT_OK) return r;
     if (e != hipSuccess) {
         evt_set_error("binarize failed: %s", hipGetErrorString(e));
         return EVT_ERR_HIP;
     }
-    if (r != EVT_OK) return r;
     r = check_errflag(c, "binarize produced values outside 1..nbins");
     if (r != EVT_OK) return r;
     c->have_xbin = true;
@@ -1459,7 +1575,6 @@ static void complete_trees(int ntrees, const int64_t *tree_off, const int64_t *f
 }
 
 // Rows binned per pass of evt_predict_f64: bounds the Float64 staging buffer to chunk * nfeats * 8 bytes.
-static const int64_t PREDICT_F64_CHUNK = 1 << 20;
 
 static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, const uint8_t *feattypes, int32_t loss, int32_t K, int32_t ntrees,
                           const int64_t *tree_off, const int64_t *feat, const uint8_t *cond_bin, const float *pred, const uint8_t *split,
@@ -1540,21 +1655,20 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
     if (e == hipSuccess && leaf_out) e = hipMalloc((void **)&d_leaf, sizeof(uint32_t) * (size_t)nobs * ntrees);
     if (e == hipSuccess && !x_f64 && !x_in_place) e = hipMemcpy(d_x, x_bin, (size_t)nobs * nfeats, hipMemcpyDefault);
     if (e == hipSuccess && x_f64) {
-        // binarize on the device, PREDICT_F64_CHUNK rows at a time: each pass copies the rows' slice of every
-        // column (a strided 2-D copy) and bins it into place
-        const int64_t chunk = std::min(nobs, PREDICT_F64_CHUNK);
+        // binarize on the device: the matrix goes up in pieces through pinned buffers and is binned into place
         double *d_xf = nullptr, *d_edges = nullptr;
         int32_t *d_eoff = nullptr;
-        e = hipMalloc((void **)&d_xf, sizeof(double) * (size_t)chunk * nfeats);
-        if (e == hipSuccess) e = hipMalloc((void **)&d_edges, sizeof(double) * eoff[nfeats]);
+        e = hipMalloc((void **)&d_edges, sizeof(double) * eoff[nfeats]);
         if (e == hipSuccess) e = hipMalloc((void **)&d_eoff, sizeof(int32_t) * (nfeats + 1));
         if (e == hipSuccess) e = hipMemcpy(d_edges, edges, sizeof(double) * eoff[nfeats], hipMemcpyDefault);
         if (e == hipSuccess) e = hipMemcpy(d_eoff, eoff.data(), sizeof(int32_t) * (nfeats + 1), hipMemcpyHostToDevice);
-        for (int64_t r0 = 0; r0 < nobs && e == hipSuccess && r == EVT_OK; r0 += chunk) {
-            const int64_t n = std::min(chunk, nobs - r0);
-            e = hipMemcpy2D(d_xf, sizeof(double) * chunk, x_f64 + r0, sizeof(double) * nobs, sizeof(double) * n, nfeats, hipMemcpyDefault);
-            if (e == hipSuccess) r = launch_binarize_cols(s, d_xf, d_edges, d_eoff, d_x + r0, n, nfeats, chunk, nobs);
-            if (e == hipSuccess) e = hipStreamSynchronize(s);
+        if (e == hipSuccess) {
+            if (on_device(x_f64)) {
+                r = launch_binarize_cols(s, x_f64, d_edges, d_eoff, d_x, nobs, nfeats, nobs, nobs);
+                if (r == EVT_OK) e = hipStreamSynchronize(s);
+            } else {
+                r = upload_binarize_f64(s, x_f64, nobs, nfeats, d_edges, d_eoff, d_x);
+            }
         }
         void *tmp[] = {d_xf, d_edges, d_eoff};
         for (void *p : tmp)

@@ -20,6 +20,11 @@
  *  - A handle is bound to the device that was current when it was created and to one HIP
  *    stream.  Calls on one handle must not overlap; different handles may be used from
  *    different threads.
+ *  - The library installs no signal handlers and never calls back into the caller's runtime.
+ *    The two calls that take a Float64 matrix from host memory (evt_binarize_f64,
+ *    evt_predict_f64) copy it into pinned memory with up to six worker threads of their own,
+ *    which only copy memory and are joined before the call returns; no other call starts a
+ *    thread.
  */
 #ifndef EVOTREES_HIP_H
 #define EVOTREES_HIP_H
@@ -130,7 +135,9 @@ int evt_set_xbin(evt_handle h, const uint8_t *x_bin_colmajor);
 
 /* Device binarize: searchsortedfirst(edges[j], x[i,j]) for every cell (src/fit-utils.jl:66-72),
  * written straight into the cache's x_bin.  x is nobs x nfeats column-major Float64; edges are
- * concatenated per feature, edge_off has nfeats+1 entries. */
+ * concatenated per feature, edge_off has nfeats+1 entries.  A matrix in host memory goes up in
+ * 32 MB pieces through pinned buffers, each binned behind its copy (8 bytes per value over the bus:
+ * 0.16 s for 10M x 100 where a plain copy from pageable memory takes 0.30 s). */
 int evt_binarize_f64(evt_handle h, const double *x_colmajor, const double *edges, const int32_t *edge_off);
 
 /* Target, weights and initial prediction: y Float32[nobs] (for mlogloss the 1-based level code of each row,

@@ -157,14 +157,17 @@ def test_early_stopping_and_offsets(evt):
     assert m4.info["logger"] is None
 
 
-def test_predict_f64_equals_host_binarize_then_predict(evt):
-    # crosses the internal row-chunk boundary (2^20 rows) and uses ragged edge counts
+@pytest.mark.parametrize("N,F", [((1 << 22) + 12345, 3), (700001, 7)])
+def test_predict_f64_equals_host_binarize_then_predict(evt, N, F):
+    # the Float64 matrix goes up in pieces of 2^22 values: a long column is cut into row ranges (first shape: two pieces per
+    # column, more pieces than upload buffers), short columns share a piece (second shape: five columns, then two); ragged
+    # edge counts
     rng = np.random.default_rng(9)
-    N, F = (1 << 20) + 12345, 3
     X = rng.standard_normal((N, F))
-    edges = [np.sort(rng.standard_normal(k)) for k in (31, 1, 254)]
+    edges = [np.sort(rng.standard_normal(k)) for k in (31, 1, 254, 7, 100, 2, 63)[:F]]
     X[:1000, 0] = edges[0][rng.integers(0, 31, 1000)]  # values equal to an edge fall in that edge's bin
     X[5, 1], X[6, 1] = np.inf, -np.inf
+    X[N - 1, F - 1] = np.nan
     xb = evt.binarize(X, edges)
     trees = []
     K = 1
@@ -182,6 +185,11 @@ def test_predict_f64_equals_host_binarize_then_predict(evt):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     with pytest.raises(evt.EvtError):
         evt._lib.predict_model_f64(np.ascontiguousarray(X[:10].T), [np.zeros(0)] * F, ft, "mse", K, trees)
+    # the training cache takes the same way up: evt_binarize_f64 leaves the bins the host computes
+    h = evt.Handle(N, F, 255, 1, 2, "mse")
+    h.binarize(np.ascontiguousarray(X.T), edges)
+    assert np.array_equal(h.get_xbin(), xb)
+    h.close()
 
 
 def test_classifier_fit_levels_logger_and_errors(evt):
