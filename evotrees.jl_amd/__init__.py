@@ -421,6 +421,8 @@ def init(config, x_train, y_train=None, w_train=None, offset_train=None, feature
     if table:  # Bool and categorical columns have no edges to search: binned on the host as the reference does
         h.set_xbin(binarize_table(x_train, feature_names, edges))
     else:
+        # the library takes the reference's memory order (column-major, a Julia matrix as it lies): free for a Fortran-ordered
+        # numpy array, a transposing host copy for a C-ordered one
         h.binarize(np.ascontiguousarray(x.T, np.float64), edges)
     mono = np.zeros(F, np.int32)
     for k, v in config.monotone_constraints.items():
