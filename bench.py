@@ -126,6 +126,7 @@ def prepare(evt, cfg, opts=None):
     h = evt.Handle(N, F, B, K, D, loss, cfg["tree_type"])
     h.binarize(x, edges)
     del x
+    h.bench_edges = edges  # for the inference probe from raw features
     mu = bias(loss, y)
     h.set_target(y, None, mu)
     for name, v in (opts or {}).items():
@@ -463,6 +464,27 @@ def main():
             hip.hipFree(d_out)
         except Exception as e:  # measurement aid only
             out["predict_model"] = {"error": str(e)}
+
+    # The reference's whole inference call m(x) from a raw Float64 matrix in host memory (binarize + 200 trees + link, its
+    # published "infer" figure; src/predict.jl:118-136): evt_predict_f64, everything included - the 8 GB upload through pinned
+    # buffers, device binarize, the traversal, the predictions' way back.  The matrix is generated again (it was dropped after
+    # the set-up to free host memory).
+    if args.workload == "cfg3" and not args.rows and args.side_steps > 0:
+        try:
+            x_raw, _, _ = synth(cfg)
+            m_trees = [evt.Tree.bias(mu)] + [tree] * 200
+            best = None
+            for _ in range(2):
+                tp = time.perf_counter()
+                evt._lib.predict_model_f64(x_raw, h.bench_edges, None, loss, K, m_trees, apply_link=True)
+                dt = time.perf_counter() - tp
+                best = dt if best is None else min(best, dt)
+            del x_raw
+            out["predict_f64"] = {"trees": 201, "s": round(best, 3), "rows_per_s": round(N / best, 1),
+                                  "note": "whole evt_predict_f64 call from a Float64 matrix in host memory, predictions returned to the host",
+                                  "reference_context": "published infer 10M x 100: 12.18 s CPU (Ryzen 5900X, 12 threads), 3.57 s GPU (RTX A4000), host binarize included (README.md:69,86); other hardware"}
+        except Exception as e:  # measurement aid only
+            out["predict_f64"] = {"error": str(e)}
 
     if args.predict:
         m_trees = []
