@@ -501,22 +501,6 @@ static int check_errflag(evt_ctx *c, const char *what) {
     return EVT_OK;
 }
 
-extern "C" int evt_set_xbin(evt_handle c, const uint8_t *x_bin_colmajor) {
-    return guarded([&]() -> int {
-    CTXCHK(c);
-    ARGCHK(x_bin_colmajor, "x_bin is NULL");
-    c->have_xbin = false;
-    c->planes_ready = false;
-    HIPCHK(hipMemcpyAsync(c->xcm, x_bin_colmajor, (size_t)c->N * c->F, hipMemcpyDefault, c->stream));
-    int r = launch_transpose_validate(c);
-    if (r != EVT_OK) return r;
-    r = check_errflag(c, "x_bin holds values outside 1..nbins");
-    if (r != EVT_OK) return r;
-    c->have_xbin = true;
-    return EVT_OK;
-    });
-}
-
 // A Float64 matrix in host memory (column-major, nobs x nfeats) -> bins, written in place at xcm (column j at xcm + j * nobs).
 // The matrix goes up in pieces (whole columns while they are short, row ranges of one column otherwise) through three pinned
 // buffers: a few worker threads copy piece k + 1 into its buffer while the DMA engine moves piece k, and the kernel that bins
@@ -590,25 +574,33 @@ struct UploadSlots {
             if (host[k]) (void)hipHostFree(host[k]);
         }
     }
+    int init(size_t bytes, bool with_dev) {
+        for (int k = 0; k < NS; k++) {
+            HIPCHK(hipHostMalloc(&host[k], bytes, hipHostMallocDefault));
+            if (with_dev) HIPCHK(hipMalloc((void **)&dev[k], bytes));
+            HIPCHK(hipEventCreateWithFlags(&ev[k], hipEventDisableTiming));
+        }
+        return EVT_OK;
+    }
 };
+static const int64_t UPLOAD_PIECE = (int64_t)32 << 20; // bytes
+// worker threads for an upload of this size: none below a few pieces, else up to six
+static int upload_workers(int64_t total_bytes) {
+    if (total_bytes < 2 * UPLOAD_PIECE) return 0;
+    return (int)std::min<unsigned>(6, std::max(1u, std::thread::hardware_concurrency() / 2));
+}
 static int upload_binarize_f64(hipStream_t s, const double *x, int64_t nobs, int nfeats, const double *d_edges, const int32_t *d_eoff,
                                uint8_t *xcm) {
-    const int64_t PIECE = (int64_t)32 << 20; // bytes
-    const int64_t rows_max = PIECE / 8;
+    const int64_t rows_max = UPLOAD_PIECE / 8;
     const int64_t rows_piece = std::min(nobs, rows_max);
     const int cols_piece = (nobs <= rows_max) ? (int)std::max<int64_t>(1, std::min<int64_t>(nfeats, rows_max / nobs)) : 1;
     const size_t bytes = sizeof(double) * (size_t)rows_piece * cols_piece;
     UploadSlots U;
-    for (int k = 0; k < UploadSlots::NS; k++) {
-        HIPCHK(hipHostMalloc(&U.host[k], bytes, hipHostMallocDefault));
-        HIPCHK(hipMalloc((void **)&U.dev[k], bytes));
-        HIPCHK(hipEventCreateWithFlags(&U.ev[k], hipEventDisableTiming));
-    }
+    int r0 = U.init(bytes, true);
+    if (r0 != EVT_OK) return r0;
     // small inputs are copied by the calling thread; from a few pieces on, by up to six workers
-    const int64_t total_bytes = (int64_t)sizeof(double) * nobs * nfeats;
-    const int nworkers = total_bytes < ((int64_t)64 << 20) ? 0 : (int)std::min<unsigned>(6, std::max(1u, std::thread::hardware_concurrency() / 2));
     std::unique_ptr<CopyPool> pool;
-    if (nworkers > 1) pool.reset(new CopyPool(nworkers));
+    if (upload_workers((int64_t)sizeof(double) * nobs * nfeats) > 1) pool.reset(new CopyPool(upload_workers((int64_t)sizeof(double) * nobs * nfeats)));
     std::vector<CopyJob> jobs;
     int64_t piece = 0;
     for (int j0 = 0; j0 < nfeats; j0 += cols_piece) {
@@ -634,6 +626,54 @@ static int upload_binarize_f64(hipStream_t s, const double *x, int64_t nobs, int
     }
     HIPCHK(hipStreamSynchronize(s));
     return EVT_OK;
+}
+
+// nbytes from the caller's memory to the device: large host buffers go through the pinned buffers (see upload_binarize_f64),
+// everything else is a plain copy.  The data has arrived when the call returns.
+static int upload_bytes(hipStream_t s, const void *src, void *dst, size_t nbytes) {
+    hipPointerAttribute_t attr;
+    const bool on_dev = (hipPointerGetAttributes(&attr, src) == hipSuccess) && attr.type == hipMemoryTypeDevice;
+    (void)hipGetLastError();
+    const int nworkers = on_dev ? 0 : upload_workers((int64_t)nbytes);
+    if (nworkers <= 1) {
+        HIPCHK(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDefault, s));
+        HIPCHK(hipStreamSynchronize(s));
+        return EVT_OK;
+    }
+    UploadSlots U;
+    int r = U.init((size_t)UPLOAD_PIECE, false);
+    if (r != EVT_OK) return r;
+    CopyPool pool(nworkers);
+    std::vector<CopyJob> jobs(1);
+    int64_t piece = 0;
+    for (size_t o = 0; o < nbytes; o += (size_t)UPLOAD_PIECE, piece++) {
+        const size_t n = std::min((size_t)UPLOAD_PIECE, nbytes - o);
+        const int k = (int)(piece % UploadSlots::NS);
+        if (piece >= UploadSlots::NS) HIPCHK(hipEventSynchronize(U.ev[k]));
+        jobs[0] = {static_cast<const char *>(src) + o, static_cast<char *>(U.host[k]), n};
+        pool.copy(jobs);
+        HIPCHK(hipMemcpyAsync(static_cast<char *>(dst) + o, U.host[k], n, hipMemcpyHostToDevice, s));
+        HIPCHK(hipEventRecord(U.ev[k], s));
+    }
+    HIPCHK(hipStreamSynchronize(s));
+    return EVT_OK;
+}
+
+extern "C" int evt_set_xbin(evt_handle c, const uint8_t *x_bin_colmajor) {
+    return guarded([&]() -> int {
+    CTXCHK(c);
+    ARGCHK(x_bin_colmajor, "x_bin is NULL");
+    c->have_xbin = false;
+    c->planes_ready = false;
+    int ru = upload_bytes(c->stream, x_bin_colmajor, c->xcm, (size_t)c->N * c->F);
+    if (ru != EVT_OK) return ru;
+    int r = launch_transpose_validate(c);
+    if (r != EVT_OK) return r;
+    r = check_errflag(c, "x_bin holds values outside 1..nbins");
+    if (r != EVT_OK) return r;
+    c->have_xbin = true;
+    return EVT_OK;
+    });
 }
 
 extern "C" int evt_binarize_f64(evt_handle c, const double *x_colmajor, const double *edges, const int32_t *edge_off) {
@@ -1653,7 +1693,7 @@ static int predict_common(int64_t nobs, int32_t nfeats, const uint8_t *x_bin, co
     if (out_in_place) d_out = out;
     else if (e == hipSuccess && !leaf_out) e = hipMalloc((void **)&d_out, sizeof(float) * (size_t)nobs * K);
     if (e == hipSuccess && leaf_out) e = hipMalloc((void **)&d_leaf, sizeof(uint32_t) * (size_t)nobs * ntrees);
-    if (e == hipSuccess && !x_f64 && !x_in_place) e = hipMemcpy(d_x, x_bin, (size_t)nobs * nfeats, hipMemcpyDefault);
+    if (e == hipSuccess && !x_f64 && !x_in_place) r = upload_bytes(s, x_bin, d_x, (size_t)nobs * nfeats);
     if (e == hipSuccess && x_f64) {
         // binarize on the device: the matrix goes up in pieces through pinned buffers and is binned into place
         double *d_xf = nullptr, *d_edges = nullptr;

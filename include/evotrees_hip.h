@@ -21,10 +21,10 @@
  *    stream.  Calls on one handle must not overlap; different handles may be used from
  *    different threads.
  *  - The library installs no signal handlers and never calls back into the caller's runtime.
- *    The two calls that take a Float64 matrix from host memory (evt_binarize_f64,
- *    evt_predict_f64) copy it into pinned memory with up to six worker threads of their own,
- *    which only copy memory and are joined before the call returns; no other call starts a
- *    thread.
+ *    The calls that take a whole matrix from host memory (evt_binarize_f64, evt_predict_f64,
+ *    and evt_set_xbin / evt_predict from 64 MB up) copy it into pinned memory with up to six
+ *    worker threads of their own, which only copy memory and are joined before the call
+ *    returns; no other call starts a thread.
  */
 #ifndef EVOTREES_HIP_H
 #define EVOTREES_HIP_H
