@@ -10,7 +10,9 @@
 //             counts lefts;
 //   next    : one block scans the chunk counts, sets the children's segments, picks which child
 //             is built (fewer rows; tie -> left, src/fit.jl:123-129) and writes the next level's
-//             tables (active nodes, chunk prefix, build list);
+//             tables (active nodes, chunk prefix, build list); it is the last block of the scatter
+//             kernel, except that inputs with thousands of chunks scan the counts in a kernel of
+//             its own before the scatter;
 //   scatter : one block per chunk moves row ids to their stable destination; chunks of nodes that
 //             became leaves record the node id per row (and add the leaf value to the prediction).
 // No host round trip is needed between levels.
@@ -217,15 +219,16 @@ __device__ void block_excl_scan2(long long va, long long vb, long long *pa, long
 }
 
 // One block turns the chunk counts of a level into the next level's tables (children's segments, which child is
-// built, active nodes, chunk prefix, build list).  It rides along as the last block of the scatter kernel, whose other
-// blocks need nothing from it: they add up the chunk counts of their own node themselves.  Loads that do not depend on
-// each other are issued together (fixed-trip loops over clamped indices instead of data-dependent ones).
-__device__ void level_next_block(const NextArgs &A, long long *s_tmp /* [34] */) {
+// built, active nodes, chunk prefix, build list), in two halves: the scan of the chunk counts (A) and the tables (B).  It
+// rides along as the last block of the scatter kernel, whose other blocks need nothing from it: they add up the chunk
+// counts of their own node themselves - or, with thousands of chunks per level, read the counts scanned by half A in a
+// kernel of its own just before, while half B runs beside them.  Loads that do not depend on each other are issued
+// together (fixed-trip loops over clamped indices instead of data-dependent ones).
+// A: exclusive scan of the chunks' left counts (chunk_lpre[c] = lefts in the chunks before c, chunk_lpre[n_chunks] = all)
+__device__ void chunk_scan_block(const NextArgs &A, long long *s_tmp /* [34] */) {
     const int tid = threadIdx.x, nthr = blockDim.x;
-    const int n_act = (int)A.hdr[LH_N_ACT];
     const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
     long long total;
-    // A: exclusive scan of the chunks' left counts
     {
         constexpr int SP = 8;
         const int64_t span = (n_chunks + nthr - 1) / nthr;
@@ -255,8 +258,12 @@ __device__ void level_next_block(const NextArgs &A, long long *s_tmp /* [34] */)
         }
         if (tid == 0) A.chunk_lpre[n_chunks] = total;
     }
-    __syncthreads();
-    // B: children segments + three scans over the active nodes (children count, chunks, build rows)
+}
+
+// B: children segments + three scans over the active nodes (children count, chunks, build rows) -> the next level's tables
+__device__ void level_tables_block(const NextArgs &A, long long *s_tmp /* [34] */) {
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int n_act = (int)A.hdr[LH_N_ACT];
     const int span = (n_act + nthr - 1) / nthr;
     const int i0 = tid * span, i1 = (i0 + span < n_act) ? i0 + span : n_act;
     long long s_pos = 0, s_chunks = 0, s_brows = 0;
@@ -311,11 +318,19 @@ __device__ void level_next_block(const NextArgs &A, long long *s_tmp /* [34] */)
     }
 }
 
-// The same bookkeeping as a kernel of its own (one block of 1024 threads), for inputs with thousands of chunks per level,
-// where every scatter block adding up its node's chunk counts would cost more than this launch.
-__global__ __launch_bounds__(1024) void k_level_next(NextArgs A) {
+// both halves by one block: the form that rides along in the scatter kernel for inputs of up to a thousand chunks per level
+__device__ void level_next_block(const NextArgs &A, long long *s_tmp /* [34] */) {
+    chunk_scan_block(A, s_tmp);
+    __syncthreads();
+    level_tables_block(A, s_tmp);
+}
+
+// Inputs with thousands of chunks per level: the scan of the chunk counts is a kernel of its own (one block of 1024 threads)
+// between the count and the scatter pass - every scatter block adding up its node's chunk counts would cost more than this
+// launch - and only the next level's tables, which no scatter block reads, ride along in the scatter kernel.
+__global__ __launch_bounds__(1024) void k_chunk_scan(NextArgs A) {
     __shared__ long long s_tmp[34];
-    level_next_block(A, s_tmp);
+    chunk_scan_block(A, s_tmp);
 }
 
 // HNA > 0: the pass also builds the next level's histograms (update_hist!, src/fit-utils.jl:345-394) for inputs whose
@@ -329,9 +344,12 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A, NextArgs NX) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     __shared__ long long s_tmp[34];
     extern __shared__ unsigned long long s_H[]; // HNA > 0: [HNA][sampled features][bins]
-    const bool fold = A.fold != 0;
-    if (fold && blockIdx.x == gridDim.x - 1) { // the level's bookkeeping, beside the blocks that move the rows
-        level_next_block(NX, s_tmp);
+    // fold 1: the level's bookkeeping rides along whole and the blocks add up their node's chunk counts themselves;
+    // fold 2: the chunk counts were scanned by k_chunk_scan, only the next level's tables ride along
+    const bool fold = A.fold == 1;
+    if (blockIdx.x == gridDim.x - 1) { // the level's bookkeeping, beside the blocks that move the rows
+        if (fold) level_next_block(NX, s_tmp);
+        else level_tables_block(NX, s_tmp);
         return;
     }
     // the 16 features of a record -> LDS word of their first bin (bins are 1-based); vmask bit t: feature t is sampled
@@ -348,7 +366,7 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A, NextArgs NX) {
         }
         for (int i = tid; i < HNA * plane; i += 256) s_H[i] = 0ull;
     }
-    const int64_t G = fold ? gridDim.x - 1 : gridDim.x;
+    const int64_t G = gridDim.x - 1;
     uint4 cd = A.cdesc[blockIdx.x];
     const int64_t n_chunks = A.hdr[LH_N_CHUNKS];
     __shared__ unsigned long long s_w[EVT_CHUNK_WORDS];
@@ -372,9 +390,10 @@ __global__ __launch_bounds__(256) void k_part_scatter(PartArgs A, NextArgs NX) {
                 sum_node += v;
                 sum_before += (k < c) ? v : 0;
             }
-        } else { // the bookkeeping kernel ran before this one: prefix of the chunk counts, children's sizes
-            sum_before = A.chunk_lpre[c] - A.chunk_lpre[c0];
-            sum_node = A.seg_len[2 * n];
+        } else { // the chunk counts were scanned before this kernel (the children's sizes are being written beside it)
+            const long long l0 = A.chunk_lpre[c0];
+            sum_before = A.chunk_lpre[c] - l0;
+            sum_node = A.chunk_lpre[c1] - l0;
         }
         constexpr int NI = EVT_CHUNK / 256;
         uint32_t rid[NI];
@@ -910,12 +929,12 @@ int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t 
     NextArgs NX;
     fill_next_args(c, level, NX);
     // up to a thousand chunks per level the bookkeeping rides along in the scatter kernel (one launch less per level)
-    A.fold = c->max_chunks <= 1024 + c->maxlvl ? 1 : 0;
-    if (!A.fold) {
-        hipLaunchKernelGGL(k_level_next, dim3(1), dim3(1024), 0, c->stream, NX);
+    A.fold = c->max_chunks <= 1024 + c->maxlvl ? 1 : 2;
+    if (A.fold == 2) {
+        hipLaunchKernelGGL(k_chunk_scan, dim3(1), dim3(1024), 0, c->stream, NX);
         HIPCHK(hipGetLastError());
     }
-    const dim3 grid(grid_for_chunks(c->max_chunks) + (A.fold ? 1 : 0));
+    const dim3 grid(grid_for_chunks(c->max_chunks) + 1);
     if (c->step.hist_fused) {
         // the next level's histograms are built here: no histogram kernel runs at that level
         A.xrm = c->xrm;
@@ -927,7 +946,7 @@ int launch_part_scatter(evt_ctx *c, int level, const uint32_t *is_cur, uint32_t 
         A.nfs = c->n_js_last;
         A.NAg = c->NAg;
         const size_t lds = (size_t)c->NA * c->n_js_last * c->B * 8;
-        if (!A.fold || !scatter_can_build_hist(c, c->n_js_last)) {
+        if (A.fold != 1 || !scatter_can_build_hist(c, c->n_js_last)) {
             evt_set_error("internal: scatter pass cannot build histograms for this shape");
             return EVT_ERR_STATE;
         }
