@@ -268,7 +268,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     memset(&c->tree, 0, sizeof(c->tree));
     c->tree_blob = nullptr;
     memset(c->lvl, 0, sizeof(c->lvl));
-    c->js = nullptr; c->jsmap = nullptr; c->feattypes = nullptr; c->mono = nullptr; c->absmax = nullptr; c->qexp = nullptr; c->qbits = nullptr;
+    c->js = nullptr; c->jsmap = nullptr; c->feattypes = nullptr; c->mono = nullptr; c->absmax = nullptr; c->absmax_cur = 0; c->qexp = nullptr; c->qbits = nullptr;
     c->alphas = nullptr; c->alphas_f = nullptr; c->qkeys_a = c->qkeys_b = nullptr; c->qtemp = nullptr; c->qtemp_bytes = 0;
     c->n_alphas = 1;
     for (int k = 0; k < EVT_MAX_K; k++) c->h_alphas[k] = 0.5;
@@ -384,7 +384,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ALLOC(c->jsmap, c->RS);
     ALLOC(c->feattypes, c->F);
     ALLOC(c->mono, c->F);
-    ALLOC(c->absmax, EVT_ABSMAX_STRIPES * EVT_MC_MAX_NK);
+    ALLOC(c->absmax, 2 * EVT_ABSMAX_STRIPES * EVT_MC_MAX_NK);
     ALLOC(c->alphas, EVT_MAX_K);
     ALLOC(c->alphas_f, EVT_MAX_K);
     for (int s = 0; s < 2; s++) {
@@ -423,7 +423,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
         c->h_feattypes = ft;
         hipError_t e2 = hipMemcpy(c->feattypes, ft.data(), c->F, hipMemcpyHostToDevice);
         if (e2 == hipSuccess) e2 = hipMemset(c->mono, 0, sizeof(int32_t) * c->F);
-        if (e2 == hipSuccess) e2 = hipMemset(c->absmax, 0, sizeof(uint32_t) * EVT_ABSMAX_STRIPES * EVT_MC_MAX_NK);
+        if (e2 == hipSuccess) e2 = hipMemset(c->absmax, 0, sizeof(uint32_t) * 2 * EVT_ABSMAX_STRIPES * EVT_MC_MAX_NK);
         if (e2 == hipSuccess) e2 = hipMemset(c->nidx, 0, sizeof(uint32_t) * N);
         if (e2 == hipSuccess) e2 = hipMemset(c->errflag, 0, sizeof(int32_t));
         if (e2 == hipSuccess) e2 = upload_alphas(c);

@@ -123,7 +123,8 @@ struct evt_ctx {
     uint16_t *jsmap;   // [RS] slot of feature f (0-based), 0xFFFF = not sampled / padding
     uint8_t *feattypes;
     int32_t *mono;
-    uint32_t *absmax;  // [EVT_ABSMAX_STRIPES][EVT_MC_MAX_NK] float bits
+    uint32_t *absmax;  // [2][EVT_ABSMAX_STRIPES][EVT_MC_MAX_NK] float bits: two sets, raised by alternate gradient passes
+    int absmax_cur;    // the set the next gradient pass raises
     // quantile losses: levels (Float64 for the gradients, Float32 for the metrics) and the sort buffers of the leaf pass
     double h_alphas[EVT_MAX_K];
     int32_t n_alphas;

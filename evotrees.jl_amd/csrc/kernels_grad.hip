@@ -8,6 +8,7 @@
 // first thing the next gradient pass does (4 B of node id read and 4K B written more per row) - or in
 // k_apply_leaf when something else needs the predictions first.
 #include "evt_internal.h"
+#include <algorithm>
 
 __device__ __forceinline__ float wave_max_f32(float v) {
 #pragma unroll
@@ -44,7 +45,7 @@ __device__ __forceinline__ void mle2p_grad_hess(float loc, float raw, float y, f
 // Raises the running maximum of gradient row k.  Same-address atomics from thousands of blocks queue up one behind the
 // other (about 20 ns each - 40 us for the 2048 blocks of a gradient pass), so the maximum is kept in
 // EVT_ABSMAX_STRIPES copies on different cache lines, a block raises the copy its index selects, and the one reader
-// (k_quant_setup) takes the largest.  The value only grows while a pass runs: a block whose own maximum is already
+// (the quantisation pass, k_quantize) takes the largest.  The value only grows while a pass runs: a block whose own maximum is already
 // covered by what a device-scope load shows skips the atomic.
 __device__ __forceinline__ void absmax_raise(uint32_t *absmax, int k, float m) {
     if (!(m > 0.0f)) return;
@@ -334,51 +335,61 @@ __global__ __launch_bounds__(256) void k_absmax(const float *__restrict__ grad, 
     }
 }
 
-// qexp[k] = ilogb(max) + 1 (0 for an all-zero row); qmul[k] = 2^(qbits-qexp) encodes, qscale decodes.
-// The maxima of the rows the gradient kernel rewrites every round are cleared for its next pass once they are read;
-// the weight row (last) is written once and keeps its maximum.
-__global__ void k_quant_setup(uint32_t *absmax, const int32_t *qbits, int32_t *qexp, double *qmul, double *qscale_g,
-                              int NK, int NAg, int loss, int unit_w) {
-    int k = threadIdx.x;
-    if (k < NK) {
+// Quantisation tables of a gradient pass and the fixed-point words the histogram kernel adds, in one kernel.
+// qexp[k] = ilogb(max |row k|) + 1 (0 for an all-zero row); qmul[k] = 2^(qbits - qexp) encodes, qscale decodes.  Every block
+// derives the multipliers from the striped maxima itself (a few dozen cached loads: no kernel of its own in front of this one);
+// block 0 also writes the tables for the readers that follow (split search, read-back).  The maxima live in two sets: a
+// gradient pass raises one, this kernel reads it and clears the other - which nobody uses at that moment - for the next pass,
+// so no pass starts from maxima an earlier one left behind.  The weight row (last) is written once and keeps its maximum.
+// Plane a of gq holds, per row, q = rint(v * 2^(qbits - qexp)) of gradient row chan_k[a]; with unit weights plane 0 also carries
+// the row count in its low 16 bits ((q << 16) + 1) so that one 64-bit LDS add serves both.
+// Channel a reads gradient row a, except for mse whose channels are {g, w} = rows {0, 2}.
+__global__ __launch_bounds__(256) void k_quantize(const float *__restrict__ grad, unsigned long long *__restrict__ gq, int64_t N,
+                                                 int NK, int NA, int mse, int pack, const uint32_t *__restrict__ absmax, uint32_t *absmax_next,
+                                                 const int32_t *__restrict__ qbits, int32_t *qexp, double *qmul, double *qscale_g, int NAg,
+                                                 int loss, int unit_w) {
+    __shared__ double s_qmul[EVT_MC_MAX_NK];
+    __shared__ int s_qexp[EVT_MC_MAX_NK], s_qbits[EVT_MC_MAX_NK];
+    const int t = threadIdx.x;
+    if (t < NK) {
         uint32_t mu = 0u;
         for (int st = 0; st < EVT_ABSMAX_STRIPES; st++) {
-            const uint32_t v = absmax[st * EVT_MC_MAX_NK + k]; // non-negative floats order as their bit patterns
+            const uint32_t v = absmax[st * EVT_MC_MAX_NK + t]; // non-negative floats order as their bit patterns
             mu = v > mu ? v : mu;
         }
-        float m = __uint_as_float(mu);
+        const float m = __uint_as_float(mu);
         int e = 0;
         if (m > 0.0f) {
             e = ilogbf(m) + 1;
             if (e > 128) e = 128;
             if (e < -140) e = -140;
         }
-        qexp[k] = e;
-        qmul[k] = scalbn(1.0, qbits[k] - e);
-        if (k < NK - 1)
-            for (int st = 0; st < EVT_ABSMAX_STRIPES; st++) absmax[st * EVT_MC_MAX_NK + k] = 0u;
+        const int qb = qbits[t];
+        s_qexp[t] = e;
+        s_qbits[t] = qb;
+        s_qmul[t] = scalbn(1.0, qb - e);
     }
     __syncthreads();
-    if (k < NAg) {
-        // global channel ag -> gradient row: mse {g, w}; otherwise identity; last channel is w (or the row count)
-        int kk = EVT_TWO_CHAN(loss, (NK - 1) / 2) ? (k == 0 ? 0 : 2) : k; // one-target mse / mae: channels {g, w}
-        if (k == NAg - 1 && unit_w) qscale_g[k] = 1.0;
-        else qscale_g[k] = scalbn(1.0, qexp[kk] - qbits[kk]);
+    if (blockIdx.x == 0) {
+        if (t < NK) {
+            qexp[t] = s_qexp[t];
+            qmul[t] = s_qmul[t];
+            if (t < NK - 1)
+                for (int st = 0; st < EVT_ABSMAX_STRIPES; st++) absmax_next[st * EVT_MC_MAX_NK + t] = 0u;
+        }
+        if (t < NAg) {
+            // global channel ag -> gradient row: mse {g, w}; otherwise identity; last channel is w (or the row count)
+            const int kk = EVT_TWO_CHAN(loss, (NK - 1) / 2) ? (t == 0 ? 0 : 2) : t; // one-target mse / mae: channels {g, w}
+            if (t == NAg - 1 && unit_w) qscale_g[t] = 1.0;
+            else qscale_g[t] = scalbn(1.0, s_qexp[kk] - s_qbits[kk]);
+        }
     }
-}
-
-// Stages the fixed-point words the histogram kernel adds: plane a of gq holds, per row,
-// q = rint(v * 2^(qbits-qexp)) of gradient row chan_k[a]; with unit weights plane 0 also carries
-// the row count in its low 16 bits ((q << 16) + 1) so that one 64-bit LDS add serves both.
-// Channel a reads gradient row a, except for mse whose channels are {g, w} = rows {0, 2}.
-__global__ __launch_bounds__(256) void k_quantize(const float *__restrict__ grad, unsigned long long *__restrict__ gq, int64_t N,
-                                                 int NK, int NA, int mse, const double *__restrict__ qmul, int pack) {
-    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = (int64_t)blockIdx.x * 256 + t;
     if (i >= N) return;
     const float *g = grad + (size_t)NK * i;
     for (int a = 0; a < NA; a++) {
         const int k = (mse && a == 1) ? 2 : a;
-        long long q = __double2ll_rn((double)g[k] * qmul[k]);
+        long long q = __double2ll_rn((double)g[k] * s_qmul[k]);
         if (a == 0 && pack) { // 30 bits: staged as a 32-bit word, widened to (q << 16) + 1 (the row count) by the histogram kernel
             reinterpret_cast<int32_t *>(gq)[i] = (int32_t)q;
             continue;
@@ -387,8 +398,12 @@ __global__ __launch_bounds__(256) void k_quantize(const float *__restrict__ grad
     }
 }
 
+// the set of striped maxima the next gradient pass raises (and the quantisation behind it reads)
+static uint32_t *absmax_set(evt_ctx *c, int which) { return c->absmax + (size_t)which * EVT_ABSMAX_STRIPES * EVT_MC_MAX_NK; }
+
 int launch_grads(evt_ctx *c) {
-    // absmax of the rows this kernel writes starts from zero (cleared at creation and by k_quant_setup after every use)
+    // the maxima of the rows this kernel writes start from zero (cleared at creation and by the quantisation pass before last)
+    uint32_t *const am = absmax_set(c, c->absmax_cur);
     int64_t nb = (c->N + 255) / 256;
     if (nb > 2048) nb = 2048;
     dim3 grid((unsigned)nb);
@@ -396,13 +411,13 @@ int launch_grads(evt_ctx *c) {
     c->pend_pred = false;
     if (EVT_IS_QUANTILE(c->loss)) {
         hipLaunchKernelGGL(k_grads_quantile, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->loss == EVT_LOSS_MULTIQUANTILE ? 1 : 0,
-                           c->alphas, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+                           c->alphas, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
         HIPCHK(hipGetLastError());
         return EVT_OK;
     }
     const bool multi_target = c->loss != EVT_LOSS_MLOGLOSS && c->K > (EVT_IS_MLE2P(c->loss) ? 2 : 1);
     if (multi_target) {
-#define MT(L_) hipLaunchKernelGGL(k_grads_mt<L_>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0)
+#define MT(L_) hipLaunchKernelGGL(k_grads_mt<L_>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, am, pn, c->tree.pred, c->unit_w ? 1 : 0)
         switch (c->loss) {
         case EVT_LOSS_MSE: MT(0); break;
         case EVT_LOSS_LOGLOSS: MT(1); break;
@@ -420,25 +435,25 @@ int launch_grads(evt_ctx *c) {
         return EVT_OK;
     }
     if (c->loss == EVT_LOSS_MSE)
-        hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<0>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_LOGLOSS)
-        hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<1>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_LOGISTIC_MLE)
-        hipLaunchKernelGGL(k_grads<7>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<7>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_GAUSSIAN_MLE)
-        hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<2>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_POISSON)
-        hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<3>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_GAMMA)
-        hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<4>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_MAE)
-        hipLaunchKernelGGL(k_grads<8>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<8>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (EVT_IS_CRED(c->loss))
-        hipLaunchKernelGGL(k_grads<9>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<9>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else if (c->loss == EVT_LOSS_MLOGLOSS)
-        hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads_mlogloss, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->K, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     else
-        hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, c->absmax, pn, c->tree.pred, c->unit_w ? 1 : 0);
+        hipLaunchKernelGGL(k_grads<5>, grid, dim3(256), 0, c->stream, c->pred, c->y, c->grad, c->N, am, pn, c->tree.pred, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -480,14 +495,20 @@ __global__ void k_absmax_clear(uint32_t *absmax, int k0, int k1) {
     for (int i = threadIdx.x; i < n * EVT_ABSMAX_STRIPES; i += blockDim.x) absmax[(i / n) * EVT_MC_MAX_NK + k0 + i % n] = 0u;
 }
 
-// absmax over rows [k0, k1) of the current gradient matrix
+// absmax over rows [k0, k1) of the current gradient matrix, into the set the next quantisation reads; the weight row's
+// maximum (row NK - 1) is kept in both sets, since no gradient pass renews it
 int launch_absmax_rows(evt_ctx *c, int k0, int k1) {
-    hipLaunchKernelGGL(k_absmax_clear, dim3(1), dim3(256), 0, c->stream, c->absmax, k0, k1);
-    HIPCHK(hipGetLastError());
     int64_t nb = (c->N + 255) / 256;
     if (nb > 2048) nb = 2048;
-    hipLaunchKernelGGL(k_absmax, dim3((unsigned)nb), dim3(256), 0, c->stream, c->grad, c->N, c->NK, k0, k1, c->absmax);
-    HIPCHK(hipGetLastError());
+    for (int pass = 0; pass < 2; pass++) {
+        uint32_t *am = absmax_set(c, pass == 0 ? c->absmax_cur : c->absmax_cur ^ 1);
+        const int a0 = pass == 0 ? k0 : std::max(k0, c->NK - 1);
+        if (a0 >= k1) continue;
+        hipLaunchKernelGGL(k_absmax_clear, dim3(1), dim3(256), 0, c->stream, am, a0, k1);
+        HIPCHK(hipGetLastError());
+        hipLaunchKernelGGL(k_absmax, dim3((unsigned)nb), dim3(256), 0, c->stream, c->grad, c->N, c->NK, a0, k1, am);
+        HIPCHK(hipGetLastError());
+    }
     return EVT_OK;
 }
 
@@ -497,12 +518,11 @@ int launch_quantize(evt_ctx *c) {
     c->qexp = c->qexp_buf[c->q_cur];
     c->qscale = c->qscale_buf[c->q_cur];
     double *qmul = c->qscale + EVT_MC_MAX_NK; // decode scales per global channel first, then encode multipliers per gradient row
-    hipLaunchKernelGGL(k_quant_setup, dim3(1), dim3(64), 0, c->stream, c->absmax, c->qbits, c->qexp, qmul, c->qscale, c->NK, c->NAg,
-                       c->loss, c->unit_w ? 1 : 0);
-    HIPCHK(hipGetLastError());
     hipLaunchKernelGGL(k_quantize, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, c->gq, c->N, c->NK, c->NA,
-                       EVT_TWO_CHAN(c->loss, c->K) ? 1 : 0, qmul, c->unit_w ? 1 : 0);
+                       EVT_TWO_CHAN(c->loss, c->K) ? 1 : 0, c->unit_w ? 1 : 0, absmax_set(c, c->absmax_cur), absmax_set(c, c->absmax_cur ^ 1),
+                       c->qbits, c->qexp, qmul, c->qscale, c->NAg, c->loss, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
+    c->absmax_cur ^= 1; // the next gradient pass raises the set this kernel cleared
     return EVT_OK;
 }
 
