@@ -384,17 +384,18 @@ __global__ __launch_bounds__(256) void k_quantize(const float *__restrict__ grad
             else qscale_g[t] = scalbn(1.0, s_qexp[kk] - s_qbits[kk]);
         }
     }
-    const int64_t i = (int64_t)blockIdx.x * 256 + t;
-    if (i >= N) return;
-    const float *g = grad + (size_t)NK * i;
-    for (int a = 0; a < NA; a++) {
-        const int k = (mse && a == 1) ? 2 : a;
-        long long q = __double2ll_rn((double)g[k] * s_qmul[k]);
-        if (a == 0 && pack) { // 30 bits: staged as a 32-bit word, widened to (q << 16) + 1 (the row count) by the histogram kernel
-            reinterpret_cast<int32_t *>(gq)[i] = (int32_t)q;
-            continue;
+    // a block takes many rows (grid-stride), so that the prologue above is paid a couple of thousand times, not once per 256 rows
+    for (int64_t i = (int64_t)blockIdx.x * 256 + t; i < N; i += (int64_t)gridDim.x * 256) {
+        const float *g = grad + (size_t)NK * i;
+        for (int a = 0; a < NA; a++) {
+            const int k = (mse && a == 1) ? 2 : a;
+            long long q = __double2ll_rn((double)g[k] * s_qmul[k]);
+            if (a == 0 && pack) { // 30 bits: staged as a 32-bit word, widened to (q << 16) + 1 (the row count) by the histogram kernel
+                reinterpret_cast<int32_t *>(gq)[i] = (int32_t)q;
+                continue;
+            }
+            gq[(size_t)a * N + i] = (unsigned long long)q;
         }
-        gq[(size_t)a * N + i] = (unsigned long long)q;
     }
 }
 
@@ -518,7 +519,7 @@ int launch_quantize(evt_ctx *c) {
     c->qexp = c->qexp_buf[c->q_cur];
     c->qscale = c->qscale_buf[c->q_cur];
     double *qmul = c->qscale + EVT_MC_MAX_NK; // decode scales per global channel first, then encode multipliers per gradient row
-    hipLaunchKernelGGL(k_quantize, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, c->gq, c->N, c->NK, c->NA,
+    hipLaunchKernelGGL(k_quantize, dim3((unsigned)std::min<int64_t>(4096, (c->N + 255) / 256)), dim3(256), 0, c->stream, c->grad, c->gq, c->N, c->NK, c->NA,
                        EVT_TWO_CHAN(c->loss, c->K) ? 1 : 0, c->unit_w ? 1 : 0, absmax_set(c, c->absmax_cur), absmax_set(c, c->absmax_cur ^ 1),
                        c->qbits, c->qexp, qmul, c->qscale, c->NAg, c->loss, c->unit_w ? 1 : 0);
     HIPCHK(hipGetLastError());
