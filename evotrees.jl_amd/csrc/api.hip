@@ -303,6 +303,8 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->mask_next = nullptr;
     c->copy_stream = nullptr;
     c->mask_next_valid = false;
+    c->mask_seed_valid = false;
+    c->mask_seed = 0;
     c->grads_ahead = false;
     c->grads_ready = false;
     c->last_cond = 255;
@@ -993,8 +995,14 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
     prof_begin(c, EVT_K_OTHER, 0);
     r = launch_apply_pending(c); // an earlier tree's values go in before its node ids are overwritten
     if (r != EVT_OK) return r;
-    if (mask_staged) { // uploaded by evt_stage_mask, which waited for the copy: the two buffers change places
-        std::swap(c->mask, c->mask_next);
+    bool draw = false;
+    if (mask_staged) {
+        if (c->mask_seed_valid) { // evt_draw_mask: the compaction pass below draws the bytes into the mask buffer
+            draw = true;
+            c->mask_seed_valid = false;
+        } else { // uploaded by evt_stage_mask, which waited for the copy: the two buffers change places
+            std::swap(c->mask, c->mask_next);
+        }
         c->mask_next_valid = false;
     }
     if (!all_rows) {
@@ -1002,10 +1010,10 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
             HIPCHK(hipMemcpyAsync(c->mask, mask, c->N, hipMemcpyDefault, c->stream));
             HIPCHK(hipStreamSynchronize(c->stream)); // the caller may reuse its mask buffer as soon as this call returns
         }
-        r = launch_compact_mask(c, cond);
+        r = launch_compact_mask(c, cond, draw, c->mask_seed);
         if (r == EVT_OK && rec_nidx) r = launch_fill_u32(c, c->nidx, 0u, c->N);
     }
-    if (r == EVT_OK) r = launch_tree_begin(c, all_rows);
+    if (r == EVT_OK && all_rows) r = launch_tree_begin(c); // with a row sample the compaction above has set the tree up
     prof_end(c);
     if (r != EVT_OK) return r;
 
@@ -1186,6 +1194,7 @@ extern "C" int evt_stage_mask(evt_handle c, const uint8_t *mask) {
         if (r != EVT_OK) return r;
     }
     c->mask_next_valid = false;
+    c->mask_seed_valid = false; // an uploaded mask replaces a seed given before
     HIPCHK(hipMemcpyAsync(c->mask_next, mask, c->N, hipMemcpyDefault, c->copy_stream));
     HIPCHK(hipStreamSynchronize(c->copy_stream)); // the caller may reuse its buffer; the tree in flight keeps running
     c->mask_next_valid = true;
@@ -1198,13 +1207,10 @@ extern "C" int evt_stage_mask(evt_handle c, const uint8_t *mask) {
 extern "C" int evt_draw_mask(evt_handle c, uint64_t seed) {
     return guarded([&]() -> int {
     CTXCHK_QUEUE(c);
-    if (!c->mask_next) {
-        int r = dev_alloc(&c->mask_next, (size_t)c->N);
-        if (r != EVT_OK) return r;
-    }
-    c->mask_next_valid = false;
-    int r = launch_draw_mask(c, c->mask_next, (unsigned long long)seed);
-    if (r != EVT_OK) return r;
+    // nothing is queued here: the bytes are drawn by the next staged tree's compaction pass, which writes them into the
+    // mask buffer on its way (in stream order behind whatever still reads that buffer)
+    c->mask_seed = (unsigned long long)seed;
+    c->mask_seed_valid = true;
     c->mask_next_valid = true;
     return EVT_OK;
     });

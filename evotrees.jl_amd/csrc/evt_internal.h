@@ -107,6 +107,8 @@ struct evt_ctx {
     uint8_t *mask_next;
     hipStream_t copy_stream;
     bool mask_next_valid;
+    bool mask_seed_valid;   // the next staged tree draws its mask on the device from mask_seed (evt_draw_mask) instead of using mask_next
+    unsigned long long mask_seed;
     unsigned long long *flagw;
     int32_t *chunk_nleft;
     int64_t *chunk_lpre;
@@ -328,10 +330,9 @@ int launch_binarize_cols(hipStream_t s, const double *x_dev, const double *edges
                          int F, int64_t ldx, int64_t ldo);
 int launch_eval_metric(evt_ctx *c, int metric, double *partial);
 // tree
-int launch_tree_begin(evt_ctx *c, bool all_rows);
+int launch_tree_begin(evt_ctx *c);
 int launch_iota(evt_ctx *c, uint32_t *dst, int64_t n);
-int launch_compact_mask(evt_ctx *c, uint8_t cond);
-int launch_draw_mask(evt_ctx *c, uint8_t *mask, unsigned long long seed);
+int launch_compact_mask(evt_ctx *c, uint8_t cond, bool draw, unsigned long long seed);
 int quantile_leaf_buffers(evt_ctx *c);
 int launch_quantile_leaves(evt_ctx *c, const evt_params *p);
 int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur);

@@ -627,9 +627,12 @@ struct BeginArgs {
     int js_words, map_words;
 };
 
-__global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) {
-    const int tid = threadIdx.x;
-    for (int n = tid; n < A.nnodes; n += 1024) {
+// One block prepares a tree: empty Tree arrays, node states, the root's histogram slice, the first level's tables, the
+// column sample.  A kernel of its own for a tree on every row; with a row sample it is the last block of the kernel that
+// compacts the sampled rows (k_mask_scatter), which hands it the number of rows kept.
+__device__ void tree_begin_block(BeginArgs A) {
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    for (int n = tid; n < A.nnodes; n += nthr) {
         A.tree.feat[n] = 0;
         A.tree.cond_bin[n] = 0;
         A.tree.w[n] = 0.0f;
@@ -638,11 +641,11 @@ __global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) {
         A.tree.packed[n] = 0u;
         for (int k = 0; k < A.K; k++) A.tree.pred[(int64_t)A.K * n + k] = 0.0f;
     }
-    for (int n = tid; n < A.nnodes + 2; n += 1024) A.status[n] = ST_INACTIVE;
-    for (int64_t i = tid; i < A.root_words; i += 1024) A.hist[i] = 0;
-    for (int d = tid; d <= A.D; d += 1024) A.stats[d] = 0;
-    for (int i = tid; i < A.js_words; i += 1024) A.js_dst[i] = A.js_src[i];
-    for (int i = tid; i < A.map_words; i += 1024) A.map_dst[i] = A.map_src[i];
+    for (int n = tid; n < A.nnodes + 2; n += nthr) A.status[n] = ST_INACTIVE;
+    for (int64_t i = tid; i < A.root_words; i += nthr) A.hist[i] = 0;
+    for (int d = tid; d <= A.D; d += nthr) A.stats[d] = 0;
+    for (int i = tid; i < A.js_words; i += nthr) A.js_dst[i] = A.js_src[i];
+    for (int i = tid; i < A.map_words; i += nthr) A.map_dst[i] = A.map_src[i];
     __syncthreads();
     if (tid == 0) {
         if (A.n_is_dev) A.n_is = *A.n_is_dev;
@@ -664,6 +667,8 @@ __global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) {
     }
 }
 
+__global__ __launch_bounds__(1024) void k_tree_begin(BeginArgs A) { tree_begin_block(A); }
+
 // ---- row subsampling: is = rows with mask <= cond, ascending (src/subsample.jl:6-38) -----------
 __device__ __forceinline__ int wave_sum_i32(int v) {
 #pragma unroll
@@ -672,8 +677,14 @@ __device__ __forceinline__ int wave_sum_i32(int v) {
 }
 
 // A thread takes 8 consecutive mask bytes (one load); the 8 flags of 8 neighbouring threads make one 64-row flag word.
-__global__ __launch_bounds__(256) void k_mask_count(const uint8_t *mask, uint8_t cond, int64_t N, int64_t n_chunks,
-                                                   unsigned long long *flagw, int32_t *chunk_nleft) {
+// DRAW: the bytes are not read but drawn here and written to `mask` on the way: the mask's 8-byte word w is output w of
+// SplitMix64 (Steele, Lea, Flood 2014: a Weyl sequence with increment 0x9E3779B97F4A7C15 passed through two
+// multiply-xorshift rounds) started at state `seed`, stored little end first - byte i of the mask is bits 8*(i%8).. of output
+// i/8.  Stands in for rand!(rng, mask) of src/subsample.jl:7 when the caller accepts a counter-based stream keyed by one 64-bit
+// draw of its own generator per tree.
+template <bool DRAW>
+__global__ __launch_bounds__(256) void k_mask_count(uint8_t *mask, uint8_t cond, int64_t N, int64_t n_chunks,
+                                                   unsigned long long *flagw, int32_t *chunk_nleft, unsigned long long seed) {
     static_assert(EVT_CHUNK == 2048 && EVT_CHUNK_WORDS == 32, "a chunk is 256 threads x 8 bytes");
     const int tid = threadIdx.x;
     __shared__ unsigned long long s_w[EVT_CHUNK_WORDS];
@@ -681,7 +692,18 @@ __global__ __launch_bounds__(256) void k_mask_count(const uint8_t *mask, uint8_t
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
         const int64_t p0 = c * EVT_CHUNK + (int64_t)tid * 8;
         unsigned long long v = ~0ull; // bytes past the end read as 255
-        if (p0 + 8 <= N) {
+        if (DRAW) {
+            unsigned long long z = seed + (unsigned long long)((p0 >> 3) + 1) * 0x9E3779B97F4A7C15ull;
+            z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+            z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+            z ^= z >> 31;
+            v = z;
+            if (p0 + 8 <= N) {
+                *reinterpret_cast<unsigned long long *>(mask + p0) = z;
+            } else {
+                for (int j = 0; p0 + j < N; j++) mask[p0 + j] = (uint8_t)(z >> (8 * j));
+            }
+        } else if (p0 + 8 <= N) {
             v = *reinterpret_cast<const unsigned long long *>(mask + p0);
         } else {
             for (int j = 0; j < 8; j++)
@@ -719,15 +741,34 @@ __global__ __launch_bounds__(1024) void k_mask_scan(const int32_t *chunk_nleft, 
 }
 
 // SELF: no k_mask_scan has run - every block adds up the counts of the chunks before its own (a few hundred values:
-// cheaper than the launch), and the block of the last chunk leaves the total where k_tree_begin reads it.
+// cheaper than the launch).
+// The last block of the grid prepares the tree that is grown on the sample (tree_begin_block), with the number of rows kept.
 template <bool SELF>
 __global__ __launch_bounds__(256) void k_mask_scatter(int64_t N, int64_t n_chunks, const unsigned long long *flagw,
-                                                     const int32_t *chunk_nleft, int64_t *chunk_lpre, uint32_t *is_out) {
+                                                     const int32_t *chunk_nleft, int64_t *chunk_lpre, uint32_t *is_out, BeginArgs B) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     __shared__ unsigned long long s_w[EVT_CHUNK_WORDS];
     __shared__ int s_pre[EVT_CHUNK_WORDS];
     __shared__ int s_sum[4];
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+    const int64_t G = (int64_t)gridDim.x - 1;
+    if ((int64_t)blockIdx.x == G) {
+        int64_t kept;
+        if (SELF) { // no scan has run: the chunk counts (a thousand at most) are added up here
+            int part = 0;
+            for (int64_t k = tid; k < n_chunks; k += 256) part += chunk_nleft[k];
+            part = wave_sum_i32(part);
+            if (lane == 0) s_sum[wave] = part;
+            __syncthreads();
+            kept = (int64_t)s_sum[0] + s_sum[1] + s_sum[2] + s_sum[3];
+        } else {
+            kept = chunk_lpre[n_chunks];
+        }
+        B.n_is = kept;
+        B.n_is_dev = nullptr;
+        tree_begin_block(B);
+        return;
+    }
+    for (int64_t c = blockIdx.x; c < n_chunks; c += G) {
         if (tid < EVT_CHUNK_WORDS) s_w[tid] = flagw[c * EVT_CHUNK_WORDS + tid];
         int64_t base;
         if (SELF) {
@@ -743,7 +784,6 @@ __global__ __launch_bounds__(256) void k_mask_scatter(int64_t N, int64_t n_chunk
         }
         if (SELF) {
             base = (int64_t)s_sum[0] + s_sum[1] + s_sum[2] + s_sum[3];
-            if (c == n_chunks - 1 && tid == 0) chunk_lpre[n_chunks] = base + chunk_nleft[c];
         } else {
             base = chunk_lpre[c];
         }
@@ -759,35 +799,6 @@ __global__ __launch_bounds__(256) void k_mask_scatter(int64_t N, int64_t n_chunk
     }
 }
 
-// The row mask drawn on the device instead of uploaded: the mask's 8-byte word w is output w of SplitMix64 (Steele,
-// Lea, Flood 2014: the state advances by the odd constant 0x9E3779B97F4A7C15 per output, each output is the state
-// passed through two multiply-xorshift rounds) started at state `seed`, stored little end first - byte i of the mask
-// is bits 8*(i%8).. of output i/8.  Stands in for rand!(rng, mask) of src/subsample.jl:7 when the caller accepts a
-// counter-based stream keyed by one 64-bit draw of its own generator per tree.
-__global__ __launch_bounds__(256) void k_draw_mask(uint8_t *mask, int64_t N, unsigned long long seed) {
-    const int64_t nwords = (N + 7) >> 3;
-    for (int64_t w = (int64_t)blockIdx.x * 256 + threadIdx.x; w < nwords; w += (int64_t)gridDim.x * 256) {
-        unsigned long long z = seed + (unsigned long long)(w + 1) * 0x9E3779B97F4A7C15ull;
-        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-        z ^= z >> 31;
-        if ((w + 1) * 8 <= N) {
-            reinterpret_cast<unsigned long long *>(mask)[w] = z;
-        } else {
-            for (int j = 0; w * 8 + j < N; j++) mask[w * 8 + j] = (uint8_t)(z >> (8 * j));
-        }
-    }
-}
-
-int launch_draw_mask(evt_ctx *c, uint8_t *mask, unsigned long long seed) {
-    const int64_t nwords = (c->N + 7) >> 3;
-    int64_t g = (nwords + 255) / 256;
-    if (g > 8192) g = 8192;
-    hipLaunchKernelGGL(k_draw_mask, dim3((unsigned)g), dim3(256), 0, c->stream, mask, c->N, seed);
-    HIPCHK(hipGetLastError());
-    return EVT_OK;
-}
-
 static unsigned grid_for_chunks(int64_t max_chunks) {
     int64_t g = max_chunks;
     if (g > 4096) g = 4096;
@@ -795,26 +806,8 @@ static unsigned grid_for_chunks(int64_t max_chunks) {
     return (unsigned)g;
 }
 
-int launch_compact_mask(evt_ctx *c, uint8_t cond) {
-    const int64_t n_chunks = (c->N + EVT_CHUNK - 1) / EVT_CHUNK;
-    unsigned g = grid_for_chunks(n_chunks);
-    hipLaunchKernelGGL(k_mask_count, dim3(g), dim3(256), 0, c->stream, c->mask, cond, c->N, n_chunks, c->flagw, c->chunk_nleft);
-    HIPCHK(hipGetLastError());
-    if (n_chunks <= 1024) { // the scatter's blocks add up the counts before their chunk themselves
-        hipLaunchKernelGGL(k_mask_scatter<true>, dim3(g), dim3(256), 0, c->stream, c->N, n_chunks, c->flagw, c->chunk_nleft, c->chunk_lpre, c->is_a);
-        HIPCHK(hipGetLastError());
-        return EVT_OK;
-    }
-    hipLaunchKernelGGL(k_mask_scan, dim3(1), dim3(1024), 0, c->stream, c->chunk_nleft, c->chunk_lpre, n_chunks);
-    HIPCHK(hipGetLastError());
-    hipLaunchKernelGGL(k_mask_scatter<false>, dim3(g), dim3(256), 0, c->stream, c->N, n_chunks, c->flagw, c->chunk_nleft, c->chunk_lpre, c->is_a);
-    HIPCHK(hipGetLastError());
-    return EVT_OK;
-}
-
-int launch_tree_begin(evt_ctx *c, bool all_rows) {
+static void fill_begin_args(evt_ctx *c, bool all_rows, BeginArgs &A) {
     const LevelTab &L = c->lvl[1];
-    BeginArgs A;
     A.tree = c->tree;
     A.status = c->status;
     A.seg_start = c->seg_start;
@@ -846,7 +839,35 @@ int launch_tree_begin(evt_ctx *c, bool all_rows) {
         A.map_dst = reinterpret_cast<uint32_t *>(c->jsmap);
         A.map_words = c->RS / 2;
     }
+}
+
+// a tree on every row: the set-up block as a kernel of its own
+int launch_tree_begin(evt_ctx *c) {
+    BeginArgs A;
+    fill_begin_args(c, true, A);
     hipLaunchKernelGGL(k_tree_begin, dim3(1), dim3(1024), 0, c->stream, A);
+    HIPCHK(hipGetLastError());
+    c->js_staged = false;
+    return EVT_OK;
+}
+
+// Subsampling of a tree and its set-up.  draw: the mask's bytes are drawn from `seed` by the count pass (and written to
+// c->mask) instead of read.  The tree's set-up block rides in the scatter pass.
+int launch_compact_mask(evt_ctx *c, uint8_t cond, bool draw, unsigned long long seed) {
+    const int64_t n_chunks = (c->N + EVT_CHUNK - 1) / EVT_CHUNK;
+    unsigned g = grid_for_chunks(n_chunks);
+    if (draw) hipLaunchKernelGGL(k_mask_count<true>, dim3(g), dim3(256), 0, c->stream, c->mask, cond, c->N, n_chunks, c->flagw, c->chunk_nleft, seed);
+    else hipLaunchKernelGGL(k_mask_count<false>, dim3(g), dim3(256), 0, c->stream, c->mask, cond, c->N, n_chunks, c->flagw, c->chunk_nleft, 0ull);
+    HIPCHK(hipGetLastError());
+    BeginArgs B;
+    fill_begin_args(c, false, B);
+    if (n_chunks <= 1024) { // the scatter's blocks add up the counts before their chunk themselves
+        hipLaunchKernelGGL(k_mask_scatter<true>, dim3(g + 1), dim3(256), 0, c->stream, c->N, n_chunks, c->flagw, c->chunk_nleft, c->chunk_lpre, c->is_a, B);
+    } else {
+        hipLaunchKernelGGL(k_mask_scan, dim3(1), dim3(1024), 0, c->stream, c->chunk_nleft, c->chunk_lpre, n_chunks);
+        HIPCHK(hipGetLastError());
+        hipLaunchKernelGGL(k_mask_scatter<false>, dim3(g + 1), dim3(256), 0, c->stream, c->N, n_chunks, c->flagw, c->chunk_nleft, c->chunk_lpre, c->is_a, B);
+    }
     HIPCHK(hipGetLastError());
     c->js_staged = false;
     return EVT_OK;

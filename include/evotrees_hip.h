@@ -213,9 +213,10 @@ int evt_grow_tree_begin_staged(evt_handle h, uint8_t cond, const uint32_t *js, i
  * tree from its generator and the mask's 8-byte word w becomes output w of SplitMix64 started at that seed
  * (z = seed + (w + 1) * 0x9E3779B97F4A7C15; z = (z ^ z >> 30) * 0xBF58476D1CE4E5B9; z = (z ^ z >> 27) *
  * 0x94D049BB133111EB; z ^= z >> 31), little end first: byte i of the mask is bits 8 * (i % 8) and up of word i / 8.
- * A row is kept when its byte <= cond, as with an uploaded mask, so P[keep] = (cond + 1) / 256 all the same.  Queued
- * on the handle's stream (also behind a tree in flight), no host work per row; follow it with
- * evt_grow_tree_begin_staged.  The trees equal, bit for bit, those grown from the same bytes uploaded. */
+ * A row is kept when its byte <= cond, as with an uploaded mask, so P[keep] = (cond + 1) / 256 all the same.  The call
+ * only takes note of the seed (it may come while a tree is in flight); the evt_grow_tree_begin_staged that follows draws
+ * the bytes in its subsampling pass, on the device, with no host work per row.  A later evt_stage_mask replaces the seed.
+ * The trees equal, bit for bit, those grown from the same bytes uploaded. */
 int evt_draw_mask(evt_handle h, uint64_t seed);
 
 /*
