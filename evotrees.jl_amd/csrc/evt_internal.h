@@ -346,7 +346,6 @@ int launch_final_fused(evt_ctx *c, int level, const uint32_t *is_cur, bool fuse_
 int launch_nidx_from_segments(evt_ctx *c, int level, const uint32_t *is_cur);
 int launch_copy_to_host(evt_ctx *c, const void *src_dev, void *dst_host_dev, size_t nbytes);
 int launch_copy_words(evt_ctx *c, const void *src, void *dst, size_t nbytes);
-int launch_copy_words2(evt_ctx *c, const void *src0, void *dst0, size_t nbytes0, const void *src1, void *dst1, size_t nbytes1);
 int launch_fill_u32(evt_ctx *c, uint32_t *dst, uint32_t v, int64_t n);
 int launch_fill_bytes(evt_ctx *c, void *dst, int64_t nbytes);
 // predict

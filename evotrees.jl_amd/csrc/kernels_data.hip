@@ -151,25 +151,6 @@ int launch_copy_words(evt_ctx *c, const void *src, void *dst, size_t nbytes) {
     return EVT_OK;
 }
 
-// two such uploads in one launch (a launch costs a small kernel more than its words do)
-__global__ __launch_bounds__(256) void k_copy_words2(const uint32_t *__restrict__ src0, uint32_t *__restrict__ dst0, int64_t n0,
-                                                    const uint32_t *__restrict__ src1, uint32_t *__restrict__ dst1, int64_t n1) {
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n0 + n1; i += (int64_t)gridDim.x * 256) {
-        if (i < n0) dst0[i] = src0[i];
-        else dst1[i - n0] = src1[i - n0];
-    }
-}
-int launch_copy_words2(evt_ctx *c, const void *src0, void *dst0, size_t nbytes0, const void *src1, void *dst1, size_t nbytes1) {
-    const int64_t n0 = (int64_t)(nbytes0 / 4), n1 = (int64_t)(nbytes1 / 4);
-    if (n0 + n1 <= 0) return EVT_OK;
-    int64_t nb = (n0 + n1 + 255) / 256;
-    if (nb > 64) nb = 64;
-    hipLaunchKernelGGL(k_copy_words2, dim3((unsigned)nb), dim3(256), 0, c->stream, static_cast<const uint32_t *>(src0), static_cast<uint32_t *>(dst0), n0,
-                       static_cast<const uint32_t *>(src1), static_cast<uint32_t *>(dst1), n1);
-    HIPCHK(hipGetLastError());
-    return EVT_OK;
-}
-
 __global__ __launch_bounds__(256) void k_fill_u32(uint32_t *dst, uint32_t v, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = v;
 }
