@@ -51,16 +51,24 @@ struct HistArgs {
 };
 
 // First node of a block's span: the largest i with bprefix[i] <= start.  bprefix ascends from 0, so that is the number
-// of entries <= start, less one.  Every wavefront counts them for itself, 64 entries per step with all loads
-// independent: one trip to memory where a binary search makes log2(n_build) dependent ones.
+// of entries <= start, less one.  Every wavefront counts them for itself, 64 entries per load instruction and eight
+// load instructions in flight (clamped indices, no branch between them): one trip to memory for up to 512 build nodes
+// where a binary search makes log2(n_build) dependent ones.
 __device__ __forceinline__ int first_node_of_span(const int64_t *__restrict__ bprefix, int n_build, int64_t start) {
     const int lane = threadIdx.x & 63;
     int cnt = 0;
-    for (int k0 = 0; k0 < n_build; k0 += 64) {
-        const int k = k0 + lane;
-        const bool hit = (k < n_build) && (bprefix[k < n_build ? k : 0] <= start);
-        cnt += __popcll(__ballot(hit));
+    for (int k0 = 0; k0 < n_build; k0 += 512) {
+        int64_t v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int k = k0 + j * 64 + lane;
+            v[j] = bprefix[k < n_build ? k : n_build - 1];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) cnt += (k0 + j * 64 + lane < n_build && v[j] <= start) ? 1 : 0;
     }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) cnt += __shfl_xor(cnt, o);
     return cnt - 1;
 }
 
@@ -339,12 +347,28 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     // (32-bit unsigned arithmetic throughout: one 24-bit multiply-add per LDS address)
     uint32_t coff[PB];
     unsigned vmask = 0;
+    {
+        // the slots of this lane's PB features in one load (jsmap has an entry for every byte of the record, 0xFFFF for
+        // the padding and for features outside the sample)
+        const int f0 = tb + sub * PB;
+        uint32_t mw[4] = {0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu};
+        if (f0 < A.RS) {
+            if constexpr (PB == 8) {
+                const uint4 q = *reinterpret_cast<const uint4 *>(A.jsmap + f0);
+                mw[0] = q.x; mw[1] = q.y; mw[2] = q.z; mw[3] = q.w;
+            } else if constexpr (PB == 4) {
+                const uint2 q = *reinterpret_cast<const uint2 *>(A.jsmap + f0);
+                mw[0] = q.x; mw[1] = q.y;
+            } else {
+                mw[0] = *reinterpret_cast<const uint32_t *>(A.jsmap + f0);
+            }
+        }
 #pragma unroll
-    for (int t = 0; t < PB; t++) {
-        const int f = tb + sub * PB + t;
-        const bool ok = (f < A.F) && (A.jsmap[f] != 0xFFFF);
-        coff[t] = (uint32_t)(((t * B - 1) * NS + sub) * 8);
-        vmask |= ok ? (1u << t) : 0u;
+        for (int t = 0; t < PB; t++) {
+            const bool ok = ((mw[t >> 1] >> (16 * (t & 1))) & 0xFFFFu) != 0xFFFFu;
+            coff[t] = (uint32_t)(((t * B - 1) * NS + sub) * 8);
+            vmask |= ok ? (1u << t) : 0u;
+        }
     }
     const uint32_t binmul = (uint32_t)NS * 8u;
     const bool lane_on = vmask != 0;
@@ -360,6 +384,8 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         // nodes carries proportionally fewer rows
         const int64_t nbeg = A.bprefix[i];
         const int64_t nxt = A.bprefix[i + 1];
+        int64_t bst = A.bstart[i];
+        asm volatile("" : "+v"(bst)); // requested with the two above, not behind the branch below
         const int64_t nrows_end = nxt - A.seg_cost;
         const int64_t cend = end < nxt ? end : nxt;
         const int64_t nend_all = cend < nrows_end ? cend : nrows_end;
@@ -370,7 +396,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         }
         // the packed row counter holds 16 bits: a longer run of one node is flushed in several parts
         const int64_t nend = (PACK && nend_all - start > EVT_HIST_MAX_ROWS_PER_BLOCK) ? start + EVT_HIST_MAX_ROWS_PER_BLOCK : nend_all;
-        const int64_t seg = A.bstart[i] - nbeg;
+        const int64_t seg = bst - nbeg;
         // A wave takes SR = U * RPW consecutive positions of the run per iteration (U row groups of RPW rows).
         // Row ids and gradient words are fetched one position per lane (one load instruction per SR rows instead of
         // one per group): the number of load instructions in flight, not their bytes, is what a CU runs out of
