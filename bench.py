@@ -98,19 +98,20 @@ def bias(loss, y):
     return np.array([y.mean()], np.float32)
 
 
-def measured_traffic_per_launch(path):
-    """Average HBM bytes per k_hist_build launch (scaled FETCH_SIZE + WRITE_SIZE) from the committed
-    rocprofv3 --pmc summary of the same workload; None if the summary is absent."""
+def measured_traffic_per_row(path):
+    """HBM bytes per built row of the k_hist_build launches (scaled FETCH_SIZE + WRITE_SIZE over the rows the profiled
+    tree built) from the committed rocprofv3 --pmc summary of the same workload, with the rows of that tree; (None, None)
+    if the summary is absent."""
     try:
-        tot, n = 0.0, 0
+        tot, rows = 0.0, 0
         for line in open(path):
             p = line.split()
             if len(p) == 11 and p[0].isdigit():
                 tot += (float(p[7]) + float(p[9])) * 1e6
-                n += 1
-        return tot / n if n else None
+                rows += int(p[1])
+        return (tot / rows, rows) if rows else (None, None)
     except OSError:
-        return None
+        return None, None
 
 
 def prepare(evt, cfg, opts=None):
@@ -359,16 +360,40 @@ def main():
     roofline = None
     if hist_ms > 0:
         achieved = rows_built * bytes_per_row / (hist_ms * 1e-3) / 1e9
-        traffic = None
+        # HBM bytes per launch: the counters' bytes per built row (profiled tree) times the rows THIS run built per launch
+        traffic = traffic_row = pmc_rows = None
         if args.workload == "cfg3" and not args.rows:
-            traffic = measured_traffic_per_launch(os.path.join(ROOT, "profiles", "cfg3_k_hist_build_pmc.txt"))
+            traffic_row, pmc_rows = measured_traffic_per_row(os.path.join(ROOT, "profiles", "cfg3_k_hist_build_pmc.txt"))
+            if traffic_row is not None:
+                traffic = traffic_row * rows_built / max(1, prof["hist"]["launches"])
         roofline = {"bound": "hbm", "kernel": "k_hist_build", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None if traffic is None else round(traffic),
                     "algorithmic_bytes_per_launch": round(rows_built * bytes_per_row / max(1, prof["hist"]["launches"])),
                     "launches": prof["hist"]["launches"], "avg_launch_ms": round(hist_ms / max(1, prof["hist"]["launches"]), 4),
                     "timed_rounds": "%d of the %d timed rounds (every %d%s)" % (sampled, args.steps, pe, "th" if pe > 1 else ""),
                     "rows_built_per_round": rows_built // max(1, sampled), "bytes_per_row": bytes_per_row,
+                    "traffic_bytes_per_row": None if traffic_row is None else round(traffic_row, 1), "traffic_profiled_rows": pmc_rows,
                     "rows_features_per_s": round(rows_built * nfs / (hist_ms * 1e-3), 1)}
+        # The kernel's other bound: one 64-bit LDS atomic per (built row, sampled feature) and accumulator channel.  Peak = the
+        # device's measured rate of such atomics in the kernel's own conflict-free layout with all 64 lanes issuing; the
+        # kernel's record layout lets 13 of every 16 lanes issue (100 features in 8-byte pieces), the third figure.
+        try:
+            lane16, instr16 = evt._lib.lds_atomic_rate(0, 16, 200)
+            lane13, instr13 = evt._lib.lds_atomic_rate(0, 13, 200)
+            lane_rand, _ = evt._lib.lds_atomic_rate(1, 16, 200)
+            na_lds = 1 if (loss == "mse") else (4 if loss == "gaussian_mle" else 2)  # unit weights: mse packs {g, count} into one word
+            ach = rows_built * nfs * na_lds / (hist_ms * 1e-3)
+            roofline["secondary"] = {"bound": "lds_atomic", "achieved": round(ach / 1e9, 1), "peak": round(lane16 / 1e9, 1),
+                                     "unit": "G lane-atomics/s", "frac": round(ach / lane16, 4),
+                                     "peak_with_13_of_16_lanes": round(lane13 / 1e9, 1), "frac_of_13_lane_peak": round(ach / lane13, 4),
+                                     "peak_random_banks": round(lane_rand / 1e9, 1),
+                                     "wave_instr_per_s_16_lanes": round(instr16 / 1e9, 2), "wave_instr_per_s_13_lanes": round(instr13 / 1e9, 2)}
+            # the flush: 64-bit global atomics, every block adds the 12 800 words of a node's slice (100 features x 64 bins x 2)
+            ga = evt._lib.global_atomic_rate(nfs * B * 2 // 64 * 64, 256, 4)
+            roofline["flush_global_atomics"] = {"rate_G_per_s": round(ga / 1e9, 1), "atomics_per_launch": 256 * nfs * B * 2,
+                                                "us_per_launch_at_that_rate": round(256 * nfs * B * 2 / ga * 1e6, 1)}
+        except Exception as e:  # measurement aid only
+            roofline["secondary"] = {"error": str(e)}
     nb = max(1, extra)
     kernels = {k: {"ms_per_round": round(v["ms"] / nb, 4), "launches_per_round": v["launches"] / nb} for k, v in prof_all.items()}
     if prof_all["grad"]["ms"] > 0:

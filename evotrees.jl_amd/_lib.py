@@ -11,7 +11,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libevotrees_hip.so")
 
-EVT_OK, EVT_ERR_ARG, EVT_ERR_HIP, EVT_ERR_STATE, EVT_ERR_EMPTY, EVT_ERR_NOMEM = 0, -1, -2, -3, -4, -5
+EVT_OK, EVT_ERR_ARG, EVT_ERR_HIP, EVT_ERR_STATE, EVT_ERR_EMPTY, EVT_ERR_NOMEM, EVT_ERR_INTERNAL = 0, -1, -2, -3, -4, -5, -6
 LOSS_IDS = {"mse": 0, "logloss": 1, "gaussian_mle": 2, "poisson": 3, "gamma": 4, "tweedie": 5, "mlogloss": 6, "logistic_mle": 7, "mae": 8,
             "cred_var": 9, "cred_std": 10, "quantile": 11, "multiquantile": 12}
 METRIC_IDS = {"mse": 0, "rmse": 1, "mae": 2, "logloss": 3, "gaussian_mle": 4, "poisson": 5, "gamma": 6, "tweedie": 7, "mlogloss": 8, "logistic_mle": 9, "quantile": 10, "multiquantile": 11}
@@ -27,6 +27,7 @@ EXPORTS = [
     "evt_predict_tree", "evt_get_xbin", "evt_get_pred", "evt_get_grads", "evt_get_nidx", "evt_get_hist", "evt_get_quant",
     "evt_predict", "evt_predict_f64", "evt_predict_leaf_idx", "evt_eval_metric", "evt_set_profiling", "evt_get_profile", "evt_reset_profile",
     "evt_set_option", "evt_synchronize", "evt_copy_bandwidth", "evt_read_bandwidth", "evt_predict_static",
+    "evt_lds_atomic_rate", "evt_global_atomic_rate",
 ]
 
 
@@ -102,6 +103,8 @@ def load():
         "evt_synchronize": [vp],
         "evt_copy_bandwidth": [i64, i32, vp],
         "evt_read_bandwidth": [i64, i32, vp],
+        "evt_lds_atomic_rate": [i32, i32, i32, vp, vp],
+        "evt_global_atomic_rate": [i32, i32, i32, vp],
         "evt_predict_static": [vp, i64, i32, vp, vp, i32, i32, i32, i64, vp, vp, vp, vp, vp, i32, vp, vp],
     }
     for name, args in sigs.items():
@@ -133,6 +136,20 @@ def copy_bandwidth(nbytes=1 << 30, iters=10):
     out = C.c_double(0.0)
     check(load().evt_copy_bandwidth(nbytes, iters, C.byref(out)))
     return out.value
+
+
+def lds_atomic_rate(pattern=0, lanes16=16, iters=200):
+    """(lane-atomics per second, wavefront instructions per second) of 64-bit LDS atomics, device wide."""
+    a, b = C.c_double(0.0), C.c_double(0.0)
+    check(load().evt_lds_atomic_rate(pattern, lanes16, iters, C.byref(a), C.byref(b)))
+    return a.value, b.value
+
+
+def global_atomic_rate(words=12800, blocks=256, reps=4):
+    """64-bit global atomics per second when `blocks` blocks each add `words` consecutive words of one slice."""
+    a = C.c_double(0.0)
+    check(load().evt_global_atomic_rate(words, blocks, reps, C.byref(a)))
+    return a.value
 
 
 def read_bandwidth(nbytes=1 << 30, iters=10):

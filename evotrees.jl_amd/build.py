@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libevotrees_hip.so")
 SOURCES = ["api.hip", "kernels_data.hip", "kernels_grad.hip", "kernels_hist.hip", "kernels_scan.hip", "kernels_part.hip",
-           "kernels_predict.hip", "predict_static.hip", "kernels_quantile.hip"]
+           "kernels_predict.hip", "predict_static.hip", "kernels_quantile.hip", "probes.hip"]
 # -ffp-contract=off: the split gains follow the reference's expression order without fused multiply-add.
 # packed-fp32 instructions are disabled for all device code.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang",

@@ -33,23 +33,6 @@ void evt_set_error(const char *fmt, ...) {
 
 extern "C" const char *evt_last_error(void) { return g_err; }
 
-// No C++ exception crosses the C ABI: every entry point that returns a status runs inside this guard.
-template <typename F>
-static int guarded(F &&f) {
-    try {
-        return f();
-    } catch (const std::bad_alloc &) {
-        evt_set_error("out of host memory");
-        return EVT_ERR_NOMEM;
-    } catch (const std::exception &e) {
-        evt_set_error("internal error: %s", e.what());
-        return EVT_ERR_NOMEM;
-    } catch (...) {
-        evt_set_error("internal error");
-        return EVT_ERR_NOMEM;
-    }
-}
-
 extern "C" int evt_device_count(int32_t *count) {
     return guarded([&]() -> int {
     ARGCHK(count, "count is NULL");
@@ -930,10 +913,6 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
         evt_set_error("x_bin, target and gradients must be set before evt_grow_tree");
         return EVT_ERR_STATE;
     }
-    // the tree's staging slot: the one the tree collected last (or never used) held
-    c->h_stage = c->h_stage_base + (size_t)c->slot_w * c->h_stage_bytes;
-    c->h_stage_dev = c->h_stage_dev_base + (size_t)c->slot_w * c->h_stage_bytes;
-    c->tree_seq += 1;
     // js: 1-based, strictly ascending
     std::vector<uint32_t> jsv(n_js);
     {
@@ -950,6 +929,12 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
     // LDS budget of one block: the channels of one launch x bins of a single feature must fit (more than EVT_MAX_NA
     // channels go EVT_HIST_GROUP per launch)
     ARGCHK((size_t)(c->NA <= EVT_MAX_NA ? c->NA : EVT_HIST_GROUP) * c->B * 8 <= 64 * 1024, "histogram of one feature exceeds the LDS budget");
+
+    // the arguments are in order: the tree takes its staging slot (the one the tree collected last, or never used,
+    // held) and its number in the profile
+    c->h_stage = c->h_stage_base + (size_t)c->slot_w * c->h_stage_bytes;
+    c->h_stage_dev = c->h_stage_dev_base + (size_t)c->slot_w * c->h_stage_bytes;
+    c->tree_seq += 1;
 
     // rows kept by the mask (the host owns the RNG; src/subsample.jl:7-9).  The threshold, the count and the
     // compaction run on the device; the count comes back with the finished tree.

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <atomic>
+#include <exception>
+#include <new>
 #include <string>
 #include <vector>
 
@@ -236,6 +238,22 @@ void evt_set_error(const char *fmt, ...);
             return EVT_ERR_HIP;                                                            \
         }                                                                                  \
     } while (0)
+// No C++ exception crosses the C ABI: every entry point that returns a status runs inside this guard.
+template <typename F>
+static int guarded(F &&f) {
+    try {
+        return f();
+    } catch (const std::bad_alloc &) {
+        evt_set_error("out of host memory");
+        return EVT_ERR_NOMEM;
+    } catch (const std::exception &e) {
+        evt_set_error("internal error: %s", e.what());
+        return EVT_ERR_INTERNAL;
+    } catch (...) {
+        evt_set_error("internal error");
+        return EVT_ERR_INTERNAL;
+    }
+}
 #define ARGCHK(cond, msg)                \
     do {                                 \
         if (!(cond)) {                   \

@@ -43,7 +43,8 @@ typedef enum {
     EVT_ERR_HIP = -2,   /* a HIP runtime call or kernel launch failed                      */
     EVT_ERR_STATE = -3, /* call order violated (e.g. grow before x_bin / target were set)  */
     EVT_ERR_EMPTY = -4, /* "no subsample observation" (src/subsample.jl:36)                */
-    EVT_ERR_NOMEM = -5
+    EVT_ERR_NOMEM = -5,   /* a host or device allocation failed                             */
+    EVT_ERR_INTERNAL = -6 /* any other failure inside the library (e.g. a worker thread could not start) */
 } evt_status;
 
 /* loss ids: the losses of src/loss.jl:20-34 */
@@ -366,6 +367,16 @@ int evt_synchronize(evt_handle h);
 int evt_copy_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out);
 /* Same for a read-only stream of nbytes (no write traffic). */
 int evt_read_bandwidth(int64_t nbytes, int32_t iters, double *gbps_out);
+/* Rate of 64-bit LDS atomics as the histogram kernel issues them (256 blocks of 1024 threads, one 64 KB LDS array each):
+ * pattern 0 = the kernel's layout for 128-byte records (the 16 lanes the LDS serves per pass fall on 16 different bank
+ * pairs, random bins), pattern 1 = random words; lanes16 of every 16 lanes issue (the 100-feature record of the headline
+ * workload uses 13).  Outputs: lane-atomics per second and wavefront instructions per second, device wide.  No
+ * counterpart in the reference (its histogram kernel adds into global memory, ext/.../fit-utils.jl:57-174): the ceiling
+ * the kernel's row rate is quoted beside. */
+int evt_lds_atomic_rate(int32_t pattern, int32_t lanes16, int32_t iters, double *lane_atomics_per_s, double *wave_instr_per_s);
+/* Rate of 64-bit global atomics as the histogram kernel's flush issues them: `blocks` blocks each add `words` consecutive
+ * words of one slice `reps` times.  Output: atomics per second, device wide. */
+int evt_global_atomic_rate(int32_t words, int32_t blocks, int32_t reps, double *atomics_per_s);
 
 #ifdef __cplusplus
 }

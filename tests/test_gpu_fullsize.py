@@ -190,3 +190,115 @@ def test_offsets_past_two_to_the_31(evt, N, F):
     assert np.array_equal(evt._lib.predict_leaf_idx(x_bin, ft, [t]).reshape(-1), nid.astype(np.uint32))
     raw = evt._lib.predict_model(x_bin, ft, "mse", 1, [t], apply_link=False)
     assert np.array_equal(raw[:, 0], t.pred[nid - 1, 0])
+
+
+# BASELINE.json's other configurations at their full sizes: kernel selection changes with the number of rows (streaming
+# hint, the scan of the chunk counts as a kernel of its own from about a thousand partition chunks per level, whether
+# the threshold bit planes fit), so the small parity cases do not reach the code these sizes run.
+BASELINE_CASES = [
+    # name, loss, N, F, nbins, depth, tree_type, rowsample, colsample, params
+    ("cfg2", "mse", 1_000_000, 100, 64, 6, "binary", 0.5, 0.5, {}),
+    ("cfg4", "logloss", 1_000_000, 28, 128, 8, "binary", 0.8, 1.0, dict(eta=0.05)),
+    ("cfg5", "gaussian_mle", 2_000_000, 50, 64, 7, "binary", 1.0, 1.0, dict(min_weight=8.0)),
+    ("cfg5o", "gaussian_mle", 2_000_000, 50, 64, 7, "oblivious", 1.0, 1.0, dict(min_weight=8.0)),
+]
+
+
+@pytest.mark.parametrize("name,loss,N,F,B,D,tt,rowsample,colsample,pk", BASELINE_CASES)
+def test_baseline_config_full_size(evt, name, loss, N, F, B, D, tt, rowsample, colsample, pk):
+    """One teacher-forced round of the named configuration at its full size, bit for bit against the fixed-point oracle
+    (tree arrays, node of every sampled row, predictions of all rows), and the size-independent properties: weights add
+    up, no row sits in a split node, node ids equal an independent walk of the finished tree (the rule of
+    test/predict-leaf-idx.jl:25-73), parent histogram = left + right exactly, another launch shape gives the same bits."""
+    from oracle import oracle as orc
+    from test_gpu_parity import assert_tree_bits, setup_pair
+    print("case", name, loss, N, F, B, D, tt, rowsample, colsample, flush=True)
+    rng = np.random.default_rng(2025)
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    K = 2 if loss == "gaussian_mle" else 1
+    z = (x_bin[0] / np.float32(B) + np.float32(0.5) * (x_bin[F // 2] > B // 3) + np.float32(0.25) * (x_bin[F - 1] / np.float32(B)) ** 2).astype(np.float32)
+    noise = rng.standard_normal(N).astype(np.float32)
+    if loss == "logloss":
+        y = (z + np.float32(0.4) * noise > np.float32(0.9)).astype(np.float32)
+        mu = np.array([np.log(y.mean() / (1 - y.mean()))], np.float32)
+    elif loss == "gaussian_mle":
+        y = (z + (np.float32(0.2) + np.float32(0.3) * (x_bin[2] > B // 2)) * noise).astype(np.float32)
+        s = float(y.std(ddof=1))
+        mu = np.array([y.mean(), s + np.log(-np.expm1(-s))], np.float32)
+    else:
+        y = (z + np.float32(0.1) * noise).astype(np.float32)
+        mu = np.array([y.mean()], np.float32)
+    h, o, op, gp, pred0, grad0 = setup_pair(evt, loss, x_bin, y, None, mu, B, D, tt, **pk)
+    grad = grad0.copy()
+    orc.update_grads(op, pred0, y, grad)
+    h.set_grads(grad)  # identical Float32 gradients on both sides
+    nfs = int(np.ceil(colsample * F))
+    js = np.arange(1, F + 1, dtype=np.uint32) if nfs >= F else (np.sort(rng.choice(F, nfs, replace=False)) + 1).astype(np.uint32)
+    if rowsample < 1.0:
+        mask = rng.integers(0, 256, N, dtype=np.uint8)
+        cond = int(np.rint(255 * rowsample))
+        rows = orc.subsample(mask, cond)
+    else:
+        mask, cond, rows = None, 255, np.arange(N, dtype=np.uint32)
+    h.set_option("record_nidx", 1)
+    print("growing on the device", flush=True)
+    t = h.grow_tree(js, gp, mask=mask, cond=cond)
+    nidx = h.get_nidx()
+    p_gpu = h.get_pred()
+    H = h.get_hist()
+    print("growing in the oracle", flush=True)
+    qb, qe = h.get_quant()
+    o.set_quant(grad, qb)
+    t_fx, nidx_fx = o.grow_tree(grad, rows, js, mode=1)
+    assert_tree_bits(t, t_fx)
+    assert np.array_equal(nidx, nidx_fx)
+    p_orc = pred0.copy()
+    o.predict_tree(t_fx, p_orc)
+    assert np.array_equal(p_gpu.view(np.uint32), p_orc.view(np.uint32))
+    # structure and weights (unit weights: Tree.w holds row counts)
+    split = t.split.astype(bool)
+    nn = (1 << D) - 1
+    assert split[0] and split.sum() >= (D - 1 if tt == "oblivious" else 10)
+    assert t.w[0] == np.float32(rows.shape[0])
+    for n in np.flatnonzero(split) + 1:
+        assert t.w[n - 1] == t.w[2 * n - 1] + t.w[2 * n]
+        assert t.feat[n - 1] in js and 1 <= t.cond_bin[n - 1] <= B - 1
+    if tt == "oblivious":  # every split node of a depth shares (feature, bin)
+        for d in range(D - 1):
+            lvl = np.arange(1 << d, 1 << (d + 1))
+            sp = lvl[split[lvl - 1]]
+            assert len(set(zip(t.feat[sp - 1].tolist(), t.cond_bin[sp - 1].tolist()))) <= 1
+    # node ids: sampled rows sit in leaves, and equal an independent walk of the finished tree
+    assert not split[nidx[rows] - 1].any()
+    walk = evt._lib.predict_leaf_idx(x_bin, None, [t])[:, 0]
+    assert np.array_equal(walk[rows], nidx[rows])
+    counts = np.bincount(nidx[rows], minlength=nn + 1)
+    leaves = np.array([n for n in range(1, nn + 1) if t.w[n - 1] > 0 and not split[n - 1]])
+    assert np.array_equal(counts[leaves].astype(np.float32), t.w[leaves - 1])
+    # histograms: parent == left + right exactly (integer accumulation), bins of a feature add up to the node totals
+    jz = js - 1
+    last_hist_node = (1 << (D - 1)) - 1  # nodes of the last level never get a histogram
+    checked = 0
+    for n in np.flatnonzero(split) + 1:
+        if 2 * n + 1 <= last_hist_node and split[2 * n - 1] and split[2 * n]:
+            assert np.array_equal(H[n - 1][jz], H[2 * n - 1][jz] + H[2 * n][jz])
+            checked += 1
+            if checked >= 8:
+                break
+    assert checked >= 1
+    # (the exported values are Float64: a channel's sum over 2M rows of 38-bit fixed-point words is not exact there, the
+    # row count is)
+    tot = H[0][jz].sum(axis=1)
+    mag = np.abs(H[0][jz]).sum(axis=1).max(axis=0)  # gradient sums cancel: the bound is relative to the summed magnitudes
+    assert (np.abs(tot - tot[0]) <= 1e-12 * mag).all()
+    assert (tot[:, 2 * K] == rows.shape[0]).all()
+    del H
+    # another launch shape, the other decision source of the partition: the same bits
+    h.set_option("record_nidx", 0)
+    h.set_option("hist_blocks", 193)
+    h.set_option("hist_threads", 512)
+    h.set_option("bit_planes", 0)
+    assert_tree_bits(h.grow_tree(js, gp, mask=mask, cond=cond), t_fx)  # the gradients given above are still in place
+    assert np.array_equal(h.get_nidx(), nidx_fx)
+    h.close()
+    o.close()
