@@ -213,7 +213,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     ARGCHK(out, "out handle is NULL");
     *out = nullptr;
     ARGCHK(nobs >= 1 && nobs <= (int64_t)0xFFFFFFFFll, "nobs must be in [1, 2^32-1]");
-    ARGCHK(nfeats >= 1 && nfeats <= 1024, "nfeats must be in [1, 1024]");
+    ARGCHK(nfeats >= 1 && nfeats <= EVT_MAX_FEATS, "nfeats must be in [1, 65534]");
     ARGCHK(nbins >= 2 && nbins <= 255, "nbins must be in [2, 255]");
     ARGCHK(max_depth >= 1 && max_depth <= EVT_MAX_DEPTH, "max_depth must be in [1, 16]");
     ARGCHK(loss >= 0 && loss <= EVT_LOSS_LAST,
@@ -297,11 +297,6 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     memset(c->prof_launches, 0, sizeof(c->prof_launches));
     memset(c->prof_ms, 0, sizeof(c->prof_ms));
     memset(c->prof_units, 0, sizeof(c->prof_units));
-    if (c->LPR > 64) {
-        delete c;
-        evt_set_error("nfeats too large for the record layout");
-        return EVT_ERR_ARG;
-    }
     hipError_t e = hipGetDevice(&c->device);
     if (e == hipSuccess) e = hipStreamCreate(&c->stream);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&c->tree_evs[0], hipEventDisableTiming);
@@ -1808,6 +1803,7 @@ extern "C" int evt_set_option(evt_handle c, const char *name, int64_t value) {
         c->hist_seg_cost = (int)value;
     } else if (strcmp(name, "hist_variant") == 0) {
         ARGCHK(value >= 0 && value <= 2, "hist_variant must be 0 (auto), 1 (generic) or 2 (conflict-free where it applies)");
+        ARGCHK(value != 1 || c->LPR <= 64, "hist_variant 1: the generic histogram kernel takes records of up to 1024 bytes");
         c->hist_variant = (int)value;
     } else if (strcmp(name, "bit_planes") == 0) {
         ARGCHK(value == 0 || value == 1, "bit_planes must be 0 or 1");

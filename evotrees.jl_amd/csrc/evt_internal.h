@@ -29,6 +29,7 @@
 #define EVT_HIST_GROUP 4 // accumulator channels one histogram launch handles; more channels take several launches
 #define EVT_METRIC_BLOCKS 1024 // partial sums of the evaluation metric
 #define EVT_MAX_DEPTH 16
+#define EVT_MAX_FEATS 65534 // a feature's slot in the column sample is a 16-bit word, 0xFFFF = not sampled
 #define EVT_PACK_QBITS 30     // fixed-point bits of the gradient channel that shares a word with the row count
 #define EVT_PACK_CNT_BITS 16
 // rows one LDS histogram may take between two flushes: the packed row counter has EVT_PACK_CNT_BITS bits, and

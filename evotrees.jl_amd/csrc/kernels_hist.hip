@@ -689,6 +689,10 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
         const size_t lds16 = (size_t)na * c->B * tw * 8; // channels x bins x tile bytes words
         const bool can16 = c->RS >= 32 && lds16 <= 128 * 1024;
         const bool use16 = (c->hist_variant == 1) ? false : can16;
+        if (!use16 && c->LPR > 64) { // the generic kernel reads a record with one wavefront instruction: 64 lanes of 16 bytes
+            evt_set_error("%d accumulator channels x %d bins need the generic histogram kernel, which takes at most 1024 features", na, c->B);
+            return EVT_ERR_ARG;
+        }
         int r = EVT_ERR_ARG;
         if (use16) {
             // several block columns share the launch's blocks: the same number of LDS histograms is flushed per node

@@ -522,9 +522,11 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
     }
     double bg = -INFINITY;
     int bj = NO_BIN, bb = NO_BIN;
-    if (tid < ngroups) {
-        const ScanBest r = A.sbest[(int64_t)blockIdx.x * ngroups + tid];
-        bg = r.gain; bj = r.jp; bb = r.bin;
+    // a thread takes the groups tid, tid + 256, ... (more than 1024 sampled features): ascending feature positions, so
+    // only a strictly larger gain replaces an earlier one
+    for (int g = tid; g < ngroups; g += 256) {
+        const ScanBest r = A.sbest[(int64_t)blockIdx.x * ngroups + g];
+        if (r.gain > bg) { bg = r.gain; bj = r.jp; bb = r.bin; }
     }
     s_g[tid] = bg; s_j[tid] = bj; s_b[tid] = bb;
     __syncthreads();
@@ -860,9 +862,11 @@ __global__ __launch_bounds__(256) void k_scan_fin_mc(ScanArgs A, int ngroups) {
     }
     double bg = -INFINITY;
     int bj = NO_BIN, bb = NO_BIN;
-    if (tid < ngroups) {
-        const ScanBest r = A.sbest[(int64_t)blockIdx.x * ngroups + tid];
-        bg = r.gain; bj = r.jp; bb = r.bin;
+    // a thread takes the groups tid, tid + 256, ... (more than 1024 sampled features): ascending feature positions, so
+    // only a strictly larger gain replaces an earlier one
+    for (int g = tid; g < ngroups; g += 256) {
+        const ScanBest r = A.sbest[(int64_t)blockIdx.x * ngroups + g];
+        if (r.gain > bg) { bg = r.gain; bj = r.jp; bb = r.bin; }
     }
     s_g[tid] = bg; s_j[tid] = bj; s_b[tid] = bb;
     __syncthreads();

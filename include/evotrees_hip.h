@@ -120,7 +120,10 @@ int evt_device_count(int32_t *count);
 /* ---- training cache ------------------------------------------------------------------
  * Replaces init_core(params, ::Type{<:GPU}, ...) device allocation
  * (ext/EvoTreesKernelAbstractionsExt/init.jl:1-151): sizes every device buffer.
- * nbins in [2,255] (src/learners.jl:527).  K is the number of outputs (size(pred, 1) in the reference, at most 16):
+ * nbins in [2,255] (src/learners.jl:527); nfeats in [1,65534] (a record of the observation-major copy may be any width;
+ * the one shape without a wide-record histogram kernel - more than 1024 features with accumulator channels x nbins above
+ * 512 - is refused when its first tree is grown); max_depth in [1,16] (the histogram buffer holds 2^max_depth - 1 node
+ * slices).  The reference bounds neither (src/learners.jl:525-527).  K is the number of outputs (size(pred, 1) in the reference, at most 16):
  * the number of targets for mse / logloss / poisson / gamma / tweedie / mae / quantile / cred_var / cred_std (1, or more with
  * a matrix target, src/init.jl:11-16, :104-150), twice the number of targets for gaussian_mle and logistic_mle
  * (src/init.jl:68-100), the number of classes (2..16) for mlogloss, the number of levels for multiquantile (src/init.jl:101-103). */

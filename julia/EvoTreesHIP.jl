@@ -94,7 +94,18 @@ function destroy!(c::CacheHIP)
     return nothing
 end
 
+# What the library does not take (evt_create, include/evotrees_hip.h): the reference has no such limits
+# (src/learners.jl:525-527, src/init.jl:43-67), so a fit beyond them is sent back to the CPU path by name.
+const MAX_OUTPUTS, MAX_DEPTH, MAX_FEATS = 16, 16, 65534
+function check_limits(nfeats, K, max_depth)
+    K <= MAX_OUTPUTS || error("libevotrees_hip takes at most $MAX_OUTPUTS outputs (this model has $K): fit it with device=:cpu")
+    max_depth <= MAX_DEPTH || error("libevotrees_hip takes max_depth <= $MAX_DEPTH (got $max_depth): fit it with device=:cpu")
+    nfeats <= MAX_FEATS || error("libevotrees_hip takes at most $MAX_FEATS features (got $nfeats): fit it with device=:cpu")
+    return nothing
+end
+
 function create_handle(nobs, nfeats, nbins, K, max_depth, L, tree_type)
+    check_limits(nfeats, K, max_depth)
     h = Ref{Ptr{Cvoid}}(C_NULL)
     check(ccall((:evt_create, LIB), Cint, (Int64, Cint, Cint, Cint, Cint, Cint, Cint, Ptr{Ptr{Cvoid}}),
         nobs, nfeats, nbins, K, max_depth, loss_id(L), tree_type == :oblivious ? 1 : 0, h))

@@ -557,3 +557,37 @@ def test_two_handles_on_two_threads(evt):
             assert_tree_bits(ta, tb)
         assert np.array_equal(seq[k][1].view(np.uint32), par[k][1].view(np.uint32))
         assert "js entries" in par[k][2]
+
+
+def test_size_limits_are_refused_with_a_message(evt):
+    """What the library does not take is refused before anything is sized by it, with a message that names the limit:
+    more than 16 outputs, trees deeper than 16, and - the one histogram shape without a wide-record kernel - more than 1024
+    features when channels x bins exceed 512."""
+    for args, word in (((100, 4, 8, 17, 3, "mse"), "16"), ((100, 4, 8, 1, 17, "mse"), "max_depth"), ((100, 65535, 8, 1, 3, "mse"), "nfeats"),
+                       ((100, 4, 8, 34, 3, "gaussian_mle"), "16")):
+        with pytest.raises(evt.EvtError) as ei:
+            evt.Handle(*args)
+        assert ei.value.code == evt._lib.EVT_ERR_ARG and word in str(ei.value)
+    N, F, B = 2000, 1100, 255
+    rng = np.random.default_rng(5)
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    y = rng.random(N).astype(np.float32)
+    w = (rng.random(N) + 0.5).astype(np.float32)
+    h = evt.Handle(N, F, B, 2, 3, "gaussian_mle")  # five channels x 255 bins: not even a 32-byte column tile fits the LDS
+    h.set_xbin(x_bin)
+    h.set_target(y, w, np.array([0.5, 0.1], np.float32))
+    h.update_grads()
+    with pytest.raises(evt.EvtError) as ei:
+        h.grow_tree(np.arange(1, F + 1, dtype=np.uint32), evt.make_params(min_weight=8.0))
+    assert ei.value.code == evt._lib.EVT_ERR_ARG and "1024 features" in str(ei.value)
+    with pytest.raises(evt.EvtError):
+        h.set_option("hist_variant", 1)
+    # the same shape with unit weights needs four channels and 64 bins fit: it grows
+    h.close()
+    h = evt.Handle(N, F, 64, 2, 3, "gaussian_mle")
+    h.set_xbin(np.minimum(x_bin, 64).astype(np.uint8))
+    h.set_target(y, None, np.array([0.5, 0.1], np.float32))
+    h.update_grads()
+    t = h.grow_tree(np.arange(1, F + 1, dtype=np.uint32), evt.make_params(min_weight=8.0))
+    assert t.w[0] == N
+    h.close()
