@@ -182,6 +182,7 @@ struct NextArgs {
     int32_t *n_bnode;
     int64_t *n_bstart;
     int64_t *n_bprefix;
+    int64_t *n_stats; // rows the next level builds (the level's slot of the per-tree counts; the histogram kernel writes the same figure when it runs)
     int64_t seg_cost; // cost units added per build node in the histogram kernel's span space
 };
 
@@ -315,6 +316,7 @@ __device__ void level_tables_block(const NextArgs &A, long long *s_tmp /* [34] *
         A.n_hdr[LH_N_CHUNKS] = t_chunks;
         A.n_hdr[LH_N_BUILD] = t_pos;
         A.n_hdr[LH_TOTAL_BUILD] = t_brows;
+        if (A.n_stats) *A.n_stats = t_brows - t_pos * A.seg_cost;
     }
 }
 
@@ -940,6 +942,7 @@ static void fill_next_args(evt_ctx *c, int level, NextArgs &A) {
     A.n_bnode = Nx.bnode;
     A.n_bstart = Nx.bstart;
     A.n_bprefix = Nx.bprefix;
+    A.n_stats = (level + 1 <= c->D) ? c->stats + level + 1 : nullptr;
     A.seg_cost = c->hist_seg_cost;
 }
 

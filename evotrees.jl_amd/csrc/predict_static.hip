@@ -99,11 +99,17 @@ extern "C" int evt_predict_static(void *stream, int64_t nobs, int32_t nfeats, co
                       (long long)EVT_STATIC_MAX_NODES);
         return EVT_ERR_ARG;
     }
-    ARGCHK(device_visible(x_bin_dev) && device_visible(tree_off_dev) && device_visible(feat_dev) && device_visible(cond_bin_dev) &&
-               device_visible(pred_dev) && device_visible(split_dev) && device_visible(out_dev),
-           "evt_predict_static takes device memory only (x_bin, the tree arrays, out)");
-    ARGCHK((!feattypes_dev || device_visible(feattypes_dev)) && (!status_dev || device_visible(status_dev)),
-           "feattypes and status must be device memory (or NULL)");
+    ARGCHK((apply_link & ~(1 | EVT_STATIC_TRUSTED)) == 0, "apply_link takes 0 or 1, plus EVT_STATIC_TRUSTED");
+    const bool trusted = (apply_link & EVT_STATIC_TRUSTED) != 0;
+    apply_link &= 1;
+    ARGCHK(x_bin_dev && tree_off_dev && feat_dev && cond_bin_dev && pred_dev && split_dev && out_dev, "x_bin, the tree arrays and out must not be NULL");
+    if (!trusted) { // nine pointer queries: a caller that vouches for its pointers (a serving loop, a capture) skips them
+        ARGCHK(device_visible(x_bin_dev) && device_visible(tree_off_dev) && device_visible(feat_dev) && device_visible(cond_bin_dev) &&
+                   device_visible(pred_dev) && device_visible(split_dev) && device_visible(out_dev),
+               "evt_predict_static takes device memory only (x_bin, the tree arrays, out)");
+        ARGCHK((!feattypes_dev || device_visible(feattypes_dev)) && (!status_dev || device_visible(status_dev)),
+               "feattypes and status must be device memory (or NULL)");
+    }
     unsigned char *ws = nullptr;
     const int r = static_scratch(&ws);
     if (r != EVT_OK) return r;

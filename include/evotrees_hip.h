@@ -322,8 +322,14 @@ int evt_predict_leaf_idx(int64_t nobs, int32_t nfeats, const uint8_t *x_bin_colm
  * applies on the host; a model that breaks them leaves `out` unwritten and EVT_ERR_ARG in *status (a device int32,
  * EVT_OK otherwise; may be NULL).  Results equal evt_predict's, bit for bit.  The device that is current on the calling
  * thread must be the one the pointers live on.  All calls on one GPU share the one array: calls that overlap on a GPU
- * (two streams, two threads) race, and a call must have finished before the next one is queued on another stream. */
+ * (two streams, two threads) race, and a call must have finished before the next one is queued on another stream.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress, which may load the code object) and sets
+ * kernel attributes: make it an ordinary call, outside any stream capture.  Every call queries the memory type of its
+ * nine pointers unless EVT_STATIC_TRUSTED is added to apply_link (0 or 1): a caller that vouches for device pointers -
+ * a serving loop, a call recorded into a HIP graph - skips the queries.  A captured call replays the three kernels on
+ * the same array: the rule about overlapping calls holds for replays too. */
 #define EVT_STATIC_MAX_NODES (1 << 20)
+#define EVT_STATIC_TRUSTED 2
 int evt_predict_static(void *stream, int64_t nobs, int32_t nfeats, const uint8_t *x_bin_dev, const uint8_t *feattypes_dev,
                        int32_t loss, int32_t K, int32_t ntrees, int64_t total_nodes, const int64_t *tree_off_dev,
                        const int64_t *feat_dev, const uint8_t *cond_bin_dev, const float *pred_dev, const uint8_t *split_dev,

@@ -96,3 +96,44 @@ def test_predict_static_limits_and_model_check(evt):
     rc, out, status = _static_call(evt, torch, x_bin, None, "mse", K, trees, False)
     assert rc == 0 and status == 0
     assert np.array_equal(out, evt._lib.predict_model(x_bin, None, "mse", K, trees, apply_link=False))
+
+
+def test_predict_static_recorded_into_a_graph(evt):
+    """The call recorded into a HIP graph (after one ordinary call on the device, which looks the work area up) and
+    replayed three times with eager work, other models through the same work area and synchronisations in between:
+    every replay equals evt_predict bit for bit.  The recorded call carries EVT_STATIC_TRUSTED (no pointer queries)."""
+    torch = pytest.importorskip("torch")
+    L = evt._lib.load()
+    rng = np.random.default_rng(8)
+    N, F, B, K, loss = 20_000, 12, 32, 2, "gaussian_mle"
+    x_bin = rng.integers(1, B + 1, size=(F, N), dtype=np.uint8)
+    trees = [_random_tree(rng, dd, F, B, K) for dd in (6, 2, 8, 5)]
+    want = evt._lib.predict_model(x_bin, None, loss, K, trees, apply_link=True)
+    rc, got, status = _static_call(evt, torch, x_bin, None, loss, K, trees, True)  # the ordinary first call
+    assert rc == 0 and status == 0 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    off, feat, cb, pr, sp = _model_arrays(trees, K)
+    dev = torch.device("cuda:0")
+    d = [torch.from_numpy(a).to(dev) for a in (x_bin, off, feat, cb, pr, sp)]
+    out = torch.zeros((N, K), dtype=torch.float32, device=dev)
+    status_t = torch.full((1,), 77, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = L.evt_predict_static(C.c_void_p(stream), N, F, C.c_void_p(d[0].data_ptr()), None, evt._lib.LOSS_IDS[loss], K, len(trees), int(off[-1]),
+                                  C.c_void_p(d[1].data_ptr()), C.c_void_p(d[2].data_ptr()), C.c_void_p(d[3].data_ptr()), C.c_void_p(d[4].data_ptr()),
+                                  C.c_void_p(d[5].data_ptr()), 1 | 2, C.c_void_p(out.data_ptr()), C.c_void_p(status_t.data_ptr()))
+    assert rc == 0
+    other = [_random_tree(rng, 4, F, B, K) for _ in range(2)]
+    for rep in range(3):
+        out.fill_(float("nan"))
+        status_t.fill_(77)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert int(status_t.cpu()[0]) == 0
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), rep
+        # eager work through the same work area between the replays: another model, then a synchronize
+        rc2, got2, st2 = _static_call(evt, torch, x_bin, None, loss, K, other, False)
+        assert rc2 == 0 and st2 == 0
+        assert np.array_equal(got2, evt._lib.predict_model(x_bin, None, loss, K, other, apply_link=False))
