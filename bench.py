@@ -136,6 +136,22 @@ def prepare(evt, cfg, opts=None):
     return h, y, mu, rng, {"generate_s": round(t1 - t0, 2), "edges_s": round(t2 - t1, 2), "upload_binarize_target_s": round(t3 - t2, 2)}
 
 
+def rows_built_per_level(tree, D, n_root=None):
+    """Rows the histogram kernel built at every level of a tree grown with unit weights (Tree.w holds row counts): the
+    root's rows, then the smaller child of every split (src/fit.jl:123-129), and the number of build nodes per level."""
+    rows = [int(n_root if n_root is not None else tree.w[0])]
+    nodes = [1]
+    for d in range(1, D - 1):
+        tot = cnt = 0
+        for n in range(1 << (d - 1), 1 << d):
+            if tree.split[n - 1]:
+                tot += int(min(tree.w[2 * n - 1], tree.w[2 * n]))
+                cnt += 1
+        rows.append(tot)
+        nodes.append(cnt)
+    return {"rows": rows, "build_nodes": nodes}
+
+
 class Rounds:
     """Boosting rounds on a prepared handle, as the host mirror's grow_evotree drives them: gradients, the column sample,
     the row mask drawn on the device from one 64-bit draw of the host's generator, the tree.  host_mask=True draws one
@@ -163,6 +179,7 @@ class Rounds:
         self.in_flight = 0
         self.sampled = 0
         self.prof_on = False
+        self.levels = None  # a list: every collected tree's rows built per level are appended (--levels-out)
         h.set_option("grads_ahead", 1)  # one tree per round: the next round's gradients are queued behind the tree
 
     def draw_mask(self):
@@ -211,6 +228,8 @@ class Rounds:
             self.begin()
         self.evt._lib.check(self.L.evt_grow_tree_end(h._h, self.tree_out))
         self.in_flight -= 1
+        if self.levels is not None:
+            self.levels.append(rows_built_per_level(self.tree, self.cfg["depth"], self.N if self.cond >= 255 else None))
 
     def timed(self, steps, warmup, profile_every=4, no_profile=False):
         """`warmup` untimed rounds, then `steps` timed ones.  HIP events around the histogram launches only (the kernel
@@ -282,6 +301,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
     ap.add_argument("--rows", type=int, default=0, help="override the number of rows (smoke runs)")
+    ap.add_argument("--depth", type=int, default=0, help="override max_depth (2: the root's histogram only)")
+    ap.add_argument("--levels-out", default="", help="file that receives, for every tree grown (warm-up, timed, extra rounds, in order), "
+                    "the rows built and the build nodes per level - to set beside a kernel trace of the same run")
     ap.add_argument("--cpu-rounds", type=int, default=3, help="rounds of the CPU oracle to time (0: skip)")
     ap.add_argument("--no-profile", action="store_true", help="do not record HIP events around kernels")
     ap.add_argument("--profile-every", type=int, default=4, help="rounds between two rounds whose histogram launches carry HIP events")
@@ -305,6 +327,8 @@ def main():
     cfg = dict(WORKLOADS[args.workload])
     if args.rows:
         cfg["N"] = args.rows
+    if args.depth:
+        cfg["depth"] = args.depth
     N, F, B, D, loss = cfg["N"], cfg["F"], cfg["nbins"], cfg["depth"], cfg["loss"]
     K = 2 if loss == "gaussian_mle" else 1
     NK = 2 * K + 1
@@ -334,6 +358,8 @@ def main():
     t_setup = t_init["edges_s"] + t_init["upload_binarize_target_s"]
 
     R = Rounds(evt, h, cfg, rng)
+    if args.levels_out:
+        R.levels = []
     cond, nfs, L, tree = R.cond, R.nfs, R.L, R.tree
     one_round = R.one_round
     ms_per_step, prof_hist, sampled = R.timed(args.steps, args.warmup, args.profile_every, args.no_profile)
@@ -362,7 +388,7 @@ def main():
         achieved = rows_built * bytes_per_row / (hist_ms * 1e-3) / 1e9
         # HBM bytes per launch: the counters' bytes per built row (profiled tree) times the rows THIS run built per launch
         traffic = traffic_row = pmc_rows = None
-        if args.workload == "cfg3" and not args.rows:
+        if args.workload == "cfg3" and not args.rows and not args.depth:
             traffic_row, pmc_rows = measured_traffic_per_row(os.path.join(ROOT, "profiles", "cfg3_k_hist_build_pmc.txt"))
             if traffic_row is not None:
                 traffic = traffic_row * rows_built / max(1, prof["hist"]["launches"])
@@ -403,7 +429,7 @@ def main():
         kernels["grad"]["GBps"] = round(gb * nb / (prof_all["grad"]["ms"] * 1e-3) / 1e9, 1)
 
     out = {
-        "metric": "train s/200 rounds @10Mx100 depth 11 (1 GPU)" if args.workload == "cfg3" and not args.rows
+        "metric": "train s/200 rounds @10Mx100 depth 11 (1 GPU)" if args.workload == "cfg3" and not args.rows and not args.depth
         else "train s/200 rounds (%s)" % args.workload,
         "value": round(value, 4), "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
@@ -416,14 +442,10 @@ def main():
         "init_s": t_init, "fit_total_s": round(t_setup + value, 2),
     }
     # rows built per level of the last tree (unit weights: Tree.w holds row counts): the smaller child of every split
-    per_level = [int(N if cond >= 255 else tree.w[0])]
-    for d in range(1, D - 1):
-        tot = 0
-        for n in range(1 << (d - 1), 1 << d):
-            if tree.split[n - 1]:
-                tot += int(min(tree.w[2 * n - 1], tree.w[2 * n]))
-        per_level.append(tot)
-    out["last_tree_rows_built_per_level"] = per_level
+    out["last_tree_rows_built_per_level"] = rows_built_per_level(tree, D, N if cond >= 255 else None)["rows"]
+    if args.levels_out:
+        with open(args.levels_out, "w") as f:
+            json.dump({"warmup": args.warmup, "steps": args.steps, "extra": extra, "trees": R.levels}, f)
     try:
         out["copy_kernel_GBps"] = round(evt._lib.copy_bandwidth(1 << 30, 10), 1)  # read + write bytes of a plain copy
         out["read_kernel_GBps"] = round(evt._lib.read_bandwidth(1 << 30, 10), 1)  # read-only stream
@@ -494,7 +516,7 @@ def main():
     # published "infer" figure; src/predict.jl:118-136): evt_predict_f64, everything included - the 8 GB upload through pinned
     # buffers, device binarize, the traversal, the predictions' way back.  The matrix is generated again (it was dropped after
     # the set-up to free host memory).
-    if args.workload == "cfg3" and not args.rows and args.side_steps > 0:
+    if args.workload == "cfg3" and not args.rows and not args.depth and args.side_steps > 0:
         try:
             x_raw, _, _ = synth(cfg)
             m_trees = [evt.Tree.bias(mu)] + [tree] * 200
@@ -523,7 +545,7 @@ def main():
 
     # BASELINE.json's other configurations, a few dozen rounds each (cfg3s = the headline matrix with the sampling the
     # reference's published 10M x 100 table was run with, on the same handle)
-    if args.side_steps > 0 and args.workload == "cfg3" and not args.rows:
+    if args.side_steps > 0 and args.workload == "cfg3" and not args.rows and not args.depth:
         side = {}
         try:
             side["cfg3s"] = side_workload(evt, "cfg3s", args.side_steps, h, y, mu, rng)
