@@ -157,6 +157,25 @@ static int record_stride(int F) {
     return ((F + 63) / 64) * 64;
 }
 
+// Piece layout of a record (evt_ctx::PBL, PU).  The conflict-free histogram kernel gives a row NS lanes, one per piece of
+// 8, 4 or 2 bytes, and issues one LDS atomic instruction per byte position of a piece: when the features fill the
+// record's last pieces only partly, ceil(F / pieces) features per piece use more of the lanes and take fewer instructions per row
+// (100 features: 7 per piece over 15 lanes instead of 8 over 13).  Chosen when one block's LDS histogram takes the whole
+// record for the largest channel count the loss can have (weights are only known later); densely packed otherwise.
+static void record_layout(int F, int B, int na_max, int RS, int *PBL, int *PU) {
+    *PBL = *PU = 1;
+    if (RS < 32 || RS > 512) return;
+    int tw = 32;
+    while (tw < RS) tw <<= 1;
+    const int pb = tw >= 128 ? 8 : (tw == 64 ? 4 : 2);
+    const int ns = tw / pb;      // lanes per row
+    const int pieces = RS / pb;  // of which the record fills this many
+    const int pu = (F + pieces - 1) / pieces;
+    if (pu >= pb || (size_t)na_max * B * ns * pu * 8 > 128 * 1024) return;
+    *PBL = pb;
+    *PU = pu;
+}
+
 static int ceil_log2_i64(int64_t v) {
     int b = 0;
     while (((int64_t)1 << b) < v) b++;
@@ -242,6 +261,12 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     c->maxlvl = 1 << (max_depth - 1);
     c->RS = record_stride(nfeats);
     c->LPR = c->RS / 16;
+    {
+        // accumulator channels of one histogram launch at most: every gradient row and the weights, EVT_HIST_GROUP at a time
+        // beyond EVT_MAX_NA (set_channels)
+        const int na_all = EVT_TWO_CHAN(loss, K) ? 2 : 2 * K + 1;
+        record_layout(nfeats, nbins, na_all <= EVT_MAX_NA ? na_all : EVT_HIST_GROUP, c->RS, &c->PBL, &c->PU);
+    }
     c->unit_w = true;
     c->have_xbin = c->have_target = c->have_grads = false;
     c->planes = nullptr; c->plane_words = 0; c->planes_ready = false; c->use_planes = 1;
@@ -950,7 +975,8 @@ static int tree_open(evt_ctx *c, const uint8_t *mask, bool mask_staged, uint8_t 
         for (int f = 0; f < c->RS; f++) h_map[f] = 0xFFFF;
         for (int i = 0; i < n_js; i++) {
             h_js[i] = jsv[i];
-            h_map[jsv[i] - 1] = (uint16_t)i;
+            const int f = (int)jsv[i] - 1;
+            h_map[(f / c->PU) * c->PBL + f % c->PU] = (uint16_t)i;
         }
         // k_tree_begin reads them from the pinned buffer (this tree's staging slot, not written again before the tree has
         // been collected)

@@ -81,6 +81,11 @@ struct evt_ctx {
     int32_t maxlvl;    // 2^(D-1)
     int32_t RS;        // bytes per observation-major record
     int32_t LPR;       // 16-byte lanes per record
+    // A record is made of pieces of PBL bytes (the unit one lane of the conflict-free histogram kernel loads) of which the
+    // first PU hold features: feature f sits at byte (f / PU) * PBL + f % PU, the other bytes are padding (bin 1).  PU < PBL
+    // spreads the features evenly over all the lanes a row has, so that a row costs PU LDS atomic instructions where
+    // a densely packed record costs PBL of them with its last lanes idle.  PBL == PU == 1: densely packed (byte f = feature f).
+    int32_t PBL, PU;
     bool unit_w;       // weights are all one (w == NULL at set_target)
     int32_t NA;        // LDS accumulator channels per bin
     int32_t NAg;       // global histogram channels per bin
@@ -125,7 +130,7 @@ struct evt_ctx {
     size_t blob_feat, blob_w, blob_gain, blob_pred, blob_stats, blob_bin, blob_split, blob_bytes;
     LevelTab lvl[2];
     uint32_t *js;      // [F]
-    uint16_t *jsmap;   // [RS] slot of feature f (0-based), 0xFFFF = not sampled / padding
+    uint16_t *jsmap;   // [RS] slot of the feature at byte p of a record, 0xFFFF = not sampled / padding
     uint8_t *feattypes;
     int32_t *mono;
     uint32_t *absmax;  // [2][EVT_ABSMAX_STRIPES][EVT_MC_MAX_NK] float bits: two sets, raised by alternate gradient passes

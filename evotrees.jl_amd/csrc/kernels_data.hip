@@ -5,8 +5,9 @@
 // column; the 16 bytes are written as one 128-bit store into the observation-major record.
 // Bins outside 1..B raise the device error flag (the histogram kernels index LDS with them).
 // Padding bytes of a record are set to 1, so that a kernel may index with them unchecked.
+// Byte p of a record holds feature (p / PBL) * PU + p % PBL when p % PBL < PU, padding otherwise (evt_ctx::PBL).
 __global__ __launch_bounds__(256) void k_transpose_validate(const uint8_t *__restrict__ xcm, uint8_t *__restrict__ xrm,
-                                                           int64_t N, int F, int B, int RS, int32_t *errflag) {
+                                                           int64_t N, int F, int B, int RS, int PBL, int PU, int32_t *errflag) {
     int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
     int grp = blockIdx.y;
     if (row >= N) return;
@@ -14,9 +15,10 @@ __global__ __launch_bounds__(256) void k_transpose_validate(const uint8_t *__res
     bool bad = false;
 #pragma unroll
     for (int t = 0; t < 16; t++) {
-        int f = grp * 16 + t;
-        uint32_t b = 1; // padding behind the last feature reads as bin 1: always a valid histogram index
-        if (f < F) {
+        const int p = grp * 16 + t;
+        const int f = (p / PBL) * PU + p % PBL;
+        uint32_t b = 1; // padding reads as bin 1: always a valid histogram index
+        if (p % PBL < PU && f < F) {
             b = xcm[(size_t)f * N + row];
             bad |= (b == 0 || b > (uint32_t)B);
         }
@@ -29,7 +31,7 @@ __global__ __launch_bounds__(256) void k_transpose_validate(const uint8_t *__res
 
 int launch_transpose_validate(evt_ctx *c) {
     dim3 grid((unsigned)((c->N + 255) / 256), (unsigned)(c->RS / 16));
-    hipLaunchKernelGGL(k_transpose_validate, grid, dim3(256), 0, c->stream, c->xcm, c->xrm, c->N, c->F, c->B, c->RS, c->errflag);
+    hipLaunchKernelGGL(k_transpose_validate, grid, dim3(256), 0, c->stream, c->xcm, c->xrm, c->N, c->F, c->B, c->RS, c->PBL, c->PU, c->errflag);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }

@@ -115,8 +115,7 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
     unsigned vmask = 0;
 #pragma unroll
     for (int t = 0; t < 16; t++) {
-        int f = sub * 16 + t;
-        int s = (f < A.F) ? (int)A.jsmap[f] : 0xFFFF;
+        int s = (int)A.jsmap[sub * 16 + t]; // by record byte: 0xFFFF for padding and for features outside the sample
         s = (s == 0xFFFF) ? -1 : s - slot0;
         const bool ok = (s >= 0 && s < nslots);
         off[t] = ok ? s * A.B - 1 : 0; // bins are 1-based
@@ -267,8 +266,9 @@ __global__ __launch_bounds__(1024) void k_hist_build(HistArgs A) {
 // A record is read in pieces of PB bytes, one lane each, NS = RS/PB lanes per row with PB chosen so that NS is a
 // multiple of 16 (8-byte pieces from 128-byte records up, 4-byte pieces for 64-byte records, 2-byte pieces for
 // 32-byte ones): every group of 16 consecutive lanes - the unit the LDS serves per cycle for 64-bit operations -
-// holds 16 different pieces `sub` of ONE row.  The LDS histogram is laid out as word(a, t, bin, sub) =
-// ((a*PB + t)*B + bin)*NS + sub for feature f = PB*sub + t, i.e. `sub` selects the bank pair, so the 16 lanes of a
+// holds 16 different pieces `sub` of ONE row.  The first PU bytes of a piece hold features (evt_ctx::PU; PU == PB for a
+// densely packed record); a row costs PU LDS atomic instructions.  The LDS histogram is laid out as word(a, t, bin, sub)
+// = ((a*PU + t)*B + bin)*NS + sub for byte t of piece sub, i.e. `sub` selects the bank pair, so the 16 lanes of a
 // group always fall on 16 different bank pairs whatever their bins are.  Rows that share a wave instruction sit in
 // different groups and cannot collide inside one LDS pass either.  (Two 64-byte records per 16-lane group, 8 lanes of
 // 8-byte pieces each, collide whenever their bins' words share a bank half: cfg5's histograms took 0.64 ms per round
@@ -312,9 +312,9 @@ __device__ __forceinline__ uint32_t load_id(const uint32_t *p) {
     return NT ? __builtin_nontemporal_load(p) : *p;
 }
 
-template <int NA, bool PACK, int U, bool FULL, int PB, bool NT>
+template <int NA, bool PACK, int U, bool FULL, int PB, int PU, bool NT>
 __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
-    extern __shared__ unsigned long long H[]; // [NA][PB][B][NS]
+    extern __shared__ unsigned long long H[]; // [NA][PU][B][NS]
     const int tid = threadIdx.x, nthr = blockDim.x;
     const int lane = tid & 63, wave = tid >> 6, nwaves = nthr >> 6;
     const int n_build = (int)A.hdr[LH_N_BUILD];
@@ -324,6 +324,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     if (blockIdx.x == 0 && tid == 0 && A.a0 == 0) A.stats[A.level] = total - (int64_t)n_build * A.seg_cost;
 
     static_assert(PB == 8 || PB == 4 || PB == 2, "a piece is 8, 4 or 2 bytes");
+    static_assert(PU >= 1 && PU <= PB, "features per piece");
     const int NS = A.NSL;         // lanes per row: one per piece of the record, idle ones beyond its last piece
     const int RPW = 64 / NS;      // rows per wave instruction
     const int step = nwaves * RPW;
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     int64_t end = start + T < total ? start + T : total;
 
     const int B = A.B;
-    const int plane = PB * B * NS; // words per channel
+    const int plane = PU * B * NS; // words per channel
     for (int i = tid; i < NA * plane; i += nthr) H[i] = 0ull;
 
     const int sub = lane % NS, rloc = lane / NS;
@@ -345,7 +346,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     const int subl = (tb + sub * PB < A.RS) ? sub : 0; // an idle lane loads the tile's first piece and adds nothing (no feature: vmask 0)
     // byte offset of (t, bin 0) for this lane; bins are 1-based so bin*NS*8 is added on top
     // (32-bit unsigned arithmetic throughout: one 24-bit multiply-add per LDS address)
-    uint32_t coff[PB];
+    uint32_t coff[PU];
     unsigned vmask = 0;
     {
         // the slots of this lane's PB features in one load (jsmap has an entry for every byte of the record, 0xFFFF for
@@ -364,7 +365,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             }
         }
 #pragma unroll
-        for (int t = 0; t < PB; t++) {
+        for (int t = 0; t < PU; t++) {
             const bool ok = ((mw[t >> 1] >> (16 * (t & 1))) & 0xFFFFu) != 0xFFFFu;
             coff[t] = (uint32_t)(((t * B - 1) * NS + sub) * 8);
             vmask |= ok ? (1u << t) : 0u;
@@ -463,7 +464,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             }                                                                                                         \
             if (lane_on && (pw + (u_) * RPW + rloc < nend)) {                                                          \
                 const uint32_t wds[2] = {v[ui].x, v[ui].y};                                                            \
-                _Pragma("unroll") for (int t = 0; t < PB; t++) {                                                       \
+                _Pragma("unroll") for (int t = 0; t < PU; t++) {                                                       \
                     if (FULL || (vmask & (1u << t))) {                                                                \
                         const uint32_t bo = __umul24((wds[t >> 2] >> (8 * (t & 3))) & 0xFFu, binmul) + coff[t];       \
                         _Pragma("unroll") for (int a = 0; a < NA; a++)                                                 \
@@ -492,12 +493,13 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
         const bool sole = (nbeg >= blk_start) && (nrows_end <= blk_end) && !(PACK && nrows_end - nbeg > EVT_HIST_MAX_ROWS_PER_BLOCK);
         long long *hn = A.hist + (int64_t)(A.bnode[i] - 1) * A.node_stride;
         const int nchunks = (B + 7) >> 3;
-        const int nitems = NA * PB * nchunks * NS * 8; // (channel, t, bin chunk, piece, bin in chunk), the last fastest
+        const int nitems = NA * PU * nchunks * NS * 8; // (channel, t, bin chunk, piece, bin in chunk), the last fastest
         const int rot = (int)(((int64_t)blockIdx.x * 1031) % (nitems >> 6)) << 6;
         // FU items per thread at a time: their LDS words (and, when features are sampled, their slots) are all
         // requested before the first is used, so a flush costs one LDS and one memory round trip, not FU of each
         constexpr int FU = 8;
         const bool all_feats = A.nfs == A.F; // slot of feature f is f itself
+        const int piece0 = tb / PB;          // first piece of this column tile
         const bool pow2 = (nchunks & (nchunks - 1)) == 0; // decode with shifts
         const int ns_sh = __ffs(NS) - 1, nc_sh = __ffs(nchunks) - 1;
         for (int k0 = tid; k0 < nitems; k0 += FU * nthr) {
@@ -525,15 +527,15 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                         chunk = rest % nchunks;
                         rest /= nchunks;
                     }
-                    const int t = rest & (PB - 1);
-                    const int a = rest / PB;
+                    const int t = rest % PU;
+                    const int a = rest / PU;
                     const int b = chunk * 8 + bl;
-                    const int f = tb + sidx * PB + t;
+                    const int f = (piece0 + sidx) * PU + t; // the feature at byte t of the piece
                     if (b < B) {
                         hwv[j] = &H[(size_t)a * plane + ((size_t)t * B + b) * NS + sidx];
                         wv[j] = *hwv[j];
                         av[j] = a; bv[j] = b;
-                        if (f < A.F) slotv[j] = all_feats ? f : (int)A.jsmap[f]; // a padding byte's word has no slot
+                        if (f < A.F) slotv[j] = all_feats ? f : (int)A.jsmap[tb + sidx * PB + t]; // a padding byte's word has no slot
                     }
                 }
             }
@@ -572,7 +574,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
     }
 }
 
-template <int NA, bool PACK, int U, int PB, bool NT>
+template <int NA, bool PACK, int U, int PB, int PU, bool NT>
 static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads, size_t lds) {
     // unpredicated atomics for every feature of the record pay off unless most features are left out: the words of
     // features outside the sample are simply not flushed
@@ -580,16 +582,16 @@ static int launch_hist16_q(evt_ctx *c, const HistArgs &A, dim3 grid, int threads
     if (lds > 64 * 1024) { // one block per CU may take most of its 160 KB
         static EvtDevOnce once;
         if (once.pending(c->device)) {
-            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, true, PB, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, false, PB, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, true, PB, PU, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_hist_build16<NA, PACK, U, false, PB, PU, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
             once.mark(c->device);
         }
     }
     // c->launch_e0 / launch_e1 (when profiling): the kernel's own dispatch records them
     if (full)
-        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, true, PB, NT>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
+        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, true, PB, PU, NT>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
     else
-        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, false, PB, NT>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
+        hipExtLaunchKernelGGL((k_hist_build16<NA, PACK, U, false, PB, PU, NT>), grid, dim3(threads), (uint32_t)lds, c->stream, c->launch_e0, c->launch_e1, 0, A);
     HIPCHK(hipGetLastError());
     return EVT_OK;
 }
@@ -600,9 +602,16 @@ static int launch_hist16_t(evt_ctx *c, const HistArgs &A, dim3 grid, int threads
     constexpr int U = (NA <= 2) ? 16 : 8;
     // records larger in total than the last-level cache (256 MB) are streamed past it
     const bool nt = (size_t)c->N * c->RS > ((size_t)256 << 20);
-    if (A.TW >= 128) return nt ? launch_hist16_q<NA, PACK, U, 8, true>(c, A, grid, threads, lds) : launch_hist16_q<NA, PACK, U, 8, false>(c, A, grid, threads, lds);
-    if (A.TW == 64) return nt ? launch_hist16_q<NA, PACK, U, 4, true>(c, A, grid, threads, lds) : launch_hist16_q<NA, PACK, U, 4, false>(c, A, grid, threads, lds);
-    return nt ? launch_hist16_q<NA, PACK, U, 2, true>(c, A, grid, threads, lds) : launch_hist16_q<NA, PACK, U, 2, false>(c, A, grid, threads, lds); // 32-byte tiles
+    // (piece bytes, features per piece): a densely packed record has PU == PB, record_layout() picks the others
+    const int pb = A.TW >= 128 ? 8 : (A.TW == 64 ? 4 : 2);
+    const int pu = c->PU < c->PBL ? c->PU : pb;
+#define H16Q(PB_, PU_)                                                                                                     \
+    if (pb == PB_ && pu == PU_)                                                                                            \
+        return nt ? launch_hist16_q<NA, PACK, U, PB_, PU_, true>(c, A, grid, threads, lds) : launch_hist16_q<NA, PACK, U, PB_, PU_, false>(c, A, grid, threads, lds);
+    H16Q(8, 8) H16Q(8, 7) H16Q(8, 6) H16Q(8, 5) H16Q(4, 4) H16Q(4, 3) H16Q(2, 2)
+#undef H16Q
+    evt_set_error("no histogram kernel for pieces of %d bytes holding %d features", pb, pu);
+    return EVT_ERR_INTERNAL;
 }
 
 template <int NA, bool PACK>
@@ -681,13 +690,14 @@ int launch_hist_build(evt_ctx *c, int level, const uint32_t *is_cur) {
         // generic kernel.)
         int tw = 32;
         while (tw < c->RS && tw < 512) tw <<= 1;
-        while (tw > 32 && (size_t)na * c->B * tw * 8 > 128 * 1024) tw >>= 1;
+        const bool spread = c->PU < c->PBL; // features spread over all pieces: one tile takes the whole record (record_layout)
+        while (!spread && tw > 32 && (size_t)na * c->B * tw * 8 > 128 * 1024) tw >>= 1;
         const int pb16 = tw >= 128 ? 8 : (tw == 64 ? 4 : 2);
         A.TW = tw;
         A.NSL = tw / pb16;
         const int ntiles16 = (c->RS + tw - 1) / tw;
-        const size_t lds16 = (size_t)na * c->B * tw * 8; // channels x bins x tile bytes words
-        const bool can16 = c->RS >= 32 && lds16 <= 128 * 1024;
+        const size_t lds16 = (size_t)na * c->B * A.NSL * (spread ? c->PU : pb16) * 8; // channels x bins x feature bytes of a tile, words
+        const bool can16 = c->RS >= 32 && lds16 <= 128 * 1024 && (!spread || (pb16 == c->PBL && ntiles16 == 1));
         const bool use16 = (c->hist_variant == 1) ? false : can16;
         if (!use16 && c->LPR > 64) { // the generic kernel reads a record with one wavefront instruction: 64 lanes of 16 bytes
             evt_set_error("%d accumulator channels x %d bins need the generic histogram kernel, which takes at most 1024 features", na, c->B);

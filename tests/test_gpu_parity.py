@@ -135,6 +135,12 @@ CASES = [
     ("logistic_mle", True, 30000, 20, 32, 6, "binary", 20, 1.0, dict(min_weight=8.0)),
     ("logistic_mle", False, 20000, 100, 64, 5, "oblivious", 50, 0.5, dict(min_weight=8.0)),
     ("mse", False, 20000, 300, 16, 5, "binary", 300, 1.0, {}),
+    # records whose features are spread over all their pieces: 5, 6 and 7 features per 8-byte piece, 3 per 4-byte piece,
+    # 32 lanes per row, with and without a column sample that switches the per-feature test on
+    ("mse", False, 30000, 80, 32, 5, "binary", 80, 1.0, {}),
+    ("mse", False, 20000, 90, 64, 5, "binary", 40, 1.0, {}),
+    ("mse", True, 30000, 40, 32, 5, "binary", 15, 0.8, {}),
+    ("logloss", False, 20000, 150, 16, 5, "binary", 150, 1.0, {}),
     ("mse", False, 1000, 3, 4, 1, "binary", 3, 1.0, {}),
     ("mse", False, 300, 1, 2, 3, "binary", 1, 1.0, dict(min_weight=0.0)),
     ("poisson", True, 30000, 12, 32, 6, "binary", 9, 0.8, {}),
