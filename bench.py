@@ -114,6 +114,25 @@ def measured_traffic_per_row(path):
         return None, None
 
 
+def record_slot_fill(F, B, na_max):
+    """Share of the LDS atomic lane slots a row takes in the conflict-free histogram kernel that carry a feature: a row is
+    read as pieces of 8, 4 or 2 bytes by NS lanes (a power of two >= 16) and costs one instruction per feature byte of a
+    piece - all bytes of a piece when the record is densely packed, ceil(F / pieces) when the features are spread over the
+    record's pieces (the library's record_layout, csrc/api.hip)."""
+    RS = 16 if F <= 16 else 32 if F <= 32 else 64 if F <= 64 else (F + 63) // 64 * 64
+    if RS < 32 or RS > 512:
+        return 1.0
+    tw = 32
+    while tw < RS:
+        tw *= 2
+    pb = 8 if tw >= 128 else 4 if tw == 64 else 2
+    ns, pieces = tw // pb, RS // pb
+    pu = -(-F // pieces)
+    if pu >= pb or na_max * B * ns * pu * 8 > 128 * 1024:
+        pu = pb
+    return F / (pu * ns)
+
+
 def prepare(evt, cfg, opts=None):
     """Synthetic data of the configuration, quantile edges, handle creation, upload + device binarize, target.
     Returns the handle and the seconds spent in each part (data generation apart: it is not part of a fit)."""
@@ -401,19 +420,20 @@ def main():
                     "traffic_bytes_per_row": None if traffic_row is None else round(traffic_row, 1), "traffic_profiled_rows": pmc_rows,
                     "rows_features_per_s": round(rows_built * nfs / (hist_ms * 1e-3), 1)}
         # The kernel's other bound: one 64-bit LDS atomic per (built row, sampled feature) and accumulator channel.  Peak = the
-        # device's measured rate of such atomics in the kernel's own conflict-free layout with all 64 lanes issuing; the
-        # kernel's record layout lets 13 of every 16 lanes issue (100 features in 8-byte pieces), the third figure.
+        # device's measured rate of such atomics in the kernel's own conflict-free layout with all 64 lanes issuing.  The
+        # record layout decides how many of the issued lane slots carry a feature (layout_fill: 100 features as 7 per
+        # 8-byte piece fill 100 of the 7 x 16 slots a row takes); peak x fill is what the layout allows.
         try:
             lane16, instr16 = evt._lib.lds_atomic_rate(0, 16, 200)
-            lane13, instr13 = evt._lib.lds_atomic_rate(0, 13, 200)
             lane_rand, _ = evt._lib.lds_atomic_rate(1, 16, 200)
             na_lds = 1 if (loss == "mse") else (4 if loss == "gaussian_mle" else 2)  # unit weights: mse packs {g, count} into one word
             ach = rows_built * nfs * na_lds / (hist_ms * 1e-3)
+            fill = record_slot_fill(F, B, 2 if loss == "mse" else (5 if loss == "gaussian_mle" else 3))
             roofline["secondary"] = {"bound": "lds_atomic", "achieved": round(ach / 1e9, 1), "peak": round(lane16 / 1e9, 1),
                                      "unit": "G lane-atomics/s", "frac": round(ach / lane16, 4),
-                                     "peak_with_13_of_16_lanes": round(lane13 / 1e9, 1), "frac_of_13_lane_peak": round(ach / lane13, 4),
+                                     "layout_fill": round(fill, 4), "frac_of_peak_x_fill": round(ach / (lane16 * fill), 4),
                                      "peak_random_banks": round(lane_rand / 1e9, 1),
-                                     "wave_instr_per_s_16_lanes": round(instr16 / 1e9, 2), "wave_instr_per_s_13_lanes": round(instr13 / 1e9, 2)}
+                                     "wave_instr_per_s": round(instr16 / 1e9, 2)}
             # the flush: 64-bit global atomics, every block adds the 12 800 words of a node's slice (100 features x 64 bins x 2)
             ga = evt._lib.global_atomic_rate(nfs * B * 2 // 64 * 64, 256, 4)
             roofline["flush_global_atomics"] = {"rate_G_per_s": round(ga / 1e9, 1), "atomics_per_launch": 256 * nfs * B * 2,
