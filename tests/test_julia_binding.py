@@ -1,6 +1,6 @@
 """Keeps julia/EvoTreesHIP.jl in step with include/evotrees_hip.h without a Julia toolchain: every `ccall` of the module
 is parsed and its argument tuple compared with the C prototype it binds (arity and types), the two mirrored structs
-are compared field by field, and every `EvoTrees.<name>` the module touches must be tabulated in INTEGRATION.md."""
+are compared field by field, and every `EvoTrees.<name>` the module touches must be tabulated in the integration notes."""
 import os
 import re
 
@@ -178,9 +178,9 @@ def test_parser_notices_a_changed_prototype():
 
 
 def test_every_reference_name_is_tabulated():
-    """Every EvoTrees.<name> the module extends or calls appears in INTEGRATION.md."""
+    """Every EvoTrees.<name> the module extends or calls appears in the integration notes at the repository root."""
     s = strip_comments_jl(open(JL).read())
     names = set(re.findall(r"\bEvoTrees\.([A-Za-z_!][A-Za-z_0-9!]*)", s)) - {"Random", "Tables"}
     doc = open(INTEG).read()
     missing = sorted(n for n in names if n not in doc)
-    assert not missing, "not mentioned in INTEGRATION.md: " + ", ".join(missing)
+    assert not missing, "not tabulated in the integration notes: " + ", ".join(missing)
