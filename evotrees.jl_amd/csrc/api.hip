@@ -14,7 +14,7 @@
 
 int launch_absmax_rows(evt_ctx *c, int k0, int k1);
 int launch_check_unit_weight(evt_ctx *c);
-int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, const float *leaf_pred_dev);
+int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, int nnodes, const float *leaf_pred_dev);
 int launch_predict_model(hipStream_t s, const uint32_t *nodes, const float *leaf_pred, const int64_t *off, int ntrees, const uint8_t *xcm, int64_t N,
                          int K, int loss, int apply_link, float *out, const int32_t *skip_flag);
 int predict_lds_shape(int F, int max_int, int K, int hint);
@@ -1420,7 +1420,7 @@ extern "C" int evt_predict_tree(evt_handle c, int32_t nnodes_tree, const int64_t
     if (r != EVT_OK) return r;
     c->pt_busy = true;
     prof_begin(c, EVT_K_PREDICT, 0);
-    r = launch_predict_tree_nodes(c, c->pt_nodes, c->pt_pred);
+    r = launch_predict_tree_nodes(c, c->pt_nodes, nnodes_tree, c->pt_pred);
     prof_end(c);
     if (r != EVT_OK) return r;
     if (c->profiling) {

@@ -23,19 +23,74 @@ __device__ __forceinline__ int walk_packed(const uint32_t *__restrict__ nodes, c
 
 // one tree added to pred (K x N), all rows.  copy_blocks extra blocks at the end of the grid carry copy_n 16-byte words
 // from copy_src to copy_dst: the finished tree's way back to the host's pinned buffer, when this is the tree's last kernel.
-__global__ __launch_bounds__(256) void k_predict_tree(const uint32_t *__restrict__ nodes, const float *__restrict__ leaf_pred,
+// A row's walk is a chain of dependent loads (node word, bin byte, node word, ...), so the kernel is paced by latency, not by
+// the bytes it moves: the first n_lds node words (the upper levels of the heap, all of it for depths up to 13) are copied to
+// LDS, where a lookup costs a fraction of a trip to the caches, and a thread walks R rows side by side - R bin bytes are
+// requested before the first is used.  Rows of a thread are 256 apart: the threads of a wavefront read neighbouring bytes.
+template <int R>
+__global__ __launch_bounds__(256) void k_predict_tree(const uint32_t *__restrict__ nodes, int n_lds, const float *__restrict__ leaf_pred,
                                                      const uint8_t *__restrict__ xcm, int64_t N, int K, int loss, float *pred,
                                                      const uint4 *__restrict__ copy_src, uint4 *__restrict__ copy_dst, int64_t copy_n,
                                                      int copy_blocks) {
+    extern __shared__ uint32_t s_nodes[];
     const int64_t G = (int64_t)gridDim.x - copy_blocks;
     if ((int64_t)blockIdx.x >= G) {
         for (int64_t k = ((int64_t)blockIdx.x - G) * 256 + threadIdx.x; k < copy_n; k += (int64_t)copy_blocks * 256) copy_dst[k] = copy_src[k];
         return;
     }
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= N) return;
-    const int nid = walk_packed(nodes, xcm, N, i);
-    evt_add_leaf(pred + (size_t)K * i, leaf_pred + (size_t)K * (nid - 1), K, loss);
+    for (int k = threadIdx.x; k < n_lds; k += 256) s_nodes[k] = nodes[k];
+    __syncthreads();
+    const int64_t i0 = (int64_t)blockIdx.x * (256 * R) + threadIdx.x;
+    int nid[R];
+    uint32_t nd[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        nid[r] = 1;
+        nd[r] = (i0 + 256 * r < N) ? s_nodes[0] : 0u; // a row past the end walks nothing
+    }
+    for (;;) {
+        uint32_t xb[R];
+        bool any = false;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            xb[r] = 0;
+            if (nd[r] & EVT_NODE_SPLIT) {
+                xb[r] = xcm[(size_t)((nd[r] & 0xFFFFu) - 1) * N + (i0 + 256 * r)];
+                any = true;
+            }
+        }
+        if (!any) break;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (nd[r] & EVT_NODE_SPLIT) {
+                const uint32_t cb = (nd[r] >> 16) & 0xFFu;
+                const bool cond = (nd[r] & EVT_NODE_NUMERIC) ? (xb[r] <= cb) : (xb[r] == cb);
+                nid[r] = (nid[r] << 1) + (cond ? 0 : 1);
+                nd[r] = (nid[r] - 1 < n_lds) ? s_nodes[nid[r] - 1] : nodes[nid[r] - 1];
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int64_t i = i0 + 256 * r;
+        if (i < N) evt_add_leaf(pred + (size_t)K * i, leaf_pred + (size_t)K * (nid[r] - 1), K, loss);
+    }
+}
+
+// rows per thread: four once the rows fill the device several times over, one for small inputs (more blocks)
+static int launch_predict_tree_any(evt_ctx *c, const uint32_t *nodes, int nnodes, const float *leaf_pred, const uint4 *copy_src, uint4 *copy_dst,
+                                   int64_t copy_n, int copy_blocks) {
+    const int n_lds = nnodes < 8192 ? nnodes : 8192;
+    const size_t lds = (size_t)n_lds * sizeof(uint32_t);
+    if (c->N >= ((int64_t)1 << 21)) {
+        hipLaunchKernelGGL(k_predict_tree<4>, dim3((unsigned)((c->N + 1023) / 1024) + (unsigned)copy_blocks), dim3(256), lds, c->stream, nodes, n_lds,
+                           leaf_pred, c->xcm, c->N, c->K, c->loss, c->pred, copy_src, copy_dst, copy_n, copy_blocks);
+    } else {
+        hipLaunchKernelGGL(k_predict_tree<1>, dim3((unsigned)((c->N + 255) / 256) + (unsigned)copy_blocks), dim3(256), lds, c->stream, nodes, n_lds,
+                           leaf_pred, c->xcm, c->N, c->K, c->loss, c->pred, copy_src, copy_dst, copy_n, copy_blocks);
+    }
+    HIPCHK(hipGetLastError());
+    return EVT_OK;
 }
 
 // node each sampled row of the last tree ended in (0 outside the sample): the walk reproduces the
@@ -59,19 +114,15 @@ int launch_nidx_from_tree(evt_ctx *c, bool use_mask, uint8_t cond) {
 int launch_predict_tree_cache(evt_ctx *c, bool send_blob) {
     const int64_t copy_n = send_blob ? (int64_t)(c->blob_bytes / 16) : 0;
     const int copy_blocks = (int)std::min<int64_t>(64, (copy_n + 255) / 256);
-    hipLaunchKernelGGL(k_predict_tree, dim3((unsigned)((c->N + 255) / 256) + (unsigned)copy_blocks), dim3(256), 0, c->stream, c->tree.packed,
-                       c->tree.pred, c->xcm, c->N, c->K, c->loss, c->pred, reinterpret_cast<const uint4 *>(c->tree_blob),
-                       reinterpret_cast<uint4 *>(c->h_stage_dev), copy_n, copy_blocks);
-    HIPCHK(hipGetLastError());
+    const int r = launch_predict_tree_any(c, c->tree.packed, c->nnodes, c->tree.pred, reinterpret_cast<const uint4 *>(c->tree_blob),
+                                          reinterpret_cast<uint4 *>(c->h_stage_dev), copy_n, copy_blocks);
+    if (r != EVT_OK) return r;
     if (send_blob) c->step.blob_sent = true;
     return EVT_OK;
 }
 
-int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, const float *leaf_pred_dev) {
-    hipLaunchKernelGGL(k_predict_tree, dim3((unsigned)((c->N + 255) / 256)), dim3(256), 0, c->stream, nodes_dev, leaf_pred_dev, c->xcm, c->N,
-                       c->K, c->loss, c->pred, static_cast<const uint4 *>(nullptr), static_cast<uint4 *>(nullptr), (int64_t)0, 0);
-    HIPCHK(hipGetLastError());
-    return EVT_OK;
+int launch_predict_tree_nodes(evt_ctx *c, const uint32_t *nodes_dev, int nnodes, const float *leaf_pred_dev) {
+    return launch_predict_tree_any(c, nodes_dev, nnodes, leaf_pred_dev, static_cast<const uint4 *>(nullptr), static_cast<uint4 *>(nullptr), (int64_t)0, 0);
 }
 
 // apply_prediction_link!, src/predict.jl:105-116 (softmax!: :187-195)
