@@ -111,11 +111,15 @@ __global__ __launch_bounds__(256) void k_part_count(PartArgs A) {
             const int64_t p = p0 + it * 256 + tid;
             rid[it] = A.is_cur[p < pend ? p : pend - 1];
         }
-        if (A.status[n] != ST_SPLIT) {
+        // the node's split word is requested together with its state (and the row ids), not one trip later behind the
+        // branch on the state: a node without a split holds 0 there, which is not used
+        const int st = A.status[n];
+        uint32_t nd = A.t_packed[n - 1];
+        asm volatile("" : "+v"(nd));
+        if (st != ST_SPLIT) {
             if (tid == 0) A.chunk_nleft[c] = 0;
             continue;
         }
-        const uint32_t nd = A.t_packed[n - 1];
         const int f = (int)(nd & 0xFFFFu) - 1;
         const uint32_t cb = (nd >> 16) & 0xFFu;
         const bool numeric = (nd & EVT_NODE_NUMERIC) != 0;
@@ -555,13 +559,14 @@ __global__ __launch_bounds__(256) void k_final_fused(PartArgs A) {
             rid[it] = A.is_cur[p < pend ? p : pend - 1];
         }
         const int st = A.status[n];
+        uint32_t nd = A.t_packed[n - 1]; // requested with the state, not behind the branch on it
+        asm volatile("" : "+v"(nd));
         if (st != ST_SPLIT && st != ST_LEAF) continue;
         const bool is_split = (st == ST_SPLIT);
         int f = 0;
         uint32_t cb = 0;
         bool numeric = true;
         if (is_split) {
-            const uint32_t nd = A.t_packed[n - 1];
             f = (int)(nd & 0xFFFFu) - 1;
             cb = (nd >> 16) & 0xFFu;
             numeric = (nd & EVT_NODE_NUMERIC) != 0;
