@@ -404,7 +404,7 @@ extern "C" int evt_create(int64_t nobs, int32_t nfeats, int32_t nbins, int32_t K
     if (tree_type == EVT_TREE_OBLIVIOUS) ALLOC(c->ogains, (size_t)c->maxlvl * c->F * c->B);
     {
         uint8_t *sb = nullptr;
-        ALLOC(sb, (size_t)c->maxlvl * ((c->F + 3) / 4) * 16);
+        ALLOC(sb, (size_t)c->maxlvl * ((c->F + 3) / 4) * 64); // one 64-byte candidate (ScanBestQ, kernels_scan.hip) per node and group of 4 features
         c->sbest = sb;
     }
     // pinned staging: tree read-back + small per-tree uploads

@@ -156,7 +156,7 @@ struct evt_ctx {
     int64_t *stats;    // [D+1] rows built per level
     int32_t *errflag;  // device-side validation flag
     double *ogains;    // oblivious: [maxlvl][F][B]
-    void *sbest;       // split search: best candidate per (node of the level, feature group), 16 B each
+    void *sbest;       // split search: best candidate per (node of the level, feature group), 64 B each
 
     // host staging (pinned): two slots of h_stage_bytes each, so that a second tree can be queued before the first one
     // has been collected.  h_stage / h_stage_dev point at the slot of the tree queued last.

@@ -16,9 +16,19 @@ struct ScanBest {
     double gain;
     int jp, bin;
 };
+// The candidate as the one- and two-output kernels hand it over: with the feature (1-based id, negative when categorical)
+// and the fixed-point totals left of the split, so that the pass that decides needs neither the feature tables nor the
+// histogram again.
+struct ScanBestQ {
+    double gain;
+    int jp, bin;
+    int feat, pad;
+    long long qL[EVT_MAX_NA];
+};
+static_assert(sizeof(ScanBestQ) == 64, "one candidate per 64-byte line");
 
 struct ScanArgs {
-    ScanBest *sbest;
+    ScanBest *sbest; // ScanBestQ entries for k_scan / k_scan_fin (same buffer)
     long long *hist;
     int64_t node_stride;
     const uint32_t *js;
@@ -274,7 +284,8 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
     __shared__ double s_sc[EVT_MAX_NA];
     __shared__ double s_wg[16];
     __shared__ int s_wjp[16], s_wbin[16];
-    __shared__ int s_wfeat[16]; // FUSED: feature of each wave (1-based id, negative when categorical)
+    __shared__ int s_wfeat[16]; // feature of each wave (1-based id, negative when categorical)
+    __shared__ long long s_wq[FUSED ? 1 : 4][NAG]; // two-pass search: left totals of each wave's best candidate
     __shared__ int s_dec[3];
 
     long long pre[NAG][BPL];
@@ -347,6 +358,9 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
 
     double wbest = -INFINITY;
     int wjp = NO_BIN, wbin = NO_BIN;
+    long long wq[NAG];
+#pragma unroll
+    for (int ag = 0; ag < NAG; ag++) wq[ag] = 0;
     const int nodeidx = blockIdx.x;
 
     if (have) {
@@ -367,14 +381,19 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
         }
         double lg = -INFINITY;
         int lb = NO_BIN;
+        long long lq[NAG]; // fixed-point totals left of this lane's best candidate
+#pragma unroll
+        for (int ag = 0; ag < NAG; ag++) lq[ag] = 0;
 #pragma unroll
         for (int t = 0; t < BPL; t++) {
             const int b = lane * BPL + t;
             if (b < B) {
                 double gain = 0.0;
                 bool ok = false;
+                long long q[NAG];
+#pragma unroll
+                for (int ag = 0; ag < NAG; ag++) q[ag] = 0;
                 if (b + 1 <= bmax) {
-                    long long q[NAG];
 #pragma unroll
                     for (int ag = 0; ag < NAG; ag++) {
                         const long long prev = (t == 0) ? excl[ag] : pre[ag][t > 0 ? t - 1 : 0];
@@ -407,6 +426,8 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
                 } else if (ok && gain > lg) {
                     lg = gain;
                     lb = b + 1;
+#pragma unroll
+                    for (int ag = 0; ag < NAG; ag++) lq[ag] = q[ag];
                 }
             }
         }
@@ -418,20 +439,33 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
                 if (og > lg || (og == lg && ob < lb)) { lg = og; lb = ob; }
             }
             if (lg > wbest) { wbest = lg; wjp = jp; wbin = lb; }
+            if constexpr (!FUSED) {
+                // the lane that holds the winning bin hands its left totals to the whole wave
+                const int owner = (lb != NO_BIN) ? (lb - 1) / BPL : 0;
+#pragma unroll
+                for (int ag = 0; ag < NAG; ag++) {
+                    const int lo = __shfl((int)(lq[ag] & 0xffffffffll), owner), hi = __shfl((int)(lq[ag] >> 32), owner);
+                    wq[ag] = ((long long)hi << 32) | (unsigned int)lo;
+                }
+            }
         }
     }
     if (A.oblivious) return; // decision is taken for the whole level by k_obliv_select
 
     if (lane == 0) {
         s_wg[wave] = wbest; s_wjp[wave] = wjp; s_wbin[wave] = wbin;
-        if (FUSED) s_wfeat[wave] = numeric ? f + 1 : -(f + 1);
+        s_wfeat[wave] = numeric ? f + 1 : -(f + 1);
+        if constexpr (!FUSED) {
+#pragma unroll
+            for (int ag = 0; ag < NAG; ag++) s_wq[wave][ag] = wq[ag];
+        }
     }
     __syncthreads();
     double bg = -INFINITY;
-    int bj = NO_BIN, bb = NO_BIN;
+    int bj = NO_BIN, bb = NO_BIN, bw = 0;
     if (tid == 0) {
         for (int w = 0; w < nwaves; w++) {
-            if (s_wg[w] > bg || (s_wg[w] == bg && s_wjp[w] < bj)) { bg = s_wg[w]; bj = s_wjp[w]; bb = s_wbin[w]; }
+            if (s_wg[w] > bg || (s_wg[w] == bg && s_wjp[w] < bj)) { bg = s_wg[w]; bj = s_wjp[w]; bb = s_wbin[w]; bw = w; }
         }
     }
     if constexpr (FUSED) {
@@ -462,9 +496,12 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
         }
         if (A.zero_children) zero_children_slices<NAG>(A, n);
     } else if (tid == 0) {
-        ScanBest r;
+        ScanBestQ r;
         r.gain = bg; r.jp = bj; r.bin = bb;
-        A.sbest[(int64_t)nodeidx * gridDim.y + blockIdx.y] = r;
+        r.feat = s_wfeat[bw]; r.pad = 0;
+#pragma unroll
+        for (int ag = 0; ag < EVT_MAX_NA; ag++) r.qL[ag] = (ag < NAG) ? s_wq[bw][ag < NAG ? ag : 0] : 0;
+        reinterpret_cast<ScanBestQ *>(A.sbest)[(int64_t)nodeidx * gridDim.y + blockIdx.y] = r;
     }
 }
 
@@ -493,11 +530,29 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
         }
         return;
     }
+    // Everything the block needs is requested in one batch of unconditional loads, ahead of the branch on the node's
+    // state: the state itself, the node's totals and decode scales, and this thread's candidate (group tid, clamped).
+    const int tq = tid < NAG ? tid : 0;
+    double qs = A.qscale[tq];
+    long long nsq = A.node_sum[(int64_t)n * NAG + tq]; // not yet written at level 1, and not used there
+    union CandWords {
+        ScanBestQ q;
+        uint4 v[4];
+    };
+    CandWords cw;
+    {
+        const uint4 *cp = reinterpret_cast<const uint4 *>(reinterpret_cast<const ScanBestQ *>(A.sbest) + (int64_t)blockIdx.x * ngroups + (tid < ngroups ? tid : 0));
+#pragma unroll
+        for (int k = 0; k < 4; k++) cw.v[k] = cp[k];
+    }
+    // nodes of the last level are the children of the split nodes above them (the root when max_depth == 1)
+    int st = A.leaf_level ? (n > 1 ? A.status[n >> 1] : ST_SPLIT) : A.status[n];
+    asm volatile("" : "+v"(st), "+v"(qs), "+v"(nsq));
+#pragma unroll
+    for (int k = 0; k < 4; k++) asm volatile("" : "+v"(cw.v[k].x), "+v"(cw.v[k].y), "+v"(cw.v[k].z), "+v"(cw.v[k].w));
     if (A.leaf_level) {
-        // nodes of the last level are the children of the split nodes above them (the root when max_depth == 1)
-        if (n > 1 && A.status[n >> 1] != ST_SPLIT) return;
+        if (st != ST_SPLIT) return;
     } else {
-        const int st = A.status[n];
         if (st != ST_BUILD && st != ST_SUBTRACT) return;
     }
     const int NK = A.NK, K = A.K;
@@ -510,7 +565,23 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
     __shared__ int s_j[256], s_b[256];
     __shared__ int s_dec[3];
 
-    node_totals<NAG>(A, n, hn, true, s_Sq, s_S, s_sc);
+    if (A.level == 1) {
+        node_totals<NAG>(A, n, hn, true, s_Sq, s_S, s_sc);
+    } else {
+        if (tid < NAG) {
+            s_sc[tid] = qs;
+            s_Sq[tid] = nsq;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            double v[EVT_MAX_NK];
+            long long q[NAG];
+            for (int ag = 0; ag < NAG; ag++) q[ag] = s_Sq[ag];
+            decode_vals(q, s_sc, A.loss, NK, v);
+            for (int k = 0; k < NK; k++) s_S[k] = v[k];
+        }
+        __syncthreads();
+    }
     double S[EVT_MAX_NK];
     for (int k = 0; k < NK; k++) S[k] = s_S[k];
     if (tid == 0) A.tree.w[n - 1] = (float)S[NK - 1];
@@ -520,15 +591,19 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
         if (tid == 0) A.status[n] = ST_LEAF;
         return;
     }
-    double bg = -INFINITY;
-    int bj = NO_BIN, bb = NO_BIN;
     // a thread takes the groups tid, tid + 256, ... (more than 1024 sampled features): ascending feature positions, so
-    // only a strictly larger gain replaces an earlier one
-    for (int g = tid; g < ngroups; g += 256) {
-        const ScanBest r = A.sbest[(int64_t)blockIdx.x * ngroups + g];
-        if (r.gain > bg) { bg = r.gain; bj = r.jp; bb = r.bin; }
+    // only a strictly larger gain replaces an earlier one.  It keeps the whole candidate: the thread whose candidate wins
+    // decides the node and writes the children's totals from its own registers - no feature table, no histogram read.
+    ScanBestQ mine = cw.q;
+    if (tid >= ngroups) {
+        mine.gain = -INFINITY; mine.jp = NO_BIN; mine.bin = NO_BIN;
     }
-    s_g[tid] = bg; s_j[tid] = bj; s_b[tid] = bb;
+    const ScanBestQ *cand = reinterpret_cast<const ScanBestQ *>(A.sbest) + (int64_t)blockIdx.x * ngroups;
+    for (int g = tid + 256; g < ngroups; g += 256) {
+        const ScanBestQ r = cand[g];
+        if (r.gain > mine.gain) mine = r;
+    }
+    s_g[tid] = mine.gain; s_j[tid] = mine.jp; s_b[tid] = mine.bin;
     __syncthreads();
     for (int o = 128; o > 0; o >>= 1) {
         if (tid < o) {
@@ -538,36 +613,23 @@ __global__ __launch_bounds__(256) void k_scan_fin(ScanArgs A, int ngroups) {
         }
         __syncthreads();
     }
-    if (tid == 0) {
-        const int bj0 = s_j[0], bb0 = s_b[0];
-        int feat = 0;
-        bool numeric = true;
-        if (bb0 != NO_BIN) {
-            feat = (int)A.js[bj0];
-            numeric = A.feattypes[feat - 1] != 0;
+    const double bg = s_g[0];
+    const int bj = s_j[0], bb = s_b[0];
+    // every sampled feature belongs to one group and every group to one thread: exactly one thread holds the winner;
+    // without any candidate the first thread turns the node into a leaf
+    const bool found = (bb != NO_BIN && bg > A.gamma);
+    const bool owner = found ? (mine.jp == bj && mine.bin != NO_BIN) : (tid == 0);
+    if (owner) {
+        const int feat = found ? (mine.feat < 0 ? -mine.feat : mine.feat) : 1;
+        scan_decide(A, n, s_S, s_dec, bg, bj, bb, feat, found ? mine.feat > 0 : true);
+        if (found) {
+            long long qL[NAG];
+#pragma unroll
+            for (int ag = 0; ag < NAG; ag++) qL[ag] = mine.qL[ag];
+            write_children<NAG>(A, n, qL, s_Sq, s_sc);
         }
-        scan_decide(A, n, s_S, s_dec, s_g[0], bj0, bb0, feat, numeric);
     }
-    __syncthreads();
-    if (!s_dec[0]) return;
-    bj = s_dec[1]; bb = s_dec[2];
-    if (tid < 64) { // wave 0; pass 1 already materialised h[n] for subtract nodes
-        const int lane = tid;
-        const int B = A.B;
-        const int f = (int)A.js[bj] - 1;
-        const bool numeric = A.feattypes[f] != 0;
-        long long qL[NAG];
-        for (int ag = 0; ag < NAG; ag++) {
-            const int64_t o = ((int64_t)bj * NAG + ag) * B;
-            long long sL = 0;
-            for (int b = lane; b < B; b += 64) {
-                const bool in = numeric ? (b + 1 <= bb) : (b + 1 == bb);
-                if (in) sL += hn[o + b];
-            }
-            qL[ag] = wave_sum_i64(sL);
-        }
-        if (lane == 0) write_children<NAG>(A, n, qL, s_Sq, s_sc);
-    }
+    if (!found) return;
     // with one block per node this block clears the children's slices, otherwise the node's other blocks have
     if (A.zero_children && gridDim.y == 1) zero_children_slices<NAG>(A, n);
 }
