@@ -412,6 +412,8 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             const int SR = U * RPW; // positions per wave iteration (<= 64)
             const int64_t itstride = (int64_t)nwaves * SR;
             const uint32_t *isp = A.is + seg;
+            // a record's address: row id times record size as one 32 x 32 -> 64 bit multiply-add, plus the piece's byte offset
+            const uint32_t rs32 = (uint32_t)A.RS, pofs = (uint32_t)(tb + subl * PB);
             const int64_t lastp = nend - 1;          // >= start
             int64_t pw = start + (int64_t)wave * SR; // first position of this wave's iteration
             // lane j of a DPP row fetches for row group j the row its DPP row belongs to (a record wider than a DPP row is
@@ -436,13 +438,16 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
 #define EVT_H16_PRO(u_)                                                                                               \
     if constexpr ((u_) < U) {                                                                                         \
         const uint32_t row = grp_bcast<(u_) < U ? (u_) : 0>(idc);                                               \
-        v[(u_) < U ? (u_) : 0] = load_piece<PB, NT>(A.xrm + (size_t)row * A.RS + tb + subl * PB);           \
+        v[(u_) < U ? (u_) : 0] = load_piece<PB, NT>(A.xrm + ((size_t)row * rs32 + pofs));                   \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
             EVT_H16_PRO(0) EVT_H16_PRO(1) EVT_H16_PRO(2) EVT_H16_PRO(3) EVT_H16_PRO(4) EVT_H16_PRO(5) EVT_H16_PRO(6) EVT_H16_PRO(7)
             EVT_H16_PRO(8) EVT_H16_PRO(9) EVT_H16_PRO(10) EVT_H16_PRO(11) EVT_H16_PRO(12) EVT_H16_PRO(13) EVT_H16_PRO(14) EVT_H16_PRO(15)
 #undef EVT_H16_PRO
             for (; pw < nend; pw += itstride) {
+                // positions of this lane's rows left in the run, as a 32-bit number: group u is inside while u * RPW < rem
+                const int64_t rem64 = nend - pw - rloc;
+                const int rem = rem64 > 0x7fffffff ? 0x7fffffff : (int)rem64;
                 // next iteration's gradient words and the row ids of the one after: ahead of the records in issue order
 #pragma unroll
                 for (int a = 0; a < NA; a++) gn[a] = evt_load_gq<PACK>(A.gq, A.N, a, idn);
@@ -462,7 +467,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
                 const uint32_t ghi = grp_bcast<ui>((uint32_t)(gc[a] >> 32));                                    \
                 gg[a] = ((unsigned long long)ghi << 32) | glo;                                                         \
             }                                                                                                         \
-            if (lane_on && (pw + (u_) * RPW + rloc < nend)) {                                                          \
+            if (lane_on && ((u_) * RPW < rem)) {                                                                       \
                 const uint32_t wds[2] = {v[ui].x, v[ui].y};                                                            \
                 _Pragma("unroll") for (int t = 0; t < PU; t++) {                                                       \
                     if (FULL || (vmask & (1u << t))) {                                                                \
@@ -474,7 +479,7 @@ __global__ __launch_bounds__(1024) void k_hist_build16(HistArgs A) {
             }                                                                                                         \
         }                                                                                                             \
         const uint32_t row = grp_bcast<ui>(idn);                                                                \
-        v[ui] = load_piece<PB, NT>(A.xrm + (size_t)row * A.RS + tb + subl * PB);                          \
+        v[ui] = load_piece<PB, NT>(A.xrm + ((size_t)row * rs32 + pofs));                                  \
         __builtin_amdgcn_sched_barrier(0);                                                                            \
     }
                 EVT_H16_STEP(0) EVT_H16_STEP(1) EVT_H16_STEP(2) EVT_H16_STEP(3) EVT_H16_STEP(4) EVT_H16_STEP(5) EVT_H16_STEP(6) EVT_H16_STEP(7)
