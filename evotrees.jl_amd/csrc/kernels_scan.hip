@@ -82,11 +82,32 @@ __device__ __forceinline__ long long wave_sum_i64(long long x) {
     return x;
 }
 
-__device__ __forceinline__ double shfl_xor_f64(double v, int o) {
-    long long b = __double_as_longlong(v);
-    int lo = __shfl_xor((int)(b & 0xffffffffll), o), hi = __shfl_xor((int)(b >> 32), o);
-    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+// Arg-max over the 64 lanes of a wavefront: highest gain, of equal gains the lowest bin; every lane gets the result.
+// Same data movement as the prefix scan above (row shifts, then row broadcasts; a lane without a source combines with
+// the identity), so the reduction ends in lane 63 - VALU moves only, where a butterfly of cross-lane shuffles goes
+// through the LDS crossbar eighteen times, each a dependent round trip.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ void argmax_step(double &g, int &b) {
+    const long long gb = __double_as_longlong(g);
+    const int olo = __builtin_amdgcn_update_dpp(0, (int)(gb & 0xffffffffll), CTRL, ROW_MASK, 0xf, false);
+    const int ohi = __builtin_amdgcn_update_dpp((int)0xFFF00000, (int)(gb >> 32), CTRL, ROW_MASK, 0xf, false); // -inf
+    const int ob = __builtin_amdgcn_update_dpp(NO_BIN, b, CTRL, ROW_MASK, 0xf, false);
+    const double og = __longlong_as_double(((long long)ohi << 32) | (unsigned int)olo);
+    if (og > g || (og == g && ob < b)) { g = og; b = ob; }
 }
+__device__ __forceinline__ void wave_argmax(double &g, int &b) {
+    argmax_step<0x111, 0xf>(g, b); // row_shr:1
+    argmax_step<0x112, 0xf>(g, b); // row_shr:2
+    argmax_step<0x114, 0xf>(g, b); // row_shr:4
+    argmax_step<0x118, 0xf>(g, b); // row_shr:8
+    argmax_step<0x142, 0xa>(g, b); // row_bcast:15 into rows 1 and 3
+    argmax_step<0x143, 0xc>(g, b); // row_bcast:31 into rows 2 and 3
+    const long long gb = __double_as_longlong(g);
+    const int lo = __builtin_amdgcn_readlane((int)(gb & 0xffffffffll), 63), hi = __builtin_amdgcn_readlane((int)(gb >> 32), 63);
+    g = __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+    b = __builtin_amdgcn_readlane(b, 63);
+}
+
 
 // ---- Float64 gain algebra, expression order as in the reference ------------------------------
 __device__ __forceinline__ double term_gh(double g, double h, double w, double lambda, double L2) {
@@ -432,12 +453,7 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
             }
         }
         if (!A.oblivious) {
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const double og = shfl_xor_f64(lg, o);
-                const int ob = __shfl_xor(lb, o);
-                if (og > lg || (og == lg && ob < lb)) { lg = og; lb = ob; }
-            }
+            wave_argmax(lg, lb);
             if (lg > wbest) { wbest = lg; wjp = jp; wbin = lb; }
             if constexpr (!FUSED) {
                 // the lane that holds the winning bin hands its left totals to the whole wave
@@ -874,12 +890,7 @@ __global__ __launch_bounds__(256) void k_scan_mc(ScanArgs A) {
             }
         }
         if (!A.oblivious) {
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const double og = shfl_xor_f64(lg, o);
-                const int ob = __shfl_xor(lb, o);
-                if (og > lg || (og == lg && ob < lb)) { lg = og; lb = ob; }
-            }
+            wave_argmax(lg, lb);
             if (lg > wbest) { wbest = lg; wjp = jp; wbin = lb; }
         }
     }
