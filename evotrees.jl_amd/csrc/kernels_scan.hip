@@ -337,9 +337,15 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
     }
     const bool numeric = A.feattypes[f] != 0;
     const int constraint = A.mono[f];
-    const int tq = tid < NAG ? tid : 0;
-    const double qs = A.qscale[tq];
-    const long long nsq = A.node_sum[(int64_t)n * NAG + tq]; // not yet written at level 1, and not used there
+    // node totals and decode scales: the same few words for every thread of the block (scalar loads), so that below the
+    // root no thread waits at a barrier for another to decode them
+    long long nsq[NAG];
+    double sc[NAG];
+#pragma unroll
+    for (int ag = 0; ag < NAG; ag++) {
+        sc[ag] = A.qscale[ag];
+        nsq[ag] = A.node_sum[(int64_t)n * NAG + ag]; // not yet written at level 1, and not used there
+    }
 
 #pragma unroll
     for (int ag = 0; ag < NAG; ag++) {
@@ -352,26 +358,24 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
         }
     }
 
-    // node totals -> Float64 statistics (as node_totals, with the values requested above)
-    if (A.level == 1) {
-        node_totals<NAG>(A, n, hn, blockIdx.y == 0, s_Sq, s_S, s_sc);
-    } else {
-        if (tid < NAG) {
-            s_sc[tid] = qs;
-            s_Sq[tid] = nsq;
-        }
-        __syncthreads();
-        if (tid == 0) {
-            double v[NK];
-            long long q[NAG];
-            for (int ag = 0; ag < NAG; ag++) q[ag] = s_Sq[ag];
-            decode_vals(q, s_sc, A.loss, NK, v);
-            for (int k = 0; k < NK; k++) s_S[k] = v[k];
-        }
-        __syncthreads();
-    }
+    // node totals -> Float64 statistics
     double S[NK];
-    for (int k = 0; k < NK; k++) S[k] = s_S[k];
+    if (A.level == 1) { // the root's totals are the bin sums of its first sampled feature
+        node_totals<NAG>(A, n, hn, blockIdx.y == 0, s_Sq, s_S, s_sc);
+        for (int k = 0; k < NK; k++) S[k] = s_S[k];
+#pragma unroll
+        for (int ag = 0; ag < NAG; ag++) sc[ag] = s_sc[ag];
+    } else {
+        decode_vals(nsq, sc, A.loss, NK, S);
+        if (FUSED && tid == 0) { // the block's last step reads them from shared memory, behind the barriers below
+#pragma unroll
+            for (int ag = 0; ag < NAG; ag++) {
+                s_sc[ag] = sc[ag];
+                s_Sq[ag] = nsq[ag];
+            }
+            for (int k = 0; k < NK; k++) s_S[k] = S[k];
+        }
+    }
 
     double gain_p = 0.0;
     for (int k = 0; k < K; k++) gain_p += node_gain_k(A.loss, S[k], S[K + k], S[2 * K], A.lambda, A.L2);
@@ -421,7 +425,7 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void k_scan(ScanArgs A) {
                         q[ag] = numeric ? pre[ag][t] : (pre[ag][t] - prev); // _acc_left!: accumulate vs single bin
                     }
                     double SL[NK];
-                    decode_vals(q, s_sc, A.loss, NK, SL);
+                    decode_vals(q, sc, A.loss, NK, SL);
                     const double w_l = SL[NK - 1];
                     const double w_r = w_p - w_l;
                     if (w_l > A.min_weight && w_r > A.min_weight) {
